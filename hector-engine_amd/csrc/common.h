@@ -1,0 +1,94 @@
+// Shared helpers of the gfx950 kernel library: storage types, conversions,
+// wave/block reductions and the error channel of the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+// dtype codes used across the C ABI
+#define HE_F32 0
+#define HE_BF16 1
+
+// Tokens per page of the key/value cache. The pools are laid out
+// [page][kv_head][PAGE_TOKENS][head_dim].
+#define HE_PAGE_TOKENS 64
+#define HE_PAGE_SHIFT 6
+
+#define HE_WAVE 64
+
+struct bf16_t {
+  uint16_t v;
+};
+
+__device__ __forceinline__ float bf16_bits_to_float(uint16_t b) {
+  return __uint_as_float(((uint32_t)b) << 16);
+}
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float to_float(float x) { return x; }
+__device__ __forceinline__ float to_float(bf16_t x) { return bf16_bits_to_float(x.v); }
+
+template <typename T>
+__device__ __forceinline__ T from_float(float f);
+template <>
+__device__ __forceinline__ float from_float<float>(float f) {
+  return f;
+}
+template <>
+__device__ __forceinline__ bf16_t from_float<bf16_t>(float f) {
+  bf16_t r;
+  r.v = float_to_bf16_bits(f);
+  return r;
+}
+
+// A small parameter vector (norm gain, bias) may be stored in either dtype
+// independently of the activation dtype.
+__device__ __forceinline__ float load_param(const void* p, int64_t i, int dtype) {
+  return dtype == HE_BF16 ? bf16_bits_to_float(((const uint16_t*)p)[i]) : ((const float*)p)[i];
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = HE_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, HE_WAVE);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = HE_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, HE_WAVE));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; every thread gets the result.
+// `scratch` needs 16 floats of shared memory. The order of the additions is
+// fixed by the block shape alone.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x & (HE_WAVE - 1);
+  const int wave = threadIdx.x >> 6;
+  const int nwaves = (blockDim.x + HE_WAVE - 1) >> 6;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < nwaves; ++w) total += scratch[w];
+  return total;
+}
+
+// ---- error channel -------------------------------------------------------
+void he_set_error(const char* fmt, ...);
+int he_check_launch(const char* what);
+
+#define HE_REQUIRE(cond, ...)      \
+  do {                             \
+    if (!(cond)) {                 \
+      he_set_error(__VA_ARGS__);   \
+      return -1;                   \
+    }                              \
+  } while (0)

@@ -1,0 +1,125 @@
+// Row-wise kernels without reductions: embedding gather into the fp32 residual
+// stream, row gather, gated activation (SiLU(gate) * up) and the materialising
+// residual add.
+#include "common.h"
+#include "hector_kernels.h"
+
+// out[t, :] = table[ids[t], :] as fp32; an id outside [0, V) gives a zero row
+// (reference: kernels/linear.cu:36-69).
+template <typename T>
+__global__ void embedding_kernel(float* __restrict__ out, const T* __restrict__ table,
+                                 const int32_t* __restrict__ ids, int D, int V) {
+  const int64_t t = blockIdx.x;
+  const int id = ids[t];
+  float* o = out + t * (int64_t)D;
+  if (id < 0 || id >= V) {
+    for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = 0.f;
+    return;
+  }
+  const T* row = table + (int64_t)id * D;
+  for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = to_float(row[i]);
+}
+
+extern "C" int he_embedding(void* out_f32, const void* table, const void* ids, int rows, int D,
+                            int V, int table_dtype, void* stream) {
+  HE_REQUIRE(rows >= 0 && D > 0 && V > 0, "he_embedding: bad sizes rows=%d D=%d V=%d", rows, D, V);
+  if (rows == 0) return 0;
+  const int threads = D >= 1024 ? 256 : (D >= 256 ? 128 : 64);
+  hipStream_t s = (hipStream_t)stream;
+  if (table_dtype == HE_BF16)
+    embedding_kernel<bf16_t><<<rows, threads, 0, s>>>((float*)out_f32, (const bf16_t*)table,
+                                                      (const int32_t*)ids, D, V);
+  else if (table_dtype == HE_F32)
+    embedding_kernel<float><<<rows, threads, 0, s>>>((float*)out_f32, (const float*)table,
+                                                     (const int32_t*)ids, D, V);
+  else
+    HE_REQUIRE(false, "he_embedding: unknown dtype %d", table_dtype);
+  return he_check_launch("he_embedding");
+}
+
+// out[r, :] = src[rows[r], :]; a negative row index gives a zero row.
+__global__ void gather_rows_f32_kernel(float* __restrict__ out, const float* __restrict__ src,
+                                       const int32_t* __restrict__ rows, int D, int n_src) {
+  const int64_t r = blockIdx.x;
+  const int idx = rows[r];
+  float* o = out + r * (int64_t)D;
+  if (idx < 0 || idx >= n_src) {
+    for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = 0.f;
+    return;
+  }
+  const float* in = src + (int64_t)idx * D;
+  for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = in[i];
+}
+
+extern "C" int he_gather_rows_f32(void* out, const void* src, const void* rows, int n_out, int D,
+                                  int n_src, void* stream) {
+  HE_REQUIRE(n_out >= 0 && D > 0 && n_src >= 0, "he_gather_rows_f32: bad sizes");
+  if (n_out == 0) return 0;
+  gather_rows_f32_kernel<<<n_out, 256, 0, (hipStream_t)stream>>>(
+      (float*)out, (const float*)src, (const int32_t*)rows, D, n_src);
+  return he_check_launch("he_gather_rows_f32");
+}
+
+// resid[r, :] += delta[r, :], the residual sum in fp32.
+template <typename T>
+__global__ void residual_add_kernel(float* __restrict__ resid, const T* __restrict__ delta,
+                                    int64_t n) {
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) resid[i] += to_float(delta[i]);
+}
+
+extern "C" int he_residual_add(void* resid_f32, const void* delta, int64_t n, int delta_dtype,
+                               void* stream) {
+  HE_REQUIRE(n >= 0, "he_residual_add: bad size");
+  if (n == 0) return 0;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 65535) blocks = 65535;
+  hipStream_t s = (hipStream_t)stream;
+  if (delta_dtype == HE_BF16)
+    residual_add_kernel<bf16_t><<<(int)blocks, 256, 0, s>>>((float*)resid_f32,
+                                                            (const bf16_t*)delta, n);
+  else if (delta_dtype == HE_F32)
+    residual_add_kernel<float><<<(int)blocks, 256, 0, s>>>((float*)resid_f32, (const float*)delta,
+                                                           n);
+  else
+    HE_REQUIRE(false, "he_residual_add: unknown dtype %d", delta_dtype);
+  return he_check_launch("he_residual_add");
+}
+
+// out[r, i] = silu(x[r, i]) * x[r, I + i] with x = [rows, 2I] (gate then up),
+// silu(z) = z / (1 + exp(-z)) in fp32 (reference: kernels/activations.cu:19-21,183-198).
+template <typename T>
+__global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ x, int64_t rows,
+                                int I) {
+  const int64_t n = rows * (int64_t)I;
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) {
+    const int64_t r = i / I;
+    const int c = (int)(i - r * I);
+    const float g = to_float(x[r * 2 * (int64_t)I + c]);
+    const float u = to_float(x[r * 2 * (int64_t)I + I + c]);
+    const float y = g / (1.f + expf(-g)) * u;
+    out[i] = from_float<T>(y);
+  }
+}
+
+extern "C" int he_silu_mul(void* out, const void* gate_up, int rows, int I, int dtype,
+                           void* stream) {
+  HE_REQUIRE(rows >= 0 && I > 0, "he_silu_mul: bad sizes rows=%d I=%d", rows, I);
+  if (rows == 0) return 0;
+  const int64_t n = (int64_t)rows * I;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 65535 * 4) blocks = 65535 * 4;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == HE_BF16)
+    silu_mul_kernel<bf16_t><<<(int)blocks, 256, 0, s>>>((bf16_t*)out, (const bf16_t*)gate_up, rows,
+                                                        I);
+  else if (dtype == HE_F32)
+    silu_mul_kernel<float><<<(int)blocks, 256, 0, s>>>((float*)out, (const float*)gate_up, rows,
+                                                       I);
+  else
+    HE_REQUIRE(false, "he_silu_mul: unknown dtype %d", dtype);
+  return he_check_launch("he_silu_mul");
+}

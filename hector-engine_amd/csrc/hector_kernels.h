@@ -1,0 +1,84 @@
+// C ABI of the gfx950 kernel library. Every function launches on the given HIP
+// stream and returns 0, or non-zero after recording a message for
+// he_last_error(). Pointers are device pointers unless named host_*. Shapes
+// are validated on the host before any launch. dtype codes: 0 = float32,
+// 1 = bfloat16.
+#pragma once
+#include <stdint.h>
+
+#define HE_ABI_VERSION 3
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* he_last_error(void);
+int he_abi_version(void);
+
+// ---- row-wise ------------------------------------------------------------
+int he_embedding(void* out_f32, const void* table, const void* ids, int rows, int D, int V,
+                 int table_dtype, void* stream);
+int he_gather_rows_f32(void* out, const void* src, const void* rows, int n_out, int D, int n_src,
+                       void* stream);
+int he_residual_add(void* resid_f32, const void* delta, int64_t n, int delta_dtype, void* stream);
+int he_silu_mul(void* out, const void* gate_up, int rows, int I, int dtype, void* stream);
+
+// ---- norms ---------------------------------------------------------------
+// resid (fp32, in place) += delta (may be null); out (may be null) = rmsnorm(resid) * weight
+int he_add_rmsnorm(void* resid_f32, const void* delta, const void* weight, void* out, int rows,
+                   int D, float eps, int act_dtype, int w_dtype, void* stream);
+int he_rmsnorm_rows(void* out, const void* x, const void* weight, int rows, int D,
+                    int64_t x_stride, int64_t out_stride, float eps, int dtype, int w_dtype,
+                    void* stream);
+
+// ---- matrix products: C[M,N] = A[M,K] * W[N,K]^T (+ bias) -------------------
+int he_gemm_plain(void* C, const void* A, const void* W, const void* bias, int M, int N, int K,
+                  int64_t lda, int64_t ldw, int64_t ldc, int in_dtype, int out_dtype,
+                  int bias_dtype, void* stream);
+// bf16 MFMA product for M <= HE_SKINNY_MAX_M rows: every weight element is read once.
+#define HE_SKINNY_MAX_M 64
+int he_gemm_skinny_bf16(void* C, const void* A, const void* W, const void* bias, int M, int N,
+                        int K, int out_dtype, int bias_dtype, void* workspace_f32,
+                        int64_t workspace_floats, void* stream);
+int64_t he_gemm_skinny_workspace_floats(int M, int N, int K);
+
+// ---- position encoding + cache write -------------------------------------
+int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const void* q_in, const void* k_in,
+                      const void* v_in, int64_t in_stride, const void* q_bias, const void* k_bias,
+                      const void* v_bias, int bias_dtype, const void* positions,
+                      const void* row_seq, const void* seq_slot, const void* page_table,
+                      int max_blocks, int num_pages, const void* inv_freq, int rotary_dim, int rows,
+                      int H, int KVH, int hd, int dtype, void* stream);
+
+// ---- attention over the paged cache ----------------------------------------
+int he_attention_plain(void* out, const void* q, const void* kpool, const void* vpool,
+                       const void* positions, const void* row_seq, const void* seq_slot,
+                       const void* page_table, int max_blocks, int num_pages, int rows, int H,
+                       int KVH, int hd, int window, float scale, int dtype, void* stream);
+// bf16, one query row per sequence (decode): split over the keys, then merged.
+int he_attention_decode_bf16(void* out, const void* q, const void* kpool, const void* vpool,
+                             const void* positions, const void* row_seq, const void* seq_slot,
+                             const void* page_table, int max_blocks, int num_pages, int rows,
+                             int H, int KVH, int hd, int window, float scale, int max_keys,
+                             void* workspace_f32, int64_t workspace_floats, void* stream);
+int64_t he_attention_decode_workspace_floats(int rows, int H, int hd, int max_keys);
+// bf16, prompt steps: tiles of queries of one sequence against its cache rows.
+int he_attention_prefill_bf16(void* out, const void* q, const void* kpool, const void* vpool,
+                              const void* cu_seqlens, const void* seq_slot, const void* seq_start,
+                              const void* page_table, int max_blocks, int num_pages, int num_seqs,
+                              int max_q_len, int H, int KVH, int hd, int window, float scale,
+                              void* stream);
+
+// ---- sampling ------------------------------------------------------------
+int he_argmax_rows(void* out_i32, const void* logits_f32, int rows, int V, int64_t row_stride,
+                   void* stream);
+int he_apply_penalties(void* logits_f32, int rows, int V, int64_t row_stride, const void* ids,
+                       const void* counts, const void* offsets, float rep, float freq, float pres,
+                       void* stream);
+int he_sample_rows(void* out_i32, const void* logits_f32, int rows, int V, int64_t row_stride,
+                   const void* uniforms_u32, float temperature, int top_k, float top_p,
+                   void* stream);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,103 @@
+// RMS normalisation. The residual stream is fp32 in both precisions; the fused
+// kernel adds the pending branch output to it and normalises the sum in one
+// pass over the row:
+//   r = resid + delta          (fp32, stored back as the new residual)
+//   y = r * (1/sqrt(mean(r^2) + eps)) * w
+// Reference formulas: kernels/normalization.cu:36-63 (norm) and
+// kernels/fused_add_rmsnorm.cu:47-81 (add + norm, two outputs).
+#include "common.h"
+#include "hector_kernels.h"
+
+template <typename TD, typename TO>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
+                                   const void* __restrict__ w, int w_dtype, TO* __restrict__ out,
+                                   int D, float eps) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  float* r = resid + row * (int64_t)D;
+  float ss = 0.f;
+  if (delta != nullptr) {
+    const TD* d = delta + row * (int64_t)D;
+    for (int i = threadIdx.x; i < D; i += blockDim.x) {
+      const float v = r[i] + to_float(d[i]);
+      r[i] = v;
+      ss += v * v;
+    }
+  } else {
+    for (int i = threadIdx.x; i < D; i += blockDim.x) {
+      const float v = r[i];
+      ss += v * v;
+    }
+  }
+  const float total = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(total / (float)D + eps);
+  if (out == nullptr) return;
+  TO* o = out + row * (int64_t)D;
+  // each thread re-reads exactly the elements it wrote above
+  for (int i = threadIdx.x; i < D; i += blockDim.x) {
+    o[i] = from_float<TO>(r[i] * inv * load_param(w, i, w_dtype));
+  }
+}
+
+static int norm_threads(int D) { return D >= 2048 ? 512 : (D >= 512 ? 256 : (D >= 128 ? 128 : 64)); }
+
+extern "C" int he_add_rmsnorm(void* resid_f32, const void* delta, const void* weight, void* out,
+                              int rows, int D, float eps, int act_dtype, int w_dtype,
+                              void* stream) {
+  HE_REQUIRE(rows >= 0 && D > 0, "he_add_rmsnorm: bad sizes rows=%d D=%d", rows, D);
+  HE_REQUIRE(w_dtype == HE_F32 || w_dtype == HE_BF16, "he_add_rmsnorm: bad weight dtype");
+  if (rows == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int threads = norm_threads(D);
+  if (act_dtype == HE_BF16)
+    add_rmsnorm_kernel<bf16_t, bf16_t><<<rows, threads, 0, s>>>(
+        (float*)resid_f32, (const bf16_t*)delta, weight, w_dtype, (bf16_t*)out, D, eps);
+  else if (act_dtype == HE_F32)
+    add_rmsnorm_kernel<float, float><<<rows, threads, 0, s>>>(
+        (float*)resid_f32, (const float*)delta, weight, w_dtype, (float*)out, D, eps);
+  else
+    HE_REQUIRE(false, "he_add_rmsnorm: unknown dtype %d", act_dtype);
+  return he_check_launch("he_add_rmsnorm");
+}
+
+// Plain row-wise RMS norm of an activation tensor with a row stride (for
+// normalising slices such as per-head vectors): x viewed as [rows, D].
+template <typename T>
+__global__ void rmsnorm_rows_kernel(T* __restrict__ out, const T* __restrict__ x,
+                                    const void* __restrict__ w, int w_dtype, int D,
+                                    int64_t x_stride, int64_t out_stride, float eps) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  const T* xi = x + row * x_stride;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < D; i += blockDim.x) {
+    const float v = to_float(xi[i]);
+    ss += v * v;
+  }
+  const float total = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(total / (float)D + eps);
+  T* o = out + row * out_stride;
+  for (int i = threadIdx.x; i < D; i += blockDim.x) {
+    const float g = w ? load_param(w, i, w_dtype) : 1.f;
+    o[i] = from_float<T>(to_float(xi[i]) * inv * g);
+  }
+}
+
+extern "C" int he_rmsnorm_rows(void* out, const void* x, const void* weight, int rows, int D,
+                               int64_t x_stride, int64_t out_stride, float eps, int dtype,
+                               int w_dtype, void* stream) {
+  HE_REQUIRE(rows >= 0 && D > 0 && x_stride >= D && out_stride >= D,
+             "he_rmsnorm_rows: bad sizes rows=%d D=%d", rows, D);
+  if (rows == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int threads = norm_threads(D);
+  if (dtype == HE_BF16)
+    rmsnorm_rows_kernel<bf16_t><<<rows, threads, 0, s>>>((bf16_t*)out, (const bf16_t*)x, weight,
+                                                         w_dtype, D, x_stride, out_stride, eps);
+  else if (dtype == HE_F32)
+    rmsnorm_rows_kernel<float><<<rows, threads, 0, s>>>((float*)out, (const float*)x, weight,
+                                                        w_dtype, D, x_stride, out_stride, eps);
+  else
+    HE_REQUIRE(false, "he_rmsnorm_rows: unknown dtype %d", dtype);
+  return he_check_launch("he_rmsnorm_rows");
+}

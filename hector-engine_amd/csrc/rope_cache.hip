@@ -1,0 +1,147 @@
+// One pass over the projected q/k/v rows of a step: add the projection bias,
+// rotate q and k by each row's own position, write q out densely and scatter
+// k and v into the paged cache at (slot, position). It replaces the reference's
+// add_bias, rope and kv_cache_update launches (kernels/elementwise.cu:307-323,
+// kernels/attention.cu:516-558, kernels/attention.cu:1067-1097).
+//
+// Rotation (half-split pairing): for i < r/2, a = pos * inv_freq[i],
+//   y[i]       = x[i] * cos a - x[i + r/2] * sin a
+//   y[i + r/2] = x[i] * sin a + x[i + r/2] * cos a
+// and dims >= r pass through. All of it in fp32.
+#include "common.h"
+#include "hector_kernels.h"
+
+#define ROPE_MAX_HALF 256
+
+template <typename T>
+__global__ void qkv_rope_cache_kernel(
+    T* __restrict__ q_out, T* __restrict__ kpool, T* __restrict__ vpool,
+    const T* __restrict__ q_in, const T* __restrict__ k_in, const T* __restrict__ v_in,
+    int64_t in_stride, const void* __restrict__ q_bias, const void* __restrict__ k_bias,
+    const void* __restrict__ v_bias, int bias_dtype, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ row_seq, const int32_t* __restrict__ seq_slot,
+    const int32_t* __restrict__ page_table, int max_blocks, int num_pages,
+    const float* __restrict__ inv_freq, int rotary_dim, int H, int KVH, int hd) {
+  __shared__ float cs[2][ROPE_MAX_HALF];
+  const int64_t row = blockIdx.x;
+  const int seq = row_seq[row];
+  if (seq < 0) return;  // padding row
+  const int pos = positions[row];
+  const int half = rotary_dim >> 1;
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    const float a = (float)pos * inv_freq[i];
+    float sn, c;
+    sincosf(a, &sn, &c);
+    cs[0][i] = c;
+    cs[1][i] = sn;
+  }
+  __syncthreads();
+
+  // ---- q: rotate and store densely
+  {
+    const T* in = q_in + row * in_stride;
+    T* out = q_out + row * (int64_t)H * hd;
+    const int per_head = half + (hd - rotary_dim);
+    for (int it = threadIdx.x; it < H * per_head; it += blockDim.x) {
+      const int h = it / per_head;
+      const int j = it - h * per_head;
+      const int base = h * hd;
+      if (j < half) {
+        float x0 = to_float(in[base + j]);
+        float x1 = to_float(in[base + j + half]);
+        if (q_bias) {
+          x0 += load_param(q_bias, base + j, bias_dtype);
+          x1 += load_param(q_bias, base + j + half, bias_dtype);
+        }
+        const float c = cs[0][j], sn = cs[1][j];
+        out[base + j] = from_float<T>(x0 * c - x1 * sn);
+        out[base + j + half] = from_float<T>(x0 * sn + x1 * c);
+      } else {
+        const int d = rotary_dim + (j - half);
+        float x = to_float(in[base + d]);
+        if (q_bias) x += load_param(q_bias, base + d, bias_dtype);
+        out[base + d] = from_float<T>(x);
+      }
+    }
+  }
+  if (k_in == nullptr) return;  // this layer reads another layer's cache
+
+  const int slot = seq_slot[seq];
+  const int page = page_table[(int64_t)slot * max_blocks + (pos >> HE_PAGE_SHIFT)];
+  if (page < 0 || page >= num_pages) return;  // never for a batch the host has admitted
+  const int off = pos & (HE_PAGE_TOKENS - 1);
+  // ---- k: rotate and scatter
+  {
+    const T* in = k_in + row * in_stride;
+    const int per_head = half + (hd - rotary_dim);
+    for (int it = threadIdx.x; it < KVH * per_head; it += blockDim.x) {
+      const int h = it / per_head;
+      const int j = it - h * per_head;
+      const int base = h * hd;
+      T* out = kpool + (((int64_t)page * KVH + h) * HE_PAGE_TOKENS + off) * hd;
+      if (j < half) {
+        float x0 = to_float(in[base + j]);
+        float x1 = to_float(in[base + j + half]);
+        if (k_bias) {
+          x0 += load_param(k_bias, base + j, bias_dtype);
+          x1 += load_param(k_bias, base + j + half, bias_dtype);
+        }
+        const float c = cs[0][j], sn = cs[1][j];
+        out[j] = from_float<T>(x0 * c - x1 * sn);
+        out[j + half] = from_float<T>(x0 * sn + x1 * c);
+      } else {
+        const int d = rotary_dim + (j - half);
+        float x = to_float(in[base + d]);
+        if (k_bias) x += load_param(k_bias, base + d, bias_dtype);
+        out[d] = from_float<T>(x);
+      }
+    }
+  }
+  // ---- v: bias and scatter
+  {
+    const T* in = v_in + row * in_stride;
+    for (int it = threadIdx.x; it < KVH * hd; it += blockDim.x) {
+      const int h = it / hd;
+      const int d = it - h * hd;
+      float x = to_float(in[it]);
+      if (v_bias) x += load_param(v_bias, it, bias_dtype);
+      vpool[(((int64_t)page * KVH + h) * HE_PAGE_TOKENS + off) * hd + d] = from_float<T>(x);
+    }
+  }
+}
+
+extern "C" int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const void* q_in,
+                                 const void* k_in, const void* v_in, int64_t in_stride,
+                                 const void* q_bias, const void* k_bias, const void* v_bias,
+                                 int bias_dtype, const void* positions, const void* row_seq,
+                                 const void* seq_slot, const void* page_table, int max_blocks,
+                                 int num_pages, const void* inv_freq, int rotary_dim, int rows,
+                                 int H, int KVH, int hd, int dtype, void* stream) {
+  HE_REQUIRE(rows >= 0 && H > 0 && KVH >= 0 && hd > 0, "he_qkv_rope_cache: bad sizes");
+  HE_REQUIRE(rotary_dim >= 0 && rotary_dim <= hd && (rotary_dim & 1) == 0,
+             "he_qkv_rope_cache: rotary_dim %d must be even and at most head_dim %d", rotary_dim,
+             hd);
+  HE_REQUIRE(rotary_dim / 2 <= ROPE_MAX_HALF, "he_qkv_rope_cache: rotary_dim %d above %d",
+             rotary_dim, 2 * ROPE_MAX_HALF);
+  HE_REQUIRE(rotary_dim == 0 || inv_freq != nullptr, "he_qkv_rope_cache: missing inv_freq");
+  HE_REQUIRE((k_in == nullptr) == (v_in == nullptr), "he_qkv_rope_cache: k and v go together");
+  HE_REQUIRE(k_in == nullptr || (kpool && vpool && page_table && max_blocks > 0 && KVH > 0),
+             "he_qkv_rope_cache: cache arguments missing");
+  if (rows == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int threads = 256;
+#define ROPE_LAUNCH(T)                                                                          \
+  qkv_rope_cache_kernel<T><<<rows, threads, 0, s>>>(                                            \
+      (T*)q_out, (T*)kpool, (T*)vpool, (const T*)q_in, (const T*)k_in, (const T*)v_in,          \
+      in_stride, q_bias, k_bias, v_bias, bias_dtype, (const int32_t*)positions,                 \
+      (const int32_t*)row_seq, (const int32_t*)seq_slot, (const int32_t*)page_table, max_blocks, \
+      num_pages, (const float*)inv_freq, rotary_dim, H, KVH, hd)
+  if (dtype == HE_BF16)
+    ROPE_LAUNCH(bf16_t);
+  else if (dtype == HE_F32)
+    ROPE_LAUNCH(float);
+  else
+    HE_REQUIRE(false, "he_qkv_rope_cache: unknown dtype %d", dtype);
+#undef ROPE_LAUNCH
+  return he_check_launch("he_qkv_rope_cache");
+}

@@ -1,0 +1,286 @@
+"""The engine: a model, its cache and the one step function.
+
+A step takes, for each sequence of a batch, its slot, its next tokens (a whole
+prompt, one token, or any run of tokens) and the places whose logits are wanted.
+It runs exactly those tokens, packed without padding, against the cache that
+earlier steps left, and returns fp32 logits at the wanted places. The reference
+runs one sequence with one position scalar (src/graph_builder.hpp:222-231,
+src/engine.cpp:138-145); packing, slots and per-row positions are this
+engine's own. One-token steps are captured once per batch-size bucket into a
+HIP graph and replayed (the reference's build-once, replay-many decode:
+src/engine.cpp:151-269).
+"""
+from __future__ import annotations
+
+import dataclasses
+import time
+
+import numpy as np
+import torch
+
+from ..cache.paged import PagedCache
+from ..cache.pages import CacheError, CacheFull  # noqa: F401
+from ..config.base import ModelConfig
+from ..kernels import lib as kernel_lib
+from ..parts.base import BuildEnv, StepContext
+from ..registry import build_model, load_config
+from ..weights.loader import load_tensors
+from ..weights.random_init import random_tensors
+from .scratch import ScratchPool
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32,
+           "fp32": torch.float32}
+
+GRAPH_MAX_BUCKET = 256
+
+
+class StepError(ValueError):
+    """A step that cannot run as asked; nothing has been changed."""
+
+
+@dataclasses.dataclass
+class StepEntry:
+    slot: int
+    tokens: list
+    want: list = dataclasses.field(default_factory=list)   # places among `tokens`
+
+
+class _Meta:
+    """Packed int32 metadata of a step: one host buffer, one copy, views on the device."""
+
+    FIELDS = ("tokens", "positions", "row_seq", "seq_slot", "cu_seqlens", "seq_start", "want_rows")
+
+    def __init__(self, rows: int, seqs: int, wants: int):
+        sizes = (rows, rows, rows, seqs, seqs + 1, seqs, max(wants, 1))
+        self.offsets = {}
+        off = 0
+        for name, n in zip(self.FIELDS, sizes):
+            self.offsets[name] = (off, n)
+            off += n
+        self.total = off
+
+    def views(self, buf):
+        return {name: buf[o:o + n] for name, (o, n) in self.offsets.items()}
+
+
+class _GraphBucket:
+    def __init__(self, size: int, device):
+        self.size = size
+        self.meta = _Meta(size, size, size)
+        self.dev = torch.zeros(self.meta.total, dtype=torch.int32, device=device)
+        self.views = self.meta.views(self.dev)
+        self.pool = ScratchPool(device)
+        self.graph: torch.cuda.CUDAGraph | None = None
+        self.logits: torch.Tensor | None = None
+        self.uses = 0
+
+
+class Engine:
+    def __init__(self, model_dir: str | None = None, *, config: ModelConfig | None = None,
+                 seed: int | None = None, dtype: str = "bfloat16", max_tokens: int = 8192,
+                 max_slots: int | None = None, max_seq_len: int | None = None,
+                 device: str = "cuda:0", fast_kernels: bool = True, use_graphs: bool = True):
+        if dtype not in _DTYPES:
+            raise ValueError(f"dtype must be one of {sorted(_DTYPES)}, got {dtype!r}")
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU: this engine runs its HIP kernels on an MI355X only")
+        kernel_lib.load()   # fails loudly when the kernel library is missing
+        self.device = torch.device(device)
+        torch.cuda.set_device(self.device)
+        self.dtype = _DTYPES[dtype]
+        if self.dtype == torch.float32:
+            # the library matrix product is not on the float32 path; make sure no
+            # reduced-precision mode could slip in through torch either
+            torch.backends.cuda.matmul.allow_tf32 = False
+        self.env = BuildEnv(self.device, self.dtype, fast_kernels)
+        if model_dir is not None:
+            self.config = load_config(model_dir)
+        elif config is not None:
+            self.config = config
+        else:
+            raise ValueError("give a model folder, or a configuration and a seed")
+        self.model = build_model(self.config, self.env)
+        specs = self.model.tensor_specs()
+        if model_dir is not None:
+            extra = {"lm_head.weight"} if getattr(self.config, "tie_word_embeddings", False) else set()
+            tensors = load_tensors(model_dir, specs, self.dtype, self.device, extra)
+        else:
+            if seed is None:
+                raise ValueError("random weights need a seed")
+            tensors = random_tensors(specs, seed, self.dtype, self.device)
+        self.model.bind(tensors)
+        del tensors
+        self.vocab_size = self.model.spec.vocab_size
+        max_seq_len = max_seq_len or self.model.spec.max_positions
+        self.cache = PagedCache(self.model.run_plans(), max_tokens=max_tokens,
+                                max_slots=max_slots or 256, max_seq_len=min(max_seq_len, max_tokens),
+                                dtype=self.dtype, device=self.device)
+        self.caches = [self.cache.layer_cache(r) for r in range(len(self.model.schedule))]
+        self.scratch = ScratchPool(self.device)
+        self.use_graphs = use_graphs
+        self._buckets: dict[int, _GraphBucket] = {}
+        self._pinned = [torch.empty(1 << 16, dtype=torch.int32).pin_memory() for _ in range(4)]
+        self._pinned_events: list[torch.cuda.Event | None] = [None] * 4
+        self._pinned_next = 0
+        self.stats = {"steps": 0, "graph_replays": 0, "graph_captures": 0, "eager_steps": 0}
+
+    # -- slots ----------------------------------------------------------------
+    def acquire(self) -> int:
+        return self.cache.acquire()
+
+    def release(self, slot: int) -> None:
+        self.cache.release(slot)
+
+    def length(self, slot: int) -> int:
+        return self.cache.length(slot)
+
+    @property
+    def max_seq_len(self) -> int:
+        return self.cache.max_seq_len
+
+    # -- the step function -------------------------------------------------------
+    def step(self, entries: list[StepEntry]) -> torch.Tensor | None:
+        """Runs the entries' tokens as one batch. Returns fp32 logits
+        [number of wanted places, vocab] in the order of the entries and of their
+        `want`, or None if nothing is wanted. The tensor is valid until the next step."""
+        if not entries:
+            raise StepError("a step needs at least one entry")
+        seen = set()
+        growth = []
+        for e in entries:
+            if e.slot in seen:
+                raise StepError(f"slot {e.slot} appears twice in one step")
+            seen.add(e.slot)
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"slot {e.slot}: an entry needs at least one token")
+            start = self.cache.length(e.slot)
+            if start + n > self.cache.max_seq_len:
+                raise StepError(f"slot {e.slot}: {start} cached + {n} new tokens exceed the "
+                                f"longest sequence {self.cache.max_seq_len}")
+            toks = np.asarray(e.tokens, dtype=np.int64)
+            if toks.ndim != 1 or toks.min() < 0 or toks.max() >= self.vocab_size:
+                raise StepError(f"slot {e.slot}: token ids must lie in [0, {self.vocab_size})")
+            for w in e.want:
+                if not 0 <= int(w) < n:
+                    raise StepError(f"slot {e.slot}: wanted place {w} outside its {n} tokens")
+            growth.append((e.slot, start + n))
+        self.cache.reserve(growth)          # all pages or an error, before anything runs
+        all_single = all(len(e.tokens) == 1 for e in entries)
+        every_wanted = all(list(e.want) == [0] for e in entries)
+        self.stats["steps"] += 1
+        if self.use_graphs and all_single and every_wanted and len(entries) <= GRAPH_MAX_BUCKET:
+            logits = self._graph_step(entries)
+        else:
+            logits = self._eager_step(entries, all_single)
+        self.cache.commit(growth)
+        return logits
+
+    # -- packing ---------------------------------------------------------------
+    def _pack(self, entries, meta: _Meta, rows_padded: int, seqs_padded: int):
+        """Fills a pinned host buffer with the step's metadata; returns it and the
+        number of wanted rows."""
+        if meta.total > self._pinned[0].numel():
+            need = 1 << (meta.total - 1).bit_length()
+            self._pinned = [torch.empty(need, dtype=torch.int32).pin_memory() for _ in range(4)]
+            self._pinned_events = [None] * 4
+        i = self._pinned_next
+        self._pinned_next = (i + 1) % len(self._pinned)
+        if self._pinned_events[i] is not None:
+            self._pinned_events[i].synchronize()
+        host = self._pinned[i][:meta.total]
+        a = host.numpy()
+        v = meta.views(a)
+        v["row_seq"][:] = -1
+        v["tokens"][:] = 0
+        v["positions"][:] = 0
+        v["seq_slot"][:] = -1
+        v["seq_start"][:] = 0
+        row = 0
+        nw = 0
+        for s, e in enumerate(entries):
+            n = len(e.tokens)
+            start = self.cache.length(e.slot)
+            v["tokens"][row:row + n] = e.tokens
+            v["positions"][row:row + n] = np.arange(start, start + n, dtype=np.int32)
+            v["row_seq"][row:row + n] = s
+            v["seq_slot"][s] = e.slot
+            v["cu_seqlens"][s] = row
+            v["seq_start"][s] = start
+            for w in e.want:
+                v["want_rows"][nw] = row + int(w)
+                nw += 1
+            row += n
+        v["cu_seqlens"][len(entries):] = row
+        return host, i, nw
+
+    def _upload(self, host, index: int, dev: torch.Tensor) -> None:
+        dev.copy_(host, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self._pinned_events[index] = ev
+
+    def _context(self, views, rows, seqs, max_q_len, all_single, pool) -> StepContext:
+        return StepContext(rows=rows, num_seqs=seqs, positions=views["positions"],
+                           row_seq=views["row_seq"], seq_slot=views["seq_slot"],
+                           cu_seqlens=views["cu_seqlens"], seq_start=views["seq_start"],
+                           max_q_len=max_q_len, max_keys=self.cache.max_seq_len,
+                           all_single=all_single, env=self.env, scratch=pool)
+
+    def _eager_step(self, entries, all_single: bool):
+        rows = sum(len(e.tokens) for e in entries)
+        wants = sum(len(e.want) for e in entries)
+        meta = _Meta(rows, len(entries), wants)
+        host, idx, nw = self._pack(entries, meta, rows, len(entries))
+        self.scratch.reset()
+        dev = self.scratch.alloc((meta.total,), torch.int32)
+        self._upload(host, idx, dev)
+        views = meta.views(dev)
+        ctx = self._context(views, rows, len(entries), max(len(e.tokens) for e in entries),
+                            all_single, self.scratch)
+        self.stats["eager_steps"] += 1
+        return self.model.forward(views["tokens"], ctx, self.caches, views["want_rows"], nw)
+
+    def _graph_step(self, entries):
+        n = len(entries)
+        size = 1 << (n - 1).bit_length()
+        bucket = self._buckets.get(size)
+        if bucket is None:
+            bucket = self._buckets[size] = _GraphBucket(size, self.device)
+        # every row of the bucket gets logits; padding rows are inert (row_seq -1)
+        padded = [StepEntry(e.slot, e.tokens, [0]) for e in entries]
+        host, idx, _ = self._pack(padded, bucket.meta, size, size)
+        host.numpy()[bucket.meta.offsets["want_rows"][0]:][:size] = np.arange(size, dtype=np.int32)
+        self._upload(host, idx, bucket.dev)
+        bucket.uses += 1
+        if bucket.graph is None:
+            ctx = self._context(bucket.views, size, size, 1, True, bucket.pool)
+            if bucket.uses == 1:
+                # first use: run eagerly; it also sizes the bucket's scratch pool
+                bucket.pool.reset()
+                self.stats["eager_steps"] += 1
+                logits = self.model.forward(bucket.views["tokens"], ctx, self.caches,
+                                            bucket.views["want_rows"], size)
+                return logits[:n]
+            bucket.pool.frozen = True
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                bucket.pool.reset()
+                bucket.logits = self.model.forward(bucket.views["tokens"], ctx, self.caches,
+                                                   bucket.views["want_rows"], size)
+            bucket.graph = graph
+            self.stats["graph_captures"] += 1
+        bucket.graph.replay()
+        self.stats["graph_replays"] += 1
+        return bucket.logits[:n]
+
+    # -- convenience -----------------------------------------------------------
+    def synchronize(self) -> None:
+        torch.cuda.synchronize(self.device)
+
+    def memory_report(self) -> dict:
+        return {"cache_bytes_per_token": self.cache.bytes_per_token(),
+                "pages": self.cache.num_pages, "free_pages": self.cache.free_pages,
+                "slots": self.cache.max_slots, "scratch_peak": self.scratch.peak,
+                "allocated": torch.cuda.memory_allocated(self.device)}

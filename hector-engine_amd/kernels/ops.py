@@ -1,0 +1,323 @@
+"""Python faces of the HIP kernels: they check shapes, dtypes and contiguity on
+the host, then launch on torch's current stream. Tensors are torch tensors on
+the GPU; nothing here computes in torch."""
+from __future__ import annotations
+
+import torch
+
+from . import lib as _lib
+
+F32, BF16 = 0, 1
+PAGE_TOKENS = 64
+SKINNY_MAX_M = 64
+
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _CODES[dtype]
+    except KeyError:
+        raise TypeError(f"kernels take float32 or bfloat16 tensors, not {dtype}") from None
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
+    if not t.is_cuda:
+        raise ValueError(f"{name}: expected a GPU tensor")
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: expected a contiguous tensor")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name}: expected {dtype}, got {t.dtype}")
+    if shape is not None:
+        if len(shape) != t.dim() or any(s is not None and s != d for s, d in zip(shape, t.shape)):
+            raise ValueError(f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def embedding(out_f32, table, ids, rows: int) -> None:
+    V, D = table.shape
+    _need(table, "table")
+    _need(out_f32, "out", torch.float32)
+    _need(ids, "ids", torch.int32)
+    if out_f32.numel() < rows * D or ids.numel() < rows:
+        raise ValueError("embedding: buffers smaller than the row count")
+    L = _lib.load()
+    _lib.check(L.he_embedding(out_f32.data_ptr(), table.data_ptr(), ids.data_ptr(), rows, D, V,
+                              dtype_code(table.dtype), _stream()))
+
+
+def gather_rows_f32(out, src, rows_idx, n_out: int, n_src: int) -> None:
+    D = src.shape[-1]
+    _need(src, "src", torch.float32)
+    _need(out, "out", torch.float32)
+    _need(rows_idx, "rows", torch.int32)
+    if out.numel() < n_out * D or rows_idx.numel() < n_out or src.numel() < n_src * D:
+        raise ValueError("gather_rows: buffers smaller than the row counts")
+    L = _lib.load()
+    _lib.check(L.he_gather_rows_f32(out.data_ptr(), src.data_ptr(), rows_idx.data_ptr(), n_out, D,
+                                    n_src, _stream()))
+
+
+def residual_add(resid_f32, delta, rows: int) -> None:
+    D = resid_f32.shape[-1]
+    _need(resid_f32, "resid", torch.float32)
+    _need(delta, "delta")
+    if delta.shape[-1] != D or resid_f32.numel() < rows * D or delta.numel() < rows * D:
+        raise ValueError("residual_add: shape mismatch")
+    L = _lib.load()
+    _lib.check(L.he_residual_add(resid_f32.data_ptr(), delta.data_ptr(), rows * D,
+                                 dtype_code(delta.dtype), _stream()))
+
+
+def silu_mul(out, gate_up, rows: int) -> None:
+    I = out.shape[-1]
+    _need(out, "out")
+    _need(gate_up, "gate_up", out.dtype)
+    if gate_up.shape[-1] != 2 * I or out.numel() < rows * I or gate_up.numel() < rows * 2 * I:
+        raise ValueError("silu_mul: gate_up must be [rows, 2*I] for out [rows, I]")
+    L = _lib.load()
+    _lib.check(L.he_silu_mul(out.data_ptr(), gate_up.data_ptr(), rows, I, dtype_code(out.dtype),
+                             _stream()))
+
+
+def add_rmsnorm(resid_f32, delta, weight, out, rows: int, eps: float) -> None:
+    """resid += delta (if given); out = rmsnorm(resid) * weight (if out given)."""
+    D = resid_f32.shape[-1]
+    _need(resid_f32, "resid", torch.float32)
+    _need(weight, "weight", shape=(D,))
+    act = None
+    for name, t in (("delta", delta), ("out", out)):
+        if t is not None:
+            _need(t, name)
+            if t.shape[-1] != D or t.numel() < rows * D:
+                raise ValueError(f"add_rmsnorm: {name} does not match [rows, {D}]")
+            if act is not None and t.dtype != act:
+                raise TypeError("add_rmsnorm: delta and out must share a dtype")
+            act = t.dtype
+    if resid_f32.numel() < rows * D:
+        raise ValueError("add_rmsnorm: resid smaller than the row count")
+    L = _lib.load()
+    _lib.check(L.he_add_rmsnorm(resid_f32.data_ptr(), _ptr(delta), weight.data_ptr(), _ptr(out),
+                                rows, D, float(eps), dtype_code(act or torch.float32),
+                                dtype_code(weight.dtype), _stream()))
+
+
+def rmsnorm_rows(out, x, weight, rows: int, D: int, x_stride: int, out_stride: int,
+                 eps: float) -> None:
+    if out.dtype != x.dtype:
+        raise TypeError("rmsnorm_rows: out and x must share a dtype")
+    if weight is not None:
+        _need(weight, "weight", shape=(D,))
+    if rows > 0 and (x.numel() < (rows - 1) * x_stride + D or out.numel() < (rows - 1) * out_stride + D):
+        raise ValueError("rmsnorm_rows: buffers smaller than rows and strides need")
+    L = _lib.load()
+    _lib.check(L.he_rmsnorm_rows(out.data_ptr(), x.data_ptr(), _ptr(weight), rows, D, x_stride,
+                                 out_stride, float(eps), dtype_code(x.dtype),
+                                 dtype_code(weight.dtype) if weight is not None else F32, _stream()))
+
+
+def gemm_plain(out, a, w, bias, M: int) -> None:
+    """out[M,N] = a[M,K] . w[N,K]^T (+ bias), fixed summation order."""
+    N, K = w.shape
+    _need(a, "a")
+    _need(w, "w", a.dtype)
+    _need(out, "out")
+    if a.shape[-1] != K or out.shape[-1] != N or a.numel() < M * K or out.numel() < M * N:
+        raise ValueError(f"gemm_plain: shapes a{tuple(a.shape)} w{tuple(w.shape)} out{tuple(out.shape)} M={M}")
+    if bias is not None:
+        _need(bias, "bias", shape=(N,))
+    L = _lib.load()
+    _lib.check(L.he_gemm_plain(out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, K,
+                               K, N, dtype_code(a.dtype), dtype_code(out.dtype),
+                               dtype_code(bias.dtype) if bias is not None else F32, _stream()))
+
+
+def gemm_skinny_workspace_floats(M: int, N: int, K: int) -> int:
+    return int(_lib.load().he_gemm_skinny_workspace_floats(M, N, K))
+
+
+def gemm_skinny(out, a, w, bias, M: int, workspace) -> None:
+    """bf16 MFMA product for M <= 64; out is bf16 or fp32."""
+    N, K = w.shape
+    _need(a, "a", torch.bfloat16)
+    _need(w, "w", torch.bfloat16)
+    _need(out, "out")
+    if M > SKINNY_MAX_M:
+        raise ValueError(f"gemm_skinny: M={M} above {SKINNY_MAX_M}")
+    if a.shape[-1] != K or out.shape[-1] != N or a.numel() < M * K or out.numel() < M * N:
+        raise ValueError(f"gemm_skinny: shapes a{tuple(a.shape)} w{tuple(w.shape)} out{tuple(out.shape)} M={M}")
+    if bias is not None:
+        _need(bias, "bias", shape=(N,))
+    ws_floats = 0
+    if workspace is not None:
+        _need(workspace, "workspace", torch.float32)
+        ws_floats = workspace.numel()
+    L = _lib.load()
+    _lib.check(L.he_gemm_skinny_bf16(out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N,
+                                     K, dtype_code(out.dtype),
+                                     dtype_code(bias.dtype) if bias is not None else F32,
+                                     _ptr(workspace), ws_floats, _stream()))
+
+
+def qkv_rope_cache(q_out, kpool, vpool, qkv, q_cols: int, kv_cols: int, bias, positions, row_seq,
+                   seq_slot, page_table, inv_freq, rotary_dim: int, rows: int, H: int, KVH: int,
+                   hd: int, write_kv: bool) -> None:
+    """qkv: [rows, q_cols (+ 2 kv_cols)] projected rows without bias; bias (optional)
+    has the same column layout. Rotated q goes to q_out [rows, H*hd]; k, v go
+    into the pools at (slot, position) when write_kv."""
+    _need(qkv, "qkv")
+    _need(q_out, "q_out", qkv.dtype)
+    width = qkv.shape[-1]
+    if q_cols != H * hd or (write_kv and (kv_cols != KVH * hd or width != q_cols + 2 * kv_cols)):
+        raise ValueError("qkv_rope_cache: column layout does not match the head sizes")
+    if not write_kv and width < q_cols:
+        raise ValueError("qkv_rope_cache: qkv narrower than the query columns")
+    if qkv.numel() < rows * width or q_out.numel() < rows * q_cols:
+        raise ValueError("qkv_rope_cache: buffers smaller than the row count")
+    _need(positions, "positions", torch.int32)
+    _need(row_seq, "row_seq", torch.int32)
+    _need(seq_slot, "seq_slot", torch.int32)
+    if positions.numel() < rows or row_seq.numel() < rows:
+        raise ValueError("qkv_rope_cache: metadata shorter than the row count")
+    es = qkv.element_size()
+    base = qkv.data_ptr()
+    k_in = v_in = None
+    max_blocks = num_pages = 0
+    if write_kv:
+        _need(kpool, "kpool", qkv.dtype, (None, KVH, PAGE_TOKENS, hd))
+        _need(vpool, "vpool", qkv.dtype, (None, KVH, PAGE_TOKENS, hd))
+        _need(page_table, "page_table", torch.int32)
+        num_pages = kpool.shape[0]
+        max_blocks = page_table.shape[1]
+        k_in = base + q_cols * es
+        v_in = base + (q_cols + kv_cols) * es
+    qb = kb = vb = None
+    bias_code = F32
+    if bias is not None:
+        _need(bias, "bias", shape=(width,))
+        bias_code = dtype_code(bias.dtype)
+        bes = bias.element_size()
+        qb = bias.data_ptr()
+        if write_kv:
+            kb = qb + q_cols * bes
+            vb = qb + (q_cols + kv_cols) * bes
+    if rotary_dim:
+        _need(inv_freq, "inv_freq", torch.float32, (rotary_dim // 2,))
+    L = _lib.load()
+    _lib.check(L.he_qkv_rope_cache(
+        q_out.data_ptr(), _ptr(kpool) if write_kv else None, _ptr(vpool) if write_kv else None,
+        base, k_in, v_in, width, qb, kb, vb, bias_code, positions.data_ptr(), row_seq.data_ptr(),
+        seq_slot.data_ptr(), _ptr(page_table) if write_kv else None, max_blocks, num_pages,
+        _ptr(inv_freq) if rotary_dim else None, rotary_dim, rows, H, KVH if write_kv else 0, hd,
+        dtype_code(qkv.dtype), _stream()))
+
+
+def _check_attention(out, q, kpool, vpool, page_table, rows, H, KVH, hd):
+    _need(q, "q")
+    _need(out, "out", q.dtype)
+    _need(kpool, "kpool", q.dtype, (None, KVH, PAGE_TOKENS, hd))
+    _need(vpool, "vpool", q.dtype, (None, KVH, PAGE_TOKENS, hd))
+    _need(page_table, "page_table", torch.int32)
+    if page_table.dim() != 2:
+        raise ValueError("attention: page_table must be [slots, blocks]")
+    if q.numel() < rows * H * hd or out.numel() < rows * H * hd:
+        raise ValueError("attention: q/out smaller than the row count")
+
+
+def attention_plain(out, q, kpool, vpool, positions, row_seq, seq_slot, page_table, rows: int,
+                    H: int, KVH: int, hd: int, window: int, scale: float) -> None:
+    _check_attention(out, q, kpool, vpool, page_table, rows, H, KVH, hd)
+    for name, t in (("positions", positions), ("row_seq", row_seq), ("seq_slot", seq_slot)):
+        _need(t, name, torch.int32)
+    if positions.numel() < rows or row_seq.numel() < rows:
+        raise ValueError("attention: metadata shorter than the row count")
+    L = _lib.load()
+    _lib.check(L.he_attention_plain(
+        out.data_ptr(), q.data_ptr(), kpool.data_ptr(), vpool.data_ptr(), positions.data_ptr(),
+        row_seq.data_ptr(), seq_slot.data_ptr(), page_table.data_ptr(), page_table.shape[1],
+        kpool.shape[0], rows, H, KVH, hd, window, float(scale), dtype_code(q.dtype), _stream()))
+
+
+def attention_decode_workspace_floats(rows: int, H: int, hd: int, max_keys: int) -> int:
+    return int(_lib.load().he_attention_decode_workspace_floats(rows, H, hd, max_keys))
+
+
+def attention_decode(out, q, kpool, vpool, positions, row_seq, seq_slot, page_table, rows: int,
+                     H: int, KVH: int, hd: int, window: int, scale: float, max_keys: int,
+                     workspace) -> None:
+    _check_attention(out, q, kpool, vpool, page_table, rows, H, KVH, hd)
+    _need(q, "q", torch.bfloat16)
+    for name, t in (("positions", positions), ("row_seq", row_seq), ("seq_slot", seq_slot)):
+        _need(t, name, torch.int32)
+    if positions.numel() < rows or row_seq.numel() < rows:
+        raise ValueError("attention: metadata shorter than the row count")
+    _need(workspace, "workspace", torch.float32)
+    L = _lib.load()
+    _lib.check(L.he_attention_decode_bf16(
+        out.data_ptr(), q.data_ptr(), kpool.data_ptr(), vpool.data_ptr(), positions.data_ptr(),
+        row_seq.data_ptr(), seq_slot.data_ptr(), page_table.data_ptr(), page_table.shape[1],
+        kpool.shape[0], rows, H, KVH, hd, window, float(scale), max_keys, workspace.data_ptr(),
+        workspace.numel(), _stream()))
+
+
+def attention_prefill(out, q, kpool, vpool, cu_seqlens, seq_slot, seq_start, page_table,
+                      num_seqs: int, max_q_len: int, total_rows: int, H: int, KVH: int, hd: int,
+                      window: int, scale: float) -> None:
+    _check_attention(out, q, kpool, vpool, page_table, total_rows, H, KVH, hd)
+    _need(q, "q", torch.bfloat16)
+    for name, t in (("cu_seqlens", cu_seqlens), ("seq_slot", seq_slot), ("seq_start", seq_start)):
+        _need(t, name, torch.int32)
+    if cu_seqlens.numel() < num_seqs + 1 or seq_slot.numel() < num_seqs or seq_start.numel() < num_seqs:
+        raise ValueError("attention_prefill: metadata shorter than the sequence count")
+    L = _lib.load()
+    _lib.check(L.he_attention_prefill_bf16(
+        out.data_ptr(), q.data_ptr(), kpool.data_ptr(), vpool.data_ptr(), cu_seqlens.data_ptr(),
+        seq_slot.data_ptr(), seq_start.data_ptr(), page_table.data_ptr(), page_table.shape[1],
+        kpool.shape[0], num_seqs, max_q_len, H, KVH, hd, window, float(scale), _stream()))
+
+
+def argmax_rows(out_i32, logits, rows: int) -> None:
+    _need(logits, "logits", torch.float32)
+    _need(out_i32, "out", torch.int32)
+    V = logits.shape[-1]
+    if logits.numel() < rows * V or out_i32.numel() < rows:
+        raise ValueError("argmax_rows: buffers smaller than the row count")
+    L = _lib.load()
+    _lib.check(L.he_argmax_rows(out_i32.data_ptr(), logits.data_ptr(), rows, V, V, _stream()))
+
+
+def apply_penalties(logits, rows: int, ids, counts, offsets, rep: float, freq: float,
+                    pres: float) -> None:
+    _need(logits, "logits", torch.float32)
+    for name, t in (("ids", ids), ("counts", counts), ("offsets", offsets)):
+        _need(t, name, torch.int32)
+    V = logits.shape[-1]
+    if logits.numel() < rows * V or offsets.numel() < rows + 1 or ids.numel() != counts.numel():
+        raise ValueError("apply_penalties: buffers do not match the row count")
+    L = _lib.load()
+    _lib.check(L.he_apply_penalties(logits.data_ptr(), rows, V, V, ids.data_ptr(),
+                                    counts.data_ptr(), offsets.data_ptr(), float(rep), float(freq),
+                                    float(pres), _stream()))
+
+
+def sample_rows(out_i32, logits, rows: int, uniforms_u32, temperature: float, top_k: int,
+                top_p: float) -> None:
+    _need(logits, "logits", torch.float32)
+    _need(out_i32, "out", torch.int32)
+    _need(uniforms_u32, "uniforms")
+    if uniforms_u32.element_size() != 4 or uniforms_u32.numel() < rows:
+        raise ValueError("sample_rows: uniforms must be one 32-bit word per row")
+    V = logits.shape[-1]
+    if logits.numel() < rows * V or out_i32.numel() < rows:
+        raise ValueError("sample_rows: buffers smaller than the row count")
+    L = _lib.load()
+    _lib.check(L.he_sample_rows(out_i32.data_ptr(), logits.data_ptr(), rows, V, V,
+                                uniforms_u32.data_ptr(), float(temperature), int(top_k),
+                                float(top_p), _stream()))

@@ -1,0 +1,126 @@
+"""Grouped-query attention over the paged cache.
+
+q = n Wq^T + bq, k = n Wk^T + bk, v = n Wv^T + bv (one product over q||k||v, the
+reference's optional fusion: src/graph_builder.cpp:1543-1670); q and k are
+encoded by the position part after the bias and before the cache write, v is
+not (src/graph_builder.cpp:1213-1326); the new keys and values are written
+before attention so that a query sees its own key (:1318-1326); the query at
+position p attends the keys (p - window, p], all of [0, p] without a window
+(kernels/attention.cu:60, :196, :696); kv head = h // (H / KVH) (:180);
+scale 1/sqrt(head_dim) (src/graph_builder.cpp:1328); then o = a Wo^T.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..kernels import ops
+from .base import (BuildEnv, KVNeed, LayerCache, Mixer, PartSpec, StepContext, TensorSpec,
+                   build_part, param, register_part)
+from .linear import Linear
+
+
+@register_part("mixer", "attention")
+class Attention(Mixer):
+    def __init__(self, params: dict, prefix: str, env: BuildEnv):
+        super().__init__(prefix, env)
+        self.hidden = param(params, "hidden_size", int)
+        self.H = param(params, "num_heads", int)
+        self.KVH = param(params, "num_kv_heads", int)
+        self.hd = param(params, "head_dim", int)
+        self.qkv_bias = param(params, "qkv_bias", bool, False)
+        self.out_bias = param(params, "out_bias", bool, False)
+        self.window = param(params, "window", int, 0)
+        self.kv_projection = param(params, "kv_projection", bool, True)
+        self.scale = param(params, "scale", float, 1.0 / math.sqrt(self.hd))
+        if self.H % self.KVH:
+            raise ValueError(f"attention: {self.H} heads are not a multiple of {self.KVH} kv heads")
+        self.position = build_part("position", param(params, "position", PartSpec, PartSpec("none")),
+                                   prefix, env)
+        self.qkv: Linear | None = None
+        self.q_only: Linear | None = None
+        self.o_proj: Linear | None = None
+        self.fast = env.dtype == torch.bfloat16 and getattr(env, "fast_kernels", True) \
+            and self.hd % 16 == 0 and self.hd <= 256
+
+    def children(self):
+        return [self.position]
+
+    def kv_need(self):
+        return KVNeed(self.KVH, self.hd, self.window)
+
+    def tensor_specs(self):
+        p, hd = self.prefix, self.hd
+        specs = {p + "q_proj.weight": TensorSpec((self.H * hd, self.hidden)),
+                 p + "o_proj.weight": TensorSpec((self.hidden, self.H * hd))}
+        if self.kv_projection:
+            specs[p + "k_proj.weight"] = TensorSpec((self.KVH * hd, self.hidden))
+            specs[p + "v_proj.weight"] = TensorSpec((self.KVH * hd, self.hidden))
+        if self.qkv_bias:
+            specs[p + "q_proj.bias"] = TensorSpec((self.H * hd,))
+            if self.kv_projection:
+                specs[p + "k_proj.bias"] = TensorSpec((self.KVH * hd,))
+                specs[p + "v_proj.bias"] = TensorSpec((self.KVH * hd,))
+        if self.out_bias:
+            specs[p + "o_proj.bias"] = TensorSpec((self.hidden,))
+        specs.update(self.position.tensor_specs())
+        return specs
+
+    def bind(self, tensors):
+        p = self.prefix
+        names = ["q_proj"] + (["k_proj", "v_proj"] if self.kv_projection else [])
+        ws = [tensors.pop(p + n + ".weight") for n in names]
+        if len({w.dtype for w in ws}) != 1:
+            raise TypeError(f"{p}q/k/v projections are stored in different dtypes")
+        w = torch.cat(ws, 0).contiguous() if len(ws) > 1 else ws[0]
+        b = None
+        if self.qkv_bias:
+            bs = [tensors.pop(p + n + ".bias") for n in names]
+            if len({x.dtype for x in bs}) != 1:
+                raise TypeError(f"{p}q/k/v biases are stored in different dtypes")
+            b = torch.cat(bs, 0).contiguous() if len(bs) > 1 else bs[0]
+        del ws
+        self.qkv = Linear(w, b)
+        q_rows = self.H * self.hd
+        self.q_only = Linear(w[:q_rows], None if b is None else b[:q_rows])
+        self.o_proj = Linear(tensors[p + "o_proj.weight"], tensors.get(p + "o_proj.bias"))
+        self.position.bind(tensors)
+
+    def forward(self, x, ctx: StepContext, cache: LayerCache):
+        rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.hd
+        writes = cache.writes
+        if writes and not self.kv_projection:
+            raise RuntimeError(f"{self.prefix}: a mixer without k/v projections must read another run's cache")
+        proj = self.qkv if writes else self.q_only
+        rot = self.position.rotary()
+        fused_bias = not self.position.custom
+        # With a rotation (or no encoding) the bias is added inside the fused kernel;
+        # any other encoding sees q and k with their bias already added.
+        qkv = proj(x, rows, ctx, use_bias=not fused_bias)
+        if not fused_bias:
+            q_cols, kv_cols = H * hd, KVH * hd
+            qv = qkv[:, :q_cols].unflatten(1, (H, hd))
+            kv = qkv[:, q_cols:q_cols + kv_cols].unflatten(1, (KVH, hd)) if writes else None
+            self.position.apply(qv, kv, ctx)
+        q = ctx.alloc((rows, H * hd))
+        inv_freq, r = rot if rot is not None else (None, 0)
+        ops.qkv_rope_cache(q, cache.kpool, cache.vpool, qkv, H * hd, KVH * hd,
+                           proj.bias if fused_bias else None, ctx.positions, ctx.row_seq,
+                           ctx.seq_slot, cache.page_table, inv_freq, r, rows, H, KVH, hd, writes)
+        out = ctx.alloc((rows, H * hd))
+        if not self.fast:
+            ops.attention_plain(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
+                                ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,
+                                self.scale)
+        elif ctx.all_single:
+            floats = ops.attention_decode_workspace_floats(rows, H, hd, ctx.max_keys)
+            ws = ctx.alloc((max(floats, 1),), torch.float32)
+            ops.attention_decode(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
+                                 ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,
+                                 self.scale, ctx.max_keys, ws)
+        else:
+            ops.attention_prefill(out, q, cache.kpool, cache.vpool, ctx.cu_seqlens, ctx.seq_slot,
+                                  ctx.seq_start, cache.page_table, ctx.num_seqs, ctx.max_q_len,
+                                  rows, H, KVH, hd, self.window, self.scale)
+        return self.o_proj(out, rows, ctx)

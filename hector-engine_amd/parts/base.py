@@ -1,0 +1,281 @@
+"""What a layer is made of: the interfaces of the parts, their registries and
+the data that selects them.
+
+A model is described by data (:class:`ModelSpec`): one :class:`PartSpec` per
+part with its sizes and constants, one block per layer, and a schedule that
+says in which order layers run and whose cache each run reads. Parts are built
+from that data through the registries below and never learn which model they
+are in. Another mixer, feed-forward, norm, position encoding or block is a
+class registered under a new kind; nothing else changes.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Any, Callable
+
+import torch
+
+# ----------------------------------------------------------------------------
+# data
+# ----------------------------------------------------------------------------
+
+
+@dataclasses.dataclass(frozen=True)
+class PartSpec:
+    """Selects a part (`kind` is the registry key) and gives its parameters."""
+
+    kind: str
+    params: dict = dataclasses.field(default_factory=dict)
+
+
+@dataclasses.dataclass(frozen=True)
+class TensorSpec:
+    """A weight tensor a part expects: shape, and how the random mode fills it.
+
+    init: ("normal", std) | ("gain", mean, std) | ("zeros",)
+    integer: integer tables are kept as int32, everything else follows the run dtype rule.
+    """
+
+    shape: tuple
+    init: tuple = ("normal", 0.02)
+    integer: bool = False
+
+
+@dataclasses.dataclass(frozen=True)
+class LayerSpec:
+    prefix: str       # tensor name prefix of the layer, e.g. "model.layers.3."
+    block: PartSpec   # arrangement of mixer, feed-forward and norms
+
+
+@dataclasses.dataclass(frozen=True)
+class ScheduleEntry:
+    """One run of a layer. cache_from names an earlier entry of the schedule
+    whose cache this run reads instead of writing one of its own."""
+
+    layer: int
+    cache_from: int | None = None
+
+
+@dataclasses.dataclass
+class ModelSpec:
+    hidden_size: int
+    vocab_size: int
+    embedding: PartSpec
+    embedding_prefix: str
+    layers: list[LayerSpec]
+    schedule: list[ScheduleEntry]
+    final_norm: PartSpec
+    final_norm_prefix: str
+    head: PartSpec
+    head_prefix: str
+    max_positions: int
+
+
+@dataclasses.dataclass(frozen=True)
+class KVNeed:
+    """What a mixer keeps per token in the cache: keys and values of this shape,
+    all of them (window 0) or only the last `window`."""
+
+    kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclasses.dataclass
+class BuildEnv:
+    """Where and in which precision parts live."""
+
+    device: torch.device
+    dtype: torch.dtype            # activation dtype: torch.float32 or torch.bfloat16
+    fast_kernels: bool = True     # False: the plain kernels also under bfloat16
+
+
+# ----------------------------------------------------------------------------
+# per-step context handed to every part
+# ----------------------------------------------------------------------------
+
+
+class StepContext:
+    """The packed batch of one step, on the device. Rows are tokens; a padding
+    row has row_seq -1. Every part receives this and nothing model-specific."""
+
+    def __init__(self, *, rows: int, num_seqs: int, positions, row_seq, seq_slot, cu_seqlens,
+                 seq_start, max_q_len: int, max_keys: int, all_single: bool, env: BuildEnv,
+                 scratch, host=None):
+        self.rows = rows                  # token rows in this step (with padding rows)
+        self.num_seqs = num_seqs          # sequences (with padding sequences)
+        self.positions = positions        # int32 [rows] absolute position of each row
+        self.row_seq = row_seq            # int32 [rows] index into seq_slot, -1 = padding
+        self.seq_slot = seq_slot          # int32 [num_seqs] cache slot of each sequence
+        self.cu_seqlens = cu_seqlens      # int32 [num_seqs + 1] first row of each sequence
+        self.seq_start = seq_start        # int32 [num_seqs] cached length before this step
+        self.max_q_len = max_q_len        # longest run of new tokens of one sequence
+        self.max_keys = max_keys          # upper bound of any sequence's length after the step
+        self.all_single = all_single      # every sequence brings exactly one token
+        self.env = env
+        self.scratch = scratch            # ScratchPool: alloc(shape, dtype)
+        self.host = host                  # host-side copy of the batch (lists), for parts that plan on the host
+
+    def alloc(self, shape, dtype=None) -> torch.Tensor:
+        return self.scratch.alloc(shape, dtype or self.env.dtype)
+
+
+@dataclasses.dataclass
+class LayerCache:
+    """The cache as one run of a layer sees it."""
+
+    kpool: torch.Tensor | None        # [pages, kv_heads, 64, head_dim]
+    vpool: torch.Tensor | None
+    page_table: torch.Tensor | None   # int32 [slots, blocks] of the layer's group
+    writes: bool                      # False: the keys/values are another run's
+    state: torch.Tensor | None        # uint8 [slots, state_bytes] of this run, or None
+
+
+# ----------------------------------------------------------------------------
+# interfaces
+# ----------------------------------------------------------------------------
+
+
+class Part:
+    """Base of all parts: declares its tensors by full name and receives them."""
+
+    def __init__(self, prefix: str, env: BuildEnv):
+        self.prefix = prefix
+        self.env = env
+
+    def tensor_specs(self) -> dict[str, TensorSpec]:
+        """Full tensor name -> spec, children included."""
+        return {}
+
+    def bind(self, tensors: dict[str, torch.Tensor]) -> None:
+        """Takes its tensors (on the device, in their run dtype); may fuse them."""
+
+    def children(self) -> list["Part"]:
+        return []
+
+
+class Norm(Part):
+    def add_norm(self, resid: torch.Tensor, delta: torch.Tensor | None, rows: int,
+                 ctx: StepContext, want_out: bool = True) -> torch.Tensor | None:
+        """resid (fp32 [rows, D], in place) += delta; returns norm(resid) in the
+        activation dtype (or None when want_out is False)."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    # True for an encoding that must run through apply() on q and k; False for a
+    # rotation the fused q/k kernel applies (rotary() gives its table) or for none.
+    custom = False
+
+    def rotary(self) -> tuple[torch.Tensor, int] | None:
+        """(inv_freq fp32 [r/2], r) when the encoding is a rotation the fused
+        q/k kernel can apply; None otherwise."""
+        return None
+
+    def apply(self, q: torch.Tensor, k: torch.Tensor | None, ctx: StepContext) -> None:
+        """In-place encoding of q [rows, H, hd] and k [rows, KVH, hd] for
+        encodings that are not a plain rotation. Default: none."""
+
+
+class Mixer(Part):
+    def kv_need(self) -> KVNeed | None:
+        """Keys/values per token this mixer keeps, or None."""
+        return None
+
+    def state_bytes(self) -> int:
+        """Bytes of fixed-size state per sequence."""
+        return 0
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """Arrangement of a layer's parts around the residual stream."""
+
+    mixer: Mixer
+
+    def forward(self, stream: "ResidualStream", ctx: StepContext, cache: LayerCache) -> None:
+        raise NotImplementedError
+
+
+class ResidualStream:
+    """The fp32 residual rows of a step plus one branch output not yet added:
+    the add is fused into the next norm."""
+
+    def __init__(self, resid: torch.Tensor, rows: int):
+        self.resid = resid
+        self.rows = rows
+        self.pending: torch.Tensor | None = None
+
+    def add(self, delta: torch.Tensor) -> None:
+        if self.pending is not None:
+            self.materialize()
+        self.pending = delta
+
+    def normed(self, norm: Norm, ctx: StepContext) -> torch.Tensor:
+        out = norm.add_norm(self.resid, self.pending, self.rows, ctx)
+        self.pending = None
+        return out
+
+    def materialize(self) -> torch.Tensor:
+        if self.pending is not None:
+            from ..kernels import ops
+            ops.residual_add(self.resid, self.pending, self.rows)
+            self.pending = None
+        return self.resid
+
+
+# ----------------------------------------------------------------------------
+# registries
+# ----------------------------------------------------------------------------
+
+CATEGORIES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head")
+_registries: dict[str, dict[str, Callable[..., Part]]] = {c: {} for c in CATEGORIES}
+
+
+def register_part(category: str, kind: str, factory: Callable[..., Part] | None = None):
+    """Registers `factory(params: dict, prefix: str, env: BuildEnv) -> Part` under
+    (category, kind); usable as a decorator on a class with that constructor."""
+    if category not in _registries:
+        raise KeyError(f"unknown part category '{category}', have {CATEGORIES}")
+
+    def deco(f):
+        _registries[category][kind] = f
+        return f
+
+    return deco(factory) if factory is not None else deco
+
+
+def build_part(category: str, spec: PartSpec, prefix: str, env: BuildEnv) -> Part:
+    try:
+        factory = _registries[category][spec.kind]
+    except KeyError:
+        raise KeyError(f"no {category} of kind '{spec.kind}' is registered; "
+                       f"registered: {sorted(_registries.get(category, {}))}") from None
+    return factory(dict(spec.params), prefix, env)
+
+
+def registered(category: str) -> list[str]:
+    return sorted(_registries[category])
+
+
+def param(params: dict, key: str, kind: type, default: Any = dataclasses.MISSING) -> Any:
+    """A part's own typed parameter access with a clear error."""
+    if key not in params or params[key] is None:
+        if default is dataclasses.MISSING:
+            raise KeyError(f"part parameter '{key}' is required")
+        return default
+    value = params[key]
+    if kind in (int, float) and isinstance(value, bool):
+        raise TypeError(f"part parameter '{key}': expected {kind.__name__}, got {value!r}")
+    if kind is float and isinstance(value, int):
+        value = float(value)
+    if not isinstance(value, kind):
+        raise TypeError(f"part parameter '{key}': expected {kind.__name__}, got {value!r}")
+    return value

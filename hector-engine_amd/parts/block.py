@@ -1,0 +1,42 @@
+"""Arrangement of a layer: pre-norm residual block
+    x = x + mixer(norm1(x));  x = x + feed_forward(norm2(x))
+(reference: src/graph_builder.cpp:1195, :1366-1374, :1396, :1443). Each
+residual add is carried as pending and fused into the next norm."""
+from __future__ import annotations
+
+from .base import (Block, BuildEnv, LayerCache, PartSpec, ResidualStream, StepContext,
+                   build_part, param, register_part)
+
+
+@register_part("block", "pre_norm")
+class PreNormBlock(Block):
+    def __init__(self, params: dict, prefix: str, env: BuildEnv):
+        super().__init__(prefix, env)
+        names = param(params, "names", dict)
+        self.mixer_norm = build_part("norm", param(params, "mixer_norm", PartSpec),
+                                     prefix + names["mixer_norm"] + ".", env)
+        self.mixer = build_part("mixer", param(params, "mixer", PartSpec),
+                                prefix + names["mixer"] + ".", env)
+        self.ff_norm = build_part("norm", param(params, "feed_forward_norm", PartSpec),
+                                  prefix + names["feed_forward_norm"] + ".", env)
+        self.feed_forward = build_part("feed_forward", param(params, "feed_forward", PartSpec),
+                                       prefix + names["feed_forward"] + ".", env)
+
+    def children(self):
+        return [self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward]
+
+    def tensor_specs(self):
+        specs = {}
+        for c in self.children():
+            specs.update(c.tensor_specs())
+        return specs
+
+    def bind(self, tensors):
+        for c in self.children():
+            c.bind(tensors)
+
+    def forward(self, stream: ResidualStream, ctx: StepContext, cache: LayerCache) -> None:
+        n = stream.normed(self.mixer_norm, ctx)
+        stream.add(self.mixer.forward(n, ctx, cache))
+        n = stream.normed(self.ff_norm, ctx)
+        stream.add(self.feed_forward.forward(n, ctx))
