@@ -3,7 +3,8 @@
 Keys and values live in pages of 64 tokens. Layers are partitioned into groups
 by what they keep (kv heads, head size, all keys or a window of them); each
 group has pools of its own, [runs][pages][kv_heads][64][head_dim] for K and for
-V, and one page table [slots][blocks] shared by its runs. A sequence holds a
+V (V transposed inside a page: [head_dim][64]), and one page table [slots][blocks]
+shared by its runs. A sequence holds a
 slot: its row of every page table, its length, and its row of the fixed-size
 state area. Slots and pages go back to the free lists when a sequence ends and
 are handed out again, lowest first; nothing is cleared, because attention only
@@ -36,9 +37,13 @@ class _Group:
                  max_blocks: int, dtype, device):
         self.need = need
         self.runs = runs
-        shape = (len(runs), num_pages, need.kv_heads, PAGE_TOKENS, need.head_dim)
-        self.kpool = torch.empty(shape, dtype=dtype, device=device)
-        self.vpool = torch.empty(shape, dtype=dtype, device=device)
+        # zero-filled once (as the reference's cache is: src/kv_cache.hpp:161-203): a masked
+        # key still enters the matrix products with weight 0, so it must never be NaN
+        self.kpool = torch.zeros((len(runs), num_pages, need.kv_heads, PAGE_TOKENS, need.head_dim),
+                                 dtype=dtype, device=device)
+        # V is transposed inside a page so that 8 consecutive tokens of one dim are contiguous
+        self.vpool = torch.zeros((len(runs), num_pages, need.kv_heads, need.head_dim, PAGE_TOKENS),
+                                 dtype=dtype, device=device)
         self.page_table = torch.full((max_slots, max_blocks), -1, dtype=torch.int32, device=device)
 
 

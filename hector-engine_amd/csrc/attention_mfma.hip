@@ -1,0 +1,377 @@
+// bf16 attention over the paged cache on the matrix cores, for prompt steps
+// (tiles of 16 queries of one sequence and head) and for one-token steps (the
+// query heads of one kv group, the keys split over workgroups and merged).
+// They replace the reference's attention_prefill_cached_kernel
+// (kernels/attention.cu:664-773: one block per query and head, no tile reuse)
+// and attention_cached_v2_kernel_dp (kernels/attention.cu:337-494); the
+// online-softmax algebra and its merge are the reference's
+// (kernels/attention.cu:279-314).
+//
+// Both kernels work on transposed tiles so that no operand ever has to change
+// lanes. With v_mfma_f32_16x16x32_bf16 (A: lane l holds A[l%16][8*(l/16)..+8),
+// B: lane l holds B[8*(l/16)..+8)[l%16], D: lane l holds D[4*(l/16)+i][l%16]):
+//   S^T[key][q] = sum_d K[key][d] Q[q][d]      A = K rows (d contiguous), B = Q rows
+//   O^T[d][q]   = sum_key V^T[d][key] P^T[key][q]   A = V^T rows, B = P^T
+// The cache stores V transposed inside a page, [head_dim][64 tokens], so a V^T
+// row's 8 consecutive keys are 16 contiguous bytes. The 32 keys of a step are
+// assigned to the rows of the two S^T tiles as key = 8*(row/4) + 4*tile + row%4,
+// which leaves lane group g with exactly the keys 8g..8g+7 that the B operand of
+// the P^T V product wants from it. A query is a column (l%16), so its softmax
+// statistics are reduced over registers and two lane swaps (xor 16, 32) only.
+// Softmax, its running maximum and sum, and both accumulators are fp32.
+#include "common.h"
+#include "hector_kernels.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+__device__ __forceinline__ bf16x8 ld8(const uint16_t* p, bool ok) {
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (ok) v = *reinterpret_cast<const uint4*>(p);
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+template <int NT>
+struct AttnState {
+  floatx4 o[NT];  // O^T[16*dt + 4*lg + i][q], unnormalised
+  float m;        // running maximum of the query of this lane's column
+  float l;        // this lane's share of the running sum
+};
+
+// One step of 32 keys starting at absolute position key_base (a multiple of 32).
+// kpage: K of (page, kv head), [64][hd]; vpage: V^T of the same, [hd][64].
+// The lane's query sees the keys in [lo, hi].
+template <int NT>
+__device__ __forceinline__ void attend32(AttnState<NT>& st, const bf16x8* qf,
+                                         const uint16_t* __restrict__ kpage,
+                                         const uint16_t* __restrict__ vpage, int koff,
+                                         int key_base, int lo, int hi, float scale, int lr,
+                                         int lg) {
+  constexpr int HD = 16 * NT;
+  constexpr int KS = (HD + 31) / 32;
+  floatx4 s[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    const int key_local = 8 * (lr >> 2) + 4 * t + (lr & 3);
+    const uint16_t* krow = kpage + (koff + key_local) * HD + 8 * lg;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const bf16x8 a = ld8(krow + 32 * ks, 32 * ks + 8 * lg < HD);
+      s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[ks], s[t], 0, 0, 0);
+    }
+  }
+  float p[2][4];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int key = key_base + 8 * lg + 4 * t + r;
+      const float v = (key >= lo && key <= hi) ? s[t][r] * scale : -INFINITY;
+      p[t][r] = v;
+      mx = fmaxf(mx, v);
+    }
+  mx = fmaxf(mx, __shfl_xor(mx, 16, HE_WAVE));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, HE_WAVE));
+  const float m_new = fmaxf(st.m, mx);
+  const float m_use = m_new == -INFINITY ? 0.f : m_new;
+  const float alpha = __expf(st.m - m_use);
+  float sum = 0.f;
+  uint32_t packed[4];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int r = 0; r < 4; r += 2) {
+      const float e0 = __expf(p[t][r] - m_use);
+      const float e1 = __expf(p[t][r + 1] - m_use);
+      sum += e0 + e1;
+      packed[2 * t + (r >> 1)] =
+          (uint32_t)float_to_bf16_bits(e0) | ((uint32_t)float_to_bf16_bits(e1) << 16);
+    }
+  st.l = st.l * alpha + sum;
+  st.m = m_new;
+  const bf16x8 pb =
+      __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
+#pragma unroll
+  for (int dt = 0; dt < NT; ++dt) {
+    st.o[dt] *= alpha;
+    const bf16x8 a = ld8(vpage + (16 * dt + lr) * HE_PAGE_TOKENS + koff + 8 * lg, true);
+    st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, st.o[dt], 0, 0, 0);
+  }
+}
+
+template <int NT>
+__device__ __forceinline__ void load_q(bf16x8* qf, const uint16_t* qrow, bool valid, int lg) {
+  constexpr int HD = 16 * NT;
+  constexpr int KS = (HD + 31) / 32;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) qf[ks] = ld8(qrow + 32 * ks + 8 * lg, valid && 32 * ks + 8 * lg < HD);
+}
+
+// ------------------------------------------------------------------ prefill
+// grid (ceil(max_q_len / 64), H, num_seqs), 256 threads: wave w takes the 16
+// queries q0 = 64*blockIdx.x + 16*w of the sequence.
+template <int NT>
+__global__ __launch_bounds__(256) void attention_prefill_kernel(
+    uint16_t* __restrict__ out, const uint16_t* __restrict__ q,
+    const uint16_t* __restrict__ kpool, const uint16_t* __restrict__ vpool,
+    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_slot,
+    const int32_t* __restrict__ seq_start, const int32_t* __restrict__ page_table, int max_blocks,
+    int num_pages, int H, int KVH, int window, float scale) {
+  constexpr int HD = 16 * NT;
+  constexpr int KS = (HD + 31) / 32;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lr = lane & 15, lg = lane >> 4;
+  const int seq = blockIdx.z, h = blockIdx.y;
+  const int slot = seq_slot[seq];
+  if (slot < 0) return;
+  const int row0 = cu_seqlens[seq];
+  const int q_len = cu_seqlens[seq + 1] - row0;
+  const int q0 = 64 * blockIdx.x + 16 * wave;
+  if (q0 >= q_len) return;
+  const int start = seq_start[seq];
+  const int kvh = h / (H / KVH);
+  const int32_t* pt = page_table + (int64_t)slot * max_blocks;
+
+  const int qi = q0 + lr;                 // this lane's query (column)
+  const bool q_ok = qi < q_len;
+  const int pos = start + qi;             // its absolute position
+  const int hi = q_ok ? pos : -1;
+  const int lo = (window > 0 && q_ok) ? max(0, pos + 1 - window) : 0;
+  bf16x8 qf[KS];
+  load_q<NT>(qf, q + ((int64_t)(row0 + min(qi, q_len - 1)) * H + h) * HD, q_ok, lg);
+
+  AttnState<NT> st;
+#pragma unroll
+  for (int dt = 0; dt < NT; ++dt) st.o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  st.m = -INFINITY;
+  st.l = 0.f;
+
+  const int last_pos = start + min(q0 + 15, q_len - 1);
+  const int first_pos = start + q0;
+  const int tile_lo = window > 0 ? max(0, first_pos + 1 - window) : 0;
+  for (int kb = tile_lo & ~31; kb <= last_pos; kb += 32) {
+    const int page = pt[kb >> HE_PAGE_SHIFT];
+    if (page < 0 || page >= num_pages) continue;  // never for an admitted batch
+    const int64_t pbase = ((int64_t)page * KVH + kvh) * (HE_PAGE_TOKENS * HD);
+    attend32<NT>(st, qf, kpool + pbase, vpool + pbase, kb & 32, kb, lo, hi, scale, lr, lg);
+  }
+  float l = st.l;
+  l += __shfl_xor(l, 16, HE_WAVE);
+  l += __shfl_xor(l, 32, HE_WAVE);
+  if (!q_ok) return;
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  uint16_t* orow = out + ((int64_t)(row0 + qi) * H + h) * HD;
+#pragma unroll
+  for (int dt = 0; dt < NT; ++dt) {
+    uint2 w;
+    w.x = (uint32_t)float_to_bf16_bits(st.o[dt][0] * inv) |
+          ((uint32_t)float_to_bf16_bits(st.o[dt][1] * inv) << 16);
+    w.y = (uint32_t)float_to_bf16_bits(st.o[dt][2] * inv) |
+          ((uint32_t)float_to_bf16_bits(st.o[dt][3] * inv) << 16);
+    *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * lg) = w;
+  }
+}
+
+// ------------------------------------------------------------------ decode
+// grid (nsplit, KVH * head_tiles, rows), 64 threads. Columns are the query heads
+// of one kv group (16 per head tile). Each workgroup takes one slice of the keys
+// and writes (m, l, unnormalised O) for its heads; the merge kernel joins them.
+template <int NT>
+__global__ __launch_bounds__(64) void attention_decode_kernel(
+    float* __restrict__ ws_o, float* __restrict__ ws_ml, const uint16_t* __restrict__ q,
+    const uint16_t* __restrict__ kpool, const uint16_t* __restrict__ vpool,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
+    const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ page_table, int max_blocks,
+    int num_pages, int H, int KVH, int head_tiles, int window, float scale) {
+  constexpr int HD = 16 * NT;
+  constexpr int KS = (HD + 31) / 32;
+  const int lane = threadIdx.x;
+  const int lr = lane & 15, lg = lane >> 4;
+  const int split = blockIdx.x, nsplit = gridDim.x;
+  const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y % head_tiles;
+  const int row = blockIdx.z;
+  const int G = H / KVH;
+  const int hg = 16 * ht + lr;            // head within the group
+  const bool h_ok = hg < G;
+  const int h = kvh * G + min(hg, G - 1);
+  const int64_t wsi = ((int64_t)row * H + h) * nsplit + split;
+  const int seq = row_seq[row];
+  int n_keys = 0, first = 0, slot = -1;
+  if (seq >= 0) {
+    slot = seq_slot[seq];
+    n_keys = positions[row] + 1;
+    first = window > 0 ? max(0, n_keys - window) : 0;
+  }
+  const int span_lo = first & ~31;
+  int chunk = (n_keys - span_lo + nsplit - 1) / nsplit;
+  chunk = (chunk + 31) & ~31;
+  const int kb_begin = span_lo + split * chunk;
+  const int kb_end = min(kb_begin + chunk, n_keys);
+  if (slot < 0 || kb_begin >= kb_end) {
+    if (h_ok && lg == 0) {
+      ws_ml[2 * wsi] = -INFINITY;
+      ws_ml[2 * wsi + 1] = 0.f;
+    }
+    return;
+  }
+  const int32_t* pt = page_table + (int64_t)slot * max_blocks;
+  bf16x8 qf[KS];
+  load_q<NT>(qf, q + ((int64_t)row * H + h) * HD, h_ok, lg);
+  AttnState<NT> st;
+#pragma unroll
+  for (int dt = 0; dt < NT; ++dt) st.o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  st.m = -INFINITY;
+  st.l = 0.f;
+  const int hi = n_keys - 1;
+  for (int kb = kb_begin; kb < kb_end; kb += 32) {
+    const int page = pt[kb >> HE_PAGE_SHIFT];
+    if (page < 0 || page >= num_pages) continue;  // never for an admitted batch
+    const int64_t pbase = ((int64_t)page * KVH + kvh) * (HE_PAGE_TOKENS * HD);
+    attend32<NT>(st, qf, kpool + pbase, vpool + pbase, kb & 32, kb, first, hi, scale, lr, lg);
+  }
+  float l = st.l;
+  l += __shfl_xor(l, 16, HE_WAVE);
+  l += __shfl_xor(l, 32, HE_WAVE);
+  if (!h_ok) return;
+  if (lg == 0) {
+    ws_ml[2 * wsi] = st.m;
+    ws_ml[2 * wsi + 1] = l;
+  }
+  float* o = ws_o + wsi * HD;
+#pragma unroll
+  for (int dt = 0; dt < NT; ++dt)
+    *reinterpret_cast<float4*>(o + 16 * dt + 4 * lg) =
+        make_float4(st.o[dt][0], st.o[dt][1], st.o[dt][2], st.o[dt][3]);
+}
+
+// out[row][h][:] = sum_s O_s e^(m_s - M) / sum_s l_s e^(m_s - M); grid (H, rows).
+__global__ void attention_merge_kernel(uint16_t* __restrict__ out, const float* __restrict__ ws_o,
+                                       const float* __restrict__ ws_ml, int H, int HD,
+                                       int nsplit) {
+  const int h = blockIdx.x;
+  const int64_t row = blockIdx.y;
+  const int64_t base = (row * H + h) * nsplit;
+  float M = -INFINITY;
+  for (int s = 0; s < nsplit; ++s) M = fmaxf(M, ws_ml[2 * (base + s)]);
+  float L = 0.f;
+  for (int s = 0; s < nsplit; ++s) {
+    const float m = ws_ml[2 * (base + s)];
+    if (m > -INFINITY) L += ws_ml[2 * (base + s) + 1] * __expf(m - M);
+  }
+  const float inv = L > 0.f ? 1.f / L : 0.f;
+  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+    float acc = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+      const float m = ws_ml[2 * (base + s)];
+      if (m > -INFINITY) acc += ws_o[(base + s) * HD + d] * __expf(m - M);
+    }
+    out[(row * H + h) * (int64_t)HD + d] = float_to_bf16_bits(acc * inv);
+  }
+}
+
+static int decode_splits(int rows, int KVH, int head_tiles, int max_keys) {
+  const int groups = rows * KVH * head_tiles;
+  int s = (1024 + groups - 1) / groups;
+  const int max_s = (max_keys + 63) / 64;
+  if (s > max_s) s = max_s;
+  if (s > 64) s = 64;
+  if (s < 1) s = 1;
+  return s;
+}
+
+extern "C" int64_t he_attention_decode_workspace_floats(int rows, int H, int KVH, int hd,
+                                                        int max_keys) {
+  if (rows <= 0 || H <= 0 || KVH <= 0 || hd <= 0 || H % KVH) return 0;
+  const int head_tiles = (H / KVH + 15) / 16;
+  return (int64_t)rows * H * decode_splits(rows, KVH, head_tiles, max_keys) * (hd + 2);
+}
+
+#define ATTN_DISPATCH(NTV, CALL) \
+  case NTV: {                    \
+    constexpr int NT = NTV;      \
+    CALL;                        \
+    break;                       \
+  }
+#define ATTN_SWITCH(nt, CALL)                                                              \
+  switch (nt) {                                                                            \
+    ATTN_DISPATCH(1, CALL) ATTN_DISPATCH(2, CALL) ATTN_DISPATCH(3, CALL)                   \
+    ATTN_DISPATCH(4, CALL) ATTN_DISPATCH(5, CALL) ATTN_DISPATCH(6, CALL)                   \
+    ATTN_DISPATCH(7, CALL) ATTN_DISPATCH(8, CALL) ATTN_DISPATCH(9, CALL)                   \
+    ATTN_DISPATCH(10, CALL) ATTN_DISPATCH(11, CALL) ATTN_DISPATCH(12, CALL)                \
+    ATTN_DISPATCH(13, CALL) ATTN_DISPATCH(14, CALL) ATTN_DISPATCH(15, CALL)                \
+    ATTN_DISPATCH(16, CALL)                                                                \
+    default:                                                                               \
+      he_set_error("attention: head_dim %d is not a multiple of 16 up to 256", 16 * (nt)); \
+      return -1;                                                                           \
+  }
+
+extern "C" int he_attention_decode_bf16(void* out, const void* q, const void* kpool,
+                                        const void* vpool, const void* positions,
+                                        const void* row_seq, const void* seq_slot,
+                                        const void* page_table, int max_blocks, int num_pages,
+                                        int rows, int H, int KVH, int hd, int window, float scale,
+                                        int max_keys, void* workspace_f32,
+                                        int64_t workspace_floats, void* stream) {
+  HE_REQUIRE(rows >= 0 && H > 0 && KVH > 0 && hd > 0 && max_keys > 0,
+             "he_attention_decode_bf16: bad sizes");
+  HE_REQUIRE(H % KVH == 0, "he_attention_decode_bf16: heads %d not a multiple of kv heads %d", H,
+             KVH);
+  HE_REQUIRE(hd % 16 == 0 && hd <= 256,
+             "he_attention_decode_bf16: head_dim %d must be a multiple of 16 up to 256", hd);
+  HE_REQUIRE(rows <= 65535, "he_attention_decode_bf16: %d rows above 65535", rows);
+  if (rows == 0) return 0;
+  const int G = H / KVH;
+  const int head_tiles = (G + 15) / 16;
+  const int nsplit = decode_splits(rows, KVH, head_tiles, max_keys);
+  const int64_t need = (int64_t)rows * H * nsplit * (hd + 2);
+  HE_REQUIRE(workspace_f32 != nullptr && workspace_floats >= need,
+             "he_attention_decode_bf16: workspace of %lld floats, need %lld",
+             (long long)workspace_floats, (long long)need);
+  HE_REQUIRE((((uintptr_t)workspace_f32) & 15) == 0 && (((uintptr_t)q) & 15) == 0 &&
+                 (((uintptr_t)kpool) & 15) == 0 && (((uintptr_t)vpool) & 15) == 0,
+             "he_attention_decode_bf16: buffers must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  float* ws_o = (float*)workspace_f32;
+  float* ws_ml = ws_o + (int64_t)rows * H * nsplit * hd;
+  dim3 grid(nsplit, KVH * head_tiles, rows);
+  ATTN_SWITCH(hd / 16, (attention_decode_kernel<NT><<<grid, 64, 0, s>>>(
+                           ws_o, ws_ml, (const uint16_t*)q, (const uint16_t*)kpool,
+                           (const uint16_t*)vpool, (const int32_t*)positions,
+                           (const int32_t*)row_seq, (const int32_t*)seq_slot,
+                           (const int32_t*)page_table, max_blocks, num_pages, H, KVH, head_tiles,
+                           window, scale)));
+  int rc = he_check_launch("he_attention_decode_bf16");
+  if (rc) return rc;
+  attention_merge_kernel<<<dim3(H, rows), 64, 0, s>>>((uint16_t*)out, ws_o, ws_ml, H, hd, nsplit);
+  return he_check_launch("he_attention_decode_bf16 merge");
+}
+
+extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* kpool,
+                                         const void* vpool, const void* cu_seqlens,
+                                         const void* seq_slot, const void* seq_start,
+                                         const void* page_table, int max_blocks, int num_pages,
+                                         int num_seqs, int max_q_len, int H, int KVH, int hd,
+                                         int window, float scale, void* stream) {
+  HE_REQUIRE(num_seqs >= 0 && max_q_len >= 0 && H > 0 && KVH > 0 && hd > 0,
+             "he_attention_prefill_bf16: bad sizes");
+  HE_REQUIRE(H % KVH == 0, "he_attention_prefill_bf16: heads %d not a multiple of kv heads %d", H,
+             KVH);
+  HE_REQUIRE(hd % 16 == 0 && hd <= 256,
+             "he_attention_prefill_bf16: head_dim %d must be a multiple of 16 up to 256", hd);
+  HE_REQUIRE(num_seqs <= 65535 && H <= 65535, "he_attention_prefill_bf16: grid too large");
+  HE_REQUIRE((((uintptr_t)q) & 15) == 0 && (((uintptr_t)kpool) & 15) == 0 &&
+                 (((uintptr_t)vpool) & 15) == 0 && (((uintptr_t)out) & 7) == 0,
+             "he_attention_prefill_bf16: buffers must be 16-byte aligned");
+  if (num_seqs == 0 || max_q_len == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid((max_q_len + 63) / 64, H, num_seqs);
+  ATTN_SWITCH(hd / 16, (attention_prefill_kernel<NT><<<grid, 256, 0, s>>>(
+                           (uint16_t*)out, (const uint16_t*)q, (const uint16_t*)kpool,
+                           (const uint16_t*)vpool, (const int32_t*)cu_seqlens,
+                           (const int32_t*)seq_slot, (const int32_t*)seq_start,
+                           (const int32_t*)page_table, max_blocks, num_pages, H, KVH, window,
+                           scale)));
+  return he_check_launch("he_attention_prefill_bf16");
+}

@@ -52,8 +52,10 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(
   for (int j = first; j <= p; ++j) {
     const int page = pt[j >> HE_PAGE_SHIFT];
     if (page < 0 || page >= num_pages) continue;  // never for an admitted batch
-    const int64_t base =
-        (((int64_t)page * KVH + kvh) * HE_PAGE_TOKENS + (j & (HE_PAGE_TOKENS - 1))) * hd;
+    const int off = j & (HE_PAGE_TOKENS - 1);
+    const int64_t base = (((int64_t)page * KVH + kvh) * HE_PAGE_TOKENS + off) * hd;
+    // V is stored transposed inside a page: [head_dim][tokens]
+    const int64_t vbase = ((int64_t)page * KVH + kvh) * hd * HE_PAGE_TOKENS + off;
     float part = 0.f;
 #pragma unroll
     for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
@@ -68,7 +70,7 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(
 #pragma unroll
     for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
       const int d = lane + i * HE_WAVE;
-      if (i < npl && d < hd) acc[i] = acc[i] * alpha + w * to_float(vpool[base + d]);
+      if (i < npl && d < hd) acc[i] = acc[i] * alpha + w * to_float(vpool[vbase + (int64_t)d * HE_PAGE_TOKENS]);
     }
     m = m_new;
   }

@@ -8,8 +8,9 @@
 #define HE_F32 0
 #define HE_BF16 1
 
-// Tokens per page of the key/value cache. The pools are laid out
-// [page][kv_head][PAGE_TOKENS][head_dim].
+// Tokens per page of the key/value cache. The K pool is laid out
+// [page][kv_head][PAGE_TOKENS][head_dim], the V pool transposed inside a page:
+// [page][kv_head][head_dim][PAGE_TOKENS].
 #define HE_PAGE_TOKENS 64
 #define HE_PAGE_SHIFT 6
 

@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 3
+#define HE_ABI_VERSION 4
 
 #ifdef __cplusplus
 extern "C" {
@@ -61,7 +61,7 @@ int he_attention_decode_bf16(void* out, const void* q, const void* kpool, const 
                              const void* page_table, int max_blocks, int num_pages, int rows,
                              int H, int KVH, int hd, int window, float scale, int max_keys,
                              void* workspace_f32, int64_t workspace_floats, void* stream);
-int64_t he_attention_decode_workspace_floats(int rows, int H, int hd, int max_keys);
+int64_t he_attention_decode_workspace_floats(int rows, int H, int KVH, int hd, int max_keys);
 // bf16, prompt steps: tiles of queries of one sequence against its cache rows.
 int he_attention_prefill_bf16(void* out, const void* q, const void* kpool, const void* vpool,
                               const void* cu_seqlens, const void* seq_slot, const void* seq_start,

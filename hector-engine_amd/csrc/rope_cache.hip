@@ -105,7 +105,8 @@ __global__ void qkv_rope_cache_kernel(
       const int d = it - h * hd;
       float x = to_float(in[it]);
       if (v_bias) x += load_param(v_bias, it, bias_dtype);
-      vpool[(((int64_t)page * KVH + h) * HE_PAGE_TOKENS + off) * hd + d] = from_float<T>(x);
+      // V is stored transposed inside a page: [head_dim][tokens]
+      vpool[(((int64_t)page * KVH + h) * hd + d) * HE_PAGE_TOKENS + off] = from_float<T>(x);
     }
   }
 }

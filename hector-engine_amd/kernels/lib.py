@@ -16,7 +16,7 @@ _lib = None
 
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 
-EXPECTED_ABI = 3
+EXPECTED_ABI = 4
 
 c_int, c_i64, c_f32, c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
@@ -42,7 +42,7 @@ _SIGNATURES = {
     "he_attention_decode_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_int, c_ptr,
                                  c_i64, c_ptr],
-    "he_attention_decode_workspace_floats": [c_int, c_int, c_int, c_int],
+    "he_attention_decode_workspace_floats": [c_int, c_int, c_int, c_int, c_int],
     "he_attention_prefill_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int,
                                   c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_ptr],
     "he_argmax_rows": [c_ptr, c_ptr, c_int, c_int, c_i64, c_ptr],
@@ -50,8 +50,6 @@ _SIGNATURES = {
                            c_ptr],
     "he_sample_rows": [c_ptr, c_ptr, c_int, c_int, c_i64, c_ptr, c_f32, c_int, c_f32, c_ptr],
 }
-_PENDING = {"he_gemm_skinny_bf16", "he_gemm_skinny_workspace_floats", "he_attention_decode_bf16",
-            "he_attention_decode_workspace_floats", "he_attention_prefill_bf16"}
 _RESTYPES = {
     "he_gemm_skinny_workspace_floats": c_i64,
     "he_attention_decode_workspace_floats": c_i64,
@@ -92,8 +90,6 @@ def load():
         for name, argtypes in _SIGNATURES.items():
             fn = getattr(lib, name, None)
             if fn is None:
-                if name in _PENDING:
-                    continue
                 raise KernelLibraryError(f"{path} lacks the entry point {name}")
             fn.argtypes = argtypes
             fn.restype = _RESTYPES.get(name, c_int)

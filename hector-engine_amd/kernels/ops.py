@@ -192,7 +192,7 @@ def qkv_rope_cache(q_out, kpool, vpool, qkv, q_cols: int, kv_cols: int, bias, po
     max_blocks = num_pages = 0
     if write_kv:
         _need(kpool, "kpool", qkv.dtype, (None, KVH, PAGE_TOKENS, hd))
-        _need(vpool, "vpool", qkv.dtype, (None, KVH, PAGE_TOKENS, hd))
+        _need(vpool, "vpool", qkv.dtype, (None, KVH, hd, PAGE_TOKENS))
         _need(page_table, "page_table", torch.int32)
         num_pages = kpool.shape[0]
         max_blocks = page_table.shape[1]
@@ -223,7 +223,7 @@ def _check_attention(out, q, kpool, vpool, page_table, rows, H, KVH, hd):
     _need(q, "q")
     _need(out, "out", q.dtype)
     _need(kpool, "kpool", q.dtype, (None, KVH, PAGE_TOKENS, hd))
-    _need(vpool, "vpool", q.dtype, (None, KVH, PAGE_TOKENS, hd))
+    _need(vpool, "vpool", q.dtype, (None, KVH, hd, PAGE_TOKENS))
     _need(page_table, "page_table", torch.int32)
     if page_table.dim() != 2:
         raise ValueError("attention: page_table must be [slots, blocks]")
@@ -245,8 +245,8 @@ def attention_plain(out, q, kpool, vpool, positions, row_seq, seq_slot, page_tab
         kpool.shape[0], rows, H, KVH, hd, window, float(scale), dtype_code(q.dtype), _stream()))
 
 
-def attention_decode_workspace_floats(rows: int, H: int, hd: int, max_keys: int) -> int:
-    return int(_lib.load().he_attention_decode_workspace_floats(rows, H, hd, max_keys))
+def attention_decode_workspace_floats(rows: int, H: int, KVH: int, hd: int, max_keys: int) -> int:
+    return int(_lib.load().he_attention_decode_workspace_floats(rows, H, KVH, hd, max_keys))
 
 
 def attention_decode(out, q, kpool, vpool, positions, row_seq, seq_slot, page_table, rows: int,

@@ -114,7 +114,7 @@ class Attention(Mixer):
                                 ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,
                                 self.scale)
         elif ctx.all_single:
-            floats = ops.attention_decode_workspace_floats(rows, H, hd, ctx.max_keys)
+            floats = ops.attention_decode_workspace_floats(rows, H, KVH, hd, ctx.max_keys)
             ws = ctx.alloc((max(floats, 1),), torch.float32)
             ops.attention_decode(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
                                  ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,

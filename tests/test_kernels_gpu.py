@@ -1,0 +1,404 @@
+"""Each HIP kernel alone against a plain fp32/fp64 torch reference of the same
+op, at sizes other than the engine's tiny models (widths that are no power of
+two, head sizes in steps of 16, odd row counts, scattered cache pages)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from tests.plain import qwen2_plain as P
+
+pytestmark = pytest.mark.gpu
+PAGE = 64
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import hector_engine_amd  # noqa: F401
+    from hector_engine_amd.kernels import lib, ops as _ops
+    lib.load()
+    assert lib.loaded_path().endswith(".so")
+    return _ops
+
+
+def dev(t):
+    return t.to("cuda")
+
+
+def rnd(*shape, seed=0, scale=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+# ------------------------------------------------------------------ row-wise
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embedding_rows_and_bad_ids(ops, dtype):
+    V, D = 301, 80
+    table = rnd(V, D, seed=1).to(dtype)
+    ids = torch.tensor([2, 300, 0, -1, 301, 17], dtype=torch.int32)
+    out = torch.empty(len(ids), D, device="cuda")
+    ops.embedding(out, dev(table), dev(ids), len(ids))
+    ref = P.embedding(ids.long(), table.float())
+    assert torch.equal(out.cpu(), ref)           # a copy: exact
+    assert torch.equal(out.cpu()[0], table[2].float())   # the reference's own row check
+    assert out.cpu()[3].abs().max() == 0 and out.cpu()[4].abs().max() == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_silu_mul(ops, dtype):
+    rows, I = 7, 136
+    x = rnd(rows, 2 * I, seed=2, scale=2.0).to(dtype)
+    out = torch.empty(rows, I, dtype=dtype, device="cuda")
+    ops.silu_mul(out, dev(x), rows)
+    xf = x.double()
+    ref = P.silu(xf[:, :I]) * xf[:, I:]
+    tol = 1e-6 if dtype == torch.float32 else 2 ** -7
+    assert torch.allclose(out.cpu().double(), ref, rtol=tol, atol=tol)
+
+
+def test_gather_rows(ops):
+    src = rnd(9, 50, seed=3)
+    idx = torch.tensor([8, 0, 3, 3], dtype=torch.int32)
+    out = torch.empty(4, 50, device="cuda")
+    ops.gather_rows_f32(out, dev(src), dev(idx), 4, 9)
+    assert torch.equal(out.cpu(), src[idx.long()])
+
+
+@pytest.mark.parametrize("dtype,wdtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                          (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("D,eps", [(80, 3e-6), (3584, 1e-6), (100, 1e-5)])
+def test_add_rmsnorm(ops, dtype, wdtype, D, eps):
+    rows = 5
+    resid = rnd(rows, D, seed=4)
+    delta = rnd(rows, D, seed=5).to(dtype)
+    w = (1 + 0.1 * rnd(D, seed=6)).to(wdtype)
+    r = dev(resid.clone())
+    out = torch.empty(rows, D, dtype=dtype, device="cuda")
+    ops.add_rmsnorm(r, dev(delta), dev(w), out, rows, eps)
+    want_r = resid.double() + delta.double()
+    assert torch.allclose(r.cpu().double(), want_r, rtol=1e-6, atol=1e-6)       # residual output
+    ref = P.rmsnorm(r.cpu().double(), w.double(), eps)                           # norm of the stored sum
+    tol = 2e-6 if dtype == torch.float32 else 2 ** -7
+    assert torch.allclose(out.cpu().double(), ref, rtol=tol, atol=tol)
+    # without delta: plain norm, residual untouched
+    r2 = dev(resid.clone())
+    ops.add_rmsnorm(r2, None, dev(w), out, rows, eps)
+    assert torch.equal(r2.cpu(), resid)
+    assert torch.allclose(out.cpu().double(), P.rmsnorm(resid.double(), w.double(), eps), rtol=tol, atol=tol)
+
+
+def test_rmsnorm_rows_strided(ops):
+    rows, D, stride = 6, 48, 100
+    x = rnd(rows, stride, seed=7)
+    w = 1 + 0.1 * rnd(D, seed=8)
+    out = torch.zeros(rows, stride, device="cuda")
+    ops.rmsnorm_rows(out, dev(x), dev(w), rows, D, stride, stride, 1e-5)
+    ref = P.rmsnorm(x[:, :D].double(), w.double(), 1e-5)
+    assert torch.allclose(out.cpu()[:, :D].double(), ref, rtol=2e-6, atol=2e-6)
+    assert out.cpu()[:, D:].abs().max() == 0
+
+
+# ------------------------------------------------------------------ matrix products
+@pytest.mark.parametrize("M,N,K", [(1, 33, 100), (7, 130, 65), (64, 64, 16), (70, 301, 136)])
+def test_gemm_plain_f32(ops, M, N, K):
+    a, w, b = rnd(M, K, seed=9), rnd(N, K, seed=10), rnd(N, seed=11)
+    out = torch.empty(M, N, device="cuda")
+    ops.gemm_plain(out, dev(a), dev(w), dev(b), M)
+    ref = a.double() @ w.double().T + b.double()
+    assert torch.allclose(out.cpu().double(), ref, rtol=1e-5, atol=1e-5)
+    # all-ones gives K (the reference's own matmul check, tests/test_kernels.cu:244-262)
+    ones = torch.ones(M, K), torch.ones(N, K)
+    ops.gemm_plain(out, dev(ones[0]), dev(ones[1]), None, M)
+    assert torch.equal(out.cpu(), torch.full((M, N), float(K)))
+
+
+def test_gemm_plain_rows_do_not_depend_on_the_batch(ops):
+    a, w = rnd(70, 136, seed=12), rnd(301, 136, seed=13)
+    full = torch.empty(70, 301, device="cuda")
+    ops.gemm_plain(full, dev(a), dev(w), None, 70)
+    one = torch.empty(1, 301, device="cuda")
+    for r in (0, 37, 69):
+        ops.gemm_plain(one, dev(a[r:r + 1].contiguous()), dev(w), None, 1)
+        assert torch.equal(one.cpu()[0], full.cpu()[r])      # bit-equal
+
+
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(301, 136), (1000, 520), (37, 4104), (4608, 3584)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_gemm_skinny(ops, M, N, K, out_dtype):
+    if (N, K) == (4608, 3584) and M not in (1, 8, 64):
+        pytest.skip("large shape at three row counts only")
+    a = rnd(M, K, seed=14).to(torch.bfloat16)
+    w = rnd(N, K, seed=15, scale=0.05).to(torch.bfloat16)
+    b = rnd(N, seed=16).to(torch.bfloat16)
+    out = torch.empty(M, N, dtype=out_dtype, device="cuda")
+    floats = ops.gemm_skinny_workspace_floats(M, N, K)
+    ws = torch.empty(max(floats, 1), device="cuda")
+    ops.gemm_skinny(out, dev(a), dev(w), dev(b), M, ws)
+    ref = a.double() @ w.double().T + b.double()
+    scale = ref.abs().max().item()
+    err = (out.cpu().double() - ref).abs().max().item()
+    tol = 2e-5 * scale * math.sqrt(K / 64) if out_dtype == torch.float32 else 2 ** -8 * scale + 1e-6
+    assert err <= tol, (err, tol)
+    # the plain kernel agrees too (same inputs, fp32 accumulation)
+    plain = torch.empty(M, N, dtype=out_dtype, device="cuda")
+    ops.gemm_plain(plain, dev(a), dev(w), dev(b), M)
+    assert (plain.cpu().double() - ref).abs().max().item() <= tol
+
+
+def test_gemm_skinny_refuses_bad_sizes(ops):
+    from hector_engine_amd.kernels.lib import KernelLibraryError
+    a = torch.zeros(2, 20, dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(16, 20, dtype=torch.bfloat16, device="cuda")
+    out = torch.empty(2, 16, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(KernelLibraryError, match="multiple of 8"):
+        ops.gemm_skinny(out, a, w, None, 2, torch.empty(1, device="cuda"))
+
+
+# ------------------------------------------------------------------ rope + cache + attention
+def paged_setup(lengths, KVH, hd, dtype, seed, extra_pages=3):
+    """Scattered pages: a random permutation of page ids, slots in reverse order."""
+    g = torch.Generator().manual_seed(seed)
+    B = len(lengths)
+    blocks = [(n + PAGE - 1) // PAGE for n in lengths]
+    num_pages = sum(blocks) + extra_pages
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    max_blocks = max(blocks) + 1
+    slots = list(range(B))[::-1]
+    table = torch.full((B + 1, max_blocks), -1, dtype=torch.int32)
+    it = iter(perm)
+    for s, nb in zip(slots, blocks):
+        for b in range(nb):
+            table[s, b] = next(it)
+    kpool = torch.zeros(num_pages, KVH, PAGE, hd, dtype=dtype)
+    vpool = torch.zeros(num_pages, KVH, hd, PAGE, dtype=dtype)
+    return slots, table, kpool, vpool
+
+
+def fill_cache(table, slots, kpool, vpool, ks, vs):
+    for s, k, v in zip(slots, ks, vs):
+        for p in range(k.shape[0]):
+            page = table[s, p // PAGE].item()
+            kpool[page, :, p % PAGE, :] = k[p]
+            vpool[page, :, :, p % PAGE] = v[p]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,KVH,hd,rot", [(6, 3, 48, 48), (4, 1, 64, 32), (5, 5, 16, 0)])
+def test_qkv_rope_cache(ops, dtype, H, KVH, hd, rot):
+    lengths = [70, 5, 130]           # new tokens start at these offsets
+    new = [3, 64, 1]
+    theta = 50000.0
+    slots, table, kpool, vpool = paged_setup([a + b for a, b in zip(lengths, new)], KVH, hd, dtype, 20)
+    rows = sum(new)
+    width = (H + 2 * KVH) * hd
+    qkv = rnd(rows, width, seed=21).to(dtype)
+    bias = rnd(width, seed=22).to(dtype)
+    positions = torch.cat([torch.arange(a, a + b) for a, b in zip(lengths, new)]).int()
+    row_seq = torch.cat([torch.full((b,), i) for i, b in enumerate(new)]).int()
+    # a padding row at the end must be left alone
+    qkv = torch.cat([qkv, torch.zeros(1, width, dtype=dtype)])
+    positions = torch.cat([positions, torch.zeros(1, dtype=torch.int32)])
+    row_seq = torch.cat([row_seq, torch.full((1,), -1, dtype=torch.int32)])
+    seq_slot = torch.tensor(slots, dtype=torch.int32)
+    inv = P.rope_inv_freq(rot, theta) if rot else None
+    q_out = torch.zeros(rows + 1, H * hd, dtype=dtype, device="cuda")
+    kp, vp = dev(kpool), dev(vpool)
+    ops.qkv_rope_cache(q_out, kp, vp, dev(qkv), H * hd, KVH * hd, dev(bias), dev(positions),
+                       dev(row_seq), dev(seq_slot), dev(table), dev(inv) if rot else None, rot,
+                       rows + 1, H, KVH, hd, True)
+    x = (qkv[:rows].double() + bias.double())
+    q = x[:, :H * hd].reshape(rows, H, hd)
+    k = x[:, H * hd:(H + KVH) * hd].reshape(rows, KVH, hd)
+    v = x[:, (H + KVH) * hd:].reshape(rows, KVH, hd)
+    pos = positions[:rows]
+    if rot:
+        q, k = P.rope(q, pos, theta, rot), P.rope(k, pos, theta, rot)
+    tol = 3e-6 if dtype == torch.float32 else 2 ** -7
+    assert torch.allclose(q_out.cpu()[:rows].double().reshape(rows, H, hd), q, rtol=tol, atol=tol * 4)
+    kp, vp = kp.cpu(), vp.cpu()
+    for r in range(rows):
+        s = slots[row_seq[r]]
+        page = table[s, pos[r] // PAGE].item()
+        assert torch.allclose(kp[page, :, pos[r] % PAGE, :].double(), k[r], rtol=tol, atol=tol * 4)
+        assert torch.allclose(vp[page, :, :, pos[r] % PAGE].double(), v[r], rtol=tol, atol=tol * 4)
+    # nothing else in the pools was touched
+    assert (kp != 0).sum().item() <= rows * KVH * hd
+
+
+def attention_case(ops, kind, dtype, H, KVH, hd, window, lengths, q_lens, seed, pad=0):
+    """Runs one attention kernel over a crafted cache; returns (got, want) lists per sequence."""
+    B = len(lengths)
+    slots, table, kpool, vpool = paged_setup(lengths, KVH, hd, dtype, seed)
+    ks = [rnd(n, KVH, hd, seed=seed + 10 + i).to(dtype) for i, n in enumerate(lengths)]
+    vs = [rnd(n, KVH, hd, seed=seed + 20 + i).to(dtype) for i, n in enumerate(lengths)]
+    fill_cache(table, slots, kpool, vpool, ks, vs)
+    qs = [rnd(m, H, hd, seed=seed + 30 + i, scale=2.0).to(dtype) for i, m in enumerate(q_lens)]
+    rows = sum(q_lens)
+    q = torch.cat(qs + [torch.zeros(pad, H, hd, dtype=dtype)]).reshape(rows + pad, H * hd)
+    positions = torch.cat([torch.arange(n - m, n) for n, m in zip(lengths, q_lens)] +
+                          [torch.zeros(pad, dtype=torch.int64)]).int()
+    row_seq = torch.cat([torch.full((m,), i) for i, m in enumerate(q_lens)] +
+                        [torch.full((pad,), -1)]).int()
+    cu = torch.tensor([0] + list(np.cumsum(q_lens)), dtype=torch.int32)
+    seq_start = torch.tensor([n - m for n, m in zip(lengths, q_lens)], dtype=torch.int32)
+    seq_slot = torch.tensor(slots, dtype=torch.int32)
+    out = torch.full((rows + pad, H * hd), 7.0, dtype=dtype, device="cuda")
+    scale = 1.0 / math.sqrt(hd)
+    args = (dev(kpool), dev(vpool))
+    if kind == "plain":
+        ops.attention_plain(out, dev(q), *args, dev(positions), dev(row_seq), dev(seq_slot),
+                            dev(table), rows + pad, H, KVH, hd, window, scale)
+    elif kind == "decode":
+        max_keys = 4096
+        ws = torch.empty(ops.attention_decode_workspace_floats(rows + pad, H, KVH, hd, max_keys), device="cuda")
+        ops.attention_decode(out, dev(q), *args, dev(positions), dev(row_seq), dev(seq_slot),
+                             dev(table), rows + pad, H, KVH, hd, window, scale, max_keys, ws)
+    else:
+        ops.attention_prefill(out, dev(q), *args, dev(cu), dev(seq_slot), dev(seq_start), dev(table),
+                              B, max(q_lens), rows, H, KVH, hd, window, scale)
+    got, want = [], []
+    r = 0
+    for i, (n, m) in enumerate(zip(lengths, q_lens)):
+        got.append(out.cpu()[r:r + m].double())
+        want.append(P.attention(qs[i].double(), ks[i].double(), vs[i].double(),
+                                torch.arange(n - m, n), torch.arange(n), window))
+        r += m
+    if pad and kind != "prefill":
+        assert out.cpu()[rows:].abs().max() == 0     # padding rows give zeros
+    return got, want
+
+
+ATT_SHAPES = [(6, 3, 48), (4, 1, 64), (28, 4, 128), (5, 5, 16), (2, 1, 80)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,KVH,hd", ATT_SHAPES)
+@pytest.mark.parametrize("window", [0, 70])
+def test_attention_plain(ops, dtype, H, KVH, hd, window):
+    got, want = attention_case(ops, "plain", dtype, H, KVH, hd, window, [200, 3, 65], [5, 3, 1], 40, pad=2)
+    tol = 3e-6 if dtype == torch.float32 else 2 ** -6
+    for g, w in zip(got, want):
+        assert torch.allclose(g, w, rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("H,KVH,hd", ATT_SHAPES + [(40, 2, 32)])
+@pytest.mark.parametrize("window", [0, 70])
+def test_attention_decode(ops, H, KVH, hd, window):
+    got, want = attention_case(ops, "decode", torch.bfloat16, H, KVH, hd, window,
+                               [700, 1, 64, 65, 300], [1, 1, 1, 1, 1], 41, pad=3)
+    for g, w in zip(got, want):
+        assert torch.allclose(g, w, rtol=2 ** -6, atol=2 ** -6)
+
+
+@pytest.mark.parametrize("H,KVH,hd", ATT_SHAPES)
+@pytest.mark.parametrize("window", [0, 70])
+def test_attention_prefill(ops, H, KVH, hd, window):
+    # whole prompts, a continuation (200 cached + 37 new) and a single token
+    got, want = attention_case(ops, "prefill", torch.bfloat16, H, KVH, hd, window,
+                               [150, 237, 3, 66], [150, 37, 3, 1], 42)
+    for g, w in zip(got, want):
+        assert torch.allclose(g, w, rtol=2 ** -6, atol=2 ** -6)
+
+
+def test_attention_far_key_stands_out(ops):
+    """One far key is made to dominate: a kernel that drops or misplaces it fails."""
+    H, KVH, hd, n = 4, 2, 64, 900
+    for kind in ("plain", "decode", "prefill"):
+        slots, table, kpool, vpool = paged_setup([n], KVH, hd, torch.bfloat16, 50)
+        k = rnd(n, KVH, hd, seed=51, scale=0.1).to(torch.bfloat16)
+        v = rnd(n, KVH, hd, seed=52).to(torch.bfloat16)
+        q = rnd(1, H, hd, seed=53, scale=0.1).to(torch.bfloat16)
+        far = 17
+        k[far] = (q[0, ::2] * 300).to(torch.bfloat16)      # aligned with the query of each group's first head
+        fill_cache(table, slots, kpool, vpool, [k], [v])
+        out = torch.empty(1, H * hd, dtype=torch.bfloat16, device="cuda")
+        pos = torch.tensor([n - 1], dtype=torch.int32)
+        zero = torch.zeros(1, dtype=torch.int32)
+        scale = 1 / math.sqrt(hd)
+        if kind == "plain":
+            ops.attention_plain(out, dev(q.reshape(1, -1)), dev(kpool), dev(vpool), dev(pos), dev(zero),
+                                dev(torch.tensor(slots, dtype=torch.int32)), dev(table), 1, H, KVH, hd, 0, scale)
+        elif kind == "decode":
+            ws = torch.empty(ops.attention_decode_workspace_floats(1, H, KVH, hd, 4096), device="cuda")
+            ops.attention_decode(out, dev(q.reshape(1, -1)), dev(kpool), dev(vpool), dev(pos), dev(zero),
+                                 dev(torch.tensor(slots, dtype=torch.int32)), dev(table), 1, H, KVH, hd, 0,
+                                 scale, 4096, ws)
+        else:
+            ops.attention_prefill(out, dev(q.reshape(1, -1)), dev(kpool), dev(vpool),
+                                  dev(torch.tensor([0, 1], dtype=torch.int32)),
+                                  dev(torch.tensor(slots, dtype=torch.int32)),
+                                  dev(torch.tensor([n - 1], dtype=torch.int32)), dev(table), 1, 1, 1,
+                                  H, KVH, hd, 0, scale)
+        want = P.attention(q.double(), k.double(), v.double(), torch.tensor([n - 1]), torch.arange(n), 0)
+        got = out.cpu().double()
+        assert torch.allclose(got, want, rtol=2 ** -6, atol=2 ** -6), kind
+        # heads 0 and 2 must return (almost) the far value
+        assert torch.allclose(got.reshape(H, hd)[0], v[far, 0].double(), atol=0.05), kind
+
+
+# ------------------------------------------------------------------ sampling
+def test_argmax_lowest_index_on_ties(ops):
+    V = 1000
+    x = rnd(4, V, seed=60)
+    x[0, 500] = x[0, 77] = 9.0
+    x[1, :] = 1.0                          # all equal -> index 0
+    x[2, 999] = 50.0
+    x[3, 3] = x[3, 2] = x[3, 998] = 8.0
+    out = torch.empty(4, dtype=torch.int32, device="cuda")
+    ops.argmax_rows(out, dev(x), 4)
+    assert out.tolist() == [77, 0, 999, 2]
+    assert out.tolist() == [P.argmax_lowest(r) for r in x]
+
+
+def test_penalties(ops):
+    V = 50
+    x = rnd(2, V, seed=61)
+    ctx = [[3, 3, 7, 49], [0]]
+    ids = torch.tensor([3, 7, 49, 0], dtype=torch.int32)
+    counts = torch.tensor([2, 1, 1, 1], dtype=torch.int32)
+    offsets = torch.tensor([0, 3, 4], dtype=torch.int32)
+    d = dev(x.clone())
+    ops.apply_penalties(d, 2, dev(ids), dev(counts), dev(offsets), 1.15, 0.1, 0.05)
+    for r in range(2):
+        want = P.apply_penalties(x[r], ctx[r], 384, 1.15, 0.1, 0.05)
+        assert torch.allclose(d.cpu()[r], want, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("V", [301, 5000, 152064])
+@pytest.mark.parametrize("temperature,top_k,top_p", [(0.8, 0, 1.0), (1.0, 50, 0.9), (0.7, 40, 1.0),
+                                                     (1.3, 0, 0.5), (0.05, 0, 1.0), (1.0, 1, 1.0)])
+def test_sample_rows_equals_plain(ops, V, temperature, top_k, top_p):
+    rows = 6
+    x = rnd(rows, V, seed=62, scale=2.0)
+    x[1, 5] = x[1, 9] = x[1].max() + 1          # a tie at the top
+    us = [0, 1, 2 ** 31, 2 ** 32 - 1, 123456789, 3000000000]
+    u = torch.tensor(us, dtype=torch.int64).to(torch.uint32)
+    out = torch.empty(rows, dtype=torch.int32, device="cuda")
+    ops.sample_rows(out, dev(x), rows, dev(u), temperature, top_k, top_p)
+    got = out.tolist()
+    want = [P.sample(x[r], temperature, top_k, top_p, us[r]) for r in range(rows)]
+    if got != want:
+        # exp() may differ in the last bit between the GPU and the CPU; then the draw must lie on
+        # a boundary: both tokens adjacent in the sorted order
+        for r in range(rows):
+            if got[r] != want[r]:
+                order = torch.argsort(-x[r].double(), stable=True).tolist()
+                assert abs(order.index(got[r]) - order.index(want[r])) == 1, (r, got[r], want[r])
+    if top_k == 1:
+        assert got == [P.argmax_lowest(r) for r in x]
+
+
+def test_sample_frequencies(ops):
+    """Empirical frequencies follow softmax(logits / T) on a small vocabulary."""
+    V, n = 8, 20000
+    logits = torch.tensor([2.0, 1.0, 0.5, 0.0, -1.0, 1.5, -3.0, 0.2])
+    x = logits.repeat(n, 1).contiguous()
+    u = torch.tensor([P.uniform_u32(7, 0, i) for i in range(n)], dtype=torch.int64).to(torch.uint32)
+    out = torch.empty(n, dtype=torch.int32, device="cuda")
+    ops.sample_rows(out, dev(x), n, dev(u), 0.8, 0, 1.0)
+    freq = torch.bincount(out.cpu().long(), minlength=V).double() / n
+    p = torch.softmax(logits.double() / 0.8, 0)
+    chi2 = (n * (freq - p) ** 2 / p).sum().item()
+    assert chi2 < 30, chi2                        # 7 degrees of freedom; 30 is far in the tail
