@@ -1,0 +1,172 @@
+#!/usr/bin/env python3
+"""Decode throughput of the Qwen2.5-7B shape (bf16, random weights, synthetic
+token ids) on one MI355X, with prefill and roofline figures on the same line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+
+A step is one decode step of the whole batch: the engine's step function (HIP
+graph replay) plus greedy sampling and the copy of the chosen ids to the host.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+import numpy as np
+
+# Qwen2.5-7B layer sizes (BASELINE.json configs[2])
+SHAPE = dict(num_hidden_layers=28, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
+             head_dim=128, intermediate_size=18944, vocab_size=152064, rope_theta=1000000.0,
+             rms_norm_eps=1e-6, max_position_embeddings=32768, tie_word_embeddings=False)
+FULL_LAYERS = 28
+CONTEXT = 8192
+PROMPT = 2048
+HBM_PEAK_GBS = 8000.0
+BF16_PEAK_FLOPS = 2.5e15
+
+
+def weight_bytes(c, layers):
+    D, H, KVH, hd, I, V = (c["hidden_size"], c["num_attention_heads"], c["num_key_value_heads"],
+                           c["head_dim"], c["intermediate_size"], c["vocab_size"])
+    per_layer = D * (H + 2 * KVH) * hd + (H + 2 * KVH) * hd + H * hd * D + 3 * D * I + 2 * D
+    return 2 * (layers * per_layer + D + V * D)      # lm_head read once; embedding rows are negligible
+
+
+def kv_bytes_per_token(c, layers):
+    return 2 * layers * c["num_key_value_heads"] * c["head_dim"] * 2
+
+
+def prefill_flops(c, layers, T):
+    D, H, KVH, hd, I, V = (c["hidden_size"], c["num_attention_heads"], c["num_key_value_heads"],
+                           c["head_dim"], c["intermediate_size"], c["vocab_size"])
+    gemm = 2 * T * (D * (H + 2 * KVH) * hd + H * hd * D + 3 * D * I)
+    attn = 4 * H * hd * T * (T + 1) // 2
+    return layers * (gemm + attn) + 2 * D * V
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    import hector_engine_amd as he
+    from hector_engine_amd.config.qwen2 import Qwen2Config
+    from hector_engine_amd.engine.engine import StepEntry
+
+    cfg_dict = dict(SHAPE, num_hidden_layers=args.layers, architectures=["Qwen2ForCausalLM"])
+    config = Qwen2Config.from_dict(cfg_dict)
+    max_batch = args.batch if args.no_points else max(args.batch, 64)
+    t_load = time.perf_counter()
+    engine = he.Engine(config=config, seed=0, dtype="bfloat16", max_tokens=max_batch * CONTEXT,
+                       max_slots=max_batch, max_seq_len=CONTEXT)
+    sampler = he.Sampler(he.SamplingConfig.deterministic(), engine.device)
+    torch.cuda.synchronize()
+    load_s = time.perf_counter() - t_load
+    rng = np.random.default_rng(0)
+
+    def prompts(n):
+        return [rng.integers(0, SHAPE["vocab_size"], PROMPT).tolist() for _ in range(n)]
+
+    def prefill(ps, slots):
+        """Prompts in groups of 8 sequences a step; returns the first sampled tokens."""
+        toks = []
+        for g in range(0, len(ps), 8):
+            entries = [StepEntry(s, p, [len(p) - 1]) for s, p in zip(slots[g:g + 8], ps[g:g + 8])]
+            logits = engine.step(entries)
+            toks += sampler.sample(logits, list(range(len(entries))), [0] * len(entries))
+        return toks
+
+    def decode_run(batch, steps, warmup):
+        slots = [engine.acquire() for _ in range(batch)]
+        toks = prefill(prompts(batch), slots)
+        seqs = list(range(batch))
+
+        def one(toks):
+            logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)])
+            return sampler.sample(logits, seqs, [0] * batch)
+
+        for _ in range(warmup):
+            toks = one(toks)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            toks = one(toks)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        avg_len = PROMPT + warmup + steps / 2
+        for s in slots:
+            engine.release(s)
+        return dt / steps, avg_len
+
+    # ---- prefill of one 2,048-token prompt (second run timed; the first warms the library GEMMs)
+    slot = engine.acquire()
+    p = prompts(1)[0]
+    engine.step([StepEntry(slot, p, [PROMPT - 1])])
+    engine.release(slot)
+    slot = engine.acquire()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    engine.step([StepEntry(slot, p, [PROMPT - 1])])
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t0
+    engine.release(slot)
+    flops = prefill_flops(SHAPE, args.layers, PROMPT)
+
+    # ---- decode at the headline batch
+    step_s, avg_len = decode_run(args.batch, args.steps, args.warmup)
+    wbytes = weight_bytes(SHAPE, args.layers)
+    step_bytes = wbytes + args.batch * avg_len * kv_bytes_per_token(SHAPE, args.layers)
+    achieved = step_bytes / step_s / 1e9
+
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            s, _ = decode_run(b, max(8, args.steps // 2), max(3, args.warmup // 2))
+            points[f"decode_b{b}"] = round(b / s, 1)
+
+    line = {
+        "metric": "decode tok/s @ bs 8, Qwen2.5-7B shape bf16, context 8192, prompts 2048",
+        "value": round(args.batch / step_s, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic token ids (uniform), random N(0, 0.02) weights",
+        "config": {
+            "model": "Qwen2.5-7B shape", "layers": args.layers, "layers_full": FULL_LAYERS,
+            "hidden_size": SHAPE["hidden_size"], "heads": SHAPE["num_attention_heads"],
+            "kv_heads": SHAPE["num_key_value_heads"], "head_dim": SHAPE["head_dim"],
+            "intermediate_size": SHAPE["intermediate_size"], "vocab_size": SHAPE["vocab_size"],
+            "rope_theta": SHAPE["rope_theta"], "rms_norm_eps": SHAPE["rms_norm_eps"],
+            "global_batch": args.batch, "seq_len": CONTEXT, "prompt_len": PROMPT,
+            "parallelism": "single GPU", "sampling": "greedy", "load_s": round(load_s, 1),
+        },
+        "prefill": {"value": round(PROMPT / prefill_s, 1), "tokens": PROMPT,
+                    "ms": round(prefill_s * 1e3, 3),
+                    "frac": round(flops / prefill_s / BF16_PEAK_FLOPS, 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,138 @@
+"""The generation loop above the step function: batches of unequal prompts,
+stop tokens, sequences that end earlier, and as many batches one after another
+as there are requests.
+
+Reference loop: prefill gives the first token; then, per token, stop checks,
+record, sample the next (src/inference_session.cpp:597-660). A stop token ends
+its sequence, is not fed back and is not part of the result (:611-615). Finish
+reasons follow the reference's names (:59-67): "eos", "max_tokens", "stop"
+(the sequence has filled its cache room; the reference stops at pos + 4 >=
+max_seq, :616-619), "cancelled", and "context_full" for a request that is
+refused at admission (:530-534).
+"""
+from __future__ import annotations
+
+import dataclasses
+import time
+from typing import Callable
+
+from ..cache.pages import PAGE_TOKENS, blocks_for
+from .engine import StepEntry
+
+
+@dataclasses.dataclass
+class GenerationResult:
+    tokens: list[int]
+    finish_reason: str
+    prompt_tokens: int
+    prefill_ms: float = 0.0
+    decode_ms: float = 0.0
+
+
+def plan_batch(pending: list[tuple[int, int]], max_new_tokens: int, free_pages: int,
+               free_slots: int, max_seq_len: int, batch_size: int | None) -> tuple[list[int], list[int]]:
+    """pending: (request index, prompt length) in order. Returns (admitted, refused)
+    for the next batch: requests are admitted in order while slots and pages for
+    prompt + max_new_tokens remain; a request that can never run is refused."""
+    admitted, refused = [], []
+    pages_left = free_pages
+    limit = free_slots if batch_size is None else min(free_slots, batch_size)
+    for idx, n in pending:
+        if n < 1 or n + 1 > max_seq_len:
+            refused.append(idx)
+            continue
+        need = blocks_for(min(n + max_new_tokens, max_seq_len))
+        if need > free_pages and not admitted:
+            refused.append(idx)          # would not fit even in an empty cache
+            continue
+        if len(admitted) >= limit or need > pages_left:
+            break
+        admitted.append(idx)
+        pages_left -= need
+    return admitted, refused
+
+
+def after_token(token: int, generated: int, max_new_tokens: int, length: int, max_seq_len: int,
+                stop_ids) -> tuple[bool, str | None]:
+    """Decision after sampling `token` as the (generated+1)-th new token of a
+    sequence whose cache holds `length` tokens. Returns (keep the token, finish
+    reason or None to go on)."""
+    if token in stop_ids:
+        return False, "eos"
+    if generated + 1 >= max_new_tokens:
+        return True, "max_tokens"
+    if length + 1 > max_seq_len:
+        return True, "stop"              # no room to feed this token back
+    return True, None
+
+
+def generate(engine, prompts: list[list[int]], *, max_new_tokens: int = 100, sampling=None,
+             stop_ids=(), include_stop: bool = False, batch_size: int | None = None,
+             cancel: Callable[[], bool] | None = None, sample_fn=None) -> list[GenerationResult]:
+    """Generates for every prompt; returns results in the order of `prompts`."""
+    from ..sampling import Sampler, SamplingConfig
+    if sample_fn is None:
+        sampler = Sampler(sampling or SamplingConfig.deterministic(), engine.device)
+        sample_fn = sampler.sample
+    stop_ids = frozenset(int(s) for s in stop_ids)
+    results: list[GenerationResult | None] = [None] * len(prompts)
+    pending = [(i, len(p)) for i, p in enumerate(prompts)]
+    if max_new_tokens < 1:
+        return [GenerationResult([], "max_tokens", len(p)) for p in prompts]
+    while pending:
+        admitted, refused = plan_batch(pending, max_new_tokens, engine.cache.free_pages,
+                                       engine.cache.book.slots.available, engine.max_seq_len,
+                                       batch_size)
+        for i in refused:
+            results[i] = GenerationResult([], "context_full", len(prompts[i]))
+        done = set(admitted) | set(refused)
+        pending = [p for p in pending if p[0] not in done]
+        if not admitted:
+            if not refused:
+                raise RuntimeError("the cache holds other sequences and no request fits beside them")
+            continue
+        _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, include_stop,
+                   cancel, sample_fn)
+    return results
+
+
+def _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, include_stop, cancel,
+               sample_fn) -> None:
+    slots = {i: engine.acquire() for i in admitted}
+    out: dict[int, list[int]] = {i: [] for i in admitted}
+    t0 = time.perf_counter()
+    try:
+        logits = engine.step([StepEntry(slots[i], prompts[i], [len(prompts[i]) - 1]) for i in admitted])
+        active = list(admitted)
+        tokens = sample_fn(logits, active, [0] * len(active), [out[i] for i in active])
+        prefill_ms = (time.perf_counter() - t0) * 1e3
+        t1 = time.perf_counter()
+
+        def finish(i, reason):
+            results[i] = GenerationResult(out[i], reason, len(prompts[i]), prefill_ms,
+                                          (time.perf_counter() - t1) * 1e3)
+            engine.release(slots.pop(i))     # the slot goes back at once
+
+        while active:
+            if cancel is not None and cancel():
+                for i in active:
+                    finish(i, "cancelled")
+                break
+            feed = []
+            for i, tok in zip(active, tokens):
+                keep, reason = after_token(tok, len(out[i]), max_new_tokens, engine.length(slots[i]),
+                                           engine.max_seq_len, stop_ids)
+                if keep or include_stop:
+                    out[i].append(tok)
+                if reason is not None:
+                    finish(i, reason)
+                else:
+                    feed.append((i, tok))
+            active = [i for i, _ in feed]
+            if not active:
+                break
+            logits = engine.step([StepEntry(slots[i], [tok], [0]) for i, tok in feed])
+            tokens = sample_fn(logits, active, [len(out[i]) for i in active], [out[i] for i in active])
+    finally:
+        for i in list(slots):
+            engine.release(slots.pop(i))

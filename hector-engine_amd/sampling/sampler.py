@@ -1,0 +1,118 @@
+"""Sampling options and the batched sampler.
+
+The options carry the reference's names, defaults and presets
+(src/sampler.hpp:26-52): temperature (below 0.01 means greedy,
+src/sampler.cpp:141), top_k (0 = off), top_p (1.0 = off), repetition_penalty,
+frequency_penalty, presence_penalty, seed; penalties look back over the last
+`penalty_window` generated tokens (src/sampler.hpp:134, src/sampler.cpp:41-91).
+With top_k = 0 the whole vocabulary is sampled (the reference's kernel puts 50
+in its place: src/sampler.cpp:172-174). All rows of a step are sampled by one
+launch and only the chosen ids come back to the host.
+"""
+from __future__ import annotations
+
+import dataclasses
+
+import numpy as np
+import torch
+
+from ..kernels import ops
+from .rng import uniform_u32
+
+GREEDY_BELOW = 0.01
+
+
+@dataclasses.dataclass
+class SamplingConfig:
+    temperature: float = 1.0
+    top_k: int = 0
+    top_p: float = 1.0
+    repetition_penalty: float = 1.0
+    frequency_penalty: float = 0.0
+    presence_penalty: float = 0.0
+    seed: int = 0
+    penalty_window: int = 128
+
+    @classmethod
+    def greedy(cls):
+        return cls(temperature=0.0, repetition_penalty=1.2)
+
+    @classmethod
+    def creative(cls, temp: float = 0.8, k: int = 50, p: float = 0.9):
+        return cls(temperature=temp, top_k=k, top_p=p, repetition_penalty=1.15, frequency_penalty=0.1)
+
+    @classmethod
+    def balanced(cls, temp: float = 0.7, k: int = 40):
+        return cls(temperature=temp, top_k=k, repetition_penalty=1.2)
+
+    @classmethod
+    def deterministic(cls):
+        return cls(temperature=0.0)
+
+    @property
+    def is_greedy(self) -> bool:
+        return self.temperature < GREEDY_BELOW
+
+    @property
+    def has_penalties(self) -> bool:
+        return (self.repetition_penalty != 1.0 or self.frequency_penalty != 0.0
+                or self.presence_penalty != 0.0)
+
+    def validate(self) -> None:
+        if self.temperature < 0:
+            raise ValueError("temperature must not be negative")
+        if self.top_k < 0:
+            raise ValueError("top_k must not be negative")
+        if not 0.0 < self.top_p <= 1.0:
+            raise ValueError("top_p must lie in (0, 1]")
+        if self.repetition_penalty <= 0:
+            raise ValueError("repetition_penalty must be positive")
+        if self.penalty_window < 0:
+            raise ValueError("penalty_window must not be negative")
+
+
+def window_counts(context: list[int], window: int, vocab: int) -> tuple[list[int], list[int]]:
+    """Distinct ids of the last `window` context tokens with their counts, in
+    order of first appearance (src/sampler.cpp:55-74)."""
+    counts: dict[int, int] = {}
+    for t in context[max(0, len(context) - window):]:
+        if 0 <= t < vocab:
+            counts[t] = counts.get(t, 0) + 1
+    return list(counts.keys()), list(counts.values())
+
+
+class Sampler:
+    def __init__(self, config: SamplingConfig, device):
+        config.validate()
+        self.config = config
+        self.device = device
+
+    def sample(self, logits: torch.Tensor, sequences: list[int], steps: list[int],
+               contexts: list[list[int]] | None = None) -> list[int]:
+        """logits: fp32 [rows, vocab] on the device; sequences[r] and steps[r] key
+        the row's random draw; contexts[r] are the row's generated tokens so far.
+        Returns the chosen ids (one device-to-host copy, which synchronises)."""
+        cfg = self.config
+        rows, V = logits.shape
+        if cfg.has_penalties and contexts is not None and any(contexts):
+            ids, counts, offsets = [], [], [0]
+            for ctx in contexts:
+                i, c = window_counts(ctx, cfg.penalty_window, V)
+                ids += i
+                counts += c
+                offsets.append(len(ids))
+            packed = torch.tensor([ids + offsets, counts + [0] * len(offsets)], dtype=torch.int32)
+            packed = packed.to(self.device)
+            n = len(ids)
+            logits = logits.clone()     # penalties work on a copy (src/sampler.cpp:126-139)
+            ops.apply_penalties(logits, rows, packed[0, :n].contiguous(), packed[1, :n].contiguous(),
+                                packed[0, n:].contiguous(), cfg.repetition_penalty,
+                                cfg.frequency_penalty, cfg.presence_penalty)
+        out = torch.empty(rows, dtype=torch.int32, device=self.device)
+        if cfg.is_greedy:
+            ops.argmax_rows(out, logits, rows)
+        else:
+            u = np.array([uniform_u32(cfg.seed, s, t) for s, t in zip(sequences, steps)], dtype=np.uint32)
+            ud = torch.from_numpy(u.view(np.int32)).to(self.device)
+            ops.sample_rows(out, logits, rows, ud, cfg.temperature, cfg.top_k, cfg.top_p)
+        return out.tolist()
