@@ -262,6 +262,7 @@ class Engine:
                 logits = self.model.forward(bucket.views["tokens"], ctx, self.caches,
                                             bucket.views["want_rows"], size)
                 return logits[:n]
+            bucket.pool.reset()          # sized by the eager run; from here on it must not move
             bucket.pool.frozen = True
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()

@@ -17,6 +17,7 @@ class ScratchPool:
         self.capacity = 0
         self.offset = 0
         self.peak = 0
+        self.step_total = 0
         self.frozen = False
         self._arena: torch.Tensor | None = None
         self._grow(initial_bytes)
@@ -29,7 +30,13 @@ class ScratchPool:
         self.offset = 0
 
     def reset(self) -> None:
+        """Starts a new step. If the last step outgrew the arena on its way, the arena
+        is made large enough to hold a whole such step in one piece."""
+        if self.step_total > self.capacity and not self.frozen:
+            self.capacity = 0
+            self._grow(self.step_total + self.step_total // 8)
         self.offset = 0
+        self.step_total = 0
 
     def alloc(self, shape, dtype: torch.dtype) -> torch.Tensor:
         numel = 1
@@ -41,5 +48,6 @@ class ScratchPool:
             self._grow(self.offset + padded)
         view = self._arena[self.offset:self.offset + nbytes].view(dtype).view(*shape)
         self.offset += padded
-        self.peak = max(self.peak, self.offset)
+        self.step_total += padded
+        self.peak = max(self.peak, self.step_total)
         return view

@@ -1,0 +1,120 @@
+"""The cache's bookkeeping on the host: no slot or page is lost, held twice or
+freed twice; windowed groups give back pages that left the window; a step gets
+all its pages or none."""
+import random
+
+import pytest
+
+import hector_engine_amd  # noqa: F401
+from hector_engine_amd.cache import CacheError, CacheFull, FreeList, GroupPages, SlotBook, blocks_for
+
+
+def book(pages=16, slots=4, max_blocks=8, windows=(0,)):
+    return SlotBook(slots, max_blocks, [GroupPages(pages, w, str(i)) for i, w in enumerate(windows)])
+
+
+def test_free_list_lowest_first_and_double_free():
+    f = FreeList(3, "thing")
+    assert [f.take(), f.take(), f.take()] == [0, 1, 2]
+    with pytest.raises(CacheFull):
+        f.take()
+    f.give_back(1)
+    f.give_back(0)
+    with pytest.raises(CacheError, match="not held"):
+        f.give_back(0)
+    assert f.take() == 0 and f.take() == 1          # reuse is deterministic: lowest first
+    with pytest.raises(CacheError):
+        f.give_back(7)
+
+
+def test_slots_are_reused_and_pages_come_back():
+    b = book()
+    s0, s1 = b.acquire(), b.acquire()
+    assert (s0, s1) == (0, 1)
+    added = b.reserve(s0, 130)
+    assert [(g, s, blk) for g, s, blk, _ in added] == [(0, 0, 0), (0, 0, 1), (0, 0, 2)]
+    b.commit(s0, 130)
+    b.reserve(s1, 64)
+    b.commit(s1, 64)
+    b.check_invariants()
+    assert b.groups[0].pool.available == 16 - 4
+    cleared = b.release(s0)
+    assert len(cleared) == 3 and b.groups[0].pool.available == 15
+    assert b.acquire() == 0                            # the freed slot is handed out again
+    with pytest.raises(CacheError):
+        b.release(3)                                   # never acquired
+    b.check_invariants()
+
+
+def test_reserve_is_all_or_nothing():
+    b = book(pages=4, windows=(0, 0))
+    s = b.acquire()
+    b.reserve(s, 200)                                  # 4 pages in each group... exactly fits
+    t = b.acquire()
+    with pytest.raises(CacheFull):
+        b.reserve(t, 1)
+    assert b.groups[0].table[t] == [] and b.groups[1].table[t] == []
+    b.check_invariants()
+    with pytest.raises(CacheFull, match="longest sequence"):
+        _too_long()
+
+
+def _too_long():
+    b = book(pages=64, max_blocks=2)
+    b.reserve(b.acquire(), 129)
+
+
+def test_cannot_shrink():
+    b = book()
+    s = b.acquire()
+    b.reserve(s, 10)
+    b.commit(s, 10)
+    with pytest.raises(CacheError, match="shrink"):
+        b.reserve(s, 5)
+
+
+@pytest.mark.parametrize("window", [1, 8, 64, 70, 129])
+def test_window_group_frees_exactly_the_dead_blocks(window):
+    b = book(pages=32, max_blocks=16, windows=(0, window))
+    s = b.acquire()
+    for new_len in (3, 64, 65, 130, 200, 512, 513, 700):
+        b.reserve(s, new_len)
+        b.commit(s, new_len)
+        b.check_invariants()
+        full, win = b.groups[0].table[s], b.groups[1].table[s]
+        assert all(p >= 0 for p in full) and len(full) == blocks_for(new_len)
+        for blk, page in enumerate(win):
+            last_pos = 64 * blk + 63
+            # a later query at p >= new_len sees keys > p - window >= new_len - window
+            dead = last_pos <= new_len - window
+            assert (page < 0) == dead, (new_len, blk)
+    b.release(s)
+    assert b.groups[1].pool.available == 32 and b.groups[0].pool.available == 32
+
+
+def test_random_traffic_keeps_every_invariant():
+    rng = random.Random(0)
+    b = book(pages=40, slots=6, max_blocks=12, windows=(0, 70))
+    live = {}
+    for _ in range(3000):
+        op = rng.random()
+        if op < 0.25 and len(live) < 6:
+            live[b.acquire()] = 0
+        elif op < 0.45 and live:
+            s = rng.choice(list(live))
+            b.release(s)
+            del live[s]
+        elif live:
+            s = rng.choice(list(live))
+            new = live[s] + rng.choice([1, 1, 1, 5, 64, 100])
+            try:
+                b.reserve(s, new)
+                b.commit(s, new)
+                live[s] = new
+            except CacheFull:
+                pass
+        b.check_invariants()
+        assert set(b.length) == set(live) and all(b.length[s] == n for s, n in live.items())
+    for s in list(live):
+        b.release(s)
+    assert all(g.pool.available == 40 for g in b.groups) and b.slots.available == 6

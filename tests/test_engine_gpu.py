@@ -1,0 +1,301 @@
+"""The engine against the plain implementation on the GPU, in 32-bit and in
+bfloat16, for three tiny configurations: each request alone and whole; the last
+32 tokens one by one; batches of unequal lengths whose shorter requests end
+earlier, one batch after another so that slots are used again; long decoding;
+the first tokens of a sequence; and that cutting, batching, padding and slot
+numbers change nothing."""
+import pytest
+import torch
+
+from tests.conftest import TINY
+from tests.helpers import argmax_agrees_where_clear, close, rand_ids
+from tests.plain import qwen2_plain as P
+
+pytestmark = pytest.mark.gpu
+DTYPES = ["float32", "bfloat16"]
+NAMES = list(TINY)
+
+
+@pytest.fixture(scope="module")
+def engines(model_dirs):
+    import hector_engine_amd as he
+    cache = {}
+
+    def get(name, dtype, **kw):
+        key = (name, dtype, tuple(sorted(kw.items())))
+        if key not in cache:
+            opts = dict(max_tokens=4096, max_slots=8, max_seq_len=1024)
+            opts.update(kw)
+            cache[key] = he.Engine(model_dirs[name], dtype=dtype, **opts)
+        return cache[key]
+
+    return get
+
+
+def entry(slot, tokens, want):
+    from hector_engine_amd.engine.engine import StepEntry
+    return StepEntry(slot, list(tokens), list(want))
+
+
+def plain_logits(plain_models, name, ids):
+    cfg, w = plain_models[name]
+    return P.forward(cfg, w, ids)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_each_request_alone_and_whole(engines, plain_models, name, dtype):
+    eng = engines(name, dtype)
+    vocab = plain_models[name][0]["vocab_size"]
+    for seed, n in enumerate([1, 2, 13, 64, 65, 150]):
+        ids = rand_ids(vocab, n, seed)
+        s = eng.acquire()
+        got = eng.step([entry(s, ids, range(n))])
+        want = plain_logits(plain_models, name, ids)
+        close(got, want, dtype)
+        argmax_agrees_where_clear(got, want, 0.05 * want.abs().max().item())
+        eng.release(s)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_last_32_tokens_one_by_one(engines, plain_models, name, dtype):
+    eng = engines(name, dtype)
+    vocab = plain_models[name][0]["vocab_size"]
+    n = 200 if name == "C" else 100
+    ids = rand_ids(vocab, n, 7)
+    want = plain_logits(plain_models, name, ids)
+    s = eng.acquire()
+    whole = eng.step([entry(s, ids, range(n))]).clone()
+    eng.release(s)
+    s = eng.acquire()
+    assert eng.step([entry(s, ids[:n - 32], [])]) is None
+    rows = [eng.step([entry(s, [t], [0])]).clone() for t in ids[n - 32:]]
+    eng.release(s)
+    dec = torch.cat(rows)
+    close(dec, want[n - 32:], dtype)
+    if dtype == "float32":
+        assert torch.equal(dec, whole[n - 32:])       # the 32-bit path does not depend on the cut
+    else:
+        close(dec, whole[n - 32:].cpu(), dtype)
+
+
+def run_batches(eng, requests, batch_sizes):
+    """requests: token lists. Batches of the given sizes run one after another; in a batch
+    all prompts (the first half of each request, at least one token) go in one step, then
+    every request feeds its own next given token each step; a request whose tokens are
+    used up leaves the batch and gives its slot back. Returns each request's logits at
+    all positions, and the slots used."""
+    out = {i: [] for i in range(len(requests))}
+    used = []
+    nxt = 0
+    for bs in batch_sizes:
+        batch = list(range(nxt, min(nxt + bs, len(requests))))
+        nxt += bs
+        slots = {i: eng.acquire() for i in batch}
+        used += list(slots.values())
+        fed = {i: max(1, len(requests[i]) // 2) for i in batch}
+        logits = eng.step([entry(slots[i], requests[i][:fed[i]], range(fed[i])) for i in batch])
+        r = 0
+        for i in batch:
+            out[i].append(logits[r:r + fed[i]].clone())
+            r += fed[i]
+        live = list(batch)
+        while True:
+            for i in list(live):
+                if fed[i] == len(requests[i]):
+                    eng.release(slots.pop(i))
+                    live.remove(i)
+            if not live:
+                break
+            logits = eng.step([entry(slots[i], [requests[i][fed[i]]], [0]) for i in live])
+            for r, i in enumerate(live):
+                out[i].append(logits[r:r + 1].clone())
+                fed[i] += 1
+    return {i: torch.cat(v) for i, v in out.items()}, used
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_unequal_batches_early_finishers_and_slot_reuse(engines, plain_models, name, dtype):
+    eng = engines(name, dtype, max_slots=4)
+    vocab = plain_models[name][0]["vocab_size"]
+    lengths = [6, 18, 26, 3, 14, 34, 60, 9, 130, 2]
+    requests = [rand_ids(vocab, n, 20 + i) for i, n in enumerate(lengths)]
+    got, used = run_batches(eng, requests, [3, 4, 3])
+    assert set(used) <= {0, 1, 2, 3} and len(used) == 10          # four slots serve ten requests
+    for i, ids in enumerate(requests):
+        close(got[i], plain_logits(plain_models, name, ids), dtype)
+    assert eng.cache.book.slots.available == 4 and eng.cache.free_pages == eng.cache.num_pages
+    eng.cache.book.check_invariants()
+    if dtype == "float32":
+        # each request alone gives the same bits as in its batch
+        for i in (0, 5, 8):
+            s = eng.acquire()
+            alone = eng.step([entry(s, requests[i], range(len(requests[i])))]).clone()
+            eng.release(s)
+            assert torch.equal(alone, got[i])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_long_decoding(engines, plain_models, name, dtype):
+    """Five prompt tokens, then 250 single-token steps: page boundaries at 64, 128 and 192
+    are crossed, and configuration C's window of 70 slides and gives pages back."""
+    eng = engines(name, dtype)
+    vocab = plain_models[name][0]["vocab_size"]
+    ids = rand_ids(vocab, 255, 3)
+    want = plain_logits(plain_models, name, ids)
+    s = eng.acquire()
+    rows = [eng.step([entry(s, ids[:5], range(5))]).clone()]
+    rows += [eng.step([entry(s, [t], [0])]).clone() for t in ids[5:]]
+    close(torch.cat(rows), want, dtype)
+    windowed = [g for g in eng.cache.book.groups if g.window > 0]
+    for g in windowed:
+        dead = [p for p in g.table[s] if p < 0]
+        assert len(dead) == (255 - g.window - 63) // 64 + 1 if 255 - g.window >= 63 else not dead
+    eng.release(s)
+    assert eng.cache.free_pages == eng.cache.num_pages
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_first_tokens_of_a_sequence(engines, plain_models, name, dtype):
+    """A sequence that starts with a single token, and the first decoded tokens after
+    prompts of one and two tokens."""
+    eng = engines(name, dtype)
+    vocab = plain_models[name][0]["vocab_size"]
+    ids = rand_ids(vocab, 6, 11)
+    want = plain_logits(plain_models, name, ids)
+    for first in (1, 2):
+        s = eng.acquire()
+        rows = [eng.step([entry(s, ids[:first], range(first))]).clone()]
+        rows += [eng.step([entry(s, [t], [0])]).clone() for t in ids[first:]]
+        close(torch.cat(rows), want, dtype)
+        eng.release(s)
+
+
+@pytest.mark.parametrize("name", NAMES)
+def test_cutting_batching_order_and_slots_change_no_bit_in_32_bit(engines, plain_models, name):
+    eng = engines(name, "float32")
+    vocab = plain_models[name][0]["vocab_size"]
+    reqs = [rand_ids(vocab, n, 40 + n) for n in (70, 9, 33)]
+
+    def run(order, chunks, burn):
+        burned = [eng.acquire() for _ in range(burn)]              # shifts the slot numbers
+        slots = {i: eng.acquire() for i in order}
+        got = {i: [] for i in order}
+        pos = {i: 0 for i in order}
+        while any(pos[i] < len(reqs[i]) for i in order):
+            live = [i for i in order if pos[i] < len(reqs[i])]
+            ents = []
+            for i in live:
+                n = min(chunks, len(reqs[i]) - pos[i])
+                ents.append(entry(slots[i], reqs[i][pos[i]:pos[i] + n], range(n)))
+            logits = eng.step(ents)
+            r = 0
+            for i, e in zip(live, ents):
+                got[i].append(logits[r:r + len(e.tokens)].clone())
+                r += len(e.tokens)
+                pos[i] += len(e.tokens)
+        for s in list(slots.values()) + burned:
+            eng.release(s)
+        return {i: torch.cat(v) for i, v in got.items()}
+
+    base = run([0, 1, 2], 1000, 0)
+    for order, chunks, burn in (([2, 0, 1], 1000, 0), ([0, 1, 2], 7, 0), ([1, 2, 0], 64, 3), ([0, 1, 2], 1, 2)):
+        other = run(order, chunks, burn)
+        for i in range(3):
+            assert torch.equal(other[i], base[i]), (order, chunks, burn, i)
+    for i in range(3):
+        close(base[i], plain_logits(plain_models, name, reqs[i]), "float32")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_chunked_prompts_equal_whole_prompts(engines, plain_models, dtype):
+    eng = engines("C", dtype)
+    vocab = plain_models["C"][0]["vocab_size"]
+    ids = rand_ids(vocab, 230, 5)
+    want = plain_logits(plain_models, "C", ids)
+    s = eng.acquire()
+    rows = []
+    for a in range(0, 230, 50):
+        chunk = ids[a:a + 50]
+        rows.append(eng.step([entry(s, chunk, range(len(chunk)))]).clone())
+    eng.release(s)
+    close(torch.cat(rows), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_graph_replay_and_padding_change_no_result(model_dirs, plain_models, name, dtype):
+    """One-token steps of 3 sequences run in a bucket of 4 (one padding row) as a
+    captured graph; the same steps run eagerly without padding. Same bits."""
+    import hector_engine_amd as he
+    vocab = plain_models[name][0]["vocab_size"]
+    reqs = [rand_ids(vocab, n, 60 + n) for n in (40, 75, 12)]
+    outs = []
+    for graphs in (True, False):
+        eng = he.Engine(model_dirs[name], dtype=dtype, max_tokens=2048, max_slots=4, max_seq_len=512,
+                        use_graphs=graphs)
+        slots = [eng.acquire() for _ in reqs]
+        eng.step([entry(s, r[:6], []) for s, r in zip(slots, reqs)])
+        rows = []
+        for t in range(6, 12):
+            rows.append(eng.step([entry(s, [r[t]], [0]) for s, r in zip(slots, reqs)]).clone())
+        outs.append(torch.stack(rows))                # [6 steps, 3, vocab]
+        if graphs:
+            assert eng.stats["graph_replays"] >= 4 and eng.stats["graph_captures"] == 1
+        else:
+            assert eng.stats["graph_replays"] == 0
+    assert torch.equal(outs[0], outs[1])
+    for i, r in enumerate(reqs):
+        close(outs[0][:, i], plain_logits(plain_models, name, r[:12])[6:12], dtype)
+
+
+def test_errors_leave_the_cache_untouched(engines, plain_models):
+    from hector_engine_amd.cache import CacheError, CacheFull
+    from hector_engine_amd.engine.engine import StepError
+    eng = engines("A", "float32", max_tokens=256, max_slots=4)       # four pages
+    s, t = eng.acquire(), eng.acquire()
+    with pytest.raises(StepError, match="token ids"):
+        eng.step([entry(s, [1, 999], [0])])
+    with pytest.raises(StepError, match="twice"):
+        eng.step([entry(s, [1], [0]), entry(s, [2], [0])])
+    with pytest.raises(StepError, match="wanted place"):
+        eng.step([entry(s, [1, 2], [2])])
+    with pytest.raises(StepError, match="at least one token"):
+        eng.step([entry(s, [], [])])
+    with pytest.raises(CacheError, match="not held"):
+        eng.step([entry(3, [1], [0])])
+    with pytest.raises(CacheFull):
+        eng.step([entry(s, [1] * 130, []), entry(t, [1] * 130, [])])     # 3 + 3 pages, 4 exist
+    assert eng.length(s) == 0 and eng.length(t) == 0 and eng.cache.free_pages == 4
+    eng.step([entry(s, [1] * 130, [])])
+    with pytest.raises(StepError, match="longest sequence"):
+        eng.step([entry(s, [1] * 127, [])])
+    eng.release(s)
+    eng.release(t)
+    with pytest.raises(CacheError):
+        eng.release(t)
+    eng.cache.book.check_invariants()
+
+
+def test_a_reused_slot_holds_nothing_of_its_past(engines, plain_models):
+    """A long request fills pages; after release a short request gets the same slot and
+    pages. Its logits equal those of a fresh engine bit for bit (32-bit)."""
+    eng = engines("B", "float32", max_tokens=512, max_slots=2)
+    vocab = plain_models["B"][0]["vocab_size"]
+    long, short = rand_ids(vocab, 300, 1), rand_ids(vocab, 70, 2)
+    s = eng.acquire()
+    first = eng.step([entry(s, short, range(70))]).clone()
+    eng.release(s)
+    s = eng.acquire()
+    eng.step([entry(s, long, [])])
+    eng.release(s)
+    s2 = eng.acquire()
+    assert s2 == s
+    again = eng.step([entry(s2, short, range(70))]).clone()
+    eng.release(s2)
+    assert torch.equal(first, again)
+    close(again, plain_logits(plain_models, "B", short), "float32")

@@ -1,0 +1,159 @@
+"""The generation loop's decisions, with a fake engine on the CPU: admission,
+batches one after another, stop tokens, sequences that end earlier and give
+their slot back at once, the token budget and the cache-room stop."""
+import pytest
+
+import hector_engine_amd  # noqa: F401
+from hector_engine_amd.cache import GroupPages, SlotBook
+from hector_engine_amd.engine.generate import after_token, generate, plan_batch
+
+V = 50
+
+
+class FakeCache:
+    def __init__(self, pages, slots, max_blocks):
+        self.book = SlotBook(slots, max_blocks, [GroupPages(pages, 0, "0")])
+
+    @property
+    def free_pages(self):
+        return self.book.groups[0].pool.available
+
+
+class FakeEngine:
+    """next token of a sequence = (sum of its tokens + its length) % V."""
+
+    device = "cpu"
+
+    def __init__(self, pages=16, slots=3, max_blocks=4):
+        self.cache = FakeCache(pages, slots, max_blocks)
+        self.max_seq_len = max_blocks * 64
+        self.history = {}
+        self.log = []          # (slots in the step, tokens per slot)
+        self.max_live = 0
+
+    def acquire(self):
+        s = self.cache.book.acquire()
+        self.history[s] = []
+        self.max_live = max(self.max_live, len(self.history))
+        return s
+
+    def release(self, s):
+        self.cache.book.release(s)
+        del self.history[s]
+
+    def length(self, s):
+        return self.cache.book.length[s]
+
+    def step(self, entries):
+        self.log.append([(e.slot, len(e.tokens)) for e in entries])
+        rows = []
+        for e in entries:
+            new = self.length(e.slot) + len(e.tokens)
+            self.cache.book.reserve(e.slot, new)
+            self.cache.book.commit(e.slot, new)
+            self.history[e.slot] += list(e.tokens)
+            assert list(e.want) == [len(e.tokens) - 1]
+            h = self.history[e.slot]
+            rows.append((sum(h) + len(h)) % V)
+        self.cache.book.check_invariants()
+        return rows
+
+
+def pick(rows, sequences, steps, contexts):
+    return list(rows)
+
+
+def expected(prompt, n, stop=()):
+    h, out = list(prompt), []
+    for _ in range(n):
+        t = (sum(h) + len(h)) % V
+        if t in stop:
+            return out, "eos"
+        out.append(t)
+        h.append(t)
+    return out, "max_tokens"
+
+
+def test_plan_batch():
+    # slots limit, page limit, refusals
+    assert plan_batch([(0, 10), (1, 20), (2, 30)], 5, 100, 2, 256, None) == ([0, 1], [])
+    assert plan_batch([(0, 10), (1, 20), (2, 30)], 5, 100, 3, 256, 2) == ([0, 1], [])
+    assert plan_batch([(0, 100), (1, 100)], 60, 3, 8, 256, None) == ([0], [])      # 3 pages: one request of 160
+    assert plan_batch([(0, 0), (1, 256), (2, 5)], 5, 100, 8, 256, None) == ([2], [0, 1])
+    assert plan_batch([(0, 200)], 100, 2, 8, 256, None) == ([], [0])               # never fits
+    # room is counted up to max_seq_len only
+    assert plan_batch([(0, 250)], 100, 4, 8, 256, None) == ([0], [])
+
+
+def test_after_token():
+    assert after_token(7, 0, 5, 10, 64, {7}) == (False, "eos")
+    assert after_token(3, 4, 5, 10, 64, {7}) == (True, "max_tokens")
+    assert after_token(3, 0, 5, 64, 64, {7}) == (True, "stop")
+    assert after_token(3, 0, 5, 63, 64, {7}) == (True, None)
+
+
+def test_unequal_prompts_stop_tokens_and_early_finishers():
+    eng = FakeEngine()
+    prompts = [[1, 2, 3], [4] * 9, [7, 7, 7, 7, 7]]
+    stop = {expected(prompts[1], 3)[0][2]}            # the third token of request 1 is a stop token
+    res = generate(eng, prompts, max_new_tokens=6, stop_ids=stop, sample_fn=pick)
+    for p, r in zip(prompts, res):
+        want, reason = expected(p, 6, stop)
+        assert r.tokens == want and r.finish_reason == reason and r.prompt_tokens == len(p)
+    assert res[1].finish_reason == "eos" and len(res[1].tokens) == 2
+    # the first step holds all prompts; after request 1 ended the steps hold two sequences
+    assert [n for _, n in eng.log[0]] == [3, 9, 5]
+    sizes = [len(step) for step in eng.log[1:]]
+    assert sizes[:2] == [3, 3] and set(sizes[2:]) == {2}
+    assert eng.cache.book.slots.available == 3 and eng.cache.free_pages == 16 and not eng.history
+
+
+def test_more_requests_than_slots_run_batch_after_batch():
+    eng = FakeEngine(slots=2)
+    prompts = [[i + 1] * (i + 2) for i in range(5)]
+    res = generate(eng, prompts, max_new_tokens=4, sample_fn=pick)
+    for p, r in zip(prompts, res):
+        assert (r.tokens, r.finish_reason) == expected(p, 4)
+    assert eng.max_live == 2
+    firsts = [step for step in eng.log if any(n > 1 for _, n in step)]
+    assert [len(s) for s in firsts] == [2, 2, 1]       # three batches
+    assert {s for step in eng.log for s, _ in step} == {0, 1}          # slots are used again
+
+
+def test_include_stop_and_refusals_and_cache_room():
+    eng = FakeEngine(max_blocks=1)                     # 64 positions per sequence
+    p = [3, 1, 4]
+    stop = {expected(p, 2)[0][1]}
+    r = generate(eng, [p], max_new_tokens=5, stop_ids=stop, include_stop=True, sample_fn=pick)[0]
+    assert r.finish_reason == "eos" and r.tokens == expected(p, 2)[0]
+    long = [1] * 64
+    r = generate(eng, [long, [2] * 60], max_new_tokens=10, sample_fn=pick)
+    assert r[0].finish_reason == "context_full" and r[0].tokens == []
+    want, _ = expected([2] * 60, 5)                    # 60 + 4 fed tokens fill the 64 positions
+    assert r[1].finish_reason == "stop" and r[1].tokens == want
+    assert eng.cache.book.slots.available == 3
+
+
+def test_cancel_and_zero_budget():
+    eng = FakeEngine()
+    calls = {"n": 0}
+
+    def cancel():
+        calls["n"] += 1
+        return calls["n"] > 2
+
+    r = generate(eng, [[1, 2]], max_new_tokens=50, cancel=cancel, sample_fn=pick)[0]
+    assert r.finish_reason == "cancelled" and len(r.tokens) == 2
+    assert eng.cache.book.slots.available == 3
+    assert generate(eng, [[1]], max_new_tokens=0, sample_fn=pick)[0].finish_reason == "max_tokens"
+
+
+def test_slots_are_released_when_a_step_fails():
+    eng = FakeEngine()
+
+    def boom(rows, *a):
+        raise RuntimeError("sampler failed")
+
+    with pytest.raises(RuntimeError, match="sampler failed"):
+        generate(eng, [[1, 2], [3]], max_new_tokens=3, sample_fn=boom)
+    assert eng.cache.book.slots.available == 3 and eng.cache.free_pages == 16
