@@ -117,7 +117,7 @@ class Engine:
                                 dtype=self.dtype, device=self.device)
         self.caches = [self.cache.layer_cache(r) for r in range(len(self.model.schedule))]
         self.scratch = ScratchPool(self.device)
-        self.use_graphs = use_graphs
+        self.use_graphs = use_graphs and self.model.graph_safe()
         self._buckets: dict[int, _GraphBucket] = {}
         self._pinned = [torch.empty(1 << 16, dtype=torch.int32).pin_memory() for _ in range(4)]
         self._pinned_events: list[torch.cuda.Event | None] = [None] * 4
@@ -238,6 +238,9 @@ class Engine:
         views = meta.views(dev)
         ctx = self._context(views, rows, len(entries), max(len(e.tokens) for e in entries),
                             all_single, self.scratch)
+        ctx.host = {"q_lens": [len(e.tokens) for e in entries],
+                    "starts": [self.cache.length(e.slot) for e in entries],
+                    "slots": [e.slot for e in entries]}
         self.stats["eager_steps"] += 1
         return self.model.forward(views["tokens"], ctx, self.caches, views["want_rows"], nw)
 

@@ -38,6 +38,16 @@ class DecoderModel:
     def parts(self):
         return [self.embedding, *self.blocks, self.final_norm, self.head]
 
+    def graph_safe(self) -> bool:
+        """True when every part works from the device-side batch alone."""
+        todo = list(self.parts())
+        while todo:
+            p = todo.pop()
+            if not p.graph_safe:
+                return False
+            todo += p.children()
+        return True
+
     def tensor_specs(self):
         specs = {}
         for p in self.parts():

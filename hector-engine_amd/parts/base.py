@@ -114,7 +114,7 @@ class StepContext:
         self.all_single = all_single      # every sequence brings exactly one token
         self.env = env
         self.scratch = scratch            # ScratchPool: alloc(shape, dtype)
-        self.host = host                  # host-side copy of the batch (lists), for parts that plan on the host
+        self.host = host                  # {"q_lens", "starts", "slots"}: lists per sequence, eager steps only
 
     def alloc(self, shape, dtype=None) -> torch.Tensor:
         return self.scratch.alloc(shape, dtype or self.env.dtype)
@@ -138,6 +138,10 @@ class LayerCache:
 
 class Part:
     """Base of all parts: declares its tensors by full name and receives them."""
+
+    # False for a part that plans on the host from ctx.host (sequence lengths as Python
+    # lists); one-token steps of a model holding such a part are not captured into graphs.
+    graph_safe = True
 
     def __init__(self, prefix: str, env: BuildEnv):
         self.prefix = prefix

@@ -1,0 +1,130 @@
+"""Generation through the entry points on the GPU: greedy generation equals the
+plain implementation's, sampled generation equals it given the same uniforms,
+stop tokens, early finishers, batches in a row, penalties, and the command line."""
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from tests.conftest import ROOT, TINY
+from tests.helpers import rand_ids
+from tests.plain import qwen2_plain as P
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def he():
+    import hector_engine_amd
+    return hector_engine_amd
+
+
+def prompts_for(cfg, lengths, seed):
+    return [rand_ids(cfg["vocab_size"], n, seed + i) for i, n in enumerate(lengths)]
+
+
+@pytest.mark.parametrize("name,lengths,steps", [("A", [5, 9, 13], 8), ("B", [3, 7, 17, 30], 12), ("C", [60, 2, 31], 10)])
+def test_greedy_generation_equals_plain(he, model_dirs, plain_models, name, lengths, steps):
+    cfg, w = plain_models[name]
+    prompts = prompts_for(cfg, lengths, 100)
+    want = [P.generate(cfg, w, p, steps) for p in prompts]
+    eng = he.Engine(model_dirs[name], dtype="float32", max_tokens=2048, max_seq_len=512)
+    got = he.generate(eng, prompts, max_new_tokens=steps)
+    assert [r.tokens for r in got] == want
+    assert all(r.finish_reason == "max_tokens" and r.prompt_tokens == len(p) for r, p in zip(got, prompts))
+    # alone, in another order, and with two slots only (batches in a row): same tokens
+    for p, t in zip(prompts, want):
+        assert he.generate(eng, [p], max_new_tokens=steps)[0].tokens == t
+    assert [r.tokens for r in he.generate(eng, prompts[::-1], max_new_tokens=steps)] == want[::-1]
+    small = he.Engine(model_dirs[name], dtype="float32", max_tokens=2048, max_slots=2, max_seq_len=512)
+    assert [r.tokens for r in he.generate(small, prompts, max_new_tokens=steps)] == want
+    assert small.cache.free_pages == small.cache.num_pages
+    # bfloat16: the same tokens wherever the oracle's choice is clear
+    eng16 = he.Engine(model_dirs[name], dtype="bfloat16", max_tokens=2048, max_seq_len=512)
+    got16 = he.generate(eng16, prompts, max_new_tokens=steps)
+    for p, r, t in zip(prompts, got16, want):
+        seq = list(p)
+        for a, b in zip(r.tokens, t):
+            if a != b:
+                top = P.forward(cfg, w, seq)[-1].topk(2).values
+                assert (top[0] - top[1]).item() < 0.02 * top[0].abs().item() + 1e-3     # a near tie
+                break
+            seq.append(a)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("kw", [dict(temperature=0.8, seed=7), dict(temperature=1.0, top_k=5, seed=1),
+                                dict(temperature=0.7, top_k=40, top_p=0.9, seed=3)])
+def test_sampled_generation_equals_plain(he, model_dirs, plain_models, name, kw):
+    cfg, w = plain_models[name]
+    prompts = prompts_for(cfg, [3, 7, 17, 30], 200)
+    eng = he.Engine(model_dirs[name], dtype="float32", max_tokens=2048, max_seq_len=512)
+    got = he.generate(eng, prompts, max_new_tokens=12, sampling=he.SamplingConfig(**kw))
+    for i, (p, r) in enumerate(zip(prompts, got)):
+        want = P.generate(cfg, w, p, 12, temperature=kw["temperature"], top_k=kw.get("top_k", 0),
+                          top_p=kw.get("top_p", 1.0), seed=kw["seed"], sequence=i)
+        assert r.tokens == want
+    # the draw is keyed by the request's index, not by the batch: one slot at a time, same tokens
+    one = he.Engine(model_dirs[name], dtype="float32", max_tokens=2048, max_slots=1, max_seq_len=512)
+    again = he.generate(one, prompts, max_new_tokens=12, sampling=he.SamplingConfig(**kw))
+    assert [r.tokens for r in again] == [r.tokens for r in got]
+
+
+def test_stop_tokens_and_early_finishers(he, model_dirs, plain_models):
+    cfg, w = plain_models["B"]
+    prompts = prompts_for(cfg, [3, 7, 17, 30], 300)
+    free = [P.generate(cfg, w, p, 12) for p in prompts]
+    stop = {free[1][4], free[3][0]}                    # request 1 stops at its fifth token, request 3 at once
+    want = [P.generate(cfg, w, p, 12, stop_ids=stop) for p in prompts]
+    eng = he.Engine(model_dirs["B"], dtype="float32", max_tokens=2048, max_seq_len=512)
+    got = he.generate(eng, prompts, max_new_tokens=12, stop_ids=stop)
+    assert [r.tokens for r in got] == want
+    assert got[3].finish_reason == "eos" and got[3].tokens == []
+    assert got[1].finish_reason == "eos" and len(got[1].tokens) <= 4
+    assert all(t not in stop for r in got for t in r.tokens)
+    assert eng.cache.free_pages == eng.cache.num_pages and eng.cache.book.slots.available == eng.cache.max_slots
+
+
+def test_penalties(he, model_dirs, plain_models):
+    cfg, w = plain_models["A"]
+    p = prompts_for(cfg, [9], 400)[0]
+    eng = he.Engine(model_dirs["A"], dtype="float32", max_tokens=1024, max_seq_len=512)
+    plainly = he.generate(eng, [p], max_new_tokens=16)[0].tokens
+    cfg_s = he.SamplingConfig(temperature=0.0, repetition_penalty=1.3, frequency_penalty=0.2,
+                              presence_penalty=0.1, penalty_window=6)
+    got = he.generate(eng, [p], max_new_tokens=16, sampling=cfg_s)[0].tokens
+    want = P.generate(cfg, w, p, 16, rep=1.3, freq=0.2, pres=0.1, penalty_window=6)
+    assert got == want and got != plainly
+
+
+def test_cache_room_ends_a_sequence(he, model_dirs):
+    eng = he.Engine(model_dirs["A"], dtype="bfloat16", max_tokens=128, max_slots=2, max_seq_len=64)
+    r = he.generate(eng, [[1] * 60, [2] * 64], max_new_tokens=20)
+    assert r[0].finish_reason == "stop" and len(r[0].tokens) == 5      # 60 + 4 fed fill 64 positions
+    assert r[1].finish_reason == "context_full" and r[1].tokens == []
+
+
+def test_command_line(model_dirs, plain_models):
+    cfg, w = plain_models["A"]
+    exe = os.path.join(ROOT, "bin", "hector_generate")
+    out = subprocess.run([sys.executable, exe, model_dirs["A"], "5,17,3;9,2,77,13", "6", "--dtype", "float32"],
+                         capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    want = [P.generate(cfg, w, p, 6) for p in ([5, 17, 3], [9, 2, 77, 13])]
+    for i, t in enumerate(want):
+        assert f"[{i}] prompt" in out.stdout and ",".join(map(str, t)) in out.stdout
+    assert "Speed:" in out.stdout and "tok/s" in out.stdout and "Prompt: 7 tokens" in out.stdout
+    env = dict(os.environ, HELIOS_SEED="7", HELIOS_TOPK="0", HELIOS_TOPP="1.0")
+    out = subprocess.run([sys.executable, exe, "--model", model_dirs["A"], "--temp", "0.8", "5,17,3", "6",
+                          "--dtype", "float32"], capture_output=True, text=True, timeout=120, env=env)
+    assert out.returncode == 0, out.stderr
+    t = P.generate(cfg, w, [5, 17, 3], 6, temperature=0.8, seed=7)
+    assert ",".join(map(str, t)) in out.stdout
+
+
+def test_smoke_entry():
+    sys.path.insert(0, ROOT)
+    import __graft_entry__
+    __graft_entry__.smoke()

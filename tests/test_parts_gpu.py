@@ -1,0 +1,462 @@
+"""Each part alone against the plain function of the same name; and the
+generality of the assembly: a toy mixer with state of its own, a toy position
+encoding and toy schedules (a layer named twice, a layer that reads another
+layer's cache) are registered here, built and stepped without a change to the
+framework's files. The toys are test fixtures, not models."""
+import dataclasses
+import math
+import os
+
+import pytest
+import torch
+
+from tests.helpers import close, rand_ids
+from tests.plain import qwen2_plain as P
+
+pytestmark = pytest.mark.gpu
+PAGE = 64
+
+
+@pytest.fixture(scope="module")
+def fw():
+    import hector_engine_amd  # noqa: F401
+    from hector_engine_amd import parts
+    from hector_engine_amd.cache.paged import PagedCache, RunPlan
+    from hector_engine_amd.engine.scratch import ScratchPool
+
+    class NS:
+        pass
+
+    ns = NS()
+    ns.parts, ns.PagedCache, ns.RunPlan, ns.ScratchPool = parts, PagedCache, RunPlan, ScratchPool
+    return ns
+
+
+def env_for(fw, dtype, fast=True):
+    return fw.parts.BuildEnv(torch.device("cuda:0"), dtype, fast)
+
+
+def make_ctx(fw, env, q_lens, starts, slots):
+    rows = sum(q_lens)
+    positions = torch.cat([torch.arange(s, s + n) for s, n in zip(starts, q_lens)]).int().cuda()
+    row_seq = torch.cat([torch.full((n,), i) for i, n in enumerate(q_lens)]).int().cuda()
+    cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32).cuda()
+    return fw.parts.StepContext(
+        rows=rows, num_seqs=len(q_lens), positions=positions, row_seq=row_seq,
+        seq_slot=torch.tensor(slots, dtype=torch.int32).cuda(), cu_seqlens=cu,
+        seq_start=torch.tensor(starts, dtype=torch.int32).cuda(), max_q_len=max(q_lens), max_keys=1024,
+        all_single=all(n == 1 for n in q_lens), env=env, scratch=fw.ScratchPool(env.device),
+        host={"q_lens": q_lens, "starts": starts, "slots": slots})
+
+
+def rnd(*shape, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g) * scale
+
+
+DT = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype):
+    return dict(rtol=3e-6, atol=3e-6) if dtype == torch.float32 else dict(rtol=2 ** -6, atol=2 ** -6)
+
+
+def near(got, want, dtype):
+    """Error bound relative to the size of the result: a few fp32 ulp, or for bfloat16
+    2^-6 of the largest value (two bf16 ulp there; several roundings are chained)."""
+    scale = want.abs().max().item()
+    err = (got - want).abs().max().item()
+    bound = (1e-5 if dtype == torch.float32 else 2 ** -6) * max(scale, 1e-3)
+    assert err <= bound, f"max error {err:.3g} above {bound:.3g} (scale {scale:.3g})"
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_rmsnorm_part(fw, dtype):
+    env = env_for(fw, dtype)
+    norm = fw.parts.build_part("norm", fw.parts.PartSpec("rmsnorm", {"size": 80, "eps": 3e-6}), "n.", env)
+    assert list(norm.tensor_specs()) == ["n.weight"]
+    w = (1 + 0.1 * rnd(80, seed=1)).to(dtype)
+    norm.bind({"n.weight": w.cuda()})
+    ctx = make_ctx(fw, env, [5], [0], [0])
+    resid, delta = rnd(5, 80, seed=2), rnd(5, 80, seed=3).to(dtype)
+    r = resid.clone().cuda()
+    out = norm.add_norm(r, delta.cuda(), 5, ctx)
+    assert out.dtype == dtype
+    assert torch.allclose(r.cpu().double(), resid.double() + delta.double(), atol=1e-6)
+    assert torch.allclose(out.cpu().double(), P.rmsnorm(r.cpu().double(), w.double(), 3e-6), **tol(dtype))
+
+
+def test_rotary_part(fw):
+    env = env_for(fw, torch.float32)
+    rot = fw.parts.build_part("position", fw.parts.PartSpec("rotary", {"head_dim": 48, "theta": 50000.0}), "", env)
+    inv, r = rot.rotary()
+    assert r == 48 and torch.equal(inv.cpu(), P.rope_inv_freq(48, 50000.0))
+    part = fw.parts.build_part("position", fw.parts.PartSpec(
+        "rotary", {"head_dim": 64, "theta": 1e4, "partial_rotary_factor": 0.5}), "", env)
+    assert part.rotary()[1] == 32 and not rot.custom and rot.tensor_specs() == {}
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("rows", [5, 100])
+def test_gated_mlp_part(fw, dtype, rows):
+    env = env_for(fw, dtype)
+    mlp = fw.parts.build_part("feed_forward", fw.parts.PartSpec(
+        "gated_mlp", {"hidden_size": 80, "intermediate_size": 136}), "m.", env)
+    specs = mlp.tensor_specs()
+    assert {k: v.shape for k, v in specs.items()} == {
+        "m.gate_proj.weight": (136, 80), "m.up_proj.weight": (136, 80), "m.down_proj.weight": (80, 136)}
+    w = {k: rnd(*v.shape, seed=i, scale=0.1).to(dtype) for i, (k, v) in enumerate(specs.items())}
+    mlp.bind({k: v.cuda() for k, v in w.items()})
+    ctx = make_ctx(fw, env, [rows], [0], [0])
+    x = rnd(rows, 80, seed=9).to(dtype)
+    out = mlp.forward(x.cuda(), ctx)
+    want = P.swiglu(x.double(), w["m.gate_proj.weight"].double(), w["m.up_proj.weight"].double(),
+                    w["m.down_proj.weight"].double())
+    assert torch.allclose(out.cpu().double(), want, **tol(dtype))
+
+
+def attention_spec(fw, D, H, KVH, hd, window, bias=True, theta=1e4):
+    return fw.parts.PartSpec("attention", {
+        "hidden_size": D, "num_heads": H, "num_kv_heads": KVH, "head_dim": hd, "qkv_bias": bias,
+        "window": window, "position": fw.parts.PartSpec("rotary", {"head_dim": hd, "theta": theta})})
+
+
+def attention_weights(specs, dtype, seed=0):
+    return {k: rnd(*v.shape, seed=seed + i, scale=0.08).to(dtype) for i, (k, v) in enumerate(specs.items())}
+
+
+@pytest.mark.parametrize("dtype,fast", [(torch.float32, True), (torch.bfloat16, True), (torch.bfloat16, False)])
+@pytest.mark.parametrize("window", [0, 9])
+def test_attention_part_prompt_then_tokens(fw, dtype, fast, window):
+    D, H, KVH, hd = 80, 6, 3, 32
+    env = env_for(fw, dtype, fast)
+    att = fw.parts.build_part("mixer", attention_spec(fw, D, H, KVH, hd, window), "a.", env)
+    assert att.kv_need() == fw.parts.KVNeed(KVH, hd, window) and att.state_bytes() == 0
+    w = attention_weights(att.tensor_specs(), dtype)
+    att.bind({k: v.cuda() for k, v in w.items()})
+    cache = fw.PagedCache([fw.RunPlan(att.kv_need(), None)], max_tokens=1024, max_slots=4, max_seq_len=512,
+                          dtype=dtype, device=env.device)
+    lc = cache.layer_cache(0)
+    lens = [70, 3]
+    slots = [cache.acquire(), cache.acquire()]
+    xs = [rnd(n + 4, D, seed=20 + i).to(dtype) for i, n in enumerate(lens)]
+    cfg = {"num_attention_heads": H, "num_key_value_heads": KVH, "head_dim": hd, "rope_theta": 1e4}
+    wd = {k: v.double() for k, v in w.items()}
+    want = [P.attention_block(cfg, wd, "a.", x.double(), torch.arange(x.shape[0]), window)[0] for x in xs]
+    # the prompts in one step
+    cache.reserve(list(zip(slots, lens)))
+    ctx = make_ctx(fw, env, lens, [0, 0], slots)
+    out = att.forward(torch.cat([x[:n] for x, n in zip(xs, lens)]).cuda(), ctx, lc).cpu().double()
+    cache.commit(list(zip(slots, lens)))
+    near(out[:70], want[0][:70], dtype)
+    near(out[70:], want[1][:3], dtype)
+    # then four single-token steps of both sequences
+    for t in range(4):
+        new = [n + t + 1 for n in lens]
+        cache.reserve(list(zip(slots, new)))
+        ctx = make_ctx(fw, env, [1, 1], [n + t for n in lens], slots)
+        x = torch.stack([xs[0][70 + t], xs[1][3 + t]])
+        out = att.forward(x.cuda(), ctx, lc).cpu().double()
+        cache.commit(list(zip(slots, new)))
+        near(out[0], want[0][70 + t], dtype)
+        near(out[1], want[1][3 + t], dtype)
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_pre_norm_block_part(fw, dtype):
+    D, H, KVH, hd, I = 64, 4, 2, 16, 96
+    env = env_for(fw, dtype)
+    norm = fw.parts.PartSpec("rmsnorm", {"size": D, "eps": 1e-5})
+    spec = fw.parts.PartSpec("pre_norm", {
+        "mixer_norm": norm, "feed_forward_norm": norm, "mixer": attention_spec(fw, D, H, KVH, hd, 0),
+        "feed_forward": fw.parts.PartSpec("gated_mlp", {"hidden_size": D, "intermediate_size": I}),
+        "names": {"mixer_norm": "ln1", "mixer": "att", "feed_forward_norm": "ln2", "feed_forward": "ff"}})
+    block = fw.parts.build_part("block", spec, "L.", env)
+    specs = block.tensor_specs()
+    assert "L.ln1.weight" in specs and "L.att.q_proj.bias" in specs and "L.ff.down_proj.weight" in specs
+    w = {k: (1 + rnd(*v.shape, seed=i, scale=0.1) if "ln" in k else rnd(*v.shape, seed=i, scale=0.1)).to(dtype)
+         for i, (k, v) in enumerate(specs.items())}
+    block.bind({k: v.cuda() for k, v in w.items()})
+    cache = fw.PagedCache([fw.RunPlan(block.mixer.kv_need(), None)], max_tokens=256, max_slots=2,
+                          max_seq_len=128, dtype=dtype, device=env.device)
+    slot = cache.acquire()
+    cache.reserve([(slot, 20)])
+    ctx = make_ctx(fw, env, [20], [0], [slot])
+    x = rnd(20, D, seed=50)
+    stream = fw.parts.ResidualStream(x.clone().cuda(), 20)
+    block.forward(stream, ctx, cache.layer_cache(0))
+    got = stream.materialize().cpu().double()
+    wd = {k: v.double() for k, v in w.items()}
+    cfg = {"num_attention_heads": H, "num_key_value_heads": KVH, "head_dim": hd, "rope_theta": 1e4}
+    h = x.double()
+    a, _ = P.attention_block(cfg, wd, "L.att.", P.rmsnorm(h, wd["L.ln1.weight"], 1e-5), torch.arange(20), 0)
+    h = h + a
+    h = h + P.swiglu(P.rmsnorm(h, wd["L.ln2.weight"], 1e-5), wd["L.ff.gate_proj.weight"],
+                     wd["L.ff.up_proj.weight"], wd["L.ff.down_proj.weight"])
+    near(got, h, dtype)
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_embedding_and_heads(fw, dtype):
+    env = env_for(fw, dtype)
+    emb = fw.parts.build_part("embedding", fw.parts.PartSpec("token_embedding", {"vocab_size": 301, "hidden_size": 80}), "e.", env)
+    tied = fw.parts.build_part("head", fw.parts.PartSpec("linear_head", {"vocab_size": 301, "hidden_size": 80, "tied_to": "e.weight"}), "h.", env)
+    own = fw.parts.build_part("head", fw.parts.PartSpec("linear_head", {"vocab_size": 301, "hidden_size": 80}), "h.", env)
+    assert tied.tensor_specs() == {} and list(own.tensor_specs()) == ["h.weight"]
+    table, hw = rnd(301, 80, seed=1).to(dtype), rnd(301, 80, seed=2).to(dtype)
+    tensors = {"e.weight": table.cuda(), "h.weight": hw.cuda()}
+    for p in (emb, tied, own):
+        p.bind(tensors)
+    assert tied.linear.weight.data_ptr() == emb.table.data_ptr()            # an alias, not a copy
+    ctx = make_ctx(fw, env, [4], [0], [0])
+    ids = torch.tensor([3, 300, 0, 17], dtype=torch.int32).cuda()
+    h = emb.forward(ids, 4, ctx)
+    assert h.dtype == torch.float32 and torch.equal(h.cpu(), table.float()[[3, 300, 0, 17]])
+    x = rnd(4, 80, seed=3).to(dtype)
+    for head, wt in ((tied, table), (own, hw)):
+        out = head.forward(x.cuda(), 4, ctx)
+        assert out.dtype == torch.float32
+        assert torch.allclose(out.cpu().double(), x.double() @ wt.double().T, rtol=1e-4, atol=1e-4)
+    # 100 wanted rows go through in chunks of 64
+    ctx = make_ctx(fw, env, [100], [0], [0])
+    x = rnd(100, 80, seed=4).to(dtype)
+    out = own.forward(x.cuda(), 100, ctx)
+    assert torch.allclose(out.cpu().double(), x.double() @ hw.double().T, rtol=1e-4, atol=1e-4)
+
+
+def test_a_weight_stored_in_32_bit_stays_so_under_bfloat16(fw):
+    from hector_engine_amd.parts.linear import Linear
+    env = env_for(fw, torch.bfloat16)
+    w, b = rnd(37, 48, seed=1, scale=0.1), rnd(37, seed=2)
+    lin = Linear(w.cuda(), b.cuda())
+    ctx = make_ctx(fw, env, [9], [0], [0])
+    x = rnd(9, 48, seed=3).to(torch.bfloat16)
+    out = lin(x.cuda(), 9, ctx)
+    assert out.dtype == torch.bfloat16 and lin.weight.dtype == torch.float32
+    want = x.double() @ w.double().T + b.double()
+    assert torch.allclose(out.cpu().double(), want, rtol=2 ** -7, atol=2 ** -7)
+
+
+# ---------------------------------------------------------------------------
+# toys: registered here, in the test, through the public registries only
+# ---------------------------------------------------------------------------
+@pytest.fixture(scope="module")
+def toys(fw):
+    import hector_engine_amd as he
+    from hector_engine_amd.config.base import ModelConfig, architecture_name, read_field
+    parts = fw.parts
+
+    @parts.register_part("mixer", "toy_running_mean")
+    class RunningMean(parts.Mixer):
+        """out_t = Wo . mean_{j<=t} x_j. Its state, the running sum and the count, lives in the
+        cache's per-sequence state area; it keeps no keys or values."""
+        graph_safe = False
+
+        def __init__(self, params, prefix, env):
+            super().__init__(prefix, env)
+            self.D = parts.param(params, "hidden_size", int)
+
+        def state_bytes(self):
+            return 4 * (self.D + 1)
+
+        def tensor_specs(self):
+            return {self.prefix + "out.weight": parts.TensorSpec((self.D, self.D))}
+
+        def bind(self, tensors):
+            self.w = tensors[self.prefix + "out.weight"].float()
+
+        def forward(self, x, ctx, cache):
+            assert cache.kpool is None and cache.state.shape[1] == self.state_bytes()
+            out = ctx.alloc((ctx.rows, self.D))
+            r = 0
+            for n, slot in zip(ctx.host["q_lens"], ctx.host["slots"]):
+                st = cache.state[slot].view(torch.float32)          # [D + 1], zeroed at acquire
+                sums = st[:self.D] + x[r:r + n].float().cumsum(0)
+                counts = st[self.D] + torch.arange(1, n + 1, device=x.device)
+                out[r:r + n] = ((sums / counts[:, None]) @ self.w.T).to(out.dtype)
+                st[:self.D] = sums[-1]
+                st[self.D] = counts[-1]
+                r += n
+            return out
+
+    @parts.register_part("position", "toy_scale_by_position")
+    class ScaleByPosition(parts.PositionEncoding):
+        """q, k <- q, k * (1 + pos / 100): not a rotation, so it runs through apply()."""
+        custom = True
+
+        def __init__(self, params, prefix, env):
+            super().__init__(prefix, env)
+
+        def apply(self, q, k, ctx):
+            f = (1 + ctx.positions[:ctx.rows].float() / 100)[:, None, None]
+            q.copy_((q.float() * f).to(q.dtype))
+            if k is not None:
+                k.copy_((k.float() * f).to(k.dtype))
+
+    @dataclasses.dataclass
+    class ToyConfig(ModelConfig):
+        vocab_size: int = 0
+        hidden_size: int = 0
+        kind: str = "state"
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(architecture=architecture_name(d), vocab_size=read_field(d, "vocab_size", int),
+                       hidden_size=read_field(d, "hidden_size", int), kind=read_field(d, "kind", str, "state"))
+
+        def to_dict(self):
+            return {"architectures": [self.architecture], "vocab_size": self.vocab_size,
+                    "hidden_size": self.hidden_size, "kind": self.kind}
+
+    def toy_spec(cfg):
+        D, V = cfg.hidden_size, cfg.vocab_size
+        norm = parts.PartSpec("rmsnorm", {"size": D, "eps": 1e-5})
+        ff = parts.PartSpec("gated_mlp", {"hidden_size": D, "intermediate_size": 2 * D + 8})
+        names = {"mixer_norm": "ln1", "mixer": "mix", "feed_forward_norm": "ln2", "feed_forward": "ff"}
+
+        def attn(pos):
+            return parts.PartSpec("attention", {"hidden_size": D, "num_heads": 4, "num_kv_heads": 2,
+                                                "head_dim": 16, "qkv_bias": True, "position": pos})
+
+        def block(mixer):
+            return parts.PartSpec("pre_norm", {"mixer_norm": norm, "feed_forward_norm": norm, "mixer": mixer,
+                                               "feed_forward": ff, "names": names})
+
+        rotary = parts.PartSpec("rotary", {"head_dim": 16, "theta": 1e4})
+        if cfg.kind == "state":
+            mixers = [attn(rotary), parts.PartSpec("toy_running_mean", {"hidden_size": D}), attn(rotary)]
+            schedule = [parts.ScheduleEntry(0), parts.ScheduleEntry(1), parts.ScheduleEntry(2)]
+        elif cfg.kind == "position":
+            mixers = [attn(parts.PartSpec("toy_scale_by_position")), attn(parts.PartSpec("none"))]
+            schedule = [parts.ScheduleEntry(0), parts.ScheduleEntry(1)]
+        elif cfg.kind == "twice":
+            mixers = [attn(rotary), attn(rotary)]
+            schedule = [parts.ScheduleEntry(0), parts.ScheduleEntry(1), parts.ScheduleEntry(1)]
+        else:   # "shared": the third run reads the keys and values the second run wrote
+            mixers = [attn(rotary), attn(rotary)]
+            schedule = [parts.ScheduleEntry(0), parts.ScheduleEntry(1), parts.ScheduleEntry(1, cache_from=1)]
+        return parts.ModelSpec(
+            hidden_size=D, vocab_size=V,
+            embedding=parts.PartSpec("token_embedding", {"vocab_size": V, "hidden_size": D}),
+            embedding_prefix="emb.", layers=[parts.LayerSpec(f"layers.{i}.", block(m)) for i, m in enumerate(mixers)],
+            schedule=schedule, final_norm=norm, final_norm_prefix="norm.",
+            head=parts.PartSpec("linear_head", {"vocab_size": V, "hidden_size": D}), head_prefix="head.",
+            max_positions=512)
+
+    he.register_architecture("ToyForCausalLM", ToyConfig, toy_spec)
+    return ToyConfig
+
+
+def toy_plain(w, kind, ids):
+    """The toy models, whole sequences, from the plain implementation's functions."""
+    S = len(ids)
+    pos = torch.arange(S)
+    cfg = {"num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 16, "rope_theta": 1e4}
+    x = P.embedding(torch.tensor(ids), w["emb.weight"])
+    H, KVH, hd = 4, 2, 16
+
+    def attn(l, n, encode, kv=None):
+        p = f"layers.{l}.mix."
+        q = P.linear(n, w[p + "q_proj.weight"], w[p + "q_proj.bias"]).reshape(S, H, hd)
+        q = encode(q)
+        if kv is None:
+            k = encode(P.linear(n, w[p + "k_proj.weight"], w[p + "k_proj.bias"]).reshape(S, KVH, hd))
+            v = P.linear(n, w[p + "v_proj.weight"], w[p + "v_proj.bias"]).reshape(S, KVH, hd)
+        else:
+            k, v = kv
+        return P.linear(P.attention(q, k, v, pos, pos), w[p + "o_proj.weight"]), (k, v)
+
+    def ff(l, h):
+        p = f"layers.{l}."
+        return h + P.swiglu(P.rmsnorm(h, w[p + "ln2.weight"], 1e-5), w[p + "ff.gate_proj.weight"],
+                            w[p + "ff.up_proj.weight"], w[p + "ff.down_proj.weight"])
+
+    rot = lambda t: P.rope(t, pos, 1e4)
+    scale = lambda t: t * (1 + pos.double() / 100)[:, None, None]
+    same = lambda t: t
+    if kind == "state":
+        runs = [(0, rot, None), (1, "mean", None), (2, rot, None)]
+    elif kind == "position":
+        runs = [(0, scale, None), (1, same, None)]
+    elif kind == "twice":
+        runs = [(0, rot, None), (1, rot, None), (1, rot, None)]
+    else:
+        runs = [(0, rot, None), (1, rot, None), (1, rot, 1)]
+    kvs = {}
+    for e, (l, enc, src) in enumerate(runs):
+        n = P.rmsnorm(x, w[f"layers.{l}.ln1.weight"], 1e-5)
+        if enc == "mean":
+            a = (n.cumsum(0) / torch.arange(1, S + 1)[:, None]) @ w[f"layers.{l}.mix.out.weight"].T
+        else:
+            a, kvs[e] = attn(l, n, enc, kvs[src] if src is not None else None)
+        x = ff(l, x + a)
+    return P.linear(P.rmsnorm(x, w["norm.weight"], 1e-5), w["head.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("kind", ["state", "position", "twice", "shared"])
+def test_toy_models_build_and_step(fw, toys, tmp_path, kind, dtype):
+    import hector_engine_amd as he
+    from hector_engine_amd.engine.engine import StepEntry
+    cfg = toys(architecture="ToyForCausalLM", vocab_size=97, hidden_size=64, kind=kind)
+    folder = str(tmp_path / kind)
+    he.write_random_model(cfg, 5, folder)
+    assert he.load_config(folder) == cfg
+    w = {k: v.double() for k, v in P.read_safetensors(os.path.join(folder, "model.safetensors")).items()}
+    eng = he.Engine(folder, dtype=dtype, max_tokens=1024, max_slots=2, max_seq_len=256)
+    assert eng.use_graphs == (kind != "state")            # the host-planning toy switches graphs off
+    if kind == "state":
+        assert eng.cache.state_bytes_per_slot >= 4 * 65 and eng.model.run_plans()[1].kv is None
+        assert len(eng.cache.groups) == 1 and len(eng.cache.groups[0].runs) == 2
+    if kind == "twice":
+        assert len(eng.cache.groups[0].runs) == 3          # a layer named twice has two caches
+    if kind == "shared":
+        assert len(eng.cache.groups[0].runs) == 2 and not eng.caches[2].writes
+        assert eng.caches[2].kpool.data_ptr() == eng.caches[1].kpool.data_ptr()
+    reqs = [rand_ids(97, n, 70 + n) for n in (70, 9, 33, 20)]
+    want = [toy_plain(w, kind, r) for r in reqs]
+    # whole, alone
+    for r, t in zip(reqs, want):
+        s = eng.acquire()
+        close(eng.step([StepEntry(s, r, list(range(len(r))))]), t, dtype)
+        eng.release(s)
+    # two batches through two slots: prompts together, then one token each; shorter ones leave;
+    # the second batch takes the slots (and their state rows) that the first gave back
+    for batch in ([0, 1], [2, 3]):
+        slots = {i: eng.acquire() for i in batch}
+        fed = {i: len(reqs[i]) // 2 for i in batch}
+        got = {i: [] for i in batch}
+        logits = eng.step([StepEntry(slots[i], reqs[i][:fed[i]], list(range(fed[i]))) for i in batch])
+        r0 = 0
+        for i in batch:
+            got[i].append(logits[r0:r0 + fed[i]].clone())
+            r0 += fed[i]
+        live = list(batch)
+        while live:
+            logits = eng.step([StepEntry(slots[i], [reqs[i][fed[i]]], [0]) for i in live])
+            for j, i in enumerate(live):
+                got[i].append(logits[j:j + 1].clone())
+                fed[i] += 1
+            for i in list(live):
+                if fed[i] == len(reqs[i]):
+                    eng.release(slots.pop(i))
+                    live.remove(i)
+        for i in batch:
+            close(torch.cat(got[i]), want[i], dtype)
+
+
+def test_bad_schedules_are_refused(fw, toys):
+    import hector_engine_amd as he
+    from hector_engine_amd.registry import model_spec
+    from hector_engine_amd.engine.model import DecoderModel
+    cfg = toys(architecture="ToyForCausalLM", vocab_size=50, hidden_size=64, kind="shared")
+    env = env_for(fw, torch.float32)
+    spec = model_spec(cfg)
+    spec.schedule = [fw.parts.ScheduleEntry(0), fw.parts.ScheduleEntry(1, cache_from=1)]
+    with pytest.raises(ValueError, match="earlier"):
+        DecoderModel(spec, env)
+    spec.schedule = [fw.parts.ScheduleEntry(0), fw.parts.ScheduleEntry(5)]
+    with pytest.raises(ValueError, match="names layer 5"):
+        DecoderModel(spec, env)
+    with pytest.raises(KeyError, match="registered"):
+        fw.parts.build_part("mixer", fw.parts.PartSpec("no_such_mixer"), "", env)
