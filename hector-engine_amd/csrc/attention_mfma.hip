@@ -176,11 +176,18 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 
 // ------------------------------------------------------------------ decode
 // grid (nsplit, KVH * head_tiles, rows), 64 threads. Columns are the query heads
-// of one kv group (16 per head tile). Each workgroup takes one slice of the keys
-// and writes (m, l, unnormalised O) for its heads; the merge kernel joins them.
+// of one kv group (16 per head tile). The keys of a sequence are cut into slices
+// of at least DECODE_MIN_CHUNK keys, at most nsplit of them; each workgroup takes
+// one slice and writes (m, l, unnormalised O) for its heads; the merge kernel
+// joins the slices in the order of their index:
+//   out = sum_s O_s e^(m_s - M) / sum_s l_s e^(m_s - M)
+// With a single slice in the grid the result is written directly.
+#define DECODE_MIN_CHUNK 128
+
 template <int NT>
 __global__ __launch_bounds__(64) void attention_decode_kernel(
-    float* __restrict__ ws_o, float* __restrict__ ws_ml, const uint16_t* __restrict__ q,
+    uint16_t* __restrict__ out, float* __restrict__ ws_o, float* __restrict__ ws_ml,
+    const uint16_t* __restrict__ q,
     const uint16_t* __restrict__ kpool, const uint16_t* __restrict__ vpool,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
     const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ page_table, int max_blocks,
@@ -196,26 +203,25 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   const int hg = 16 * ht + lr;            // head within the group
   const bool h_ok = hg < G;
   const int h = kvh * G + min(hg, G - 1);
-  const int64_t wsi = ((int64_t)row * H + h) * nsplit + split;
+  uint16_t* orow = out + ((int64_t)row * H + h) * HD;
   const int seq = row_seq[row];
-  int n_keys = 0, first = 0, slot = -1;
-  if (seq >= 0) {
-    slot = seq_slot[seq];
-    n_keys = positions[row] + 1;
-    first = window > 0 ? max(0, n_keys - window) : 0;
-  }
-  const int span_lo = first & ~31;
-  int chunk = (n_keys - span_lo + nsplit - 1) / nsplit;
-  chunk = (chunk + 31) & ~31;
-  const int kb_begin = span_lo + split * chunk;
-  const int kb_end = min(kb_begin + chunk, n_keys);
-  if (slot < 0 || kb_begin >= kb_end) {
-    if (h_ok && lg == 0) {
-      ws_ml[2 * wsi] = -INFINITY;
-      ws_ml[2 * wsi + 1] = 0.f;
-    }
+  if (seq < 0) {                          // padding row: zeros (the merge kernel writes them if there is one)
+    if (nsplit == 1 && h_ok)
+#pragma unroll
+      for (int dt = 0; dt < NT; ++dt)
+        *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * lg) = make_uint2(0u, 0u);
     return;
   }
+  const int slot = seq_slot[seq];
+  const int n_keys = positions[row] + 1;
+  const int first = window > 0 ? max(0, n_keys - window) : 0;
+  const int span_lo = first & ~31;
+  int chunk = (n_keys - span_lo + nsplit - 1) / nsplit;
+  chunk = max(DECODE_MIN_CHUNK, (chunk + 31) & ~31);
+  const int active = (n_keys - span_lo + chunk - 1) / chunk;   // slices that hold keys
+  if (split >= active) return;
+  const int kb_begin = span_lo + split * chunk;
+  const int kb_end = min(kb_begin + chunk, n_keys);
   const int32_t* pt = page_table + (int64_t)slot * max_blocks;
   bf16x8 qf[KS];
   load_q<NT>(qf, q + ((int64_t)row * H + h) * HD, h_ok, lg);
@@ -234,47 +240,74 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   float l = st.l;
   l += __shfl_xor(l, 16, HE_WAVE);
   l += __shfl_xor(l, 32, HE_WAVE);
-  if (!h_ok) return;
-  if (lg == 0) {
-    ws_ml[2 * wsi] = st.m;
-    ws_ml[2 * wsi + 1] = l;
-  }
-  float* o = ws_o + wsi * HD;
+  if (nsplit == 1) {                      // nothing to merge
+    if (!h_ok) return;
+    const float inv = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll
-  for (int dt = 0; dt < NT; ++dt)
-    *reinterpret_cast<float4*>(o + 16 * dt + 4 * lg) =
-        make_float4(st.o[dt][0], st.o[dt][1], st.o[dt][2], st.o[dt][3]);
+    for (int dt = 0; dt < NT; ++dt) {
+      uint2 w;
+      w.x = (uint32_t)float_to_bf16_bits(st.o[dt][0] * inv) |
+            ((uint32_t)float_to_bf16_bits(st.o[dt][1] * inv) << 16);
+      w.y = (uint32_t)float_to_bf16_bits(st.o[dt][2] * inv) |
+            ((uint32_t)float_to_bf16_bits(st.o[dt][3] * inv) << 16);
+      *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * lg) = w;
+    }
+    return;
+  }
+  const int64_t wbase = ((int64_t)row * H + h) * nsplit;
+  if (h_ok) {
+    if (lg == 0) {
+      ws_ml[2 * (wbase + split)] = st.m;
+      ws_ml[2 * (wbase + split) + 1] = l;
+    }
+    float* o = ws_o + (wbase + split) * HD;
+#pragma unroll
+    for (int dt = 0; dt < NT; ++dt)
+      *reinterpret_cast<float4*>(o + 16 * dt + 4 * lg) =
+          make_float4(st.o[dt][0], st.o[dt][1], st.o[dt][2], st.o[dt][3]);
+  }
 }
 
-// out[row][h][:] = sum_s O_s e^(m_s - M) / sum_s l_s e^(m_s - M); grid (H, rows).
-__global__ void attention_merge_kernel(uint16_t* __restrict__ out, const float* __restrict__ ws_o,
-                                       const float* __restrict__ ws_ml, int H, int HD,
-                                       int nsplit) {
-  const int h = blockIdx.x;
+// Joins the slices of one (row, head): grid (H, rows), one wavefront. The number of
+// slices that hold keys is recomputed exactly as the decode kernel computes it.
+__global__ __launch_bounds__(64) void attention_merge_kernel(
+    uint16_t* __restrict__ out, const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq, int H, int HD,
+    int nsplit, int window) {
+  __shared__ float wgt[64];
+  const int h = blockIdx.x, lane = threadIdx.x;
   const int64_t row = blockIdx.y;
-  const int64_t base = (row * H + h) * nsplit;
-  float M = -INFINITY;
-  for (int s = 0; s < nsplit; ++s) M = fmaxf(M, ws_ml[2 * (base + s)]);
-  float L = 0.f;
-  for (int s = 0; s < nsplit; ++s) {
-    const float m = ws_ml[2 * (base + s)];
-    if (m > -INFINITY) L += ws_ml[2 * (base + s) + 1] * __expf(m - M);
+  uint16_t* orow = out + (row * H + h) * (int64_t)HD;
+  if (row_seq[row] < 0) {
+    for (int d = lane; d < HD; d += 64) orow[d] = 0;
+    return;
   }
+  const int n_keys = positions[row] + 1;
+  const int first = window > 0 ? max(0, n_keys - window) : 0;
+  const int span_lo = first & ~31;
+  int chunk = (n_keys - span_lo + nsplit - 1) / nsplit;
+  chunk = max(DECODE_MIN_CHUNK, (chunk + 31) & ~31);
+  const int active = (n_keys - span_lo + chunk - 1) / chunk;
+  const int64_t base = (row * H + h) * nsplit;
+  const float m = lane < active ? ws_ml[2 * (base + lane)] : -INFINITY;
+  const float l = lane < active ? ws_ml[2 * (base + lane) + 1] : 0.f;
+  const float M = wave_max(m);
+  const float w = m > -INFINITY ? __expf(m - M) : 0.f;
+  const float L = wave_sum(l * w);
+  wgt[lane] = w;
+  __syncthreads();
   const float inv = L > 0.f ? 1.f / L : 0.f;
-  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+  for (int d = lane; d < HD; d += 64) {
     float acc = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-      const float m = ws_ml[2 * (base + s)];
-      if (m > -INFINITY) acc += ws_o[(base + s) * HD + d] * __expf(m - M);
-    }
-    out[(row * H + h) * (int64_t)HD + d] = float_to_bf16_bits(acc * inv);
+    for (int s = 0; s < active; ++s) acc += ws_o[(base + s) * HD + d] * wgt[s];
+    orow[d] = float_to_bf16_bits(acc * inv);
   }
 }
 
 static int decode_splits(int rows, int KVH, int head_tiles, int max_keys) {
   const int groups = rows * KVH * head_tiles;
-  int s = (1024 + groups - 1) / groups;
-  const int max_s = (max_keys + 63) / 64;
+  int s = (4096 + groups - 1) / groups;
+  const int max_s = (max_keys + DECODE_MIN_CHUNK - 1) / DECODE_MIN_CHUNK;
   if (s > max_s) s = max_s;
   if (s > 64) s = 64;
   if (s < 1) s = 1;
@@ -330,21 +363,24 @@ extern "C" int he_attention_decode_bf16(void* out, const void* q, const void* kp
              "he_attention_decode_bf16: workspace of %lld floats, need %lld",
              (long long)workspace_floats, (long long)need);
   HE_REQUIRE((((uintptr_t)workspace_f32) & 15) == 0 && (((uintptr_t)q) & 15) == 0 &&
-                 (((uintptr_t)kpool) & 15) == 0 && (((uintptr_t)vpool) & 15) == 0,
+                 (((uintptr_t)kpool) & 15) == 0 && (((uintptr_t)vpool) & 15) == 0 &&
+                 (((uintptr_t)out) & 7) == 0,
              "he_attention_decode_bf16: buffers must be 16-byte aligned");
   hipStream_t s = (hipStream_t)stream;
   float* ws_o = (float*)workspace_f32;
   float* ws_ml = ws_o + (int64_t)rows * H * nsplit * hd;
   dim3 grid(nsplit, KVH * head_tiles, rows);
   ATTN_SWITCH(hd / 16, (attention_decode_kernel<NT><<<grid, 64, 0, s>>>(
-                           ws_o, ws_ml, (const uint16_t*)q, (const uint16_t*)kpool,
-                           (const uint16_t*)vpool, (const int32_t*)positions,
-                           (const int32_t*)row_seq, (const int32_t*)seq_slot,
-                           (const int32_t*)page_table, max_blocks, num_pages, H, KVH, head_tiles,
-                           window, scale)));
+                           (uint16_t*)out, ws_o, ws_ml, (const uint16_t*)q,
+                           (const uint16_t*)kpool, (const uint16_t*)vpool,
+                           (const int32_t*)positions, (const int32_t*)row_seq,
+                           (const int32_t*)seq_slot, (const int32_t*)page_table, max_blocks,
+                           num_pages, H, KVH, head_tiles, window, scale)));
   int rc = he_check_launch("he_attention_decode_bf16");
-  if (rc) return rc;
-  attention_merge_kernel<<<dim3(H, rows), 64, 0, s>>>((uint16_t*)out, ws_o, ws_ml, H, hd, nsplit);
+  if (rc || nsplit == 1) return rc;
+  attention_merge_kernel<<<dim3(H, rows), 64, 0, s>>>(
+      (uint16_t*)out, ws_o, ws_ml, (const int32_t*)positions, (const int32_t*)row_seq, H, hd,
+      nsplit, window);
   return he_check_launch("he_attention_decode_bf16 merge");
 }
 

@@ -87,39 +87,61 @@ extern "C" int he_residual_add(void* resid_f32, const void* delta, int64_t n, in
   return he_check_launch("he_residual_add");
 }
 
-// out[r, i] = silu(x[r, i]) * x[r, I + i] with x = [rows, 2I] (gate then up),
+// out[r, i] = silu(gate[r, i]) * up[r, i] with x = [rows, 2I],
 // silu(z) = z / (1 + exp(-z)) in fp32 (reference: kernels/activations.cu:19-21,183-198).
-template <typename T>
-__global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ x, int64_t rows,
-                                int I) {
+// Column layout of x: gate then up (x[r, i], x[r, I + i]); or, interleaved in
+// blocks of 16 as the fused gate||up weight of the MFMA path lays its rows out:
+// gate i at column 32*(i/16) + i%16, its up 16 columns later.
+// With splits > 0, x is the fp32 K slices [splits][rows][2I] of the gate||up product,
+// added here in the order of the slice index.
+template <typename T, typename TI>
+__global__ void silu_mul_kernel(T* __restrict__ out, const TI* __restrict__ x, int64_t rows,
+                                int I, int interleaved, int splits) {
   const int64_t n = rows * (int64_t)I;
+  const int64_t split_stride = rows * 2 * (int64_t)I;
   int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (; i < n; i += stride) {
     const int64_t r = i / I;
     const int c = (int)(i - r * I);
-    const float g = to_float(x[r * 2 * (int64_t)I + c]);
-    const float u = to_float(x[r * 2 * (int64_t)I + I + c]);
+    const int gc = interleaved ? 32 * (c >> 4) + (c & 15) : c;
+    const int uc = interleaved ? gc + 16 : I + c;
+    const TI* row = x + r * 2 * (int64_t)I;
+    float g = to_float(row[gc]), u = to_float(row[uc]);
+    for (int s = 1; s < splits; ++s) {
+      g += to_float(row[s * split_stride + gc]);
+      u += to_float(row[s * split_stride + uc]);
+    }
     const float y = g / (1.f + expf(-g)) * u;
     out[i] = from_float<T>(y);
   }
 }
 
-extern "C" int he_silu_mul(void* out, const void* gate_up, int rows, int I, int dtype,
-                           void* stream) {
+extern "C" int he_silu_mul(void* out, const void* gate_up, int rows, int I, int interleaved,
+                           int splits, int dtype, void* stream) {
   HE_REQUIRE(rows >= 0 && I > 0, "he_silu_mul: bad sizes rows=%d I=%d", rows, I);
+  HE_REQUIRE(!interleaved || (I & 15) == 0,
+             "he_silu_mul: interleaved layout needs I=%d a multiple of 16", I);
+  HE_REQUIRE(splits >= 0 && splits <= 64, "he_silu_mul: bad slice count %d", splits);
+  HE_REQUIRE(dtype == HE_BF16 || dtype == HE_F32, "he_silu_mul: unknown dtype %d", dtype);
   if (rows == 0) return 0;
   const int64_t n = (int64_t)rows * I;
   int64_t blocks = (n + 255) / 256;
   if (blocks > 65535 * 4) blocks = 65535 * 4;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == HE_BF16)
-    silu_mul_kernel<bf16_t><<<(int)blocks, 256, 0, s>>>((bf16_t*)out, (const bf16_t*)gate_up, rows,
-                                                        I);
-  else if (dtype == HE_F32)
-    silu_mul_kernel<float><<<(int)blocks, 256, 0, s>>>((float*)out, (const float*)gate_up, rows,
-                                                       I);
-  else
-    HE_REQUIRE(false, "he_silu_mul: unknown dtype %d", dtype);
+  if (splits > 0) {  // fp32 partial sums in
+    if (dtype == HE_BF16)
+      silu_mul_kernel<bf16_t, float><<<(int)blocks, 256, 0, s>>>(
+          (bf16_t*)out, (const float*)gate_up, rows, I, interleaved, splits);
+    else
+      silu_mul_kernel<float, float><<<(int)blocks, 256, 0, s>>>(
+          (float*)out, (const float*)gate_up, rows, I, interleaved, splits);
+  } else if (dtype == HE_BF16) {
+    silu_mul_kernel<bf16_t, bf16_t><<<(int)blocks, 256, 0, s>>>(
+        (bf16_t*)out, (const bf16_t*)gate_up, rows, I, interleaved, 1);
+  } else {
+    silu_mul_kernel<float, float><<<(int)blocks, 256, 0, s>>>((float*)out, (const float*)gate_up,
+                                                              rows, I, interleaved, 1);
+  }
   return he_check_launch("he_silu_mul");
 }

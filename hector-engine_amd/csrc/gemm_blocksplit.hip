@@ -1,0 +1,248 @@
+// bf16 matrix product for few rows (M <= 32) with K cut inside the workgroup:
+// C[M,N] = X[M,K] * W[N,K]^T (+ bias), or the gated activation of a gate||up
+// weight. One workgroup owns 16*R weight rows; its NW wavefronts take one K slice
+// each (operands straight from global memory into the MFMA registers, as in
+// gemm_skinny.hip, whose operand layout this kernel shares), leave their fp32
+// tiles in LDS, and the workgroup adds the slices in wavefront order and writes
+// the result. The sum is complete inside one launch: no partial sums in global
+// memory, no second kernel, no atomics, and the order of the additions is fixed.
+// With 16 wavefronts a product as small as 3584 x 3584 still puts 3584
+// wavefronts on the chip.
+//
+// Gated epilogue: the weight interleaves gate and up rows in blocks of 16, the
+// two row tiles of a workgroup (R = 2) are a gate block and its up block, and the
+// output is silu(gate) * up, [M, N/2] (reference: kernels/activations.cu:183-198
+// as a kernel of its own).
+#include "common.h"
+#include "hector_kernels.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+__device__ __forceinline__ bf16x8 bs_load8(const uint16_t* p, bool ok) {
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (ok) v = *reinterpret_cast<const uint4*>(p);
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+template <typename TC>
+__device__ __forceinline__ void bs_store4(TC* p, const float v[4], bool vec, int valid);
+template <>
+__device__ __forceinline__ void bs_store4<float>(float* p, const float v[4], bool vec, int valid) {
+  if (vec && valid == 4) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  } else {
+    for (int i = 0; i < valid; ++i) p[i] = v[i];
+  }
+}
+template <>
+__device__ __forceinline__ void bs_store4<bf16_t>(bf16_t* p, const float v[4], bool vec,
+                                                  int valid) {
+  if (vec && valid == 4) {
+    uint2 w;
+    w.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+    w.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+    *reinterpret_cast<uint2*>(p) = w;
+  } else {
+    for (int i = 0; i < valid; ++i) p[i].v = float_to_bf16_bits(v[i]);
+  }
+}
+
+// grid: one workgroup per 16*R weight rows; block: 64 * NW threads.
+template <int MT, int R, int U, bool GATED, typename TC>
+__global__ __launch_bounds__(1024) void gemm_blocksplit_kernel(
+    TC* __restrict__ C, const uint16_t* __restrict__ X, const uint16_t* __restrict__ W,
+    const void* __restrict__ bias, int bias_dtype, int M, int N, int K, int kslice) {
+  extern __shared__ float4 tiles[];   // [NW][R*MT][64]
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int n0 = blockIdx.x * 16 * R;
+  const int k_begin = wave * kslice;
+  const int k_end = min(K, k_begin + kslice);
+  const int lr = lane & 15, lg = lane >> 4;
+
+  const uint16_t* wp[R];
+  const uint16_t* xp[MT];
+#pragma unroll
+  for (int r = 0; r < R; ++r) wp[r] = W + (int64_t)min(n0 + 16 * r + lr, N - 1) * K + lg * 16;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) xp[t] = X + (int64_t)min(16 * t + lr, M - 1) * K + lg * 16;
+
+  floatx4 acc[R][MT];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[r][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  for (int k = k_begin; k < k_end; k += 64 * U) {
+    bf16x8 a[U][R][2], b[U][MT][2];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kk = k + 64 * u + lg * 16;   // this lane's 16 k values of the step
+      const bool ok0 = kk + 8 <= k_end, ok1 = kk + 16 <= k_end;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        a[u][r][0] = bs_load8(wp[r] + k + 64 * u, ok0);
+        a[u][r][1] = bs_load8(wp[r] + k + 64 * u + 8, ok1);
+      }
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        b[u][t][0] = bs_load8(xp[t] + k + 64 * u, ok0);
+        b[u][t][1] = bs_load8(xp[t] + k + 64 * u + 8, ok1);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+          for (int t = 0; t < MT; ++t)
+            acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][r][h], b[u][t][h], acc[r][t],
+                                                                0, 0, 0);
+  }
+
+  // every wavefront leaves its tiles; acc[r][t][i] = D[n0 + 16r + 4lg + i][16t + lr]
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+      tiles[(wave * (R * MT) + r * MT + t) * 64 + lane] =
+          make_float4(acc[r][t][0], acc[r][t][1], acc[r][t][2], acc[r][t][3]);
+  __syncthreads();
+
+  // thread (tile, lane) adds the slices in wavefront order and writes 4 outputs
+  constexpr int OUT_TILES = GATED ? (R / 2) * MT : R * MT;
+  for (int item = threadIdx.x; item < OUT_TILES * 64; item += blockDim.x) {
+    const int ot = item >> 6, ol = item & 63;
+    const int olr = ol & 15, olg = ol >> 4;
+    const int t = ot % MT;
+    const int r = GATED ? 2 * (ot / MT) : ot / MT;
+    const int m = 16 * t + olr;
+    if (m >= M) continue;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f), s2 = s;
+    for (int w = 0; w < nw; ++w) {
+      const float4 v = tiles[(w * (R * MT) + r * MT + t) * 64 + ol];
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+      if (GATED) {
+        const float4 u2 = tiles[(w * (R * MT) + (r + 1) * MT + t) * 64 + ol];
+        s2.x += u2.x; s2.y += u2.y; s2.z += u2.z; s2.w += u2.w;
+      }
+    }
+    float v[4] = {s.x, s.y, s.z, s.w};
+    if (GATED) {
+      const float up[4] = {s2.x, s2.y, s2.z, s2.w};
+      const int NO = N >> 1;
+      const int n = (n0 >> 1) + 8 * r + 4 * olg;
+      const int valid = min(4, NO - n);
+      if (valid <= 0) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = v[i] / (1.f + expf(-v[i])) * up[i];
+      bs_store4<TC>(C + (int64_t)m * NO + n, v, (NO & 3) == 0, valid);
+    } else {
+      const int n = n0 + 16 * r + 4 * olg;
+      const int valid = min(4, N - n);
+      if (valid <= 0) continue;
+      if (bias != nullptr)
+        for (int i = 0; i < valid; ++i) v[i] += load_param(bias, n + i, bias_dtype);
+      bs_store4<TC>(C + (int64_t)m * N + n, v, (N & 3) == 0, valid);
+    }
+  }
+}
+
+struct BlockSplitPlan {
+  int MT, R, U, NW, kslice;
+};
+
+// Tilings measured on MI355X (graph-timed sweeps over R, U and NW at the Qwen2.5-7B
+// shapes). The rule depends on the sizes only, so a product always runs the same way.
+static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int U, int NW) {
+  BlockSplitPlan p;
+  p.MT = (M + 15) / 16;
+  int r, u, nw;
+  if (N >= 65536) {                 // output head
+    if (p.MT == 1 && M <= 4) r = 1, u = 2, nw = 16;
+    else if (p.MT == 1) r = 2, u = 4, nw = 8;
+    else r = 2, u = 2, nw = 2;
+  } else if (K >= 8192) {           // long K (down projection)
+    if (p.MT == 1) r = 1, u = 2, nw = 8;
+    else r = 1, u = 1, nw = 8;
+  } else if (N >= 16384) {          // wide N (gate||up)
+    r = 2, u = 1, nw = p.MT == 1 ? 8 : 4;
+  } else {                          // small products (q||k||v, o)
+    r = 1, u = 1, nw = p.MT == 1 ? 16 : 8;
+  }
+  if (gated) r = 2, u = u > 2 ? 2 : u;
+  p.R = R > 0 ? R : r;
+  p.U = U > 0 ? U : u;
+  if (NW <= 0) {
+    NW = nw;
+    while (NW > 1 && K / NW < 128) NW >>= 1;
+  }
+  p.NW = NW;
+  int ks = (K + NW - 1) / NW;
+  p.kslice = (ks + 63) / 64 * 64;
+  return p;
+}
+
+template <int MT, int R, int U, bool GATED, typename TC>
+static void launch_blocksplit(const BlockSplitPlan& p, void* C, const void* X, const void* W,
+                              const void* bias, int bias_dtype, int M, int N, int K,
+                              hipStream_t s) {
+  const int blocks = (N + 16 * R - 1) / (16 * R);
+  const size_t lds = (size_t)p.NW * R * MT * 64 * sizeof(float4);
+  gemm_blocksplit_kernel<MT, R, U, GATED, TC><<<blocks, 64 * p.NW, lds, s>>>(
+      (TC*)C, (const uint16_t*)X, (const uint16_t*)W, bias, bias_dtype, M, N, K, p.kslice);
+}
+
+template <bool GATED, typename TC>
+static int dispatch_blocksplit(const BlockSplitPlan& p, void* C, const void* X, const void* W,
+                               const void* bias, int bias_dtype, int M, int N, int K,
+                               hipStream_t s) {
+#define BS(MT_, R_, U_)                                                              \
+  if (p.MT == MT_ && p.R == R_ && p.U == U_) {                                       \
+    launch_blocksplit<MT_, R_, U_, GATED, TC>(p, C, X, W, bias, bias_dtype, M, N, K, s); \
+    return 0;                                                                        \
+  }
+  if (!GATED) {
+    BS(1, 1, 1) BS(1, 1, 2) BS(1, 1, 4) BS(2, 1, 1) BS(2, 1, 2)
+  }
+  BS(1, 2, 1) BS(1, 2, 2) BS(1, 2, 4) BS(2, 2, 1) BS(2, 2, 2)
+#undef BS
+  he_set_error("he_gemm_blocksplit_bf16: no kernel for MT=%d R=%d U=%d", p.MT, p.R, p.U);
+  return -1;
+}
+
+// R, U, NW <= 0 choose the heuristic tiling (NW wavefronts = K slices per workgroup).
+extern "C" int he_gemm_blocksplit_bf16(void* C, const void* A, const void* W, const void* bias,
+                                       int M, int N, int K, int out_dtype, int bias_dtype,
+                                       int gated, int R, int U, int NW, void* stream) {
+  HE_REQUIRE(M > 0 && M <= HE_BLOCKSPLIT_MAX_M, "he_gemm_blocksplit_bf16: M=%d outside [1, %d]", M,
+             HE_BLOCKSPLIT_MAX_M);
+  HE_REQUIRE(N > 0 && K > 0, "he_gemm_blocksplit_bf16: bad sizes N=%d K=%d", N, K);
+  HE_REQUIRE((K & 7) == 0, "he_gemm_blocksplit_bf16: K=%d must be a multiple of 8", K);
+  HE_REQUIRE(out_dtype == HE_BF16 || out_dtype == HE_F32, "he_gemm_blocksplit_bf16: bad out dtype");
+  HE_REQUIRE((((uintptr_t)A | (uintptr_t)W) & 15) == 0,
+             "he_gemm_blocksplit_bf16: operands must be 16-byte aligned");
+  HE_REQUIRE(!gated || ((N & 31) == 0 && bias == nullptr),
+             "he_gemm_blocksplit_bf16: the gated epilogue needs N=%d a multiple of 32 and no bias",
+             N);
+  const BlockSplitPlan p = blocksplit_plan(M, N, K, gated, R, U, NW);
+  HE_REQUIRE(p.NW >= 1 && p.NW <= 16, "he_gemm_blocksplit_bf16: %d wavefronts outside [1, 16]",
+             p.NW);
+  HE_REQUIRE(!gated || p.R == 2, "he_gemm_blocksplit_bf16: the gated epilogue needs R = 2");
+  hipStream_t s = (hipStream_t)stream;
+  int rc;
+  if (gated)
+    rc = out_dtype == HE_BF16
+             ? dispatch_blocksplit<true, bf16_t>(p, C, A, W, bias, bias_dtype, M, N, K, s)
+             : dispatch_blocksplit<true, float>(p, C, A, W, bias, bias_dtype, M, N, K, s);
+  else
+    rc = out_dtype == HE_BF16
+             ? dispatch_blocksplit<false, bf16_t>(p, C, A, W, bias, bias_dtype, M, N, K, s)
+             : dispatch_blocksplit<false, float>(p, C, A, W, bias, bias_dtype, M, N, K, s);
+  if (rc) return rc;
+  return he_check_launch("he_gemm_blocksplit_bf16");
+}

@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 4
+#define HE_ABI_VERSION 8
 
 #ifdef __cplusplus
 extern "C" {
@@ -21,12 +21,17 @@ int he_embedding(void* out_f32, const void* table, const void* ids, int rows, in
 int he_gather_rows_f32(void* out, const void* src, const void* rows, int n_out, int D, int n_src,
                        void* stream);
 int he_residual_add(void* resid_f32, const void* delta, int64_t n, int delta_dtype, void* stream);
-int he_silu_mul(void* out, const void* gate_up, int rows, int I, int dtype, void* stream);
+// splits > 0: gate_up is fp32 [splits][rows][2I], the K slices of the product.
+int he_silu_mul(void* out, const void* gate_up, int rows, int I, int interleaved, int splits,
+                int dtype, void* stream);
 
 // ---- norms ---------------------------------------------------------------
-// resid (fp32, in place) += delta (may be null); out (may be null) = rmsnorm(resid) * weight
-int he_add_rmsnorm(void* resid_f32, const void* delta, const void* weight, void* out, int rows,
-                   int D, float eps, int act_dtype, int w_dtype, void* stream);
+// resid (fp32, in place) += delta (may be null); out (may be null) = rmsnorm(resid) * weight.
+// delta_splits > 0: delta is fp32 [delta_splits][rows][D], the K slices of a product, added
+// in index order together with delta_bias[D] (may be null).
+int he_add_rmsnorm(void* resid_f32, const void* delta, int delta_splits, const void* delta_bias,
+                   int bias_dtype, const void* weight, void* out, int rows, int D, float eps,
+                   int act_dtype, int w_dtype, void* stream);
 int he_rmsnorm_rows(void* out, const void* x, const void* weight, int rows, int D,
                     int64_t x_stride, int64_t out_stride, float eps, int dtype, int w_dtype,
                     void* stream);
@@ -37,14 +42,28 @@ int he_gemm_plain(void* C, const void* A, const void* W, const void* bias, int M
                   int bias_dtype, void* stream);
 // bf16 MFMA product for M <= HE_SKINNY_MAX_M rows: every weight element is read once.
 #define HE_SKINNY_MAX_M 64
-int he_gemm_skinny_bf16(void* C, const void* A, const void* W, const void* bias, int M, int N,
-                        int K, int out_dtype, int bias_dtype, void* workspace_f32,
-                        int64_t workspace_floats, void* stream);
-int64_t he_gemm_skinny_workspace_floats(int M, int N, int K);
+// gated: W's rows interleave gate and up in blocks of 16 and C is [M, N/2] = silu(gate) * up.
+// R, U, splits <= 0 choose the heuristic tiling. When K is cut into more than one slice, C is
+// not written: partial_f32 receives fp32 [slices][M][N] (bias not added) and *splits_used says
+// how many; the reader adds them in index order (he_splitk_reduce, he_add_rmsnorm, he_qkv_rope_cache).
+int he_gemm_skinny_bf16(void* C, void* partial_f32, int64_t partial_floats, const void* A,
+                        const void* W, const void* bias, int M, int N, int K, int out_dtype,
+                        int bias_dtype, int gated, int R, int U, int splits, int* splits_used,
+                        void* stream);
+int he_gemm_skinny_splits(int M, int N, int K);
+// bf16 MFMA product for M <= HE_BLOCKSPLIT_MAX_M with K cut inside the workgroup (NW
+// wavefronts, one slice each, added in LDS): complete in one launch.
+#define HE_BLOCKSPLIT_MAX_M 32
+int he_gemm_blocksplit_bf16(void* C, const void* A, const void* W, const void* bias, int M, int N,
+                            int K, int out_dtype, int bias_dtype, int gated, int R, int U, int NW,
+                            void* stream);
+int he_splitk_reduce(void* C, const void* partial_f32, const void* bias, int M, int N, int splits,
+                     int out_dtype, int bias_dtype, void* stream);
 
 // ---- position encoding + cache write -------------------------------------
 int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const void* q_in, const void* k_in,
-                      const void* v_in, int64_t in_stride, const void* q_bias, const void* k_bias,
+                      const void* v_in, int64_t in_stride, int in_splits, const void* q_bias,
+                      const void* k_bias,
                       const void* v_bias, int bias_dtype, const void* positions,
                       const void* row_seq, const void* seq_slot, const void* page_table,
                       int max_blocks, int num_pages, const void* inv_freq, int rotary_dim, int rows,

@@ -8,16 +8,27 @@
 //   y[i]       = x[i] * cos a - x[i + r/2] * sin a
 //   y[i + r/2] = x[i] * sin a + x[i + r/2] * cos a
 // and dims >= r pass through. All of it in fp32.
+//
+// The projected rows may arrive as the fp32 partial sums [splits][rows][width]
+// of a product cut along K; they are added here in the order of the slice index.
 #include "common.h"
 #include "hector_kernels.h"
 
 #define ROPE_MAX_HALF 256
 
-template <typename T>
+template <typename TI>
+__device__ __forceinline__ float load_in(const TI* p, int splits, int64_t split_stride) {
+  if (splits <= 1) return to_float(p[0]);
+  float s = 0.f;
+  for (int i = 0; i < splits; ++i) s += to_float(p[i * split_stride]);
+  return s;
+}
+
+template <typename T, typename TI>
 __global__ void qkv_rope_cache_kernel(
     T* __restrict__ q_out, T* __restrict__ kpool, T* __restrict__ vpool,
-    const T* __restrict__ q_in, const T* __restrict__ k_in, const T* __restrict__ v_in,
-    int64_t in_stride, const void* __restrict__ q_bias, const void* __restrict__ k_bias,
+    const TI* __restrict__ q_in, const TI* __restrict__ k_in, const TI* __restrict__ v_in,
+    int64_t in_stride, int splits, int64_t split_stride, const void* __restrict__ q_bias, const void* __restrict__ k_bias,
     const void* __restrict__ v_bias, int bias_dtype, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ row_seq, const int32_t* __restrict__ seq_slot,
     const int32_t* __restrict__ page_table, int max_blocks, int num_pages,
@@ -39,7 +50,7 @@ __global__ void qkv_rope_cache_kernel(
 
   // ---- q: rotate and store densely
   {
-    const T* in = q_in + row * in_stride;
+    const TI* in = q_in + row * in_stride;
     T* out = q_out + row * (int64_t)H * hd;
     const int per_head = half + (hd - rotary_dim);
     for (int it = threadIdx.x; it < H * per_head; it += blockDim.x) {
@@ -47,8 +58,8 @@ __global__ void qkv_rope_cache_kernel(
       const int j = it - h * per_head;
       const int base = h * hd;
       if (j < half) {
-        float x0 = to_float(in[base + j]);
-        float x1 = to_float(in[base + j + half]);
+        float x0 = load_in(in + base + j, splits, split_stride);
+        float x1 = load_in(in + base + j + half, splits, split_stride);
         if (q_bias) {
           x0 += load_param(q_bias, base + j, bias_dtype);
           x1 += load_param(q_bias, base + j + half, bias_dtype);
@@ -58,7 +69,7 @@ __global__ void qkv_rope_cache_kernel(
         out[base + j + half] = from_float<T>(x0 * sn + x1 * c);
       } else {
         const int d = rotary_dim + (j - half);
-        float x = to_float(in[base + d]);
+        float x = load_in(in + base + d, splits, split_stride);
         if (q_bias) x += load_param(q_bias, base + d, bias_dtype);
         out[base + d] = from_float<T>(x);
       }
@@ -72,7 +83,7 @@ __global__ void qkv_rope_cache_kernel(
   const int off = pos & (HE_PAGE_TOKENS - 1);
   // ---- k: rotate and scatter
   {
-    const T* in = k_in + row * in_stride;
+    const TI* in = k_in + row * in_stride;
     const int per_head = half + (hd - rotary_dim);
     for (int it = threadIdx.x; it < KVH * per_head; it += blockDim.x) {
       const int h = it / per_head;
@@ -80,8 +91,8 @@ __global__ void qkv_rope_cache_kernel(
       const int base = h * hd;
       T* out = kpool + (((int64_t)page * KVH + h) * HE_PAGE_TOKENS + off) * hd;
       if (j < half) {
-        float x0 = to_float(in[base + j]);
-        float x1 = to_float(in[base + j + half]);
+        float x0 = load_in(in + base + j, splits, split_stride);
+        float x1 = load_in(in + base + j + half, splits, split_stride);
         if (k_bias) {
           x0 += load_param(k_bias, base + j, bias_dtype);
           x1 += load_param(k_bias, base + j + half, bias_dtype);
@@ -91,7 +102,7 @@ __global__ void qkv_rope_cache_kernel(
         out[j + half] = from_float<T>(x0 * sn + x1 * c);
       } else {
         const int d = rotary_dim + (j - half);
-        float x = to_float(in[base + d]);
+        float x = load_in(in + base + d, splits, split_stride);
         if (k_bias) x += load_param(k_bias, base + d, bias_dtype);
         out[d] = from_float<T>(x);
       }
@@ -99,11 +110,11 @@ __global__ void qkv_rope_cache_kernel(
   }
   // ---- v: bias and scatter
   {
-    const T* in = v_in + row * in_stride;
+    const TI* in = v_in + row * in_stride;
     for (int it = threadIdx.x; it < KVH * hd; it += blockDim.x) {
       const int h = it / hd;
       const int d = it - h * hd;
-      float x = to_float(in[it]);
+      float x = load_in(in + it, splits, split_stride);
       if (v_bias) x += load_param(v_bias, it, bias_dtype);
       // V is stored transposed inside a page: [head_dim][tokens]
       vpool[(((int64_t)page * KVH + h) * hd + d) * HE_PAGE_TOKENS + off] = from_float<T>(x);
@@ -113,7 +124,7 @@ __global__ void qkv_rope_cache_kernel(
 
 extern "C" int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const void* q_in,
                                  const void* k_in, const void* v_in, int64_t in_stride,
-                                 const void* q_bias, const void* k_bias, const void* v_bias,
+                                 int in_splits, const void* q_bias, const void* k_bias, const void* v_bias,
                                  int bias_dtype, const void* positions, const void* row_seq,
                                  const void* seq_slot, const void* page_table, int max_blocks,
                                  int num_pages, const void* inv_freq, int rotary_dim, int rows,
@@ -128,21 +139,29 @@ extern "C" int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const vo
   HE_REQUIRE((k_in == nullptr) == (v_in == nullptr), "he_qkv_rope_cache: k and v go together");
   HE_REQUIRE(k_in == nullptr || (kpool && vpool && page_table && max_blocks > 0 && KVH > 0),
              "he_qkv_rope_cache: cache arguments missing");
+  HE_REQUIRE(in_splits >= 0 && in_splits <= 64, "he_qkv_rope_cache: bad slice count %d", in_splits);
+  HE_REQUIRE(dtype == HE_BF16 || dtype == HE_F32, "he_qkv_rope_cache: unknown dtype %d", dtype);
   if (rows == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const int threads = 256;
-#define ROPE_LAUNCH(T)                                                                          \
-  qkv_rope_cache_kernel<T><<<rows, threads, 0, s>>>(                                            \
-      (T*)q_out, (T*)kpool, (T*)vpool, (const T*)q_in, (const T*)k_in, (const T*)v_in,          \
-      in_stride, q_bias, k_bias, v_bias, bias_dtype, (const int32_t*)positions,                 \
-      (const int32_t*)row_seq, (const int32_t*)seq_slot, (const int32_t*)page_table, max_blocks, \
-      num_pages, (const float*)inv_freq, rotary_dim, H, KVH, hd)
-  if (dtype == HE_BF16)
-    ROPE_LAUNCH(bf16_t);
-  else if (dtype == HE_F32)
-    ROPE_LAUNCH(float);
-  else
-    HE_REQUIRE(false, "he_qkv_rope_cache: unknown dtype %d", dtype);
+  const int64_t split_stride = (int64_t)rows * in_stride;
+#define ROPE_LAUNCH(T, TI)                                                                      \
+  qkv_rope_cache_kernel<T, TI><<<rows, threads, 0, s>>>(                                        \
+      (T*)q_out, (T*)kpool, (T*)vpool, (const TI*)q_in, (const TI*)k_in, (const TI*)v_in,       \
+      in_stride, in_splits, split_stride, q_bias, k_bias, v_bias, bias_dtype,                   \
+      (const int32_t*)positions, (const int32_t*)row_seq, (const int32_t*)seq_slot,             \
+      (const int32_t*)page_table, max_blocks, num_pages, (const float*)inv_freq, rotary_dim, H, \
+      KVH, hd)
+  if (in_splits > 0) {  // the input rows are fp32 partial sums
+    if (dtype == HE_BF16)
+      ROPE_LAUNCH(bf16_t, float);
+    else
+      ROPE_LAUNCH(float, float);
+  } else if (dtype == HE_BF16) {
+    ROPE_LAUNCH(bf16_t, bf16_t);
+  } else {
+    ROPE_LAUNCH(float, float);
+  }
 #undef ROPE_LAUNCH
   return he_check_launch("he_qkv_rope_cache");
 }

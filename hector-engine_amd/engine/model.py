@@ -77,7 +77,7 @@ class DecoderModel:
         stream = ResidualStream(resid, rows)
         for e, entry in enumerate(self.schedule):
             self.blocks[entry.layer].forward(stream, ctx, caches[e])
-        stream.materialize()
+        stream.materialize(ctx)
         if n_want == 0:
             return None
         sel = ctx.alloc((n_want, self.spec.hidden_size), torch.float32)

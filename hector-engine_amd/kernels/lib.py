@@ -16,7 +16,7 @@ _lib = None
 
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 
-EXPECTED_ABI = 4
+EXPECTED_ABI = 8
 
 c_int, c_i64, c_f32, c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
@@ -26,15 +26,19 @@ _SIGNATURES = {
     "he_embedding": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_ptr],
     "he_gather_rows_f32": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_ptr],
     "he_residual_add": [c_ptr, c_ptr, c_i64, c_int, c_ptr],
-    "he_silu_mul": [c_ptr, c_ptr, c_int, c_int, c_int, c_ptr],
-    "he_add_rmsnorm": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_f32, c_int, c_int, c_ptr],
+    "he_silu_mul": [c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_ptr],
+    "he_add_rmsnorm": [c_ptr, c_ptr, c_int, c_ptr, c_int, c_ptr, c_ptr, c_int, c_int, c_f32, c_int,
+                       c_int, c_ptr],
     "he_rmsnorm_rows": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_i64, c_i64, c_f32, c_int, c_int, c_ptr],
     "he_gemm_plain": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_i64, c_i64, c_i64,
                       c_int, c_int, c_int, c_ptr],
-    "he_gemm_skinny_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int,
-                            c_ptr, c_i64, c_ptr],
-    "he_gemm_skinny_workspace_floats": [c_int, c_int, c_int],
-    "he_qkv_rope_cache": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_ptr,
+    "he_gemm_skinny_bf16": [c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int,
+                            c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(c_int), c_ptr],
+    "he_gemm_skinny_splits": [c_int, c_int, c_int],
+    "he_gemm_blocksplit_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_int,
+                                c_int, c_int, c_int, c_ptr],
+    "he_splitk_reduce": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_ptr],
+    "he_qkv_rope_cache": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_int, c_ptr, c_ptr, c_ptr,
                           c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_ptr, c_int, c_int,
                           c_int, c_int, c_int, c_int, c_ptr],
     "he_attention_plain": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int,
@@ -51,7 +55,6 @@ _SIGNATURES = {
     "he_sample_rows": [c_ptr, c_ptr, c_int, c_int, c_i64, c_ptr, c_f32, c_int, c_f32, c_ptr],
 }
 _RESTYPES = {
-    "he_gemm_skinny_workspace_floats": c_i64,
     "he_attention_decode_workspace_floats": c_i64,
 }
 

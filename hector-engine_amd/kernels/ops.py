@@ -76,37 +76,56 @@ def residual_add(resid_f32, delta, rows: int) -> None:
                                  dtype_code(delta.dtype), _stream()))
 
 
-def silu_mul(out, gate_up, rows: int) -> None:
+def silu_mul(out, gate_up, rows: int, interleaved: bool = False, splits: int = 0) -> None:
+    """out[rows, I] = silu(gate) * up. gate_up: [rows, 2I] in out's dtype, or with
+    splits > 0 the fp32 K slices [splits, rows, 2I] of the product."""
     I = out.shape[-1]
     _need(out, "out")
-    _need(gate_up, "gate_up", out.dtype)
-    if gate_up.shape[-1] != 2 * I or out.numel() < rows * I or gate_up.numel() < rows * 2 * I:
+    _need(gate_up, "gate_up", torch.float32 if splits > 0 else out.dtype)
+    if gate_up.shape[-1] != 2 * I or out.numel() < rows * I or \
+            gate_up.numel() < max(splits, 1) * rows * 2 * I:
         raise ValueError("silu_mul: gate_up must be [rows, 2*I] for out [rows, I]")
+    if splits > 0 and tuple(gate_up.shape) != (splits, rows, 2 * I):
+        raise ValueError("silu_mul: split sums must be [splits, rows, 2*I]")
     L = _lib.load()
-    _lib.check(L.he_silu_mul(out.data_ptr(), gate_up.data_ptr(), rows, I, dtype_code(out.dtype),
-                             _stream()))
+    _lib.check(L.he_silu_mul(out.data_ptr(), gate_up.data_ptr(), rows, I, int(interleaved), splits,
+                             dtype_code(out.dtype), _stream()))
 
 
-def add_rmsnorm(resid_f32, delta, weight, out, rows: int, eps: float) -> None:
-    """resid += delta (if given); out = rmsnorm(resid) * weight (if out given)."""
+def add_rmsnorm(resid_f32, delta, weight, out, rows: int, eps: float, delta_splits: int = 0,
+                delta_bias=None) -> None:
+    """resid += delta (if given); out = rmsnorm(resid) * weight (if out given).
+    delta_splits > 0: delta is fp32 [delta_splits, rows, D], the K slices of a product,
+    added in index order with delta_bias."""
     D = resid_f32.shape[-1]
     _need(resid_f32, "resid", torch.float32)
     _need(weight, "weight", shape=(D,))
-    act = None
-    for name, t in (("delta", delta), ("out", out)):
-        if t is not None:
-            _need(t, name)
-            if t.shape[-1] != D or t.numel() < rows * D:
-                raise ValueError(f"add_rmsnorm: {name} does not match [rows, {D}]")
-            if act is not None and t.dtype != act:
-                raise TypeError("add_rmsnorm: delta and out must share a dtype")
-            act = t.dtype
     if resid_f32.numel() < rows * D:
         raise ValueError("add_rmsnorm: resid smaller than the row count")
+    act = None
+    if out is not None:
+        _need(out, "out")
+        if out.shape[-1] != D or out.numel() < rows * D:
+            raise ValueError(f"add_rmsnorm: out does not match [rows, {D}]")
+        act = out.dtype
+    if delta is not None:
+        _need(delta, "delta")
+        if delta_splits > 0:
+            if delta.dtype != torch.float32 or tuple(delta.shape) != (delta_splits, rows, D):
+                raise ValueError(f"add_rmsnorm: split sums must be fp32 [{delta_splits}, {rows}, {D}]")
+            if delta_bias is not None:
+                _need(delta_bias, "delta_bias", shape=(D,))
+        else:
+            if delta.shape[-1] != D or delta.numel() < rows * D:
+                raise ValueError(f"add_rmsnorm: delta does not match [rows, {D}]")
+            if act is not None and delta.dtype != act:
+                raise TypeError("add_rmsnorm: delta and out must share a dtype")
+            act = delta.dtype
     L = _lib.load()
-    _lib.check(L.he_add_rmsnorm(resid_f32.data_ptr(), _ptr(delta), weight.data_ptr(), _ptr(out),
-                                rows, D, float(eps), dtype_code(act or torch.float32),
-                                dtype_code(weight.dtype), _stream()))
+    _lib.check(L.he_add_rmsnorm(resid_f32.data_ptr(), _ptr(delta), delta_splits if delta is not None else 0,
+                                _ptr(delta_bias), dtype_code(delta_bias.dtype) if delta_bias is not None else F32,
+                                weight.data_ptr(), _ptr(out), rows, D, float(eps),
+                                dtype_code(act or torch.float32), dtype_code(weight.dtype), _stream()))
 
 
 def rmsnorm_rows(out, x, weight, rows: int, D: int, x_stride: int, out_stride: int,
@@ -139,47 +158,112 @@ def gemm_plain(out, a, w, bias, M: int) -> None:
                                dtype_code(bias.dtype) if bias is not None else F32, _stream()))
 
 
-def gemm_skinny_workspace_floats(M: int, N: int, K: int) -> int:
-    return int(_lib.load().he_gemm_skinny_workspace_floats(M, N, K))
+def gemm_skinny_splits(M: int, N: int, K: int) -> int:
+    """K slices the heuristic cuts this product into (1 = none)."""
+    return int(_lib.load().he_gemm_skinny_splits(M, N, K))
 
 
-def gemm_skinny(out, a, w, bias, M: int, workspace) -> None:
-    """bf16 MFMA product for M <= 64; out is bf16 or fp32."""
+def gemm_skinny(out, partial, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0),
+                out_dtype=None) -> int:
+    """bf16 MFMA product for M <= 64. plan = (R, U, splits), zeros for the heuristic.
+    With one K slice `out` (bf16 or fp32) is written, with bias or, gated, as
+    [M, N/2] = silu(gate) * up for a weight that interleaves gate and up rows in blocks
+    of 16. With more slices `partial` (fp32, room for [slices, M, N]) is written
+    instead, without bias. Returns the number of slices."""
+    import ctypes
     N, K = w.shape
+    NO = N // 2 if gated else N
+    _need(a, "a", torch.bfloat16)
+    _need(w, "w", torch.bfloat16)
+    if M > SKINNY_MAX_M:
+        raise ValueError(f"gemm_skinny: M={M} above {SKINNY_MAX_M}")
+    if a.shape[-1] != K or a.numel() < M * K:
+        raise ValueError(f"gemm_skinny: shapes a{tuple(a.shape)} w{tuple(w.shape)} M={M}")
+    if out is not None:
+        _need(out, "out")
+        if out.shape[-1] != NO or out.numel() < M * NO:
+            raise ValueError(f"gemm_skinny: out{tuple(out.shape)} does not hold [{M}, {NO}]")
+        out_dtype = out.dtype
+    if bias is not None:
+        _need(bias, "bias", shape=(N,))
+    pfloats = 0
+    if partial is not None:
+        _need(partial, "partial", torch.float32)
+        pfloats = partial.numel()
+    L = _lib.load()
+    used = ctypes.c_int(0)
+    if out is None and pfloats == 0:
+        raise ValueError("gemm_skinny: neither an output nor room for partial sums")
+    _lib.check(L.he_gemm_skinny_bf16(_ptr(out), _ptr(partial), pfloats, a.data_ptr(), w.data_ptr(),
+                                     _ptr(bias), M, N, K, dtype_code(out_dtype or torch.bfloat16),
+                                     dtype_code(bias.dtype) if bias is not None else F32, int(gated),
+                                     int(plan[0]), int(plan[1]), int(plan[2]), ctypes.byref(used),
+                                     _stream()))
+    if used.value == 1 and out is None:
+        raise ValueError("gemm_skinny: one K slice was chosen but no output tensor was given")
+    return used.value
+
+
+BLOCKSPLIT_MAX_M = 32
+
+
+def gemm_blocksplit(out, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0)) -> None:
+    """bf16 MFMA product for M <= 32 with K cut inside the workgroup; one launch, complete
+    result (bf16 or fp32), with bias or, gated, as [M, N/2] = silu(gate) * up for a weight
+    that interleaves gate and up rows in blocks of 16. plan = (R, U, NW), zeros = heuristic."""
+    N, K = w.shape
+    NO = N // 2 if gated else N
     _need(a, "a", torch.bfloat16)
     _need(w, "w", torch.bfloat16)
     _need(out, "out")
-    if M > SKINNY_MAX_M:
-        raise ValueError(f"gemm_skinny: M={M} above {SKINNY_MAX_M}")
-    if a.shape[-1] != K or out.shape[-1] != N or a.numel() < M * K or out.numel() < M * N:
-        raise ValueError(f"gemm_skinny: shapes a{tuple(a.shape)} w{tuple(w.shape)} out{tuple(out.shape)} M={M}")
+    if M > BLOCKSPLIT_MAX_M:
+        raise ValueError(f"gemm_blocksplit: M={M} above {BLOCKSPLIT_MAX_M}")
+    if a.shape[-1] != K or a.numel() < M * K or out.shape[-1] != NO or out.numel() < M * NO:
+        raise ValueError(f"gemm_blocksplit: shapes a{tuple(a.shape)} w{tuple(w.shape)} out{tuple(out.shape)} M={M}")
     if bias is not None:
         _need(bias, "bias", shape=(N,))
-    ws_floats = 0
-    if workspace is not None:
-        _need(workspace, "workspace", torch.float32)
-        ws_floats = workspace.numel()
     L = _lib.load()
-    _lib.check(L.he_gemm_skinny_bf16(out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N,
-                                     K, dtype_code(out.dtype),
-                                     dtype_code(bias.dtype) if bias is not None else F32,
-                                     _ptr(workspace), ws_floats, _stream()))
+    _lib.check(L.he_gemm_blocksplit_bf16(out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K,
+                                         dtype_code(out.dtype),
+                                         dtype_code(bias.dtype) if bias is not None else F32, int(gated),
+                                         int(plan[0]), int(plan[1]), int(plan[2]), _stream()))
+
+
+def splitk_reduce(out, partial, bias, M: int, splits: int) -> None:
+    """out[M, N] = sum of partial[s] over the slices in index order (+ bias)."""
+    N = out.shape[-1]
+    _need(out, "out")
+    _need(partial, "partial", torch.float32)
+    if partial.numel() < splits * M * N or out.numel() < M * N:
+        raise ValueError("splitk_reduce: buffers smaller than [splits, M, N]")
+    if bias is not None:
+        _need(bias, "bias", shape=(N,))
+    L = _lib.load()
+    _lib.check(L.he_splitk_reduce(out.data_ptr(), partial.data_ptr(), _ptr(bias), M, N, splits,
+                                  dtype_code(out.dtype),
+                                  dtype_code(bias.dtype) if bias is not None else F32, _stream()))
 
 
 def qkv_rope_cache(q_out, kpool, vpool, qkv, q_cols: int, kv_cols: int, bias, positions, row_seq,
                    seq_slot, page_table, inv_freq, rotary_dim: int, rows: int, H: int, KVH: int,
-                   hd: int, write_kv: bool) -> None:
-    """qkv: [rows, q_cols (+ 2 kv_cols)] projected rows without bias; bias (optional)
-    has the same column layout. Rotated q goes to q_out [rows, H*hd]; k, v go
-    into the pools at (slot, position) when write_kv."""
+                   hd: int, write_kv: bool, splits: int = 0) -> None:
+    """qkv: [rows, q_cols (+ 2 kv_cols)] projected rows without bias, or with splits > 0 the
+    fp32 K slices [splits, rows, width] of that product; bias (optional) has the same
+    column layout. Rotated q goes to q_out [rows, H*hd]; k, v go into the pools at
+    (slot, position) when write_kv."""
     _need(qkv, "qkv")
-    _need(q_out, "q_out", qkv.dtype)
+    _need(q_out, "q_out")
+    if splits > 0:
+        if qkv.dtype != torch.float32 or qkv.dim() != 3 or qkv.shape[0] != splits or qkv.shape[1] != rows:
+            raise ValueError("qkv_rope_cache: split sums must be fp32 [splits, rows, width]")
+    elif qkv.dtype != q_out.dtype:
+        raise TypeError("qkv_rope_cache: qkv and q_out must share a dtype")
     width = qkv.shape[-1]
     if q_cols != H * hd or (write_kv and (kv_cols != KVH * hd or width != q_cols + 2 * kv_cols)):
         raise ValueError("qkv_rope_cache: column layout does not match the head sizes")
     if not write_kv and width < q_cols:
         raise ValueError("qkv_rope_cache: qkv narrower than the query columns")
-    if qkv.numel() < rows * width or q_out.numel() < rows * q_cols:
+    if qkv.numel() < max(splits, 1) * rows * width or q_out.numel() < rows * q_cols:
         raise ValueError("qkv_rope_cache: buffers smaller than the row count")
     _need(positions, "positions", torch.int32)
     _need(row_seq, "row_seq", torch.int32)
@@ -191,8 +275,8 @@ def qkv_rope_cache(q_out, kpool, vpool, qkv, q_cols: int, kv_cols: int, bias, po
     k_in = v_in = None
     max_blocks = num_pages = 0
     if write_kv:
-        _need(kpool, "kpool", qkv.dtype, (None, KVH, PAGE_TOKENS, hd))
-        _need(vpool, "vpool", qkv.dtype, (None, KVH, hd, PAGE_TOKENS))
+        _need(kpool, "kpool", q_out.dtype, (None, KVH, PAGE_TOKENS, hd))
+        _need(vpool, "vpool", q_out.dtype, (None, KVH, hd, PAGE_TOKENS))
         _need(page_table, "page_table", torch.int32)
         num_pages = kpool.shape[0]
         max_blocks = page_table.shape[1]
@@ -213,10 +297,10 @@ def qkv_rope_cache(q_out, kpool, vpool, qkv, q_cols: int, kv_cols: int, bias, po
     L = _lib.load()
     _lib.check(L.he_qkv_rope_cache(
         q_out.data_ptr(), _ptr(kpool) if write_kv else None, _ptr(vpool) if write_kv else None,
-        base, k_in, v_in, width, qb, kb, vb, bias_code, positions.data_ptr(), row_seq.data_ptr(),
+        base, k_in, v_in, width, splits, qb, kb, vb, bias_code, positions.data_ptr(), row_seq.data_ptr(),
         seq_slot.data_ptr(), _ptr(page_table) if write_kv else None, max_blocks, num_pages,
         _ptr(inv_freq) if rotary_dim else None, rotary_dim, rows, H, KVH if write_kv else 0, hd,
-        dtype_code(qkv.dtype), _stream()))
+        dtype_code(q_out.dtype), _stream()))
 
 
 def _check_attention(out, q, kpool, vpool, page_table, rows, H, KVH, hd):

@@ -18,7 +18,7 @@ import torch
 from ..kernels import ops
 from .base import (BuildEnv, KVNeed, LayerCache, Mixer, PartSpec, StepContext, TensorSpec,
                    build_part, param, register_part)
-from .linear import Linear
+from .linear import Linear, SplitSum
 
 
 @register_part("mixer", "attention")
@@ -97,7 +97,10 @@ class Attention(Mixer):
         fused_bias = not self.position.custom
         # With a rotation (or no encoding) the bias is added inside the fused kernel;
         # any other encoding sees q and k with their bias already added.
-        qkv = proj(x, rows, ctx, use_bias=not fused_bias)
+        qkv = proj(x, rows, ctx, use_bias=not fused_bias, allow_split=fused_bias)
+        splits = 0
+        if isinstance(qkv, SplitSum):        # K slices: the q/k/v kernel adds them while it reads
+            splits, qkv = qkv.splits, qkv.partial
         if not fused_bias:
             q_cols, kv_cols = H * hd, KVH * hd
             qv = qkv[:, :q_cols].unflatten(1, (H, hd))
@@ -107,7 +110,8 @@ class Attention(Mixer):
         inv_freq, r = rot if rot is not None else (None, 0)
         ops.qkv_rope_cache(q, cache.kpool, cache.vpool, qkv, H * hd, KVH * hd,
                            proj.bias if fused_bias else None, ctx.positions, ctx.row_seq,
-                           ctx.seq_slot, cache.page_table, inv_freq, r, rows, H, KVH, hd, writes)
+                           ctx.seq_slot, cache.page_table, inv_freq, r, rows, H, KVH, hd, writes,
+                           splits)
         out = ctx.alloc((rows, H * hd))
         if not self.fast:
             ops.attention_plain(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
@@ -123,4 +127,4 @@ class Attention(Mixer):
             ops.attention_prefill(out, q, cache.kpool, cache.vpool, ctx.cu_seqlens, ctx.seq_slot,
                                   ctx.seq_start, cache.page_table, ctx.num_seqs, ctx.max_q_len,
                                   rows, H, KVH, hd, self.window, self.scale)
-        return self.o_proj(out, rows, ctx)
+        return self.o_proj(out, rows, ctx, allow_split=True)

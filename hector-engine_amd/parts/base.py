@@ -159,10 +159,12 @@ class Part:
 
 
 class Norm(Part):
-    def add_norm(self, resid: torch.Tensor, delta: torch.Tensor | None, rows: int,
-                 ctx: StepContext, want_out: bool = True) -> torch.Tensor | None:
+    def add_norm(self, resid: torch.Tensor, delta, rows: int, ctx: StepContext,
+                 want_out: bool = True) -> torch.Tensor | None:
         """resid (fp32 [rows, D], in place) += delta; returns norm(resid) in the
-        activation dtype (or None when want_out is False)."""
+        activation dtype (or None when want_out is False). delta is a tensor, None, or
+        the split sums of a product (parts.linear.SplitSum); a norm that does not add
+        slices itself turns them into a tensor with parts.linear.as_tensor."""
         raise NotImplementedError
 
 
@@ -190,12 +192,15 @@ class Mixer(Part):
         """Bytes of fixed-size state per sequence."""
         return 0
 
-    def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache):
+        """x: [rows, D] normed activations. Returns [rows, D], as a tensor or as the
+        split sums of its last product."""
         raise NotImplementedError
 
 
 class FeedForward(Part):
-    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, ctx: StepContext):
+        """Returns [rows, D], as a tensor or as the split sums of its last product."""
         raise NotImplementedError
 
 
@@ -217,9 +222,10 @@ class ResidualStream:
         self.rows = rows
         self.pending: torch.Tensor | None = None
 
-    def add(self, delta: torch.Tensor) -> None:
+    def add(self, delta, ctx: StepContext) -> None:
+        """delta: a tensor [rows, D] or the split sums of a product."""
         if self.pending is not None:
-            self.materialize()
+            self.materialize(ctx)
         self.pending = delta
 
     def normed(self, norm: Norm, ctx: StepContext) -> torch.Tensor:
@@ -227,10 +233,11 @@ class ResidualStream:
         self.pending = None
         return out
 
-    def materialize(self) -> torch.Tensor:
+    def materialize(self, ctx: StepContext) -> torch.Tensor:
         if self.pending is not None:
             from ..kernels import ops
-            ops.residual_add(self.resid, self.pending, self.rows)
+            from .linear import as_tensor
+            ops.residual_add(self.resid, as_tensor(self.pending, ctx), self.rows)
             self.pending = None
         return self.resid
 

@@ -37,6 +37,6 @@ class PreNormBlock(Block):
 
     def forward(self, stream: ResidualStream, ctx: StepContext, cache: LayerCache) -> None:
         n = stream.normed(self.mixer_norm, ctx)
-        stream.add(self.mixer.forward(n, ctx, cache))
+        stream.add(self.mixer.forward(n, ctx, cache), ctx)
         n = stream.normed(self.ff_norm, ctx)
-        stream.add(self.feed_forward.forward(n, ctx))
+        stream.add(self.feed_forward.forward(n, ctx), ctx)

@@ -7,6 +7,15 @@ Which kernel runs is decided by precision and row count:
                              BLAS library here: kernels/matmul_cublas.cu:240-277)
 A weight that was stored in 32-bit stays 32-bit; under bfloat16 activations it
 runs through the float32 kernel.
+
+Up to 16 rows (and up to 32 when K is long) the block-split kernel runs: K is cut
+inside the workgroup, one launch gives the finished result. From 33 to 64 rows the
+library is faster on MI355X except for long K, where the wavefront kernel with K
+cut across workgroups wins; its fp32 partial sums are added by a small kernel, or,
+when a caller says `allow_split` and SPLIT_TO_CONSUMER is on, handed over as a
+:class:`SplitSum` to a kernel that adds the slices while it reads (the fused norm,
+the q/k/v kernel). That hand-over is off: with few rows the reading kernel has one
+workgroup per row and adding the slices there is slower than the small kernel.
 """
 from __future__ import annotations
 
@@ -16,6 +25,38 @@ from ..kernels import ops
 from .base import StepContext
 
 
+class SplitSum:
+    """fp32 partial sums [slices, rows, N] of one product (+ a bias not yet added)."""
+
+    def __init__(self, partial: torch.Tensor, bias: torch.Tensor | None, rows: int):
+        self.partial = partial
+        self.bias = bias
+        self.rows = rows
+        self.splits = partial.shape[0]
+
+    def materialize(self, ctx: StepContext, dtype: torch.dtype | None = None,
+                    out: torch.Tensor | None = None) -> torch.Tensor:
+        if out is None:
+            out = ctx.alloc((self.rows, self.partial.shape[-1]), dtype or ctx.env.dtype)
+        ops.splitk_reduce(out, self.partial, self.bias, self.rows, self.splits)
+        return out
+
+
+def as_tensor(x, ctx: StepContext) -> torch.Tensor:
+    """A tensor, whether x is one or the split sums of one."""
+    return x.materialize(ctx) if isinstance(x, SplitSum) else x
+
+
+SPLIT_TO_CONSUMER = False
+LONG_K = 8192
+
+
+def _library_is_faster(rows: int, N: int, K: int) -> bool:
+    """Measured on MI355X at the Qwen2.5-7B shapes: above 16 rows the library's product
+    is faster than the MFMA kernels here unless K is long (the library does not cut K)."""
+    return rows > 16 and K < LONG_K
+
+
 class Linear:
     def __init__(self, weight: torch.Tensor, bias: torch.Tensor | None = None):
         if weight.dim() != 2:
@@ -23,19 +64,21 @@ class Linear:
         self.weight = weight
         self.bias = bias
         self.out_features, self.in_features = weight.shape
+        self._splits: dict[int, int] = {}
 
     def __call__(self, x: torch.Tensor, rows: int, ctx: StepContext, *, use_bias: bool = True,
-                 out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+                 out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None,
+                 allow_split: bool = False):
         w = self.weight
         N, K = w.shape
         bias = self.bias if use_bias else None
         act = x.dtype
         out_dtype = out_dtype or act
-        if out is None:
-            out = ctx.alloc((rows, N), out_dtype)
         if rows == 0:
-            return out
+            return out if out is not None else ctx.alloc((0, N), out_dtype)
         if w.dtype == torch.float32:
+            if out is None:
+                out = ctx.alloc((rows, N), out_dtype)
             if act == torch.float32:
                 if out_dtype != torch.float32:
                     raise TypeError("float32 activations give float32 outputs")
@@ -51,17 +94,21 @@ class Linear:
             return out
         if w.dtype != torch.bfloat16 or act != torch.bfloat16:
             raise TypeError(f"Linear: weight {w.dtype} with activations {act} is not supported")
-        if not ctx.env.fast_kernels:
-            ops.gemm_plain(out, x, w, bias, rows)   # the plain kernel also under bfloat16
+        if not ctx.env.fast_kernels or K % 8 != 0:
+            # the plain kernel also under bfloat16; the MFMA kernels take K in steps of 8
+            if out is None:
+                out = ctx.alloc((rows, N), out_dtype)
+            ops.gemm_plain(out, x, w, bias, rows)
             return out
-        if rows <= ops.SKINNY_MAX_M:
-            self._skinny(out, x, bias, rows, ctx)
-            return out
+        if rows <= ops.SKINNY_MAX_M and not (out_dtype == torch.bfloat16 and _library_is_faster(rows, N, K)):
+            return self._skinny(x, bias, rows, ctx, out, out_dtype, allow_split)
+        if out is None:
+            out = ctx.alloc((rows, N), out_dtype)
         if out_dtype == torch.float32:
             # fp32 results of a tall product: 64 rows at a time through the MFMA kernel
             for r0 in range(0, rows, ops.SKINNY_MAX_M):
                 r1 = min(rows, r0 + ops.SKINNY_MAX_M)
-                self._skinny(out[r0:r1], x[r0:r1], bias, r1 - r0, ctx)
+                self._skinny(x[r0:r1], bias, r1 - r0, ctx, out[r0:r1], out_dtype, False)
             return out
         if bias is not None:
             torch.addmm(bias, x[:rows], w.t(), out=out[:rows])
@@ -69,8 +116,36 @@ class Linear:
             torch.mm(x[:rows], w.t(), out=out[:rows])
         return out
 
-    def _skinny(self, out, x, bias, rows, ctx):
+    def _skinny(self, x, bias, rows, ctx, out, out_dtype, allow_split):
         N, K = self.weight.shape
-        floats = ops.gemm_skinny_workspace_floats(rows, N, K)
-        ws = ctx.alloc((max(floats, 1),), torch.float32)
-        ops.gemm_skinny(out, x, self.weight, bias, rows, ws)
+        if rows <= 16 or (rows <= ops.BLOCKSPLIT_MAX_M and K >= LONG_K):
+            if out is None:
+                out = ctx.alloc((rows, N), out_dtype)
+            ops.gemm_blocksplit(out, x, self.weight, bias, rows)
+            return out
+        splits = self._splits.get(rows)
+        if splits is None:
+            splits = self._splits[rows] = ops.gemm_skinny_splits(rows, N, K)
+        if splits == 1:
+            if out is None:
+                out = ctx.alloc((rows, N), out_dtype)
+            ops.gemm_skinny(out, None, x, self.weight, bias, rows)
+            return out
+        partial = ctx.alloc((splits, rows, N), torch.float32)
+        used = ops.gemm_skinny(None, partial, x, self.weight, None, rows, out_dtype=out_dtype)
+        if used != splits:
+            raise RuntimeError(f"Linear: planned {splits} K slices, the kernel used {used}")
+        s = SplitSum(partial, bias, rows)
+        if allow_split and SPLIT_TO_CONSUMER and out is None:
+            return s
+        return s.materialize(ctx, out_dtype, out)
+
+    def gated_silu(self, x: torch.Tensor, rows: int, ctx: StepContext, out: torch.Tensor) -> bool:
+        """out[rows, N/2] = silu(gate) * up in one kernel, for a weight whose rows
+        interleave gate and up in blocks of 16. False when that kernel does not apply."""
+        w = self.weight
+        if not (ctx.env.fast_kernels and w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
+                and 0 < rows <= 16 and w.shape[1] % 8 == 0 and w.shape[0] % 32 == 0):
+            return False
+        ops.gemm_blocksplit(out, x, w, None, rows, gated=True)
+        return True

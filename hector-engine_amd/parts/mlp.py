@@ -9,7 +9,7 @@ import torch
 
 from ..kernels import ops
 from .base import BuildEnv, FeedForward, StepContext, TensorSpec, param, register_part
-from .linear import Linear
+from .linear import Linear, SplitSum
 
 # rows of the intermediate activations held at once in a long prompt step
 _ROW_CHUNK = 8192
@@ -24,6 +24,7 @@ class GatedMLP(FeedForward):
         act = param(params, "activation", str, "silu")
         if act not in ("silu", "swish"):
             raise ValueError(f"gated_mlp: unsupported activation '{act}'")
+        self.interleaved = False
         self.gate_up: Linear | None = None
         self.down: Linear | None = None
 
@@ -40,17 +41,36 @@ class GatedMLP(FeedForward):
         g, u = tensors.pop(p + "gate_proj.weight"), tensors.pop(p + "up_proj.weight")
         if g.dtype != u.dtype:
             raise TypeError(f"{p}gate_proj and up_proj are stored in different dtypes")
-        self.gate_up = Linear(torch.cat([g, u], 0).contiguous())
-        del g, u
+        if self.inter % 16 == 0:
+            # rows interleaved in blocks of 16 (gate block j, then up block j): the tile pair
+            # of one MFMA wavefront then holds a gate and its up, and the gated activation
+            # is the product's epilogue
+            I, D = g.shape
+            w = torch.stack([g.view(I // 16, 16, D), u.view(I // 16, 16, D)], 1).reshape(2 * I, D)
+            self.interleaved = True
+        else:
+            w = torch.cat([g, u], 0)
+            self.interleaved = False
+        self.gate_up = Linear(w.contiguous())
+        del g, u, w
         self.down = Linear(tensors[p + "down_proj.weight"])
 
     def forward(self, x, ctx: StepContext):
         rows = ctx.rows
+        if rows <= _ROW_CHUNK:
+            h = ctx.alloc((rows, self.inter))
+            if not (self.interleaved and self.gate_up.gated_silu(x, rows, ctx, h)):
+                gu = self.gate_up(x, rows, ctx, allow_split=True)
+                if isinstance(gu, SplitSum):     # K slices: the activation kernel adds them while it reads
+                    ops.silu_mul(h, gu.partial, rows, self.interleaved, gu.splits)
+                else:
+                    ops.silu_mul(h, gu, rows, self.interleaved)
+            return self.down(h, rows, ctx, allow_split=True)
         out = ctx.alloc((rows, self.hidden))
         for r0 in range(0, rows, _ROW_CHUNK):
             n = min(_ROW_CHUNK, rows - r0)
-            gu = self.gate_up(x[r0:r0 + n], n, ctx)
             h = ctx.alloc((n, self.inter))
-            ops.silu_mul(h, gu, n)
+            gu = self.gate_up(x[r0:r0 + n], n, ctx)
+            ops.silu_mul(h, gu, n, self.interleaved)
             self.down(h, n, ctx, out=out[r0:r0 + n])
         return out

@@ -133,9 +133,13 @@ def test_gemm_skinny(ops, M, N, K, out_dtype):
     w = rnd(N, K, seed=15, scale=0.05).to(torch.bfloat16)
     b = rnd(N, seed=16).to(torch.bfloat16)
     out = torch.empty(M, N, dtype=out_dtype, device="cuda")
-    floats = ops.gemm_skinny_workspace_floats(M, N, K)
-    ws = torch.empty(max(floats, 1), device="cuda")
-    ops.gemm_skinny(out, dev(a), dev(w), dev(b), M, ws)
+    splits = ops.gemm_skinny_splits(M, N, K)
+    if splits == 1:
+        assert ops.gemm_skinny(out, None, dev(a), dev(w), dev(b), M) == 1
+    else:
+        partial = torch.empty(splits, M, N, device="cuda")
+        assert ops.gemm_skinny(None, partial, dev(a), dev(w), None, M) == splits
+        ops.splitk_reduce(out, partial, dev(b), M, splits)
     ref = a.double() @ w.double().T + b.double()
     scale = ref.abs().max().item()
     err = (out.cpu().double() - ref).abs().max().item()
@@ -147,13 +151,146 @@ def test_gemm_skinny(ops, M, N, K, out_dtype):
     assert (plain.cpu().double() - ref).abs().max().item() <= tol
 
 
+PLANS = [(1, 1, 1), (1, 2, 3), (1, 4, 8), (2, 1, 1), (2, 2, 5), (2, 4, 2), (4, 1, 1), (4, 2, 4)]
+
+
+@pytest.mark.parametrize("M", [1, 16, 20, 64])
+@pytest.mark.parametrize("R,U,splits", PLANS)
+def test_gemm_skinny_every_plan(ops, M, R, U, splits):
+    """Every tiling the kernel can be launched with gives the same product; K slices are
+    added in index order by the reader, so two runs agree bit for bit."""
+    MT = (M + 15) // 16
+    if (MT == 1 and (R, U) in ((4, 4),)) or (MT == 2 and (R == 1 or U == 4)) or \
+            (MT >= 3 and ((R, U) not in ((4, 1), (2, 1), (2, 2)))):
+        pytest.skip("not instantiated")
+    N, K = 1000, 1544
+    a = rnd(M, K, seed=70).to(torch.bfloat16)
+    w = rnd(N, K, seed=71, scale=0.05).to(torch.bfloat16)
+    b = rnd(N, seed=72).to(torch.bfloat16)
+    ref = a.double() @ w.double().T + b.double()
+    outs = []
+    for _ in range(2):
+        out = torch.empty(M, N, dtype=torch.float32, device="cuda")
+        partial = torch.empty(64, M, N, device="cuda")
+        used = ops.gemm_skinny(out, partial, dev(a), dev(w), dev(b), M, plan=(R, U, splits))
+        assert 1 <= used <= splits and (used > 1) == (splits > 1)
+        if used > 1:
+            ops.splitk_reduce(out, partial, dev(b), M, used)
+        outs.append(out.cpu())
+    assert torch.equal(outs[0], outs[1])
+    assert (outs[0].double() - ref).abs().max().item() <= 1e-4 * ref.abs().max().item()
+
+
+def test_split_sums_are_added_by_the_norm_and_the_qkv_kernel(ops):
+    """The fused norm and the q/k/v kernel read the K slices of a product directly and give
+    what they give for the reduced tensor."""
+    rows, D, S = 5, 96, 3
+    parts = rnd(S, rows, D, seed=76)
+    bias = rnd(D, seed=77)
+    resid = rnd(rows, D, seed=78)
+    w = 1 + 0.1 * rnd(D, seed=79)
+    a, b_ = dev(resid.clone()), dev(resid.clone())
+    out_a = torch.empty(rows, D, dtype=torch.bfloat16, device="cuda")
+    out_b = torch.empty_like(out_a)
+    ops.add_rmsnorm(a, dev(parts), dev(w), out_a, rows, 1e-6, delta_splits=S, delta_bias=dev(bias))
+    summed = torch.empty(rows, D, device="cuda")
+    ops.splitk_reduce(summed, dev(parts), dev(bias), rows, S)
+    want = resid.double() + parts.double().sum(0) + bias.double()
+    assert torch.allclose(a.cpu().double(), want, atol=1e-5)
+    ops.add_rmsnorm(b_, summed.to(torch.bfloat16), dev(w), out_b, rows, 1e-6)
+    assert torch.allclose(out_a.float(), out_b.float(), atol=2 ** -6, rtol=2 ** -6)
+    # q/k/v kernel: H=2, KVH=1, hd=32 -> width 128
+    H, KVH, hd = 2, 1, 32
+    width = (H + 2 * KVH) * hd
+    parts = rnd(S, rows, width, seed=80)
+    qb = rnd(width, seed=81).to(torch.bfloat16)
+    slots, table, kpool, vpool = paged_setup([rows], KVH, hd, torch.bfloat16, 82)
+    pos = torch.arange(rows, dtype=torch.int32)
+    meta = (dev(pos), dev(torch.zeros(rows, dtype=torch.int32)), dev(torch.tensor(slots, dtype=torch.int32)), dev(table))
+    inv = dev(P.rope_inv_freq(hd, 1e4))
+    res = []
+    for split in (True, False):
+        q_out = torch.zeros(rows, H * hd, dtype=torch.bfloat16, device="cuda")
+        kp, vp = dev(kpool), dev(vpool)
+        if split:
+            ops.qkv_rope_cache(q_out, kp, vp, dev(parts), H * hd, KVH * hd, dev(qb), *meta, inv, hd, rows,
+                               H, KVH, hd, True, splits=S)
+        else:
+            x = parts.sum(0)
+            q_ref = P.rope((x + qb.float())[:, :H * hd].reshape(rows, H, hd).double(), pos, 1e4)
+            res.append(q_ref.reshape(rows, H * hd))
+            continue
+        res.append(q_out.cpu().double())
+        assert (kp != 0).sum().item() > 0 and (vp != 0).sum().item() > 0
+    assert torch.allclose(res[0], res[1], atol=2 ** -6, rtol=2 ** -6)
+
+
+@pytest.mark.parametrize("M", [1, 8, 33, 64])
+@pytest.mark.parametrize("I,K", [(160, 64), (1008, 520)])
+def test_gemm_skinny_gated_epilogue(ops, M, I, K):
+    x = rnd(M, K, seed=73).to(torch.bfloat16)
+    g = rnd(I, K, seed=74, scale=0.1).to(torch.bfloat16)
+    u = rnd(I, K, seed=75, scale=0.1).to(torch.bfloat16)
+    w = torch.stack([g.view(I // 16, 16, K), u.view(I // 16, 16, K)], 1).reshape(2 * I, K).contiguous()
+    out = torch.empty(M, I, dtype=torch.bfloat16, device="cuda")
+    assert ops.gemm_skinny(out, None, dev(x), dev(w), None, M, gated=True) == 1
+    ref = P.silu(x.double() @ g.double().T) * (x.double() @ u.double().T)
+    assert (out.cpu().double() - ref).abs().max().item() <= 2 ** -8 * ref.abs().max().item() + 1e-6
+    # the separate kernel on the interleaved layout gives the same function
+    gu = (x.double() @ w.double().T).to(torch.bfloat16)
+    out2 = torch.empty(M, I, dtype=torch.bfloat16, device="cuda")
+    ops.silu_mul(out2, dev(gu), M, True)
+    ref2 = P.silu(gu.double().view(M, I // 16, 2, 16)[:, :, 0]) * gu.double().view(M, I // 16, 2, 16)[:, :, 1]
+    assert torch.allclose(out2.cpu().double(), ref2.reshape(M, I), rtol=2 ** -7, atol=1e-6)
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 20, 32])
+@pytest.mark.parametrize("N,K", [(301, 136), (1000, 1544), (37, 4104), (4608, 3584)])
+@pytest.mark.parametrize("plan", [(0, 0, 0), (1, 1, 1), (2, 2, 4), (1, 2, 16), (2, 1, 8)])
+def test_gemm_blocksplit(ops, M, N, K, plan):
+    """K cut inside the workgroup: every tiling gives the product, twice the same bits."""
+    if (N, K) == (4608, 3584) and (M not in (1, 32) or plan[2] not in (0, 16)):
+        pytest.skip("large shape at two row counts and two tilings only")
+    if M > 16 and plan[1] == 4:
+        pytest.skip("not instantiated")
+    a = rnd(M, K, seed=90).to(torch.bfloat16)
+    w = rnd(N, K, seed=91, scale=0.05).to(torch.bfloat16)
+    b = rnd(N, seed=92).to(torch.bfloat16)
+    ref = a.double() @ w.double().T + b.double()
+    outs = []
+    for _ in range(2):
+        out = torch.empty(M, N, dtype=torch.float32, device="cuda")
+        ops.gemm_blocksplit(out, dev(a), dev(w), dev(b), M, plan=plan)
+        outs.append(out.cpu())
+    assert torch.equal(outs[0], outs[1])
+    assert (outs[0].double() - ref).abs().max().item() <= 1e-4 * ref.abs().max().item()
+    out16 = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    ops.gemm_blocksplit(out16, dev(a), dev(w), None, M, plan=plan)
+    ref0 = a.double() @ w.double().T
+    assert (out16.cpu().double() - ref0).abs().max().item() <= 2 ** -8 * ref0.abs().max().item() + 1e-6
+
+
+@pytest.mark.parametrize("M", [1, 8, 20, 32])
+@pytest.mark.parametrize("I,K", [(160, 64), (1008, 520)])
+@pytest.mark.parametrize("nw", [0, 1, 8])
+def test_gemm_blocksplit_gated_epilogue(ops, M, I, K, nw):
+    x = rnd(M, K, seed=93).to(torch.bfloat16)
+    g = rnd(I, K, seed=94, scale=0.1).to(torch.bfloat16)
+    u = rnd(I, K, seed=95, scale=0.1).to(torch.bfloat16)
+    w = torch.stack([g.view(I // 16, 16, K), u.view(I // 16, 16, K)], 1).reshape(2 * I, K).contiguous()
+    out = torch.empty(M, I, dtype=torch.bfloat16, device="cuda")
+    ops.gemm_blocksplit(out, dev(x), dev(w), None, M, gated=True, plan=(2, 0, nw))
+    ref = P.silu(x.double() @ g.double().T) * (x.double() @ u.double().T)
+    assert (out.cpu().double() - ref).abs().max().item() <= 2 ** -8 * ref.abs().max().item() + 1e-6
+
+
 def test_gemm_skinny_refuses_bad_sizes(ops):
     from hector_engine_amd.kernels.lib import KernelLibraryError
     a = torch.zeros(2, 20, dtype=torch.bfloat16, device="cuda")
     w = torch.zeros(16, 20, dtype=torch.bfloat16, device="cuda")
     out = torch.empty(2, 16, dtype=torch.bfloat16, device="cuda")
     with pytest.raises(KernelLibraryError, match="multiple of 8"):
-        ops.gemm_skinny(out, a, w, None, 2, torch.empty(1, device="cuda"))
+        ops.gemm_skinny(out, None, a, w, None, 2)
 
 
 # ------------------------------------------------------------------ rope + cache + attention

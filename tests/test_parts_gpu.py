@@ -49,6 +49,11 @@ def make_ctx(fw, env, q_lens, starts, slots):
         host={"q_lens": q_lens, "starts": starts, "slots": slots})
 
 
+def as_tensor(x, ctx):
+    from hector_engine_amd.parts.linear import as_tensor as f
+    return f(x, ctx)
+
+
 def rnd(*shape, seed=0, scale=1.0):
     g = torch.Generator().manual_seed(seed)
     return torch.randn(*shape, generator=g) * scale
@@ -98,18 +103,20 @@ def test_rotary_part(fw):
 
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("rows", [5, 100])
-def test_gated_mlp_part(fw, dtype, rows):
+@pytest.mark.parametrize("inter", [136, 160])          # 160: gate and up interleaved in blocks of 16
+def test_gated_mlp_part(fw, dtype, rows, inter):
     env = env_for(fw, dtype)
     mlp = fw.parts.build_part("feed_forward", fw.parts.PartSpec(
-        "gated_mlp", {"hidden_size": 80, "intermediate_size": 136}), "m.", env)
+        "gated_mlp", {"hidden_size": 80, "intermediate_size": inter}), "m.", env)
     specs = mlp.tensor_specs()
     assert {k: v.shape for k, v in specs.items()} == {
-        "m.gate_proj.weight": (136, 80), "m.up_proj.weight": (136, 80), "m.down_proj.weight": (80, 136)}
+        "m.gate_proj.weight": (inter, 80), "m.up_proj.weight": (inter, 80), "m.down_proj.weight": (80, inter)}
     w = {k: rnd(*v.shape, seed=i, scale=0.1).to(dtype) for i, (k, v) in enumerate(specs.items())}
     mlp.bind({k: v.cuda() for k, v in w.items()})
+    assert mlp.interleaved == (inter % 16 == 0)
     ctx = make_ctx(fw, env, [rows], [0], [0])
     x = rnd(rows, 80, seed=9).to(dtype)
-    out = mlp.forward(x.cuda(), ctx)
+    out = as_tensor(mlp.forward(x.cuda(), ctx), ctx)
     want = P.swiglu(x.double(), w["m.gate_proj.weight"].double(), w["m.up_proj.weight"].double(),
                     w["m.down_proj.weight"].double())
     assert torch.allclose(out.cpu().double(), want, **tol(dtype))
@@ -146,7 +153,7 @@ def test_attention_part_prompt_then_tokens(fw, dtype, fast, window):
     # the prompts in one step
     cache.reserve(list(zip(slots, lens)))
     ctx = make_ctx(fw, env, lens, [0, 0], slots)
-    out = att.forward(torch.cat([x[:n] for x, n in zip(xs, lens)]).cuda(), ctx, lc).cpu().double()
+    out = as_tensor(att.forward(torch.cat([x[:n] for x, n in zip(xs, lens)]).cuda(), ctx, lc), ctx).cpu().double()
     cache.commit(list(zip(slots, lens)))
     near(out[:70], want[0][:70], dtype)
     near(out[70:], want[1][:3], dtype)
@@ -156,7 +163,7 @@ def test_attention_part_prompt_then_tokens(fw, dtype, fast, window):
         cache.reserve(list(zip(slots, new)))
         ctx = make_ctx(fw, env, [1, 1], [n + t for n in lens], slots)
         x = torch.stack([xs[0][70 + t], xs[1][3 + t]])
-        out = att.forward(x.cuda(), ctx, lc).cpu().double()
+        out = as_tensor(att.forward(x.cuda(), ctx, lc), ctx).cpu().double()
         cache.commit(list(zip(slots, new)))
         near(out[0], want[0][70 + t], dtype)
         near(out[1], want[1][3 + t], dtype)
@@ -185,7 +192,7 @@ def test_pre_norm_block_part(fw, dtype):
     x = rnd(20, D, seed=50)
     stream = fw.parts.ResidualStream(x.clone().cuda(), 20)
     block.forward(stream, ctx, cache.layer_cache(0))
-    got = stream.materialize().cpu().double()
+    got = stream.materialize(ctx).cpu().double()
     wd = {k: v.double() for k, v in w.items()}
     cfg = {"num_attention_heads": H, "num_key_value_heads": KVH, "head_dim": hd, "rope_theta": 1e4}
     h = x.double()
