@@ -38,28 +38,55 @@ struct AttnState {
   float l;        // this lane's share of the running sum
 };
 
-// One step of 32 keys starting at absolute position key_base (a multiple of 32).
-// kpage: K of (page, kv head), [64][hd]; vpage: V^T of the same, [hd][64].
-// The lane's query sees the keys in [lo, hi].
+// The K and V^T operands of one step of 32 keys, loaded ahead of their use so that the
+// loads of step i+1 are in flight while step i computes.
 template <int NT>
-__device__ __forceinline__ void attend32(AttnState<NT>& st, const bf16x8* qf,
-                                         const uint16_t* __restrict__ kpage,
-                                         const uint16_t* __restrict__ vpage, int koff,
-                                         int key_base, int lo, int hi, float scale, int lr,
-                                         int lg) {
+struct KVFrag {
+  bf16x8 k[2][(16 * NT + 31) / 32];
+  bf16x8 v[NT];
+  int ok;   // the page exists (always, for an admitted batch)
+};
+
+// kpool/vpool of this kv head; page: physical page of the 32 keys; koff: 0 or 32.
+template <int NT>
+__device__ __forceinline__ void load_frag(KVFrag<NT>& f, const uint16_t* __restrict__ kpool,
+                                          const uint16_t* __restrict__ vpool, int page,
+                                          int num_pages, int64_t page_stride, int koff, int lr,
+                                          int lg) {
   constexpr int HD = 16 * NT;
   constexpr int KS = (HD + 31) / 32;
+  f.ok = page >= 0 && page < num_pages;
+  const int64_t pbase = (int64_t)(f.ok ? page : 0) * page_stride;
+  const uint16_t* kpage = kpool + pbase;
+  const uint16_t* vpage = vpool + pbase;
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int key_local = 8 * (lr >> 2) + 4 * t + (lr & 3);
+    const uint16_t* krow = kpage + (koff + key_local) * HD + 8 * lg;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) f.k[t][ks] = ld8(krow + 32 * ks, 32 * ks + 8 * lg < HD);
+  }
+#pragma unroll
+  for (int dt = 0; dt < NT; ++dt)
+    f.v[dt] = ld8(vpage + (16 * dt + lr) * HE_PAGE_TOKENS + koff + 8 * lg, true);
+}
+
+// One step of 32 keys starting at absolute position key_base (a multiple of 32).
+// The lane's query sees the keys in [lo, hi].
+template <int NT>
+__device__ __forceinline__ void attend_frag(AttnState<NT>& st, const bf16x8* qf,
+                                            const KVFrag<NT>& f, int key_base, int lo, int hi,
+                                            float scale, int lg) {
+  constexpr int HD = 16 * NT;
+  constexpr int KS = (HD + 31) / 32;
+  if (!f.ok) hi = -1;
   floatx4 s[2];
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-    const int key_local = 8 * (lr >> 2) + 4 * t + (lr & 3);
-    const uint16_t* krow = kpage + (koff + key_local) * HD + 8 * lg;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const bf16x8 a = ld8(krow + 32 * ks, 32 * ks + 8 * lg < HD);
-      s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[ks], s[t], 0, 0, 0);
-    }
+    for (int ks = 0; ks < KS; ++ks)
+      s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k[t][ks], qf[ks], s[t], 0, 0, 0);
   }
   float p[2][4];
   float mx = -INFINITY;
@@ -96,8 +123,43 @@ __device__ __forceinline__ void attend32(AttnState<NT>& st, const bf16x8* qf,
 #pragma unroll
   for (int dt = 0; dt < NT; ++dt) {
     st.o[dt] *= alpha;
-    const bf16x8 a = ld8(vpage + (16 * dt + lr) * HE_PAGE_TOKENS + koff + 8 * lg, true);
-    st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, st.o[dt], 0, 0, 0);
+    st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.v[dt], pb, st.o[dt], 0, 0, 0);
+  }
+}
+
+// Runs the steps kb = kb_begin, kb_begin + 32, ... < kb_end (all multiples of 32) of one
+// (sequence, kv head) against the state, one step ahead with its loads and one page
+// ahead with its page-table entry.
+template <int NT>
+__device__ __forceinline__ void attend_range(AttnState<NT>& st, const bf16x8* qf,
+                                             const uint16_t* __restrict__ kpool,
+                                             const uint16_t* __restrict__ vpool,
+                                             const int32_t* __restrict__ pt, int max_blocks,
+                                             int num_pages, int KVH, int kvh, int kb_begin,
+                                             int kb_end, int lo, int hi, float scale, int lr,
+                                             int lg) {
+  constexpr int HD = 16 * NT;
+  if (kb_begin >= kb_end) return;
+  const int64_t page_stride = (int64_t)KVH * (HE_PAGE_TOKENS * HD);
+  const uint16_t* kp = kpool + (int64_t)kvh * (HE_PAGE_TOKENS * HD);
+  const uint16_t* vp = vpool + (int64_t)kvh * (HE_PAGE_TOKENS * HD);
+  int block = kb_begin >> HE_PAGE_SHIFT;
+  int page = pt[block];
+  int page_ahead = pt[min(block + 1, max_blocks - 1)];
+  KVFrag<NT> cur, nxt;
+  load_frag<NT>(cur, kp, vp, page, num_pages, page_stride, kb_begin & 32, lr, lg);
+  for (int kb = kb_begin; kb < kb_end; kb += 32) {
+    const int kn = kb + 32;
+    if (kn < kb_end) {
+      if ((kn & 32) == 0) {   // the next step starts a new page
+        ++block;
+        page = page_ahead;
+        page_ahead = pt[min(block + 1, max_blocks - 1)];
+      }
+      load_frag<NT>(nxt, kp, vp, page, num_pages, page_stride, kn & 32, lr, lg);
+    }
+    attend_frag<NT>(st, qf, cur, kb, lo, hi, scale, lg);
+    cur = nxt;
   }
 }
 
@@ -151,12 +213,8 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   const int last_pos = start + min(q0 + 15, q_len - 1);
   const int first_pos = start + q0;
   const int tile_lo = window > 0 ? max(0, first_pos + 1 - window) : 0;
-  for (int kb = tile_lo & ~31; kb <= last_pos; kb += 32) {
-    const int page = pt[kb >> HE_PAGE_SHIFT];
-    if (page < 0 || page >= num_pages) continue;  // never for an admitted batch
-    const int64_t pbase = ((int64_t)page * KVH + kvh) * (HE_PAGE_TOKENS * HD);
-    attend32<NT>(st, qf, kpool + pbase, vpool + pbase, kb & 32, kb, lo, hi, scale, lr, lg);
-  }
+  attend_range<NT>(st, qf, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, tile_lo & ~31,
+                   (last_pos & ~31) + 32, lo, hi, scale, lr, lg);
   float l = st.l;
   l += __shfl_xor(l, 16, HE_WAVE);
   l += __shfl_xor(l, 32, HE_WAVE);
@@ -182,7 +240,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 // joins the slices in the order of their index:
 //   out = sum_s O_s e^(m_s - M) / sum_s l_s e^(m_s - M)
 // With a single slice in the grid the result is written directly.
-#define DECODE_MIN_CHUNK 128
+#define DECODE_MIN_CHUNK 64
 
 template <int NT>
 __global__ __launch_bounds__(64) void attention_decode_kernel(
@@ -231,12 +289,8 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   st.m = -INFINITY;
   st.l = 0.f;
   const int hi = n_keys - 1;
-  for (int kb = kb_begin; kb < kb_end; kb += 32) {
-    const int page = pt[kb >> HE_PAGE_SHIFT];
-    if (page < 0 || page >= num_pages) continue;  // never for an admitted batch
-    const int64_t pbase = ((int64_t)page * KVH + kvh) * (HE_PAGE_TOKENS * HD);
-    attend32<NT>(st, qf, kpool + pbase, vpool + pbase, kb & 32, kb, first, hi, scale, lr, lg);
-  }
+  attend_range<NT>(st, qf, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, kb_begin,
+                   (kb_end + 31) & ~31, first, hi, scale, lr, lg);
   float l = st.l;
   l += __shfl_xor(l, 16, HE_WAVE);
   l += __shfl_xor(l, 32, HE_WAVE);
@@ -268,18 +322,20 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   }
 }
 
-// Joins the slices of one (row, head): grid (H, rows), one wavefront. The number of
-// slices that hold keys is recomputed exactly as the decode kernel computes it.
-__global__ __launch_bounds__(64) void attention_merge_kernel(
+// Joins the slices of one (row, head): grid (H, rows), four wavefronts; wavefront w adds
+// the slices s = w, w + 4, ... and the four sums are added in wavefront order. The number
+// of slices that hold keys is recomputed exactly as the decode kernel computes it.
+__global__ __launch_bounds__(256) void attention_merge_kernel(
     uint16_t* __restrict__ out, const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq, int H, int HD,
     int nsplit, int window) {
   __shared__ float wgt[64];
-  const int h = blockIdx.x, lane = threadIdx.x;
+  __shared__ float part[4][256];
+  const int h = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int64_t row = blockIdx.y;
   uint16_t* orow = out + (row * H + h) * (int64_t)HD;
   if (row_seq[row] < 0) {
-    for (int d = lane; d < HD; d += 64) orow[d] = 0;
+    for (int d = threadIdx.x; d < HD; d += 256) orow[d] = 0;
     return;
   }
   const int n_keys = positions[row] + 1;
@@ -293,14 +349,27 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(
   const float l = lane < active ? ws_ml[2 * (base + lane) + 1] : 0.f;
   const float M = wave_max(m);
   const float w = m > -INFINITY ? __expf(m - M) : 0.f;
-  const float L = wave_sum(l * w);
-  wgt[lane] = w;
+  const float L = wave_sum(l * w);          // every wavefront computes the same weights
+  if (wave == 0) wgt[lane] = w;
   __syncthreads();
   const float inv = L > 0.f ? 1.f / L : 0.f;
-  for (int d = lane; d < HD; d += 64) {
-    float acc = 0.f;
-    for (int s = 0; s < active; ++s) acc += ws_o[(base + s) * HD + d] * wgt[s];
-    orow[d] = float_to_bf16_bits(acc * inv);
+  for (int d0 = 0; d0 < HD; d0 += 256) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int d = d0 + lane + 64 * j;
+      float acc = 0.f;
+      if (d < HD)
+        for (int s = wave; s < active; s += 4) acc += ws_o[(base + s) * HD + d] * wgt[s];
+      part[wave][lane + 64 * j] = acc;
+    }
+    __syncthreads();
+    const int d = d0 + threadIdx.x;
+    if (d < HD) {
+      const float acc = ((part[0][threadIdx.x] + part[1][threadIdx.x]) + part[2][threadIdx.x]) +
+                        part[3][threadIdx.x];
+      orow[d] = float_to_bf16_bits(acc * inv);
+    }
+    __syncthreads();
   }
 }
 
@@ -378,7 +447,7 @@ extern "C" int he_attention_decode_bf16(void* out, const void* q, const void* kp
                            num_pages, H, KVH, head_tiles, window, scale)));
   int rc = he_check_launch("he_attention_decode_bf16");
   if (rc || nsplit == 1) return rc;
-  attention_merge_kernel<<<dim3(H, rows), 64, 0, s>>>(
+  attention_merge_kernel<<<dim3(H, rows), 256, 0, s>>>(
       (uint16_t*)out, ws_o, ws_ml, (const int32_t*)positions, (const int32_t*)row_seq, H, hd,
       nsplit, window);
   return he_check_launch("he_attention_decode_bf16 merge");

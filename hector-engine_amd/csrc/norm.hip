@@ -51,6 +51,50 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
   }
 }
 
+// The same with a row of at most NORM_EPT * blockDim.x elements kept in registers:
+// every load of the row is issued before the reduction, nothing is read twice.
+#define NORM_EPT 8
+template <typename TD, typename TO>
+__global__ void add_rmsnorm_reg_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
+                                       const void* __restrict__ w, int w_dtype,
+                                       TO* __restrict__ out, int D, float eps) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  float* r = resid + row * (int64_t)D;
+  const TD* d = delta ? delta + row * (int64_t)D : nullptr;
+  float v[NORM_EPT], g[NORM_EPT];
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < NORM_EPT; ++e) {
+    const int i = threadIdx.x + e * blockDim.x;
+    v[e] = 0.f;
+    g[e] = 0.f;
+    if (i < D) {
+      v[e] = r[i];
+      if (d) v[e] += to_float(d[i]);
+      if (out) g[e] = load_param(w, i, w_dtype);
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < NORM_EPT; ++e) ss += v[e] * v[e];
+  if (d) {
+#pragma unroll
+    for (int e = 0; e < NORM_EPT; ++e) {
+      const int i = threadIdx.x + e * blockDim.x;
+      if (i < D) r[i] = v[e];
+    }
+  }
+  const float total = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(total / (float)D + eps);
+  if (out == nullptr) return;
+  TO* o = out + row * (int64_t)D;
+#pragma unroll
+  for (int e = 0; e < NORM_EPT; ++e) {
+    const int i = threadIdx.x + e * blockDim.x;
+    if (i < D) o[i] = from_float<TO>(v[e] * inv * g[e]);
+  }
+}
+
 static int norm_threads(int D) { return D >= 2048 ? 512 : (D >= 512 ? 256 : (D >= 128 ? 128 : 64)); }
 
 extern "C" int he_add_rmsnorm(void* resid_f32, const void* delta, int delta_splits,
@@ -76,6 +120,13 @@ extern "C" int he_add_rmsnorm(void* resid_f32, const void* delta, int delta_spli
       add_rmsnorm_kernel<float, float, true><<<rows, threads, 0, s>>>(
           (float*)resid_f32, (const float*)delta, delta_splits, stride, delta_bias, bias_dtype,
           weight, w_dtype, (float*)out, D, eps);
+  } else if (D <= NORM_EPT * threads) {
+    if (act_dtype == HE_BF16)
+      add_rmsnorm_reg_kernel<bf16_t, bf16_t><<<rows, threads, 0, s>>>(
+          (float*)resid_f32, (const bf16_t*)delta, weight, w_dtype, (bf16_t*)out, D, eps);
+    else
+      add_rmsnorm_reg_kernel<float, float><<<rows, threads, 0, s>>>(
+          (float*)resid_f32, (const float*)delta, weight, w_dtype, (float*)out, D, eps);
   } else if (act_dtype == HE_BF16) {
     add_rmsnorm_kernel<bf16_t, bf16_t, false><<<rows, threads, 0, s>>>(
         (float*)resid_f32, (const bf16_t*)delta, 0, 0, nullptr, 0, weight, w_dtype, (bf16_t*)out, D,

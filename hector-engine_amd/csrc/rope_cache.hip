@@ -16,6 +16,24 @@
 
 #define ROPE_MAX_HALF 256
 
+// sin and cos of an fp32 angle to fp32 accuracy: the quadrant is taken off in double
+// (k = rint(a * 2/pi), r = a - k * pi/2, |r| <= pi/4), the two short series are summed
+// in double and rounded once. The library routine's path for large arguments is far
+// slower, and angles here reach tens of thousands of radians.
+__device__ __forceinline__ void sincos_angle(float a, float* sn, float* cs) {
+  const double x = (double)a;
+  const double k = rint(x * 0.63661977236758134308);
+  const double r = fma(-k, 6.123233995736766036e-17, fma(-k, 1.57079632679489655800, x));
+  const double r2 = r * r;
+  const double sp = r * (1.0 + r2 * (-1.0 / 6 + r2 * (1.0 / 120 + r2 * (-1.0 / 5040 + r2 * (1.0 / 362880 + r2 * (-1.0 / 39916800))))));
+  const double cp = 1.0 + r2 * (-0.5 + r2 * (1.0 / 24 + r2 * (-1.0 / 720 + r2 * (1.0 / 40320 + r2 * (-1.0 / 3628800 + r2 * (1.0 / 479001600))))));
+  const int q = (int)((long long)k & 3);
+  const double sv = (q & 1) ? cp : sp;
+  const double cv = (q & 1) ? sp : cp;
+  *sn = (float)((q & 2) ? -sv : sv);
+  *cs = (float)(((q + 1) & 2) ? -cv : cv);
+}
+
 template <typename TI>
 __device__ __forceinline__ float load_in(const TI* p, int splits, int64_t split_stride) {
   if (splits <= 1) return to_float(p[0]);
@@ -42,7 +60,7 @@ __global__ void qkv_rope_cache_kernel(
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
     const float a = (float)pos * inv_freq[i];
     float sn, c;
-    sincosf(a, &sn, &c);
+    sincos_angle(a, &sn, &c);
     cs[0][i] = c;
     cs[1][i] = sn;
   }
@@ -122,6 +140,120 @@ __global__ void qkv_rope_cache_kernel(
   }
 }
 
+// bf16 rows, eight elements per access: one thread rotates the pairs (j..j+7, j+half..)
+// of one head, or copies eight v elements. Needs rotary_dim/2, head_dim - rotary_dim and
+// the row stride in multiples of 8.
+__device__ __forceinline__ void unpack8(const uint4& v, float* f) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = __uint_as_float(w[i] << 16);
+    f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+__device__ __forceinline__ uint4 pack8(const float* f) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    w[i] = (uint32_t)float_to_bf16_bits(f[2 * i]) | ((uint32_t)float_to_bf16_bits(f[2 * i + 1]) << 16);
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+__global__ __launch_bounds__(256) void qkv_rope_cache_vec_kernel(
+    uint16_t* __restrict__ q_out, uint16_t* __restrict__ kpool, uint16_t* __restrict__ vpool,
+    const uint16_t* __restrict__ q_in, const uint16_t* __restrict__ k_in,
+    const uint16_t* __restrict__ v_in, int64_t in_stride, const uint16_t* __restrict__ q_bias,
+    const uint16_t* __restrict__ k_bias, const uint16_t* __restrict__ v_bias,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
+    const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ page_table, int max_blocks,
+    int num_pages, const float* __restrict__ inv_freq, int rotary_dim, int H, int KVH, int hd) {
+  __shared__ float cs[2][ROPE_MAX_HALF];
+  const int64_t row = blockIdx.x;
+  const int seq = row_seq[row];
+  const int pos = positions[row];
+  if (seq < 0) return;  // padding row
+  int page = -1;
+  if (k_in != nullptr) page = page_table[(int64_t)seq_slot[seq] * max_blocks + (pos >> HE_PAGE_SHIFT)];
+  const int half = rotary_dim >> 1;
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    float sn, c;
+    sincos_angle((float)pos * inv_freq[i], &sn, &c);
+    cs[0][i] = c;
+    cs[1][i] = sn;
+  }
+  __syncthreads();
+  const int rot8 = half >> 3;                 // groups of 8 pairs per head
+  const int pass8 = (hd - rotary_dim) >> 3;   // groups of 8 pass-through dims per head
+  const int per_head = rot8 + pass8;
+  const int q_items = H * per_head;
+  const int k_items = k_in ? KVH * per_head : 0;
+  const int v_items = k_in ? (KVH * hd) >> 3 : 0;
+  const bool cache_ok = page >= 0 && page < num_pages;
+  const int off = pos & (HE_PAGE_TOKENS - 1);
+  for (int it = threadIdx.x; it < q_items + k_items + v_items; it += blockDim.x) {
+    if (it < q_items + k_items) {
+      const bool is_q = it < q_items;
+      const int idx = is_q ? it : it - q_items;
+      const int h = idx / per_head;
+      const int g = idx - h * per_head;
+      const uint16_t* in = (is_q ? q_in : k_in) + row * in_stride + h * hd;
+      const uint16_t* bias = is_q ? q_bias : k_bias;
+      uint16_t* out;
+      if (is_q) {
+        out = q_out + row * (int64_t)H * hd + h * hd;
+      } else {
+        if (!cache_ok) continue;
+        out = kpool + (((int64_t)page * KVH + h) * HE_PAGE_TOKENS + off) * hd;
+      }
+      float x0[8], x1[8], b0[8], b1[8];
+      if (g < rot8) {
+        const int j = 8 * g;
+        unpack8(*reinterpret_cast<const uint4*>(in + j), x0);
+        unpack8(*reinterpret_cast<const uint4*>(in + j + half), x1);
+        if (bias) {
+          unpack8(*reinterpret_cast<const uint4*>(bias + h * hd + j), b0);
+          unpack8(*reinterpret_cast<const uint4*>(bias + h * hd + j + half), b1);
+        }
+        float y0[8], y1[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float a0 = bias ? x0[i] + b0[i] : x0[i];
+          const float a1 = bias ? x1[i] + b1[i] : x1[i];
+          const float c = cs[0][j + i], sn = cs[1][j + i];
+          y0[i] = a0 * c - a1 * sn;
+          y1[i] = a0 * sn + a1 * c;
+        }
+        *reinterpret_cast<uint4*>(out + j) = pack8(y0);
+        *reinterpret_cast<uint4*>(out + j + half) = pack8(y1);
+      } else {
+        const int d = rotary_dim + 8 * (g - rot8);
+        unpack8(*reinterpret_cast<const uint4*>(in + d), x0);
+        if (bias) {
+          unpack8(*reinterpret_cast<const uint4*>(bias + h * hd + d), b0);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) x0[i] += b0[i];
+        }
+        *reinterpret_cast<uint4*>(out + d) = pack8(x0);
+      }
+    } else {
+      if (!cache_ok) continue;
+      const int e = 8 * (it - q_items - k_items);   // element of the v row
+      const int h = e / hd, d = e - h * hd;
+      float x[8], b[8];
+      unpack8(*reinterpret_cast<const uint4*>(v_in + row * in_stride + e), x);
+      if (v_bias) {
+        unpack8(*reinterpret_cast<const uint4*>(v_bias + e), b);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] += b[i];
+      }
+      // V is stored transposed inside a page: [head_dim][tokens]
+      uint16_t* out = vpool + (((int64_t)page * KVH + h) * hd + d) * HE_PAGE_TOKENS + off;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) out[i * HE_PAGE_TOKENS] = float_to_bf16_bits(x[i]);
+    }
+  }
+}
+
 extern "C" int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const void* q_in,
                                  const void* k_in, const void* v_in, int64_t in_stride,
                                  int in_splits, const void* q_bias, const void* k_bias, const void* v_bias,
@@ -152,7 +284,21 @@ extern "C" int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const vo
       (const int32_t*)positions, (const int32_t*)row_seq, (const int32_t*)seq_slot,             \
       (const int32_t*)page_table, max_blocks, num_pages, (const float*)inv_freq, rotary_dim, H, \
       KVH, hd)
-  if (in_splits > 0) {  // the input rows are fp32 partial sums
+  const bool vec_ok = in_splits == 0 && dtype == HE_BF16 &&
+                      (q_bias == nullptr || bias_dtype == HE_BF16) &&
+                      ((rotary_dim >> 1) & 7) == 0 && ((hd - rotary_dim) & 7) == 0 &&
+                      (in_stride & 7) == 0 && (hd & 7) == 0 &&
+                      ((((uintptr_t)q_in) | ((uintptr_t)k_in) | ((uintptr_t)v_in) |
+                        ((uintptr_t)q_bias) | ((uintptr_t)k_bias) | ((uintptr_t)v_bias) |
+                        ((uintptr_t)q_out) | ((uintptr_t)kpool)) & 15) == 0;
+  if (vec_ok) {
+    qkv_rope_cache_vec_kernel<<<rows, threads, 0, s>>>(
+        (uint16_t*)q_out, (uint16_t*)kpool, (uint16_t*)vpool, (const uint16_t*)q_in,
+        (const uint16_t*)k_in, (const uint16_t*)v_in, in_stride, (const uint16_t*)q_bias,
+        (const uint16_t*)k_bias, (const uint16_t*)v_bias, (const int32_t*)positions,
+        (const int32_t*)row_seq, (const int32_t*)seq_slot, (const int32_t*)page_table, max_blocks,
+        num_pages, (const float*)inv_freq, rotary_dim, H, KVH, hd);
+  } else if (in_splits > 0) {  // the input rows are fp32 partial sums
     if (dtype == HE_BF16)
       ROPE_LAUNCH(bf16_t, float);
     else
