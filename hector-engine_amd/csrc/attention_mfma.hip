@@ -72,14 +72,18 @@ __device__ __forceinline__ void load_frag(KVFrag<NT>& f, const uint16_t* __restr
 }
 
 // One step of 32 keys starting at absolute position key_base (a multiple of 32).
-// The lane's query sees the keys in [lo, hi].
-template <int NT>
+// The lane's query sees the keys in [lo, hi]; with MASK false the caller has checked
+// that all 32 keys are visible to every query of the tile. Scores are kept in the
+// base-2 domain: s2 = (q . k) * scale * log2(e), p = 2^(s2 - m), so the exponential is
+// the bare hardware instruction; m is the running maximum of s2. When no query's
+// maximum moves, the rescaling of the accumulators is skipped.
+template <int NT, bool MASK>
 __device__ __forceinline__ void attend_frag(AttnState<NT>& st, const bf16x8* qf,
                                             const KVFrag<NT>& f, int key_base, int lo, int hi,
-                                            float scale, int lg) {
+                                            float scale_log2, int lg) {
   constexpr int HD = 16 * NT;
   constexpr int KS = (HD + 31) / 32;
-  if (!f.ok) hi = -1;
+  if (MASK && !f.ok) hi = -1;
   floatx4 s[2];
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
@@ -94,37 +98,44 @@ __device__ __forceinline__ void attend_frag(AttnState<NT>& st, const bf16x8* qf,
   for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int key = key_base + 8 * lg + 4 * t + r;
-      const float v = (key >= lo && key <= hi) ? s[t][r] * scale : -INFINITY;
+      float v = s[t][r] * scale_log2;
+      if (MASK) {
+        const int key = key_base + 8 * lg + 4 * t + r;
+        v = (key >= lo && key <= hi) ? v : -INFINITY;
+      }
       p[t][r] = v;
       mx = fmaxf(mx, v);
     }
   mx = fmaxf(mx, __shfl_xor(mx, 16, HE_WAVE));
   mx = fmaxf(mx, __shfl_xor(mx, 32, HE_WAVE));
   const float m_new = fmaxf(st.m, mx);
+  const bool moved = __builtin_amdgcn_ballot_w64(m_new != st.m) != 0;   // wave-uniform
   const float m_use = m_new == -INFINITY ? 0.f : m_new;
-  const float alpha = __expf(st.m - m_use);
   float sum = 0.f;
   uint32_t packed[4];
 #pragma unroll
   for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int r = 0; r < 4; r += 2) {
-      const float e0 = __expf(p[t][r] - m_use);
-      const float e1 = __expf(p[t][r + 1] - m_use);
+      const float e0 = __builtin_amdgcn_exp2f(p[t][r] - m_use);
+      const float e1 = __builtin_amdgcn_exp2f(p[t][r + 1] - m_use);
       sum += e0 + e1;
-      packed[2 * t + (r >> 1)] =
-          (uint32_t)float_to_bf16_bits(e0) | ((uint32_t)float_to_bf16_bits(e1) << 16);
+      packed[2 * t + (r >> 1)] = pack2_bf16(e0, e1);
     }
-  st.l = st.l * alpha + sum;
-  st.m = m_new;
+  if (moved) {
+    const float alpha = __builtin_amdgcn_exp2f(st.m - m_use);
+    st.l = st.l * alpha + sum;
+    st.m = m_new;
+#pragma unroll
+    for (int dt = 0; dt < NT; ++dt) st.o[dt] *= alpha;
+  } else {
+    st.l += sum;
+  }
   const bf16x8 pb =
       __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
 #pragma unroll
-  for (int dt = 0; dt < NT; ++dt) {
-    st.o[dt] *= alpha;
+  for (int dt = 0; dt < NT; ++dt)
     st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.v[dt], pb, st.o[dt], 0, 0, 0);
-  }
 }
 
 // Runs the steps kb = kb_begin, kb_begin + 32, ... < kb_end (all multiples of 32) of one
@@ -136,8 +147,8 @@ __device__ __forceinline__ void attend_range(AttnState<NT>& st, const bf16x8* qf
                                              const uint16_t* __restrict__ vpool,
                                              const int32_t* __restrict__ pt, int max_blocks,
                                              int num_pages, int KVH, int kvh, int kb_begin,
-                                             int kb_end, int lo, int hi, float scale, int lr,
-                                             int lg) {
+                                             int kb_end, int lo, int hi, int clear_lo,
+                                             int clear_hi, float scale_log2, int lr, int lg) {
   constexpr int HD = 16 * NT;
   if (kb_begin >= kb_end) return;
   const int64_t page_stride = (int64_t)KVH * (HE_PAGE_TOKENS * HD);
@@ -158,7 +169,11 @@ __device__ __forceinline__ void attend_range(AttnState<NT>& st, const bf16x8* qf
       }
       load_frag<NT>(nxt, kp, vp, page, num_pages, page_stride, kn & 32, lr, lg);
     }
-    attend_frag<NT>(st, qf, cur, kb, lo, hi, scale, lg);
+    // keys in [clear_lo, clear_hi] are visible to every query of the tile
+    if (kb >= clear_lo && kb + 31 <= clear_hi && cur.ok)
+      attend_frag<NT, false>(st, qf, cur, kb, lo, hi, scale_log2, lg);
+    else
+      attend_frag<NT, true>(st, qf, cur, kb, lo, hi, scale_log2, lg);
     cur = nxt;
   }
 }
@@ -213,8 +228,14 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   const int last_pos = start + min(q0 + 15, q_len - 1);
   const int first_pos = start + q0;
   const int tile_lo = window > 0 ? max(0, first_pos + 1 - window) : 0;
+  // every query of a full tile sees the keys from the last query's window start to the
+  // first query's position
+  const bool full_tile = q0 + 15 < q_len;
+  const int clear_lo = window > 0 ? max(0, last_pos + 1 - window) : 0;
+  const int clear_hi = full_tile ? first_pos : -1;
   attend_range<NT>(st, qf, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, tile_lo & ~31,
-                   (last_pos & ~31) + 32, lo, hi, scale, lr, lg);
+                   (last_pos & ~31) + 32, lo, hi, clear_lo, clear_hi, scale * 1.4426950408889634f,
+                   lr, lg);
   float l = st.l;
   l += __shfl_xor(l, 16, HE_WAVE);
   l += __shfl_xor(l, 32, HE_WAVE);
@@ -224,10 +245,158 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 #pragma unroll
   for (int dt = 0; dt < NT; ++dt) {
     uint2 w;
-    w.x = (uint32_t)float_to_bf16_bits(st.o[dt][0] * inv) |
-          ((uint32_t)float_to_bf16_bits(st.o[dt][1] * inv) << 16);
-    w.y = (uint32_t)float_to_bf16_bits(st.o[dt][2] * inv) |
-          ((uint32_t)float_to_bf16_bits(st.o[dt][3] * inv) << 16);
+    w.x = pack2_bf16(st.o[dt][0] * inv, st.o[dt][1] * inv);
+    w.y = pack2_bf16(st.o[dt][2] * inv, st.o[dt][3] * inv);
+    *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * lg) = w;
+  }
+}
+
+// ------------------------------------------------------------------ prefill, K/V through LDS
+// grid (ceil(max_q_len / 128), H, num_seqs), 512 threads. The workgroup takes 128
+// consecutive queries of one sequence and head, wave w the 16 queries 16w..16w+15. The
+// keys are walked a page (64 keys) at a time: the page's K and V^T are copied once into
+// LDS, already in the order the MFMA operands are read (one operand of all 64 lanes is
+// one contiguous KiB, so the reads have no bank conflicts), every wave builds its
+// operands from there, and the next page is already on its way into registers while the
+// current one is used. Head sizes up to 128.
+#define PF_WAVES 8
+#define PF_QUERIES (16 * PF_WAVES)
+template <int NT>
+__global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2))) void
+attention_prefill_lds_kernel(
+    uint16_t* __restrict__ out, const uint16_t* __restrict__ q,
+    const uint16_t* __restrict__ kpool, const uint16_t* __restrict__ vpool,
+    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_slot,
+    const int32_t* __restrict__ seq_start, const int32_t* __restrict__ page_table, int max_blocks,
+    int num_pages, int H, int KVH, int window, float scale) {
+  constexpr int HD = 16 * NT;
+  constexpr int KS = (HD + 31) / 32;
+  constexpr int CHUNKS = HE_PAGE_TOKENS * HD / 8;   // 16-byte chunks of one page of K (or V^T)
+  constexpr int THREADS = 64 * PF_WAVES;
+  constexpr int PER_THREAD = (CHUNKS + THREADS - 1) / THREADS;
+  // operand-ordered: k_lds[((hb*2 + t)*KS + ks)*64 + lane], v_lds[(hb*NT + dt)*64 + lane]
+  __shared__ uint4 k_lds[2 * 2 * KS * 64];
+  __shared__ uint4 v_lds[2 * NT * 64];
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lr = lane & 15, lg = lane >> 4;
+  const int seq = blockIdx.z, h = blockIdx.y;
+  const int slot = seq_slot[seq];
+  if (slot < 0) return;
+  const int row0 = cu_seqlens[seq];
+  const int q_len = cu_seqlens[seq + 1] - row0;
+  // long workgroups first: the last queries of a sequence have the most keys
+  const int qb = PF_QUERIES * (gridDim.x - 1 - blockIdx.x);
+  if (qb >= q_len) return;
+  const int start = seq_start[seq];
+  const int kvh = h / (H / KVH);
+  const int32_t* pt = page_table + (int64_t)slot * max_blocks;
+  const int64_t page_stride = (int64_t)KVH * (HE_PAGE_TOKENS * HD);
+  const uint16_t* kp = kpool + (int64_t)kvh * (HE_PAGE_TOKENS * HD);
+  const uint16_t* vp = vpool + (int64_t)kvh * (HE_PAGE_TOKENS * HD);
+
+  const int qw = qb + 16 * wave;                 // this wave's 16 queries
+  const bool wave_ok = qw < q_len;
+  const int qi = qw + lr;
+  const bool q_ok = qi < q_len;
+  const int pos = start + qi;
+  const int hi = q_ok ? pos : -1;
+  const int lo = (window > 0 && q_ok) ? max(0, pos + 1 - window) : 0;
+  bf16x8 qf[KS];
+  load_q<NT>(qf, q + ((int64_t)(row0 + min(qi, q_len - 1)) * H + h) * HD, q_ok, lg);
+  AttnState<NT> st;
+#pragma unroll
+  for (int dt = 0; dt < NT; ++dt) st.o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  st.m = -INFINITY;
+  st.l = 0.f;
+  const int wlast = start + min(qw + 15, q_len - 1);            // last position this wave sees
+  const int wfirst = window > 0 ? max(0, start + qw + 1 - window) : 0;
+  // keys every query of a full tile sees: from the last query's window start to the first
+  // query's position
+  const int clear_lo = window > 0 ? max(0, wlast + 1 - window) : 0;
+  const int clear_hi = qw + 15 < q_len ? start + qw : -1;
+  const float scale_log2 = scale * 1.4426950408889634f;
+
+  const int blk_last = start + min(qb + PF_QUERIES - 1, q_len - 1);
+  const int blk_first = window > 0 ? max(0, start + qb + 1 - window) : 0;
+  const int pb0 = blk_first >> HE_PAGE_SHIFT, pb1 = blk_last >> HE_PAGE_SHIFT;
+
+  uint4 kreg[PER_THREAD], vreg[PER_THREAD];
+  int page = pt[pb0];
+  if (page < 0 || page >= num_pages) page = 0;   // never for an admitted batch
+#pragma unroll
+  for (int j = 0; j < PER_THREAD; ++j) {
+    const int c = threadIdx.x + THREADS * j;
+    if (c < CHUNKS) {
+      kreg[j] = *reinterpret_cast<const uint4*>(kp + (int64_t)page * page_stride + 8 * c);
+      vreg[j] = *reinterpret_cast<const uint4*>(vp + (int64_t)page * page_stride + 8 * c);
+    }
+  }
+  for (int pb = pb0; pb <= pb1; ++pb) {
+    __syncthreads();   // everyone is done with the page in LDS
+#pragma unroll
+    for (int j = 0; j < PER_THREAD; ++j) {
+      const int c = threadIdx.x + THREADS * j;
+      if (c < CHUNKS) {
+        // K chunk: key krow, dims 8*kcol..+8 -> operand (half, tile, k step) and its lane
+        const int krow = c / (HD / 8), kcol = c % (HD / 8);
+        const int kl = krow & 31;
+        const int klane = 16 * (kcol & 3) + (((kl >> 3) << 2) | (kl & 3));
+        k_lds[(((krow >> 5) * 2 + ((kl >> 2) & 1)) * KS + (kcol >> 2)) * 64 + klane] = kreg[j];
+        // V^T chunk: dim vrow, keys 8*vcol..+8 -> operand (half, dim tile) and its lane
+        const int vrow = c / (HE_PAGE_TOKENS / 8), vcol = c % (HE_PAGE_TOKENS / 8);
+        v_lds[((vcol >> 2) * NT + (vrow >> 4)) * 64 + 16 * (vcol & 3) + (vrow & 15)] = vreg[j];
+      }
+    }
+    __syncthreads();
+    if (pb < pb1) {   // the next page is fetched while this one is used
+      page = pt[pb + 1];
+      if (page < 0 || page >= num_pages) page = 0;
+#pragma unroll
+      for (int j = 0; j < PER_THREAD; ++j) {
+        const int c = threadIdx.x + THREADS * j;
+        if (c < CHUNKS) {
+          kreg[j] = *reinterpret_cast<const uint4*>(kp + (int64_t)page * page_stride + 8 * c);
+          vreg[j] = *reinterpret_cast<const uint4*>(vp + (int64_t)page * page_stride + 8 * c);
+        }
+      }
+    }
+    const int page_lo = pb << HE_PAGE_SHIFT;
+    if (!wave_ok || page_lo > wlast || page_lo + HE_PAGE_TOKENS - 1 < wfirst) continue;
+#pragma unroll
+    for (int hb = 0; hb < 2; ++hb) {
+      const int key_base = page_lo + 32 * hb;
+      if (key_base > wlast || key_base + 31 < wfirst) continue;
+      KVFrag<NT> f;
+      f.ok = 1;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          uint4 v = make_uint4(0, 0, 0, 0);
+          if (32 * ks + 8 * lg < HD) v = k_lds[((hb * 2 + t) * KS + ks) * 64 + lane];
+          f.k[t][ks] = __builtin_bit_cast(bf16x8, v);
+        }
+#pragma unroll
+      for (int dt = 0; dt < NT; ++dt)
+        f.v[dt] = __builtin_bit_cast(bf16x8, v_lds[(hb * NT + dt) * 64 + lane]);
+      if (key_base >= clear_lo && key_base + 31 <= clear_hi)
+        attend_frag<NT, false>(st, qf, f, key_base, lo, hi, scale_log2, lg);
+      else
+        attend_frag<NT, true>(st, qf, f, key_base, lo, hi, scale_log2, lg);
+    }
+  }
+  float l = st.l;
+  l += __shfl_xor(l, 16, HE_WAVE);
+  l += __shfl_xor(l, 32, HE_WAVE);
+  if (!q_ok) return;
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  uint16_t* orow = out + ((int64_t)(row0 + qi) * H + h) * HD;
+#pragma unroll
+  for (int dt = 0; dt < NT; ++dt) {
+    uint2 w;
+    w.x = pack2_bf16(st.o[dt][0] * inv, st.o[dt][1] * inv);
+    w.y = pack2_bf16(st.o[dt][2] * inv, st.o[dt][3] * inv);
     *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * lg) = w;
   }
 }
@@ -290,7 +459,7 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   st.l = 0.f;
   const int hi = n_keys - 1;
   attend_range<NT>(st, qf, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, kb_begin,
-                   (kb_end + 31) & ~31, first, hi, scale, lr, lg);
+                   (kb_end + 31) & ~31, first, hi, first, hi, scale * 1.4426950408889634f, lr, lg);
   float l = st.l;
   l += __shfl_xor(l, 16, HE_WAVE);
   l += __shfl_xor(l, 32, HE_WAVE);
@@ -300,10 +469,8 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
 #pragma unroll
     for (int dt = 0; dt < NT; ++dt) {
       uint2 w;
-      w.x = (uint32_t)float_to_bf16_bits(st.o[dt][0] * inv) |
-            ((uint32_t)float_to_bf16_bits(st.o[dt][1] * inv) << 16);
-      w.y = (uint32_t)float_to_bf16_bits(st.o[dt][2] * inv) |
-            ((uint32_t)float_to_bf16_bits(st.o[dt][3] * inv) << 16);
+      w.x = pack2_bf16(st.o[dt][0] * inv, st.o[dt][1] * inv);
+      w.y = pack2_bf16(st.o[dt][2] * inv, st.o[dt][3] * inv);
       *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * lg) = w;
     }
     return;
@@ -348,7 +515,7 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(
   const float m = lane < active ? ws_ml[2 * (base + lane)] : -INFINITY;
   const float l = lane < active ? ws_ml[2 * (base + lane) + 1] : 0.f;
   const float M = wave_max(m);
-  const float w = m > -INFINITY ? __expf(m - M) : 0.f;
+  const float w = m > -INFINITY ? __builtin_amdgcn_exp2f(m - M) : 0.f;   // m is in the base-2 domain
   const float L = wave_sum(l * w);          // every wavefront computes the same weights
   if (wave == 0) wgt[lane] = w;
   __syncthreads();
@@ -471,6 +638,22 @@ extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* k
              "he_attention_prefill_bf16: buffers must be 16-byte aligned");
   if (num_seqs == 0 || max_q_len == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
+  if (hd <= 128 && max_q_len > 16) {   // K/V pages shared through LDS by 128 queries
+    dim3 grid128((max_q_len + 127) / 128, H, num_seqs);
+#define PREFILL_LDS(NTV)                                                                        \
+  case NTV:                                                                                     \
+    attention_prefill_lds_kernel<NTV><<<grid128, 64 * PF_WAVES, 0, s>>>(                                  \
+        (uint16_t*)out, (const uint16_t*)q, (const uint16_t*)kpool, (const uint16_t*)vpool,     \
+        (const int32_t*)cu_seqlens, (const int32_t*)seq_slot, (const int32_t*)seq_start,        \
+        (const int32_t*)page_table, max_blocks, num_pages, H, KVH, window, scale);              \
+    break;
+    switch (hd / 16) {
+      PREFILL_LDS(1) PREFILL_LDS(2) PREFILL_LDS(3) PREFILL_LDS(4)
+      PREFILL_LDS(5) PREFILL_LDS(6) PREFILL_LDS(7) PREFILL_LDS(8)
+    }
+#undef PREFILL_LDS
+    return he_check_launch("he_attention_prefill_bf16");
+  }
   dim3 grid((max_q_len + 63) / 64, H, num_seqs);
   ATTN_SWITCH(hd / 16, (attention_prefill_kernel<NT><<<grid, 256, 0, s>>>(
                            (uint16_t*)out, (const uint16_t*)q, (const uint16_t*)kpool,

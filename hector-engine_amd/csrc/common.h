@@ -32,6 +32,14 @@ __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
   return (uint16_t)(u >> 16);
 }
 
+// two floats to two bf16 in one register, round to nearest even (v_cvt_pk_bf16_f32)
+typedef __bf16 he_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float he_float2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
+  const he_float2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, he_bf16x2));
+}
+
 __device__ __forceinline__ float to_float(float x) { return x; }
 __device__ __forceinline__ float to_float(bf16_t x) { return bf16_bits_to_float(x.v); }
 

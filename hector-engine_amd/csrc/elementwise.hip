@@ -117,6 +117,34 @@ __global__ void silu_mul_kernel(T* __restrict__ out, const TI* __restrict__ x, i
   }
 }
 
+// bf16, eight outputs per thread. Both layouts keep eight consecutive gates (and their
+// ups) contiguous when I is a multiple of 8 (16 for the interleaved one).
+__global__ void silu_mul_vec_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ x,
+                                    int64_t rows, int I, int interleaved) {
+  const int64_t n8 = rows * (int64_t)(I >> 3);
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  const int per_row = I >> 3;
+  for (; i < n8; i += stride) {
+    const int64_t r = i / per_row;
+    const int c = (int)(i - r * per_row) << 3;
+    const int gc = interleaved ? 32 * (c >> 4) + (c & 15) : c;
+    const int uc = interleaved ? gc + 16 : I + c;
+    const uint16_t* row = x + r * 2 * (int64_t)I;
+    const uint4 g4 = *reinterpret_cast<const uint4*>(row + gc);
+    const uint4 u4 = *reinterpret_cast<const uint4*>(row + uc);
+    const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
+      const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
+      o[j] = pack2_bf16(g0 / (1.f + expf(-g0)) * u0, g1 / (1.f + expf(-g1)) * u1);
+    }
+    *reinterpret_cast<uint4*>(out + r * (int64_t)I + c) = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+
 extern "C" int he_silu_mul(void* out, const void* gate_up, int rows, int I, int interleaved,
                            int splits, int dtype, void* stream) {
   HE_REQUIRE(rows >= 0 && I > 0, "he_silu_mul: bad sizes rows=%d I=%d", rows, I);
@@ -129,7 +157,14 @@ extern "C" int he_silu_mul(void* out, const void* gate_up, int rows, int I, int 
   int64_t blocks = (n + 255) / 256;
   if (blocks > 65535 * 4) blocks = 65535 * 4;
   hipStream_t s = (hipStream_t)stream;
-  if (splits > 0) {  // fp32 partial sums in
+  if (splits == 0 && dtype == HE_BF16 && (I & (interleaved ? 15 : 7)) == 0 &&
+      ((((uintptr_t)out) | ((uintptr_t)gate_up)) & 15) == 0) {
+    const int64_t n8 = n >> 3;
+    int64_t vb = (n8 + 255) / 256;
+    if (vb > 65535 * 4) vb = 65535 * 4;
+    silu_mul_vec_kernel<<<(int)vb, 256, 0, s>>>((uint16_t*)out, (const uint16_t*)gate_up, rows, I,
+                                                interleaved);
+  } else if (splits > 0) {  // fp32 partial sums in
     if (dtype == HE_BF16)
       silu_mul_kernel<bf16_t, float><<<(int)blocks, 256, 0, s>>>(
           (bf16_t*)out, (const float*)gate_up, rows, I, interleaved, splits);
