@@ -141,7 +141,7 @@ __device__ __forceinline__ void attend_frag(AttnState<NT>& st, const bf16x8* qf,
 // Runs the steps kb = kb_begin, kb_begin + 32, ... < kb_end (all multiples of 32) of one
 // (sequence, kv head) against the state, one step ahead with its loads and one page
 // ahead with its page-table entry.
-template <int NT>
+template <int NT, bool UNMASKED_STEPS>
 __device__ __forceinline__ void attend_range(AttnState<NT>& st, const bf16x8* qf,
                                              const uint16_t* __restrict__ kpool,
                                              const uint16_t* __restrict__ vpool,
@@ -170,7 +170,7 @@ __device__ __forceinline__ void attend_range(AttnState<NT>& st, const bf16x8* qf
       load_frag<NT>(nxt, kp, vp, page, num_pages, page_stride, kn & 32, lr, lg);
     }
     // keys in [clear_lo, clear_hi] are visible to every query of the tile
-    if (kb >= clear_lo && kb + 31 <= clear_hi && cur.ok)
+    if (UNMASKED_STEPS && kb >= clear_lo && kb + 31 <= clear_hi && cur.ok)
       attend_frag<NT, false>(st, qf, cur, kb, lo, hi, scale_log2, lg);
     else
       attend_frag<NT, true>(st, qf, cur, kb, lo, hi, scale_log2, lg);
@@ -233,7 +233,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   const bool full_tile = q0 + 15 < q_len;
   const int clear_lo = window > 0 ? max(0, last_pos + 1 - window) : 0;
   const int clear_hi = full_tile ? first_pos : -1;
-  attend_range<NT>(st, qf, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, tile_lo & ~31,
+  attend_range<NT, true>(st, qf, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, tile_lo & ~31,
                    (last_pos & ~31) + 32, lo, hi, clear_lo, clear_hi, scale * 1.4426950408889634f,
                    lr, lg);
   float l = st.l;
@@ -262,7 +262,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 #define PF_WAVES 8
 #define PF_QUERIES (16 * PF_WAVES)
 template <int NT>
-__global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2))) void
+__global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 attention_prefill_lds_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q,
     const uint16_t* __restrict__ kpool, const uint16_t* __restrict__ vpool,
@@ -458,7 +458,7 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   st.m = -INFINITY;
   st.l = 0.f;
   const int hi = n_keys - 1;
-  attend_range<NT>(st, qf, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, kb_begin,
+  attend_range<NT, false>(st, qf, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, kb_begin,
                    (kb_end + 31) & ~31, first, hi, first, hi, scale * 1.4426950408889634f, lr, lg);
   float l = st.l;
   l += __shfl_xor(l, 16, HE_WAVE);

@@ -29,19 +29,16 @@ def random_tensor(name: str, spec: TensorSpec, seed: int, dtype: torch.dtype, de
     kind = spec.init[0]
     if kind == "zeros":
         return torch.zeros(shape, dtype=dtype, device=device)
-    numel = 1
-    for s in shape:
-        numel *= s
-    # large tensors are drawn straight in their dtype to bound peak memory
-    draw = dtype if numel > (1 << 26) else torch.float32
-    t = torch.empty(shape, dtype=draw, device=device).normal_(0.0, 1.0, generator=gen)
+    # always drawn in float32 and rounded to bfloat16 first, so that the values do not
+    # depend on the precision the model is then run in
+    t = torch.empty(shape, dtype=torch.float32, device=device).normal_(0.0, 1.0, generator=gen)
     if kind == "normal":
         t.mul_(spec.init[1])
     elif kind == "gain":
         t.mul_(spec.init[2]).add_(spec.init[1])
     else:
         raise ValueError(f"tensor '{name}': unknown init {spec.init}")
-    return t.to(dtype)
+    return t.to(torch.bfloat16).to(dtype)
 
 
 def random_tensors(expected: dict[str, TensorSpec], seed: int, dtype: torch.dtype,
