@@ -1,0 +1,301 @@
+// One-token attention in one launch: projection bias, rotary encoding of q and of the
+// new key, the cache write of the new key and value, attention over the cache and the
+// merge of the key slices. It replaces three launches (the q/k/v kernel, the split
+// attention kernel and its merge) where the encoding is a rotation of the whole head and
+// the head size is 64 or 128, so that the two elements of a rotated pair sit in
+// the same lane of the MFMA operand. Reference ops it covers: add_bias, rope, kv_cache_update,
+// attention_cached (kernels/elementwise.cu:307-323, kernels/attention.cu:516-558,
+// :1067-1097, :337-494).
+//
+// grid (KVH * head_tiles, rows, Z), 64 * NW threads. The workgroups (., ., z) own one
+// sequence and kv head; the query heads of the group are the columns of the tiles
+// (attention_tiles.h). The keys [first, p] are cut into Z * NW slices, one per wavefront.
+// The wavefront whose slice holds the new position p first writes the new key (bias,
+// rotation) and value into the cache and then reads them back with the rest of its
+// slice - the same wavefront, behind a workgroup-scope fence; no other wavefront reads
+// that row. Every wavefront leaves (m, l, O) of its slice in LDS and the workgroup joins
+// them in wavefront order: O = sum_w O_w 2^(m_w - M), L = sum_w l_w 2^(m_w - M). With
+// Z = 1 the workgroup stores O / L; with more (few sequences: one workgroup per sequence
+// and kv head would leave most of the chip, and its memory bandwidth, idle) it stores
+// (M, L, O) and attention_merge_kernel joins the Z parts in a second launch.
+#include "attention_tiles.h"
+#include "hector_kernels.h"
+
+#define FUSED_MIN_CHUNK 64
+
+// q of the group's heads as B operand, from the un-biased projection row: lane (lr =
+// head column, lg) holds dims 32ks + 8lg .. +8 of head lr for every k step ks. The partner
+// of dim d < half is d + half = the same lane's element in k step ks + half/32. sn, c: the
+// sine and cosine of angle `lane` (lanes below half), fetched from the lane that holds them.
+template <int NT>
+__device__ __forceinline__ void load_q_rotated(bf16x8* qf, const uint16_t* qrow,
+                                               const void* bias, int bias_dtype, int bias_off,
+                                               bool valid, int lg, float sn, float c) {
+  constexpr int HD = 16 * NT;
+  constexpr int KS = HD / 32;
+  constexpr int HS = KS / 2;   // k steps per half of the head
+  float x[KS][8];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d0 = 32 * ks + 8 * lg;
+    const bool ok = valid && d0 < HD;
+    uint4 raw = make_uint4(0, 0, 0, 0);
+    if (ok) raw = *reinterpret_cast<const uint4*>(qrow + d0);
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      x[ks][2 * j] = __uint_as_float(w[j] << 16);
+      x[ks][2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+    }
+    if (ok && bias != nullptr)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[ks][j] += load_param(bias, bias_off + d0 + j, bias_dtype);
+  }
+#pragma unroll
+  for (int ks = 0; ks < HS; ++ks)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int i = 32 * ks + 8 * lg + j;
+      const float si = __shfl(sn, i, HE_WAVE), ci = __shfl(c, i, HE_WAVE);
+      const float a0 = x[ks][j], a1 = x[ks + HS][j];
+      x[ks][j] = a0 * ci - a1 * si;
+      x[ks + HS][j] = a0 * si + a1 * ci;
+    }
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+    qf[ks] = __builtin_bit_cast(
+        bf16x8, make_uint4(pack2_bf16(x[ks][0], x[ks][1]), pack2_bf16(x[ks][2], x[ks][3]),
+                           pack2_bf16(x[ks][4], x[ks][5]), pack2_bf16(x[ks][6], x[ks][7])));
+}
+
+template <int NT>
+__global__ __launch_bounds__(512) void attention_decode_fused_kernel(
+    uint16_t* __restrict__ out, float* __restrict__ ws_o, float* __restrict__ ws_ml,
+    const uint16_t* __restrict__ qkv, int64_t qkv_stride,
+    const void* __restrict__ bias, int bias_dtype, uint16_t* kpool, uint16_t* vpool,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
+    const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ page_table, int max_blocks,
+    int num_pages, const float* __restrict__ inv_freq, int rotary_dim, int H, int KVH,
+    int head_tiles, int window, float scale, int write_kv) {
+  constexpr int HD = 16 * NT;
+  constexpr int KS = (HD + 31) / 32;
+  extern __shared__ __attribute__((aligned(16))) float lds[];   // [NW][GT][HD] O, then [NW][GT][2] (m, l)
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int lr = lane & 15, lg = lane >> 4;
+  const int kvh = blockIdx.x / head_tiles, ht = blockIdx.x % head_tiles;
+  const int row = blockIdx.y;
+  const int G = H / KVH;
+  const int GT = min(16, G - 16 * ht);     // heads of this tile
+  const bool h_ok = lr < GT;
+  const int h = kvh * G + 16 * ht + min(lr, GT - 1);
+  const int seq = row_seq[row];
+  const int Z = gridDim.z, z = blockIdx.z;
+  if (seq < 0) {                           // padding row: zeros (from the merge kernel if there is one)
+    if (Z == 1)
+      for (int i = threadIdx.x; i < GT * HD; i += blockDim.x)
+        out[((int64_t)row * H + kvh * G + 16 * ht) * HD + i] = 0;
+    return;
+  }
+  const int slot = seq_slot[seq];
+  const int p = positions[row];
+  const int n_keys = p + 1;
+  const int first = window > 0 ? max(0, n_keys - window) : 0;
+  const int span_lo = first & ~31;
+  const int slices = Z * nw;
+  int chunk = (n_keys - span_lo + slices - 1) / slices;
+  chunk = max(FUSED_MIN_CHUNK, (chunk + 31) & ~31);
+  const int kb_begin = span_lo + (z * nw + wave) * chunk;
+  const int kb_end = min(kb_begin + chunk, n_keys);
+  const int32_t* pt = page_table + (int64_t)slot * max_blocks;
+  const uint16_t* qkv_row = qkv + (int64_t)row * qkv_stride;
+  const bool has_keys = kb_begin < kb_end;   // uniform in the wavefront
+  float sn = 0.f, c = 1.f;                   // lane j < HD / 2: angle j of position p
+  if (has_keys && lane < HD / 2) sincos_angle((float)p * inv_freq[lane], &sn, &c);
+
+  // ---- the new key and value go into the cache, written by the wavefront that reads them
+  if (write_kv && p >= kb_begin && p < kb_end) {
+    const int page = pt[p >> HE_PAGE_SHIFT];
+    if (page >= 0 && page < num_pages) {
+      const int off = p & (HE_PAGE_TOKENS - 1);
+      const int half = rotary_dim >> 1;
+      const int k_col = H * HD + kvh * HD, v_col = (H + KVH) * HD + kvh * HD;
+      uint16_t* krow = kpool + (((int64_t)page * KVH + kvh) * HE_PAGE_TOKENS + off) * HD;
+      uint16_t* vcol = vpool + ((int64_t)page * KVH + kvh) * HD * HE_PAGE_TOKENS + off;
+      if (lane < half) {                     // half <= 64: one pair per lane
+        const int j = lane;
+        float x0 = bf16_bits_to_float(qkv_row[k_col + j]);
+        float x1 = bf16_bits_to_float(qkv_row[k_col + j + half]);
+        if (bias) {
+          x0 += load_param(bias, k_col + j, bias_dtype);
+          x1 += load_param(bias, k_col + j + half, bias_dtype);
+        }
+        krow[j] = float_to_bf16_bits(x0 * c - x1 * sn);
+        krow[j + half] = float_to_bf16_bits(x0 * sn + x1 * c);
+      }
+      for (int d = lane; d < HD; d += 64) {
+        float x = bf16_bits_to_float(qkv_row[v_col + d]);
+        if (bias) x += load_param(bias, v_col + d, bias_dtype);
+        vcol[(int64_t)d * HE_PAGE_TOKENS] = float_to_bf16_bits(x);
+      }
+    }
+    __threadfence_block();   // this wavefront reads the row back below
+  }
+
+  AttnState<NT> st;
+#pragma unroll
+  for (int dt = 0; dt < NT; ++dt) st.o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  st.m = -INFINITY;
+  st.l = 0.f;
+  if (has_keys) {
+    bf16x8 qf[KS];
+    load_q_rotated<NT>(qf, qkv_row + (int64_t)h * HD, bias, bias_dtype, h * HD, h_ok, lg, sn, c);
+    attend_range<NT, false>(st, qf, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, kb_begin,
+                            (kb_end + 31) & ~31, first, p, first, p,
+                            scale * 1.4426950408889634f, lr, lg);
+  }
+  float l = st.l;
+  l += __shfl_xor(l, 16, HE_WAVE);
+  l += __shfl_xor(l, 32, HE_WAVE);
+
+  // ---- join the slices through LDS, in wavefront order
+  float* lds_o = lds;
+  float* lds_ml = lds + (int64_t)nw * GT * HD;
+  if (h_ok) {
+    float* o = lds_o + ((int64_t)wave * GT + lr) * HD;
+#pragma unroll
+    for (int dt = 0; dt < NT; ++dt)
+      *reinterpret_cast<float4*>(o + 16 * dt + 4 * lg) =
+          make_float4(st.o[dt][0], st.o[dt][1], st.o[dt][2], st.o[dt][3]);
+    if (lg == 0) {
+      lds_ml[2 * (wave * GT + lr)] = st.m;
+      lds_ml[2 * (wave * GT + lr) + 1] = l;
+    }
+  }
+  __syncthreads();
+  for (int item = threadIdx.x; item < GT * (HD / 4); item += blockDim.x) {
+    const int hg = item / (HD / 4), d = 4 * (item % (HD / 4));
+    float M = -INFINITY;
+    for (int w = 0; w < nw; ++w) M = fmaxf(M, lds_ml[2 * (w * GT + hg)]);
+    float L = 0.f;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int w = 0; w < nw; ++w) {
+      const float m = lds_ml[2 * (w * GT + hg)];
+      if (!(m > -INFINITY)) continue;
+      const float wgt = __builtin_amdgcn_exp2f(m - M);
+      L += lds_ml[2 * (w * GT + hg) + 1] * wgt;
+      const float4 v = *reinterpret_cast<const float4*>(lds_o + ((int64_t)w * GT + hg) * HD + d);
+      acc.x += v.x * wgt;
+      acc.y += v.y * wgt;
+      acc.z += v.z * wgt;
+      acc.w += v.w * wgt;
+    }
+    const int64_t head = (int64_t)row * H + kvh * G + 16 * ht + hg;
+    if (Z == 1) {
+      const float inv = L > 0.f ? 1.f / L : 0.f;
+      uint2 w2;
+      w2.x = pack2_bf16(acc.x * inv, acc.y * inv);
+      w2.y = pack2_bf16(acc.z * inv, acc.w * inv);
+      *reinterpret_cast<uint2*>(out + head * HD + d) = w2;
+    } else {                               // a part without keys stores (-inf, 0, zeros)
+      *reinterpret_cast<float4*>(ws_o + (head * Z + z) * HD + d) = acc;
+      if (d == 0) {
+        ws_ml[2 * (head * Z + z)] = M;
+        ws_ml[2 * (head * Z + z) + 1] = L;
+      }
+    }
+  }
+}
+
+// Wavefronts per workgroup and workgroups per (sequence, kv head, head tile). Many
+// sequences: one workgroup of 8 wavefronts each, no second launch. Few: 4 wavefronts and
+// enough workgroups to put about 512 on the chip, while a slice keeps 64 keys at max_keys.
+static void fused_shape(int rows, int H, int KVH, int hd, int max_keys, int* nw, int* Z) {
+  const int G = H / KVH;
+  const int gt = G < 16 ? G : 16;
+  const int groups = rows * KVH * ((G + 15) / 16);
+  int w = (int64_t)8 * gt * (hd + 2) * 4 <= 65536 ? 8 : 4, zz = 1;
+  if (groups < 128) {
+    w = 4;
+    zz = (512 + groups - 1) / groups;
+    const int most = (max_keys + 4 * FUSED_MIN_CHUNK - 1) / (4 * FUSED_MIN_CHUNK);
+    if (zz > most) zz = most;
+    if (zz > 64) zz = 64;
+    if (zz < 1) zz = 1;
+  }
+  *nw = w;
+  *Z = zz;
+}
+
+// Whether the fused kernel takes these sizes (otherwise the caller runs the separate
+// q/k/v, attention and merge kernels).
+extern "C" int he_attention_decode_fused_ok(int H, int KVH, int hd, int rotary_dim) {
+  if (H <= 0 || KVH <= 0 || H % KVH) return 0;
+  if (hd != 64 && hd != 128) return 0;   // registers: the fragments of two steps are in flight
+  return rotary_dim == hd;
+}
+
+extern "C" int64_t he_attention_decode_fused_workspace_floats(int rows, int H, int KVH, int hd,
+                                                              int max_keys) {
+  if (rows <= 0 || !he_attention_decode_fused_ok(H, KVH, hd, hd) || max_keys <= 0) return 0;
+  int nw, Z;
+  fused_shape(rows, H, KVH, hd, max_keys, &nw, &Z);
+  return Z == 1 ? 0 : (int64_t)rows * H * Z * (hd + 2);
+}
+
+extern "C" int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_t qkv_stride,
+                                              const void* bias, int bias_dtype, void* kpool,
+                                              void* vpool, const void* positions,
+                                              const void* row_seq, const void* seq_slot,
+                                              const void* page_table, int max_blocks,
+                                              int num_pages, const void* inv_freq, int rotary_dim,
+                                              int rows, int H, int KVH, int hd, int window,
+                                              float scale, int max_keys, int write_kv,
+                                              void* workspace_f32, int64_t workspace_floats,
+                                              void* stream) {
+  HE_REQUIRE(rows >= 0 && H > 0 && KVH > 0 && hd > 0 && max_keys > 0,
+             "he_attention_decode_fused_bf16: bad sizes");
+  HE_REQUIRE(he_attention_decode_fused_ok(H, KVH, hd, rotary_dim),
+             "he_attention_decode_fused_bf16: sizes H=%d KVH=%d head_dim=%d rotary_dim=%d are not "
+             "taken (head_dim 64 or 128, rotated whole)", H, KVH, hd, rotary_dim);
+  HE_REQUIRE(rows <= 65535, "he_attention_decode_fused_bf16: %d rows above 65535", rows);
+  HE_REQUIRE((qkv_stride & 7) == 0 && (((uintptr_t)qkv) & 15) == 0 &&
+                 (((uintptr_t)kpool) & 15) == 0 && (((uintptr_t)vpool) & 15) == 0 &&
+                 (((uintptr_t)out) & 7) == 0,
+             "he_attention_decode_fused_bf16: buffers must be 16-byte aligned");
+  HE_REQUIRE(inv_freq != nullptr, "he_attention_decode_fused_bf16: missing inv_freq");
+  if (rows == 0) return 0;
+  const int G = H / KVH;
+  const int head_tiles = (G + 15) / 16;
+  const int gt = G < 16 ? G : 16;
+  int nw, Z;
+  fused_shape(rows, H, KVH, hd, max_keys, &nw, &Z);
+  const int64_t need = Z == 1 ? 0 : (int64_t)rows * H * Z * (hd + 2);
+  HE_REQUIRE(Z == 1 || (workspace_f32 != nullptr && workspace_floats >= need &&
+                        (((uintptr_t)workspace_f32) & 15) == 0),
+             "he_attention_decode_fused_bf16: workspace of %lld floats, need %lld (16-byte aligned)",
+             (long long)workspace_floats, (long long)need);
+  float* ws_o = (float*)workspace_f32;
+  float* ws_ml = ws_o ? ws_o + (int64_t)rows * H * Z * hd : nullptr;
+  const size_t lds = (size_t)nw * gt * (hd + 2) * sizeof(float);
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid(KVH * head_tiles, rows, Z);
+#define FUSED(NTV)                                                                              \
+  case NTV:                                                                                     \
+    attention_decode_fused_kernel<NTV><<<grid, 64 * nw, lds, s>>>(                              \
+        (uint16_t*)out, ws_o, ws_ml, (const uint16_t*)qkv, qkv_stride, bias, bias_dtype,        \
+        (uint16_t*)kpool,                                                                       \
+        (uint16_t*)vpool, (const int32_t*)positions, (const int32_t*)row_seq,                   \
+        (const int32_t*)seq_slot, (const int32_t*)page_table, max_blocks, num_pages,            \
+        (const float*)inv_freq, rotary_dim, H, KVH, head_tiles, window, scale, write_kv);       \
+    break;
+  switch (hd / 16) {
+    FUSED(4) FUSED(8)
+    default:
+      HE_REQUIRE(false, "he_attention_decode_fused_bf16: head_dim %d", hd);
+  }
+#undef FUSED
+  const int rc = he_check_launch("he_attention_decode_fused_bf16");
+  if (rc || Z == 1) return rc;
+  return he_attention_merge_parts(out, ws_o, ws_ml, row_seq, rows, H, hd, Z, stream);
+}

@@ -22,169 +22,7 @@
 #include "common.h"
 #include "hector_kernels.h"
 
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
-
-__device__ __forceinline__ bf16x8 ld8(const uint16_t* p, bool ok) {
-  uint4 v = make_uint4(0, 0, 0, 0);
-  if (ok) v = *reinterpret_cast<const uint4*>(p);
-  return __builtin_bit_cast(bf16x8, v);
-}
-
-template <int NT>
-struct AttnState {
-  floatx4 o[NT];  // O^T[16*dt + 4*lg + i][q], unnormalised
-  float m;        // running maximum of the query of this lane's column
-  float l;        // this lane's share of the running sum
-};
-
-// The K and V^T operands of one step of 32 keys, loaded ahead of their use so that the
-// loads of step i+1 are in flight while step i computes.
-template <int NT>
-struct KVFrag {
-  bf16x8 k[2][(16 * NT + 31) / 32];
-  bf16x8 v[NT];
-  int ok;   // the page exists (always, for an admitted batch)
-};
-
-// kpool/vpool of this kv head; page: physical page of the 32 keys; koff: 0 or 32.
-template <int NT>
-__device__ __forceinline__ void load_frag(KVFrag<NT>& f, const uint16_t* __restrict__ kpool,
-                                          const uint16_t* __restrict__ vpool, int page,
-                                          int num_pages, int64_t page_stride, int koff, int lr,
-                                          int lg) {
-  constexpr int HD = 16 * NT;
-  constexpr int KS = (HD + 31) / 32;
-  f.ok = page >= 0 && page < num_pages;
-  const int64_t pbase = (int64_t)(f.ok ? page : 0) * page_stride;
-  const uint16_t* kpage = kpool + pbase;
-  const uint16_t* vpage = vpool + pbase;
-#pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    const int key_local = 8 * (lr >> 2) + 4 * t + (lr & 3);
-    const uint16_t* krow = kpage + (koff + key_local) * HD + 8 * lg;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) f.k[t][ks] = ld8(krow + 32 * ks, 32 * ks + 8 * lg < HD);
-  }
-#pragma unroll
-  for (int dt = 0; dt < NT; ++dt)
-    f.v[dt] = ld8(vpage + (16 * dt + lr) * HE_PAGE_TOKENS + koff + 8 * lg, true);
-}
-
-// One step of 32 keys starting at absolute position key_base (a multiple of 32).
-// The lane's query sees the keys in [lo, hi]; with MASK false the caller has checked
-// that all 32 keys are visible to every query of the tile. Scores are kept in the
-// base-2 domain: s2 = (q . k) * scale * log2(e), p = 2^(s2 - m), so the exponential is
-// the bare hardware instruction; m is the running maximum of s2. When no query's
-// maximum moves, the rescaling of the accumulators is skipped.
-template <int NT, bool MASK>
-__device__ __forceinline__ void attend_frag(AttnState<NT>& st, const bf16x8* qf,
-                                            const KVFrag<NT>& f, int key_base, int lo, int hi,
-                                            float scale_log2, int lg) {
-  constexpr int HD = 16 * NT;
-  constexpr int KS = (HD + 31) / 32;
-  if (MASK && !f.ok) hi = -1;
-  floatx4 s[2];
-#pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k[t][ks], qf[ks], s[t], 0, 0, 0);
-  }
-  float p[2][4];
-  float mx = -INFINITY;
-#pragma unroll
-  for (int t = 0; t < 2; ++t)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      float v = s[t][r] * scale_log2;
-      if (MASK) {
-        const int key = key_base + 8 * lg + 4 * t + r;
-        v = (key >= lo && key <= hi) ? v : -INFINITY;
-      }
-      p[t][r] = v;
-      mx = fmaxf(mx, v);
-    }
-  mx = fmaxf(mx, __shfl_xor(mx, 16, HE_WAVE));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, HE_WAVE));
-  const float m_new = fmaxf(st.m, mx);
-  const bool moved = __builtin_amdgcn_ballot_w64(m_new != st.m) != 0;   // wave-uniform
-  const float m_use = m_new == -INFINITY ? 0.f : m_new;
-  float sum = 0.f;
-  uint32_t packed[4];
-#pragma unroll
-  for (int t = 0; t < 2; ++t)
-#pragma unroll
-    for (int r = 0; r < 4; r += 2) {
-      const float e0 = __builtin_amdgcn_exp2f(p[t][r] - m_use);
-      const float e1 = __builtin_amdgcn_exp2f(p[t][r + 1] - m_use);
-      sum += e0 + e1;
-      packed[2 * t + (r >> 1)] = pack2_bf16(e0, e1);
-    }
-  if (moved) {
-    const float alpha = __builtin_amdgcn_exp2f(st.m - m_use);
-    st.l = st.l * alpha + sum;
-    st.m = m_new;
-#pragma unroll
-    for (int dt = 0; dt < NT; ++dt) st.o[dt] *= alpha;
-  } else {
-    st.l += sum;
-  }
-  const bf16x8 pb =
-      __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
-#pragma unroll
-  for (int dt = 0; dt < NT; ++dt)
-    st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.v[dt], pb, st.o[dt], 0, 0, 0);
-}
-
-// Runs the steps kb = kb_begin, kb_begin + 32, ... < kb_end (all multiples of 32) of one
-// (sequence, kv head) against the state, one step ahead with its loads and one page
-// ahead with its page-table entry.
-template <int NT, bool UNMASKED_STEPS>
-__device__ __forceinline__ void attend_range(AttnState<NT>& st, const bf16x8* qf,
-                                             const uint16_t* __restrict__ kpool,
-                                             const uint16_t* __restrict__ vpool,
-                                             const int32_t* __restrict__ pt, int max_blocks,
-                                             int num_pages, int KVH, int kvh, int kb_begin,
-                                             int kb_end, int lo, int hi, int clear_lo,
-                                             int clear_hi, float scale_log2, int lr, int lg) {
-  constexpr int HD = 16 * NT;
-  if (kb_begin >= kb_end) return;
-  const int64_t page_stride = (int64_t)KVH * (HE_PAGE_TOKENS * HD);
-  const uint16_t* kp = kpool + (int64_t)kvh * (HE_PAGE_TOKENS * HD);
-  const uint16_t* vp = vpool + (int64_t)kvh * (HE_PAGE_TOKENS * HD);
-  int block = kb_begin >> HE_PAGE_SHIFT;
-  int page = pt[block];
-  int page_ahead = pt[min(block + 1, max_blocks - 1)];
-  KVFrag<NT> cur, nxt;
-  load_frag<NT>(cur, kp, vp, page, num_pages, page_stride, kb_begin & 32, lr, lg);
-  for (int kb = kb_begin; kb < kb_end; kb += 32) {
-    const int kn = kb + 32;
-    if (kn < kb_end) {
-      if ((kn & 32) == 0) {   // the next step starts a new page
-        ++block;
-        page = page_ahead;
-        page_ahead = pt[min(block + 1, max_blocks - 1)];
-      }
-      load_frag<NT>(nxt, kp, vp, page, num_pages, page_stride, kn & 32, lr, lg);
-    }
-    // keys in [clear_lo, clear_hi] are visible to every query of the tile
-    if (UNMASKED_STEPS && kb >= clear_lo && kb + 31 <= clear_hi && cur.ok)
-      attend_frag<NT, false>(st, qf, cur, kb, lo, hi, scale_log2, lg);
-    else
-      attend_frag<NT, true>(st, qf, cur, kb, lo, hi, scale_log2, lg);
-    cur = nxt;
-  }
-}
-
-template <int NT>
-__device__ __forceinline__ void load_q(bf16x8* qf, const uint16_t* qrow, bool valid, int lg) {
-  constexpr int HD = 16 * NT;
-  constexpr int KS = (HD + 31) / 32;
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) qf[ks] = ld8(qrow + 32 * ks + 8 * lg, valid && 32 * ks + 8 * lg < HD);
-}
+#include "attention_tiles.h"
 
 // ------------------------------------------------------------------ prefill
 // grid (ceil(max_q_len / 64), H, num_seqs), 256 threads: wave w takes the 16
@@ -495,7 +333,7 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
 __global__ __launch_bounds__(256) void attention_merge_kernel(
     uint16_t* __restrict__ out, const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq, int H, int HD,
-    int nsplit, int window) {
+    int nsplit, int window, int all_parts) {
   __shared__ float wgt[64];
   __shared__ float part[4][256];
   const int h = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -505,12 +343,15 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(
     for (int d = threadIdx.x; d < HD; d += 256) orow[d] = 0;
     return;
   }
-  const int n_keys = positions[row] + 1;
-  const int first = window > 0 ? max(0, n_keys - window) : 0;
-  const int span_lo = first & ~31;
-  int chunk = (n_keys - span_lo + nsplit - 1) / nsplit;
-  chunk = max(DECODE_MIN_CHUNK, (chunk + 31) & ~31);
-  const int active = (n_keys - span_lo + chunk - 1) / chunk;
+  int active = nsplit;                     // all_parts: every part was stored, empty ones as (-inf, 0, 0)
+  if (!all_parts) {
+    const int n_keys = positions[row] + 1;
+    const int first = window > 0 ? max(0, n_keys - window) : 0;
+    const int span_lo = first & ~31;
+    int chunk = (n_keys - span_lo + nsplit - 1) / nsplit;
+    chunk = max(DECODE_MIN_CHUNK, (chunk + 31) & ~31);
+    active = (n_keys - span_lo + chunk - 1) / chunk;
+  }
   const int64_t base = (row * H + h) * nsplit;
   const float m = lane < active ? ws_ml[2 * (base + lane)] : -INFINITY;
   const float l = lane < active ? ws_ml[2 * (base + lane) + 1] : 0.f;
@@ -616,8 +457,17 @@ extern "C" int he_attention_decode_bf16(void* out, const void* q, const void* kp
   if (rc || nsplit == 1) return rc;
   attention_merge_kernel<<<dim3(H, rows), 256, 0, s>>>(
       (uint16_t*)out, ws_o, ws_ml, (const int32_t*)positions, (const int32_t*)row_seq, H, hd,
-      nsplit, window);
+      nsplit, window, 0);
   return he_check_launch("he_attention_decode_bf16 merge");
+}
+
+// Joins parts [rows][H][parts] of (O fp32 [hd], then (m, l) pairs) that were all stored.
+int he_attention_merge_parts(void* out, const float* ws_o, const float* ws_ml, const void* row_seq,
+                             int rows, int H, int hd, int parts, void* stream) {
+  HE_REQUIRE(parts >= 1 && parts <= 64, "he_attention_merge_parts: %d parts, at most 64", parts);
+  attention_merge_kernel<<<dim3(H, rows), 256, 0, (hipStream_t)stream>>>(
+      (uint16_t*)out, ws_o, ws_ml, nullptr, (const int32_t*)row_seq, H, hd, parts, 0, 1);
+  return he_check_launch("he_attention_merge_parts");
 }
 
 extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* kpool,

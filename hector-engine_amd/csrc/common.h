@@ -62,6 +62,24 @@ __device__ __forceinline__ float load_param(const void* p, int64_t i, int dtype)
   return dtype == HE_BF16 ? bf16_bits_to_float(((const uint16_t*)p)[i]) : ((const float*)p)[i];
 }
 
+// sin and cos of an fp32 angle to fp32 accuracy: the quadrant is taken off in double
+// (k = rint(a * 2/pi), r = a - k * pi/2, |r| <= pi/4), the two short series are summed
+// in double and rounded once. The library routine's path for large arguments is far
+// slower, and angles here reach tens of thousands of radians.
+__device__ __forceinline__ void sincos_angle(float a, float* sn, float* cs) {
+  const double x = (double)a;
+  const double k = rint(x * 0.63661977236758134308);
+  const double r = fma(-k, 6.123233995736766036e-17, fma(-k, 1.57079632679489655800, x));
+  const double r2 = r * r;
+  const double sp = r * (1.0 + r2 * (-1.0 / 6 + r2 * (1.0 / 120 + r2 * (-1.0 / 5040 + r2 * (1.0 / 362880 + r2 * (-1.0 / 39916800))))));
+  const double cp = 1.0 + r2 * (-0.5 + r2 * (1.0 / 24 + r2 * (-1.0 / 720 + r2 * (1.0 / 40320 + r2 * (-1.0 / 3628800 + r2 * (1.0 / 479001600))))));
+  const int q = (int)((long long)k & 3);
+  const double sv = (q & 1) ? cp : sp;
+  const double cv = (q & 1) ? sp : cp;
+  *sn = (float)((q & 2) ? -sv : sv);
+  *cs = (float)(((q + 1) & 2) ? -cv : cv);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int off = HE_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, HE_WAVE);
@@ -93,6 +111,9 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 // ---- error channel -------------------------------------------------------
 void he_set_error(const char* fmt, ...);
 int he_check_launch(const char* what);
+// attention_mfma.hip: joins attention parts that were all stored (used by the fused one-token kernel)
+int he_attention_merge_parts(void* out, const float* ws_o, const float* ws_ml, const void* row_seq,
+                             int rows, int H, int hd, int parts, void* stream);
 
 #define HE_REQUIRE(cond, ...)      \
   do {                             \

@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 8
+#define HE_ABI_VERSION 9
 
 #ifdef __cplusplus
 extern "C" {
@@ -81,6 +81,19 @@ int he_attention_decode_bf16(void* out, const void* q, const void* kpool, const 
                              int H, int KVH, int hd, int window, float scale, int max_keys,
                              void* workspace_f32, int64_t workspace_floats, void* stream);
 int64_t he_attention_decode_workspace_floats(int rows, int H, int KVH, int hd, int max_keys);
+// bf16, one query row per sequence, one launch for bias + rotary + cache write + attention +
+// merge (a second launch joins the parts where few sequences are cut across workgroups).
+// qkv: the un-biased projection rows [rows, (H + 2 KVH) hd]. he_attention_decode_fused_ok: 1
+// when the sizes are taken (head_dim 64 or 128, rotated whole).
+int he_attention_decode_fused_ok(int H, int KVH, int hd, int rotary_dim);
+int64_t he_attention_decode_fused_workspace_floats(int rows, int H, int KVH, int hd, int max_keys);
+int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_t qkv_stride, const void* bias,
+                                   int bias_dtype, void* kpool, void* vpool, const void* positions,
+                                   const void* row_seq, const void* seq_slot,
+                                   const void* page_table, int max_blocks, int num_pages,
+                                   const void* inv_freq, int rotary_dim, int rows, int H, int KVH,
+                                   int hd, int window, float scale, int max_keys, int write_kv,
+                                   void* workspace_f32, int64_t workspace_floats, void* stream);
 // bf16, prompt steps: tiles of queries of one sequence against its cache rows.
 int he_attention_prefill_bf16(void* out, const void* q, const void* kpool, const void* vpool,
                               const void* cu_seqlens, const void* seq_slot, const void* seq_start,

@@ -16,24 +16,6 @@
 
 #define ROPE_MAX_HALF 256
 
-// sin and cos of an fp32 angle to fp32 accuracy: the quadrant is taken off in double
-// (k = rint(a * 2/pi), r = a - k * pi/2, |r| <= pi/4), the two short series are summed
-// in double and rounded once. The library routine's path for large arguments is far
-// slower, and angles here reach tens of thousands of radians.
-__device__ __forceinline__ void sincos_angle(float a, float* sn, float* cs) {
-  const double x = (double)a;
-  const double k = rint(x * 0.63661977236758134308);
-  const double r = fma(-k, 6.123233995736766036e-17, fma(-k, 1.57079632679489655800, x));
-  const double r2 = r * r;
-  const double sp = r * (1.0 + r2 * (-1.0 / 6 + r2 * (1.0 / 120 + r2 * (-1.0 / 5040 + r2 * (1.0 / 362880 + r2 * (-1.0 / 39916800))))));
-  const double cp = 1.0 + r2 * (-0.5 + r2 * (1.0 / 24 + r2 * (-1.0 / 720 + r2 * (1.0 / 40320 + r2 * (-1.0 / 3628800 + r2 * (1.0 / 479001600))))));
-  const int q = (int)((long long)k & 3);
-  const double sv = (q & 1) ? cp : sp;
-  const double cv = (q & 1) ? sp : cp;
-  *sn = (float)((q & 2) ? -sv : sv);
-  *cs = (float)(((q + 1) & 2) ? -cv : cv);
-}
-
 template <typename TI>
 __device__ __forceinline__ float load_in(const TI* p, int splits, int64_t split_stride) {
   if (splits <= 1) return to_float(p[0]);

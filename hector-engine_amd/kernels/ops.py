@@ -351,6 +351,48 @@ def attention_decode(out, q, kpool, vpool, positions, row_seq, seq_slot, page_ta
         workspace.numel(), _stream()))
 
 
+def attention_decode_fused_ok(H: int, KVH: int, hd: int, rotary_dim: int) -> bool:
+    return int(_lib.load().he_attention_decode_fused_ok(H, KVH, hd, rotary_dim)) > 0
+
+
+def attention_decode_fused_workspace_floats(rows: int, H: int, KVH: int, hd: int, max_keys: int) -> int:
+    return int(_lib.load().he_attention_decode_fused_workspace_floats(rows, H, KVH, hd, max_keys))
+
+
+def attention_decode_fused(out, qkv, bias, kpool, vpool, positions, row_seq, seq_slot, page_table,
+                           inv_freq, rotary_dim: int, rows: int, H: int, KVH: int, hd: int,
+                           window: int, scale: float, max_keys: int, write_kv: bool,
+                           workspace) -> None:
+    """One-token steps in one launch: bias, rotation of q and of the new key, cache write,
+    attention over the cache, merge. qkv: bf16 [rows, (H + 2 KVH) hd] without bias; q columns
+    alone where the run reads another run's cache (write_kv False)."""
+    width = (H + 2 * KVH) * hd if write_kv else H * hd
+    _need(qkv, "qkv", torch.bfloat16)
+    _need(out, "out", torch.bfloat16)
+    if qkv.dim() != 2 or qkv.shape[1] != width or qkv.shape[0] < rows or out.numel() < rows * H * hd:
+        raise ValueError("attention_decode_fused: qkv/out do not match the head sizes and row count")
+    _need(kpool, "kpool", torch.bfloat16, (None, KVH, PAGE_TOKENS, hd))
+    _need(vpool, "vpool", torch.bfloat16, (None, KVH, hd, PAGE_TOKENS))
+    _need(page_table, "page_table", torch.int32)
+    for name, t in (("positions", positions), ("row_seq", row_seq), ("seq_slot", seq_slot)):
+        _need(t, name, torch.int32)
+    if positions.numel() < rows or row_seq.numel() < rows or page_table.dim() != 2:
+        raise ValueError("attention_decode_fused: metadata shorter than the row count")
+    if bias is not None:
+        _need(bias, "bias", shape=(width,))
+    _need(inv_freq, "inv_freq", torch.float32, (rotary_dim // 2,))
+    if workspace is not None:
+        _need(workspace, "workspace", torch.float32)
+    L = _lib.load()
+    _lib.check(L.he_attention_decode_fused_bf16(
+        out.data_ptr(), qkv.data_ptr(), width, _ptr(bias),
+        dtype_code(bias.dtype) if bias is not None else F32, kpool.data_ptr(), vpool.data_ptr(),
+        positions.data_ptr(), row_seq.data_ptr(), seq_slot.data_ptr(), page_table.data_ptr(),
+        page_table.shape[1], kpool.shape[0], inv_freq.data_ptr(), rotary_dim, rows, H, KVH, hd,
+        window, float(scale), max_keys, int(write_kv), _ptr(workspace),
+        workspace.numel() if workspace is not None else 0, _stream()))
+
+
 def attention_prefill(out, q, kpool, vpool, cu_seqlens, seq_slot, seq_start, page_table,
                       num_seqs: int, max_q_len: int, total_rows: int, H: int, KVH: int, hd: int,
                       window: int, scale: float) -> None:

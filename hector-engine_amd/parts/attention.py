@@ -95,6 +95,18 @@ class Attention(Mixer):
         proj = self.qkv if writes else self.q_only
         rot = self.position.rotary()
         fused_bias = not self.position.custom
+        if self.fast and ctx.all_single and fused_bias and rot is not None \
+                and ops.attention_decode_fused_ok(H, KVH, hd, rot[1]):
+            # one-token steps: bias, rotation, cache write and attention in one launch
+            qkv = proj(x, rows, ctx, use_bias=False)
+            out = ctx.alloc((rows, H * hd))
+            floats = ops.attention_decode_fused_workspace_floats(rows, H, KVH, hd, ctx.max_keys)
+            ws = ctx.alloc((floats,), torch.float32) if floats else None
+            ops.attention_decode_fused(out, qkv, proj.bias, cache.kpool, cache.vpool, ctx.positions,
+                                       ctx.row_seq, ctx.seq_slot, cache.page_table, rot[0], rot[1],
+                                       rows, H, KVH, hd, self.window, self.scale, ctx.max_keys,
+                                       writes, ws)
+            return self.o_proj(out, rows, ctx, allow_split=True)
         # With a rotation (or no encoding) the bias is added inside the fused kernel;
         # any other encoding sees q and k with their bias already added.
         qkv = proj(x, rows, ctx, use_bias=not fused_bias, allow_split=fused_bias)

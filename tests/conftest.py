@@ -52,7 +52,17 @@ TINY_C = {
     "tie_word_embeddings": False, "use_sliding_window": True, "sliding_window": 70,
     "max_window_layers": 1, "hidden_act": "silu",
 }
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
+# Tiny D: head_dim 64 (the one-launch one-token attention takes it), H*hd = 2 D, window 40 on the
+# last layer, bias-free norm eps and theta of their own
+TINY_D = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "num_hidden_layers": 2, "hidden_size": 128, "num_attention_heads": 4,
+    "num_key_value_heads": 2, "head_dim": 64, "intermediate_size": 208, "vocab_size": 200,
+    "rope_theta": 20000.0, "rms_norm_eps": 2e-6, "max_position_embeddings": 512,
+    "tie_word_embeddings": True, "use_sliding_window": True, "sliding_window": 40,
+    "max_window_layers": 1, "hidden_act": "silu",
+}
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3)}
 
 
 @pytest.fixture(scope="session")

@@ -315,10 +315,11 @@ def paged_setup(lengths, KVH, hd, dtype, seed, extra_pages=3):
 
 def fill_cache(table, slots, kpool, vpool, ks, vs):
     for s, k, v in zip(slots, ks, vs):
-        for p in range(k.shape[0]):
-            page = table[s, p // PAGE].item()
-            kpool[page, :, p % PAGE, :] = k[p]
-            vpool[page, :, :, p % PAGE] = v[p]
+        for b in range((k.shape[0] + PAGE - 1) // PAGE):
+            page = table[s, b].item()
+            kb, vb = k[b * PAGE:(b + 1) * PAGE], v[b * PAGE:(b + 1) * PAGE]
+            kpool[page, :, :kb.shape[0], :] = kb.transpose(0, 1)
+            vpool[page, :, :, :vb.shape[0]] = vb.permute(1, 2, 0)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -437,6 +438,79 @@ def test_attention_prefill(ops, H, KVH, hd, window):
                                [150, 237, 3, 66], [150, 37, 3, 1], 42)
     for g, w in zip(got, want):
         assert torch.allclose(g, w, rtol=2 ** -6, atol=2 ** -6)
+
+
+@pytest.mark.parametrize("H,KVH,hd", [(4, 1, 64), (28, 4, 128), (6, 3, 64), (40, 2, 128)])
+@pytest.mark.parametrize("window", [0, 70])
+@pytest.mark.parametrize("write_kv", [True, False])
+@pytest.mark.parametrize("copies", [1, 24])
+def test_attention_decode_fused(ops, H, KVH, hd, window, write_kv, copies):
+    """Bias, rotation, cache write, attention and merge in one launch against the plain parts.
+    Lengths sit at page and slice edges; a padding row stands between the sequences. With few
+    sequences the keys are cut across workgroups and joined by a second launch; with many
+    (copies > 1) one workgroup serves a sequence and kv head."""
+    theta = 50000.0
+    lengths = [700, 1, 64, 65, 300, 129] * copies
+    if copies > 1:
+        lengths = [min(n, 200) for n in lengths]
+    B = len(lengths)
+    assert ops.attention_decode_fused_ok(H, KVH, hd, hd)
+    floats = ops.attention_decode_fused_workspace_floats(B + 1, H, KVH, hd, 4096)
+    assert (floats == 0) == ((B + 1) * KVH * ((H // KVH + 15) // 16) >= 128)
+    ws = torch.empty(floats, device="cuda") if floats else None
+    slots, table, kpool, vpool = paged_setup(lengths, KVH, hd, torch.bfloat16, 60)
+    old = [n if not write_kv else n - 1 for n in lengths]
+    ks = [rnd(n, KVH, hd, seed=61 + i).to(torch.bfloat16) for i, n in enumerate(old)]
+    vs = [rnd(n, KVH, hd, seed=71 + i).to(torch.bfloat16) for i, n in enumerate(old)]
+    fill_cache(table, slots, kpool, vpool, ks, vs)
+    width = (H + 2 * KVH) * hd if write_kv else H * hd
+    qkv = rnd(B, width, seed=81, scale=1.5).to(torch.bfloat16)
+    bias = rnd(width, seed=82).to(torch.bfloat16)
+    pad_at = 2
+    order = list(range(pad_at)) + [-1] + list(range(pad_at, B))          # row -> sequence
+    rows = len(order)
+    qkv_rows = torch.stack([qkv[s] if s >= 0 else torch.zeros(width, dtype=torch.bfloat16) for s in order])
+    positions = torch.tensor([lengths[s] - 1 if s >= 0 else 0 for s in order], dtype=torch.int32)
+    row_seq = torch.tensor(order, dtype=torch.int32)
+    seq_slot = torch.tensor(slots, dtype=torch.int32)
+    inv = P.rope_inv_freq(hd, theta)
+    out = torch.full((rows, H * hd), 7.0, dtype=torch.bfloat16, device="cuda")
+    kp, vp = dev(kpool), dev(vpool)
+    ops.attention_decode_fused(out, dev(qkv_rows), dev(bias), kp, vp, dev(positions), dev(row_seq),
+                               dev(seq_slot), dev(table), dev(inv), hd, rows, H, KVH, hd, window,
+                               1.0 / math.sqrt(hd), 4096, write_kv, ws)
+    got = out.cpu().double()
+    kp, vp = kp.cpu(), vp.cpu()
+    assert got[pad_at].abs().max() == 0
+    x = qkv.double() + bias.double()
+    for r, s in enumerate(order):
+        if s < 0:
+            continue
+        n = lengths[s]
+        pos = torch.tensor([n - 1])
+        q = P.rope(x[s, :H * hd].reshape(1, H, hd), pos, theta, hd).to(torch.bfloat16).double()
+        k_all, v_all = ks[s].double(), vs[s].double()
+        if write_kv:
+            k_new = P.rope(x[s, H * hd:(H + KVH) * hd].reshape(1, KVH, hd), pos, theta, hd)
+            v_new = x[s, (H + KVH) * hd:].reshape(1, KVH, hd)
+            k_new, v_new = k_new.to(torch.bfloat16), v_new.to(torch.bfloat16)
+            page = table[slots[s], (n - 1) // PAGE].item()
+            assert torch.allclose(kp[page, :, (n - 1) % PAGE, :].double(), k_new[0].double(),
+                                  rtol=2 ** -7, atol=2 ** -7), s
+            assert torch.allclose(vp[page, :, :, (n - 1) % PAGE].double(), v_new[0].double(),
+                                  rtol=2 ** -7, atol=2 ** -7), s
+            k_all, v_all = torch.cat([k_all, k_new.double()]), torch.cat([v_all, v_new.double()])
+        want = P.attention(q, k_all, v_all, pos, torch.arange(n), window).reshape(-1)
+        assert torch.allclose(got[r], want, rtol=2 ** -6, atol=2 ** -6), (s, (got[r] - want).abs().max())
+    if write_kv:   # nothing but the new rows was written
+        before = dev(kpool).cpu()
+        assert (kp != before).sum().item() <= B * KVH * hd
+
+
+def test_attention_decode_fused_refuses_other_sizes(ops):
+    assert not ops.attention_decode_fused_ok(4, 2, 48, 48)      # head size
+    assert not ops.attention_decode_fused_ok(4, 2, 64, 32)      # partial rotation
+    assert not ops.attention_decode_fused_ok(5, 2, 64, 64)
 
 
 def test_attention_far_key_stands_out(ops):
