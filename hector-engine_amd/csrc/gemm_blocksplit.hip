@@ -13,6 +13,15 @@
 // two row tiles of a workgroup (R = 2) are a gate block and its up block, and the
 // output is silu(gate) * up, [M, N/2] (reference: kernels/activations.cu:183-198
 // as a kernel of its own).
+//
+// Two more epilogues carry an RMS norm across a pair of products without a kernel of
+// its own (reference: kernels/fused_add_rmsnorm.cu:47-81 as a separate kernel):
+//   residual: r[m][n] += acc (+ bias), stored fp32 in place; xg[m][n] = bf16(r * g[n]) with
+//     the gain g of the norm that follows; and the sum of r^2 over the workgroup's columns
+//     per row, one partial per workgroup: sq[m][block].
+//   row scale: the consumer of xg adds the partials of a row in a fixed order,
+//     s[m] = 1 / sqrt(sum / dim + eps), and multiplies its sums by s[m] before bias or
+//     gate: W (r g s) = s W (r g). The norm's statistics stay fp32.
 #include "common.h"
 #include "hector_kernels.h"
 
@@ -48,12 +57,88 @@ __device__ __forceinline__ void bs_store4<bf16_t>(bf16_t* p, const float v[4], b
   }
 }
 
+// Registers hold the operands of two steps (the loads of the next step are issued before
+// the products of this one), 16 U (R + MT) of them; above 4 tile pairs the workgroup is
+// limited to 8 wavefronts so that each may use 256 registers.
+constexpr int bs_max_waves(int MT, int R, int U) { return U * (R + MT) <= 4 ? 16 : 8; }
+
+template <int MT, int R, int U>
+struct BsFrags {
+  bf16x8 a[U][R][2], b[U][MT][2];
+};
+
+template <int MT, int R, int U>
+__device__ __forceinline__ void bs_load(BsFrags<MT, R, U>& f, const uint16_t* const* wp,
+                                        const uint16_t* const* xp, int k, int lg, int k_end) {
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int kk = k + 64 * u + lg * 16;   // this lane's 16 k values of the step
+    const bool ok0 = kk + 8 <= k_end, ok1 = kk + 16 <= k_end;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      f.a[u][r][0] = bs_load8(wp[r] + k + 64 * u, ok0);
+      f.a[u][r][1] = bs_load8(wp[r] + k + 64 * u + 8, ok1);
+    }
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      f.b[u][t][0] = bs_load8(xp[t] + k + 64 * u, ok0);
+      f.b[u][t][1] = bs_load8(xp[t] + k + 64 * u + 8, ok1);
+    }
+  }
+}
+
+template <int MT, int R, int U>
+__device__ __forceinline__ void bs_multiply(const BsFrags<MT, R, U>& f, floatx4 (&acc)[R][MT]) {
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+          acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.a[u][r][h], f.b[u][t][h], acc[r][t],
+                                                              0, 0, 0);
+}
+
+struct BsFusion {
+  const float* scale_partials;   // [M][scale_count] or null: sums of squares of the input rows
+  int scale_count;
+  float scale_eps;
+  int scale_dim;
+  float* resid;                  // [M][N] fp32 or null: residual rows, updated in place
+  const void* gain;              // [N] gain of the following norm
+  int gain_dtype;
+  uint16_t* xg;                  // [M][N] bf16 out: resid * gain
+  float* sq_out;                 // [M][gridDim.x] out: sum of resid^2 over this workgroup's columns
+};
+
+// The residual values and gains of output item (tile, lane) of a non-gated product:
+// row m = 16 t + lane % 16, columns n0 + 16 r + 4 (lane / 16) .. + 4.
+template <int MT>
+__device__ __forceinline__ void bs_load_resid(const BsFusion& fu, int item, int n0, int M, int N,
+                                              float res[4], float gain[4]) {
+  const int ot = item >> 6, ol = item & 63;
+  const int m = 16 * (ot % MT) + (ol & 15);
+  const int n = n0 + 16 * (ot / MT) + 4 * (ol >> 4);
+  const int valid = m < M ? max(0, min(4, N - n)) : 0;
+  if (valid == 4 && (N & 3) == 0) {
+    const float4 r4 = *reinterpret_cast<const float4*>(fu.resid + (int64_t)m * N + n);
+    res[0] = r4.x, res[1] = r4.y, res[2] = r4.z, res[3] = r4.w;
+  } else {
+    for (int i = 0; i < 4; ++i) res[i] = i < valid ? fu.resid[(int64_t)m * N + n + i] : 0.f;
+  }
+  for (int i = 0; i < 4; ++i) gain[i] = i < valid ? load_param(fu.gain, n + i, fu.gain_dtype) : 0.f;
+}
+
 // grid: one workgroup per 16*R weight rows; block: 64 * NW threads.
 template <int MT, int R, int U, bool GATED, typename TC>
-__global__ __launch_bounds__(1024) void gemm_blocksplit_kernel(
+__global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_kernel(
     TC* __restrict__ C, const uint16_t* __restrict__ X, const uint16_t* __restrict__ W,
-    const void* __restrict__ bias, int bias_dtype, int M, int N, int K, int kslice) {
+    const void* __restrict__ bias, int bias_dtype, int M, int N, int K, int kslice, BsFusion fu) {
   extern __shared__ float4 tiles[];   // [NW][R*MT][64]
+  __shared__ float row_scale[16 * MT];
+  __shared__ float row_sq[R * MT][16];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
@@ -75,33 +160,59 @@ __global__ __launch_bounds__(1024) void gemm_blocksplit_kernel(
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[r][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  for (int k = k_begin; k < k_end; k += 64 * U) {
-    bf16x8 a[U][R][2], b[U][MT][2];
+  // Loads the epilogue needs are issued here, ahead of the weight stream, so that their
+  // latency is not added at the end: the partial sums of squares of the input rows
+  // (wavefront w takes the rows w and w + nw; lanes hold strided partials) and, for the
+  // residual epilogue, the residual values and gains of this thread's first outputs.
+  constexpr int OUT_TILES = GATED ? (R / 2) * MT : R * MT;
+  const bool scaled = fu.scale_partials != nullptr;
+  const bool to_resid = !GATED && fu.resid != nullptr;
+  const bool scale_early = scaled && fu.scale_count <= 256 && M <= 2 * nw;
+  float pv[2][4];
+  if (scale_early) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int kk = k + 64 * u + lg * 16;   // this lane's 16 k values of the step
-      const bool ok0 = kk + 8 <= k_end, ok1 = kk + 16 <= k_end;
+    for (int j = 0; j < 2; ++j) {
+      const int m = wave + j * nw;
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        a[u][r][0] = bs_load8(wp[r] + k + 64 * u, ok0);
-        a[u][r][1] = bs_load8(wp[r] + k + 64 * u + 8, ok1);
-      }
-#pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        b[u][t][0] = bs_load8(xp[t] + k + 64 * u, ok0);
-        b[u][t][1] = bs_load8(xp[t] + k + 64 * u + 8, ok1);
+      for (int q = 0; q < 4; ++q) {
+        const int i = lane + 64 * q;
+        pv[j][q] = (m < M && i < fu.scale_count) ? fu.scale_partials[(int64_t)m * fu.scale_count + i] : 0.f;
       }
     }
+  }
+  float res0[4] = {0.f, 0.f, 0.f, 0.f}, gain0[4] = {0.f, 0.f, 0.f, 0.f};
+  if (to_resid && threadIdx.x < OUT_TILES * 64)
+    bs_load_resid<MT>(fu, threadIdx.x, n0, M, N, res0, gain0);
+
+  // two steps of 64 U k values per turn; a step past k_end loads nothing and adds zeros
+  BsFrags<MT, R, U> f0, f1;
+  bs_load<MT, R, U>(f0, wp, xp, k_begin, lg, k_end);
+  for (int k = k_begin; k < k_end; k += 128 * U) {
+    bs_load<MT, R, U>(f1, wp, xp, k + 64 * U, lg, k_end);
+    bs_multiply<MT, R, U>(f0, acc);
+    bs_load<MT, R, U>(f0, wp, xp, k + 128 * U, lg, k_end);
+    bs_multiply<MT, R, U>(f1, acc);
+  }
+
+  if (scaled) {
+    if (scale_early) {
 #pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int h = 0; h < 2; ++h)
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-          for (int t = 0; t < MT; ++t)
-            acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][r][h], b[u][t][h], acc[r][t],
-                                                                0, 0, 0);
+      for (int j = 0; j < 2; ++j) {
+        const int m = wave + j * nw;
+        if (m < M) {
+          const float total = wave_sum(((pv[j][0] + pv[j][1]) + pv[j][2]) + pv[j][3]);
+          if (lane == 0) row_scale[m] = 1.0f / sqrtf(total / (float)fu.scale_dim + fu.scale_eps);
+        }
+      }
+    } else {
+      for (int m = wave; m < M; m += nw) {
+        float part = 0.f;
+        for (int i = lane; i < fu.scale_count; i += 64)
+          part += fu.scale_partials[(int64_t)m * fu.scale_count + i];
+        const float total = wave_sum(part);
+        if (lane == 0) row_scale[m] = 1.0f / sqrtf(total / (float)fu.scale_dim + fu.scale_eps);
+      }
+    }
   }
 
   // every wavefront leaves its tiles; acc[r][t][i] = D[n0 + 16r + 4lg + i][16t + lr]
@@ -113,15 +224,14 @@ __global__ __launch_bounds__(1024) void gemm_blocksplit_kernel(
           make_float4(acc[r][t][0], acc[r][t][1], acc[r][t][2], acc[r][t][3]);
   __syncthreads();
 
-  // thread (tile, lane) adds the slices in wavefront order and writes 4 outputs
-  constexpr int OUT_TILES = GATED ? (R / 2) * MT : R * MT;
+  // thread (tile, lane) adds the slices in wavefront order and writes 4 outputs; a
+  // wavefront works on one tile at a time (item >> 6 is the same in all its lanes)
   for (int item = threadIdx.x; item < OUT_TILES * 64; item += blockDim.x) {
     const int ot = item >> 6, ol = item & 63;
     const int olr = ol & 15, olg = ol >> 4;
     const int t = ot % MT;
     const int r = GATED ? 2 * (ot / MT) : ot / MT;
     const int m = 16 * t + olr;
-    if (m >= M) continue;
     float4 s = make_float4(0.f, 0.f, 0.f, 0.f), s2 = s;
     for (int w = 0; w < nw; ++w) {
       const float4 v = tiles[(w * (R * MT) + r * MT + t) * 64 + ol];
@@ -132,22 +242,56 @@ __global__ __launch_bounds__(1024) void gemm_blocksplit_kernel(
       }
     }
     float v[4] = {s.x, s.y, s.z, s.w};
+    const float rs = (scaled && m < M) ? row_scale[m] : 1.f;
     if (GATED) {
       const float up[4] = {s2.x, s2.y, s2.z, s2.w};
       const int NO = N >> 1;
       const int n = (n0 >> 1) + 8 * r + 4 * olg;
-      const int valid = min(4, NO - n);
+      const int valid = m < M ? min(4, NO - n) : 0;
       if (valid <= 0) continue;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = v[i] / (1.f + expf(-v[i])) * up[i];
+      for (int i = 0; i < 4; ++i) {
+        const float g = v[i] * rs;
+        v[i] = g / (1.f + expf(-g)) * (up[i] * rs);
+      }
       bs_store4<TC>(C + (int64_t)m * NO + n, v, (NO & 3) == 0, valid);
     } else {
       const int n = n0 + 16 * r + 4 * olg;
-      const int valid = min(4, N - n);
-      if (valid <= 0) continue;
+      const int valid = m < M ? max(0, min(4, N - n)) : 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] *= rs;
       if (bias != nullptr)
         for (int i = 0; i < valid; ++i) v[i] += load_param(bias, n + i, bias_dtype);
-      bs_store4<TC>(C + (int64_t)m * N + n, v, (N & 3) == 0, valid);
+      if (!to_resid) {
+        if (valid > 0) bs_store4<TC>(C + (int64_t)m * N + n, v, (N & 3) == 0, valid);
+        continue;
+      }
+      if (item != threadIdx.x) bs_load_resid<MT>(fu, item, n0, M, N, res0, gain0);
+      float sq = 0.f, x[4], xgv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        x[i] = res0[i] + v[i];
+        xgv[i] = x[i] * gain0[i];
+        if (i < valid) sq += x[i] * x[i];
+      }
+      if (valid > 0) {
+        const int64_t at = (int64_t)m * N + n;
+        bs_store4<float>(fu.resid + at, x, (N & 3) == 0, valid);
+        bs_store4<bf16_t>(reinterpret_cast<bf16_t*>(fu.xg) + at, xgv, (N & 3) == 0, valid);
+      }
+      // the four lane groups hold the row's other columns of this tile
+      sq += __shfl_xor(sq, 16, HE_WAVE);
+      sq += __shfl_xor(sq, 32, HE_WAVE);
+      if (olg == 0) row_sq[ot][olr] = sq;
+    }
+  }
+  if (to_resid) {
+    __syncthreads();
+    const int m = threadIdx.x;
+    if (m < M && m < 16 * MT) {
+      float sq = 0.f;
+      for (int r = 0; r < R; ++r) sq += row_sq[r * MT + m / 16][m % 16];
+      fu.sq_out[(int64_t)m * gridDim.x + blockIdx.x] = sq;
     }
   }
 }
@@ -181,6 +325,7 @@ static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int
     NW = nw;
     while (NW > 1 && K / NW < 128) NW >>= 1;
   }
+  if (NW > bs_max_waves(p.MT, p.R, p.U)) NW = bs_max_waves(p.MT, p.R, p.U);
   p.NW = NW;
   int ks = (K + NW - 1) / NW;
   p.kslice = (ks + 63) / 64 * 64;
@@ -190,20 +335,20 @@ static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int
 template <int MT, int R, int U, bool GATED, typename TC>
 static void launch_blocksplit(const BlockSplitPlan& p, void* C, const void* X, const void* W,
                               const void* bias, int bias_dtype, int M, int N, int K,
-                              hipStream_t s) {
+                              const BsFusion& fu, hipStream_t s) {
   const int blocks = (N + 16 * R - 1) / (16 * R);
   const size_t lds = (size_t)p.NW * R * MT * 64 * sizeof(float4);
   gemm_blocksplit_kernel<MT, R, U, GATED, TC><<<blocks, 64 * p.NW, lds, s>>>(
-      (TC*)C, (const uint16_t*)X, (const uint16_t*)W, bias, bias_dtype, M, N, K, p.kslice);
+      (TC*)C, (const uint16_t*)X, (const uint16_t*)W, bias, bias_dtype, M, N, K, p.kslice, fu);
 }
 
 template <bool GATED, typename TC>
 static int dispatch_blocksplit(const BlockSplitPlan& p, void* C, const void* X, const void* W,
                                const void* bias, int bias_dtype, int M, int N, int K,
-                               hipStream_t s) {
+                               const BsFusion& fu, hipStream_t s) {
 #define BS(MT_, R_, U_)                                                              \
   if (p.MT == MT_ && p.R == R_ && p.U == U_) {                                       \
-    launch_blocksplit<MT_, R_, U_, GATED, TC>(p, C, X, W, bias, bias_dtype, M, N, K, s); \
+    launch_blocksplit<MT_, R_, U_, GATED, TC>(p, C, X, W, bias, bias_dtype, M, N, K, fu, s); \
     return 0;                                                                        \
   }
   if (!GATED) {
@@ -215,10 +360,23 @@ static int dispatch_blocksplit(const BlockSplitPlan& p, void* C, const void* X, 
   return -1;
 }
 
+// Workgroups (= partial sums of squares per row) the residual epilogue of this product gives.
+extern "C" int he_gemm_blocksplit_blocks(int M, int N, int K) {
+  if (M <= 0 || M > HE_BLOCKSPLIT_MAX_M || N <= 0 || K <= 0) return 0;
+  const BlockSplitPlan p = blocksplit_plan(M, N, K, 0, 0, 0, 0);
+  return (N + 16 * p.R - 1) / (16 * p.R);
+}
+
 // R, U, NW <= 0 choose the heuristic tiling (NW wavefronts = K slices per workgroup).
-extern "C" int he_gemm_blocksplit_bf16(void* C, const void* A, const void* W, const void* bias,
-                                       int M, int N, int K, int out_dtype, int bias_dtype,
-                                       int gated, int R, int U, int NW, void* stream) {
+// scale_partials: sums of squares of the input rows (the rows are then scaled before
+// bias or gate); resid: the residual epilogue (C is not written; gain, xg, sq_out needed).
+extern "C" int he_gemm_blocksplit_fused_bf16(void* C, const void* A, const void* W,
+                                             const void* bias, int M, int N, int K, int out_dtype,
+                                             int bias_dtype, int gated, int R, int U, int NW,
+                                             const void* scale_partials, int scale_count,
+                                             float scale_eps, void* resid, const void* gain,
+                                             int gain_dtype, void* xg, void* sq_out,
+                                             int sq_count, void* stream) {
   HE_REQUIRE(M > 0 && M <= HE_BLOCKSPLIT_MAX_M, "he_gemm_blocksplit_bf16: M=%d outside [1, %d]", M,
              HE_BLOCKSPLIT_MAX_M);
   HE_REQUIRE(N > 0 && K > 0, "he_gemm_blocksplit_bf16: bad sizes N=%d K=%d", N, K);
@@ -229,20 +387,51 @@ extern "C" int he_gemm_blocksplit_bf16(void* C, const void* A, const void* W, co
   HE_REQUIRE(!gated || ((N & 31) == 0 && bias == nullptr),
              "he_gemm_blocksplit_bf16: the gated epilogue needs N=%d a multiple of 32 and no bias",
              N);
+  HE_REQUIRE(scale_partials == nullptr || scale_count > 0,
+             "he_gemm_blocksplit_bf16: row scale without partial sums");
   const BlockSplitPlan p = blocksplit_plan(M, N, K, gated, R, U, NW);
   HE_REQUIRE(p.NW >= 1 && p.NW <= 16, "he_gemm_blocksplit_bf16: %d wavefronts outside [1, 16]",
              p.NW);
   HE_REQUIRE(!gated || p.R == 2, "he_gemm_blocksplit_bf16: the gated epilogue needs R = 2");
+  const int blocks = (N + 16 * p.R - 1) / (16 * p.R);
+  if (resid != nullptr) {
+    HE_REQUIRE(!gated && gain != nullptr && xg != nullptr && sq_out != nullptr,
+               "he_gemm_blocksplit_bf16: the residual epilogue needs gain, xg and sq_out, and no gate");
+    HE_REQUIRE(sq_count == blocks,
+               "he_gemm_blocksplit_bf16: %d partial sums per row given, the product has %d workgroups",
+               sq_count, blocks);
+    HE_REQUIRE(gain_dtype == HE_F32 || gain_dtype == HE_BF16, "he_gemm_blocksplit_bf16: bad gain dtype");
+  } else {
+    HE_REQUIRE(C != nullptr, "he_gemm_blocksplit_bf16: no output");
+  }
+  BsFusion fu;
+  fu.scale_partials = (const float*)scale_partials;
+  fu.scale_count = scale_count;
+  fu.scale_eps = scale_eps;
+  fu.scale_dim = K;
+  fu.resid = (float*)resid;
+  fu.gain = gain;
+  fu.gain_dtype = gain_dtype;
+  fu.xg = (uint16_t*)xg;
+  fu.sq_out = (float*)sq_out;
   hipStream_t s = (hipStream_t)stream;
   int rc;
   if (gated)
     rc = out_dtype == HE_BF16
-             ? dispatch_blocksplit<true, bf16_t>(p, C, A, W, bias, bias_dtype, M, N, K, s)
-             : dispatch_blocksplit<true, float>(p, C, A, W, bias, bias_dtype, M, N, K, s);
+             ? dispatch_blocksplit<true, bf16_t>(p, C, A, W, bias, bias_dtype, M, N, K, fu, s)
+             : dispatch_blocksplit<true, float>(p, C, A, W, bias, bias_dtype, M, N, K, fu, s);
   else
     rc = out_dtype == HE_BF16
-             ? dispatch_blocksplit<false, bf16_t>(p, C, A, W, bias, bias_dtype, M, N, K, s)
-             : dispatch_blocksplit<false, float>(p, C, A, W, bias, bias_dtype, M, N, K, s);
+             ? dispatch_blocksplit<false, bf16_t>(p, C, A, W, bias, bias_dtype, M, N, K, fu, s)
+             : dispatch_blocksplit<false, float>(p, C, A, W, bias, bias_dtype, M, N, K, fu, s);
   if (rc) return rc;
   return he_check_launch("he_gemm_blocksplit_bf16");
+}
+
+extern "C" int he_gemm_blocksplit_bf16(void* C, const void* A, const void* W, const void* bias,
+                                       int M, int N, int K, int out_dtype, int bias_dtype,
+                                       int gated, int R, int U, int NW, void* stream) {
+  return he_gemm_blocksplit_fused_bf16(C, A, W, bias, M, N, K, out_dtype, bias_dtype, gated, R, U,
+                                       NW, nullptr, 0, 0.f, nullptr, nullptr, HE_F32, nullptr,
+                                       nullptr, 0, stream);
 }

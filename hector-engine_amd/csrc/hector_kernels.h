@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 9
+#define HE_ABI_VERSION 10
 
 #ifdef __cplusplus
 extern "C" {
@@ -57,6 +57,19 @@ int he_gemm_skinny_splits(int M, int N, int K);
 int he_gemm_blocksplit_bf16(void* C, const void* A, const void* W, const void* bias, int M, int N,
                             int K, int out_dtype, int bias_dtype, int gated, int R, int U, int NW,
                             void* stream);
+// The same with an RMS norm carried across a pair of products. resid != null: the residual
+// epilogue (resid[M,N] fp32 += result in place, xg[M,N] bf16 = resid * gain, sq_out[M, sq_count]
+// = sums of resid^2 per workgroup, sq_count = he_gemm_blocksplit_blocks). scale_partials != null:
+// the rows of A are such xg rows; the result is scaled by 1/sqrt(sum(partials)/K + eps) per row.
+int he_gemm_blocksplit_blocks(int M, int N, int K);
+int he_gemm_blocksplit_fused_bf16(void* C, const void* A, const void* W, const void* bias, int M,
+                                  int N, int K, int out_dtype, int bias_dtype, int gated, int R,
+                                  int U, int NW, const void* scale_partials, int scale_count,
+                                  float scale_eps, void* resid, const void* gain, int gain_dtype,
+                                  void* xg, void* sq_out, int sq_count, void* stream);
+// out = x / sqrt(sum(partials of the row)/D + eps): such xg rows as a normalised tensor.
+int he_scale_rows_bf16(void* out, const void* x, const void* partials, int count, int rows, int D,
+                       float eps, void* stream);
 int he_splitk_reduce(void* C, const void* partial_f32, const void* bias, int M, int N, int splits,
                      int out_dtype, int bias_dtype, void* stream);
 

@@ -180,3 +180,32 @@ extern "C" int he_rmsnorm_rows(void* out, const void* x, const void* weight, int
     HE_REQUIRE(false, "he_rmsnorm_rows: unknown dtype %d", dtype);
   return he_check_launch("he_rmsnorm_rows");
 }
+
+// Rows x = r * gain whose scale is still owed: out = x / sqrt(sum(partials of the row) / D + eps).
+// The partial sums of squares (one per workgroup of the product that made the rows) are
+// added as that product's consumers add them: lanes over strided partials, then the wavefront.
+__global__ void scale_rows_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ x,
+                                  const float* __restrict__ partials, int count, int D, float eps) {
+  __shared__ float inv_s;
+  const int64_t row = blockIdx.x;
+  if (threadIdx.x < 64) {
+    float part = 0.f;
+    for (int i = threadIdx.x; i < count; i += 64) part += partials[row * count + i];
+    const float total = wave_sum(part);
+    if (threadIdx.x == 0) inv_s = 1.0f / sqrtf(total / (float)D + eps);
+  }
+  __syncthreads();
+  const float inv = inv_s;
+  for (int i = threadIdx.x; i < D; i += blockDim.x)
+    out[row * D + i] = float_to_bf16_bits(bf16_bits_to_float(x[row * D + i]) * inv);
+}
+
+extern "C" int he_scale_rows_bf16(void* out, const void* x, const void* partials, int count,
+                                  int rows, int D, float eps, void* stream) {
+  HE_REQUIRE(rows >= 0 && D > 0 && count > 0, "he_scale_rows_bf16: bad sizes rows=%d D=%d count=%d",
+             rows, D, count);
+  if (rows == 0) return 0;
+  scale_rows_kernel<<<rows, norm_threads(D), 0, (hipStream_t)stream>>>(
+      (uint16_t*)out, (const uint16_t*)x, (const float*)partials, count, D, eps);
+  return he_check_launch("he_scale_rows_bf16");
+}

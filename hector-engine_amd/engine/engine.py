@@ -241,6 +241,8 @@ class Engine:
         ctx.host = {"q_lens": [len(e.tokens) for e in entries],
                     "starts": [self.cache.length(e.slot) for e in entries],
                     "slots": [e.slot for e in entries]}
+        want = meta.views(host.numpy())["want_rows"][:nw]
+        ctx.want_all = nw == rows and bool((want == np.arange(rows, dtype=np.int32)).all())
         self.stats["eager_steps"] += 1
         return self.model.forward(views["tokens"], ctx, self.caches, views["want_rows"], nw)
 
@@ -258,6 +260,7 @@ class Engine:
         bucket.uses += 1
         if bucket.graph is None:
             ctx = self._context(bucket.views, size, size, 1, True, bucket.pool)
+            ctx.want_all = True
             if bucket.uses == 1:
                 # first use: run eagerly; it also sizes the bucket's scratch pool
                 bucket.pool.reset()

@@ -75,11 +75,23 @@ class DecoderModel:
         rows = ctx.rows
         resid = self.embedding.forward(ids, rows, ctx)
         stream = ResidualStream(resid, rows)
+        last = len(self.schedule) - 1
         for e, entry in enumerate(self.schedule):
+            # the norm that reads the stream after this block: the next block's first, or the
+            # final norm when every row's logits are wanted (no gather in between)
+            if e < last:
+                ctx.next_norm = getattr(self.blocks[self.schedule[e + 1].layer], "mixer_norm", None)
+            else:
+                ctx.next_norm = self.final_norm if (ctx.want_all and n_want == rows) else None
             self.blocks[entry.layer].forward(stream, ctx, caches[e])
-        stream.materialize(ctx)
+        ctx.next_norm = None
         if n_want == 0:
+            stream.materialize(ctx)
             return None
+        if ctx.want_all and n_want == rows:
+            normed = stream.normed(self.final_norm, ctx, getattr(self.head, "accepts_normed_rows", False))
+            return self.head.forward(normed, n_want, ctx)
+        stream.materialize(ctx)
         sel = ctx.alloc((n_want, self.spec.hidden_size), torch.float32)
         ops.gather_rows_f32(sel, resid, want_rows, n_want, rows)
         normed = self.final_norm.add_norm(sel, None, n_want, ctx)

@@ -16,7 +16,7 @@ _lib = None
 
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 
-EXPECTED_ABI = 9
+EXPECTED_ABI = 10
 
 c_int, c_i64, c_f32, c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
@@ -37,6 +37,11 @@ _SIGNATURES = {
     "he_gemm_skinny_splits": [c_int, c_int, c_int],
     "he_gemm_blocksplit_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_int,
                                 c_int, c_int, c_int, c_ptr],
+    "he_gemm_blocksplit_blocks": [c_int, c_int, c_int],
+    "he_gemm_blocksplit_fused_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_int,
+                                      c_int, c_int, c_int, c_ptr, c_int, c_f32, c_ptr, c_ptr, c_int,
+                                      c_ptr, c_ptr, c_int, c_ptr],
+    "he_scale_rows_bf16": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_f32, c_ptr],
     "he_splitk_reduce": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_ptr],
     "he_qkv_rope_cache": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_int, c_ptr, c_ptr, c_ptr,
                           c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_ptr, c_int, c_int,

@@ -207,26 +207,78 @@ def gemm_skinny(out, partial, a, w, bias, M: int, gated: bool = False, plan=(0, 
 BLOCKSPLIT_MAX_M = 32
 
 
-def gemm_blocksplit(out, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0)) -> None:
+def gemm_blocksplit_blocks(M: int, N: int, K: int) -> int:
+    """Partial sums of squares per row that the residual epilogue of this product gives."""
+    return int(_lib.load().he_gemm_blocksplit_blocks(M, N, K))
+
+
+def gemm_blocksplit(out, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0), *,
+                    row_scale=None, residual=None) -> None:
     """bf16 MFMA product for M <= 32 with K cut inside the workgroup; one launch, complete
     result (bf16 or fp32), with bias or, gated, as [M, N/2] = silu(gate) * up for a weight
-    that interleaves gate and up rows in blocks of 16. plan = (R, U, NW), zeros = heuristic."""
+    that interleaves gate and up rows in blocks of 16. plan = (R, U, NW), zeros = heuristic.
+
+    row_scale = (partials fp32 [M, count], eps): the rows of `a` are r * gain of an RMS norm
+    whose 1/sqrt(mean(r^2) + eps) is applied to the sums here (mean over K).
+    residual = (resid fp32 [M, N], gain [N], xg bf16 [M, N], sq fp32 [M, blocks]): instead of
+    writing `out` (None), resid += result in place, xg = resid * gain, sq = the sums of resid^2
+    per workgroup (blocks = gemm_blocksplit_blocks(M, N, K))."""
     N, K = w.shape
     NO = N // 2 if gated else N
     _need(a, "a", torch.bfloat16)
     _need(w, "w", torch.bfloat16)
-    _need(out, "out")
     if M > BLOCKSPLIT_MAX_M:
         raise ValueError(f"gemm_blocksplit: M={M} above {BLOCKSPLIT_MAX_M}")
-    if a.shape[-1] != K or a.numel() < M * K or out.shape[-1] != NO or out.numel() < M * NO:
-        raise ValueError(f"gemm_blocksplit: shapes a{tuple(a.shape)} w{tuple(w.shape)} out{tuple(out.shape)} M={M}")
+    if a.shape[-1] != K or a.numel() < M * K:
+        raise ValueError(f"gemm_blocksplit: shapes a{tuple(a.shape)} w{tuple(w.shape)} M={M}")
+    if residual is None:
+        _need(out, "out")
+        if out.shape[-1] != NO or out.numel() < M * NO:
+            raise ValueError(f"gemm_blocksplit: out{tuple(out.shape)} for M={M} N={NO}")
+    elif out is not None or gated or plan != (0, 0, 0):
+        raise ValueError("gemm_blocksplit: the residual epilogue writes no `out`, is not gated and plans itself")
     if bias is not None:
         _need(bias, "bias", shape=(N,))
+    sp, sc, se = None, 0, 0.0
+    if row_scale is not None:
+        partials, se = row_scale
+        _need(partials, "row_scale partials", torch.float32)
+        if partials.dim() != 2 or partials.shape[0] < M:
+            raise ValueError("gemm_blocksplit: row_scale partials must be [M, count]")
+        sp, sc = partials.data_ptr(), partials.shape[1]
+    rp = gp = xp = qp = None
+    gdt, qc = F32, 0
+    if residual is not None:
+        resid, gain, xg, sq = residual
+        _need(resid, "resid", torch.float32)
+        _need(gain, "gain", shape=(N,))
+        _need(xg, "xg", torch.bfloat16)
+        _need(sq, "sq", torch.float32)
+        if resid.shape[-1] != N or resid.numel() < M * N or xg.shape[-1] != N or xg.numel() < M * N \
+                or sq.dim() != 2 or sq.shape[0] < M:
+            raise ValueError("gemm_blocksplit: residual buffers do not match [M, N]")
+        rp, gp, xp, qp = resid.data_ptr(), gain.data_ptr(), xg.data_ptr(), sq.data_ptr()
+        gdt, qc = dtype_code(gain.dtype), sq.shape[1]
     L = _lib.load()
-    _lib.check(L.he_gemm_blocksplit_bf16(out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K,
-                                         dtype_code(out.dtype),
-                                         dtype_code(bias.dtype) if bias is not None else F32, int(gated),
-                                         int(plan[0]), int(plan[1]), int(plan[2]), _stream()))
+    _lib.check(L.he_gemm_blocksplit_fused_bf16(
+        _ptr(out), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K,
+        dtype_code(out.dtype) if out is not None else BF16,
+        dtype_code(bias.dtype) if bias is not None else F32, int(gated),
+        int(plan[0]), int(plan[1]), int(plan[2]), sp, sc, float(se), rp, gp, gdt, xp, qp, qc,
+        _stream()))
+
+
+def scale_rows(out, x, partials, eps: float, rows: int) -> None:
+    """out = x / sqrt(sum(partials of the row) / D + eps) for rows x = r * gain (bf16)."""
+    D = x.shape[-1]
+    _need(out, "out", torch.bfloat16)
+    _need(x, "x", torch.bfloat16)
+    _need(partials, "partials", torch.float32)
+    if out.shape[-1] != D or out.numel() < rows * D or x.numel() < rows * D \
+            or partials.dim() != 2 or partials.shape[0] < rows:
+        raise ValueError("scale_rows: buffers do not match [rows, D]")
+    _lib.check(_lib.load().he_scale_rows_bf16(out.data_ptr(), x.data_ptr(), partials.data_ptr(),
+                                              partials.shape[1], rows, D, float(eps), _stream()))
 
 
 def splitk_reduce(out, partial, bias, M: int, splits: int) -> None:

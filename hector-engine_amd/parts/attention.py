@@ -23,6 +23,8 @@ from .linear import Linear, SplitSum
 
 @register_part("mixer", "attention")
 class Attention(Mixer):
+    accepts_normed_rows = True
+
     def __init__(self, params: dict, prefix: str, env: BuildEnv):
         super().__init__(prefix, env)
         self.hidden = param(params, "hidden_size", int)
@@ -106,7 +108,7 @@ class Attention(Mixer):
                                        ctx.row_seq, ctx.seq_slot, cache.page_table, rot[0], rot[1],
                                        rows, H, KVH, hd, self.window, self.scale, ctx.max_keys,
                                        writes, ws)
-            return self.o_proj(out, rows, ctx, allow_split=True)
+            return self.o_proj(out, rows, ctx, allow_split=True, sink=ctx.take_sink())
         # With a rotation (or no encoding) the bias is added inside the fused kernel;
         # any other encoding sees q and k with their bias already added.
         qkv = proj(x, rows, ctx, use_bias=not fused_bias, allow_split=fused_bias)
@@ -139,4 +141,4 @@ class Attention(Mixer):
             ops.attention_prefill(out, q, cache.kpool, cache.vpool, ctx.cu_seqlens, ctx.seq_slot,
                                   ctx.seq_start, cache.page_table, ctx.num_seqs, ctx.max_q_len,
                                   rows, H, KVH, hd, self.window, self.scale)
-        return self.o_proj(out, rows, ctx, allow_split=True)
+        return self.o_proj(out, rows, ctx, allow_split=True, sink=ctx.take_sink())

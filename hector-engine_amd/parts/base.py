@@ -115,9 +115,17 @@ class StepContext:
         self.env = env
         self.scratch = scratch            # ScratchPool: alloc(shape, dtype)
         self.host = host                  # {"q_lens", "starts", "slots"}: lists per sequence, eager steps only
+        self.want_all = False             # the wanted rows are all rows, in order
+        self.next_norm = None             # the norm that reads the stream after the running block (set by the model)
+        self.sink = None                  # ResidualSink offered to the running mixer / feed-forward
 
     def alloc(self, shape, dtype=None) -> torch.Tensor:
         return self.scratch.alloc(shape, dtype or self.env.dtype)
+
+    def take_sink(self):
+        """The residual sink offered to the running part, at most once (see ResidualSink)."""
+        sink, self.sink = self.sink, None
+        return sink
 
 
 @dataclasses.dataclass
@@ -159,6 +167,11 @@ class Part:
 
 
 class Norm(Part):
+    def carried(self) -> tuple[torch.Tensor, float] | None:
+        """(gain [D], eps) when the norm is y = x * gain / sqrt(mean(x^2) + eps), so that a
+        pair of products can carry it (ResidualSink, NormedRows); None otherwise."""
+        return None
+
     def add_norm(self, resid: torch.Tensor, delta, rows: int, ctx: StepContext,
                  want_out: bool = True) -> torch.Tensor | None:
         """resid (fp32 [rows, D], in place) += delta; returns norm(resid) in the
@@ -184,6 +197,10 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    # True for a part whose forward takes x as NormedRows as well as a tensor
+    # (its first product applies the row scale); others get a tensor.
+    accepts_normed_rows = False
+
     def kv_need(self) -> KVNeed | None:
         """Keys/values per token this mixer keeps, or None."""
         return None
@@ -199,6 +216,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    accepts_normed_rows = False
+
     def forward(self, x: torch.Tensor, ctx: StepContext):
         """Returns [rows, D], as a tensor or as the split sums of its last product."""
         raise NotImplementedError
@@ -213,6 +232,37 @@ class Block(Part):
         raise NotImplementedError
 
 
+@dataclasses.dataclass
+class NormedRows:
+    """Rows of an RMS norm whose per-row scale is still owed: `scaled` = r * gain in the
+    activation dtype, and the sum of r^2 of a row as `partials[row, :]` (fp32, added in
+    index order by lanes of 64, then across the lanes). norm(r) = scaled / sqrt(sum / dim +
+    eps). A product applies the scale to its sums (parts.linear.Linear); tensor() gives the
+    normalised rows to anything else."""
+
+    scaled: torch.Tensor
+    partials: torch.Tensor
+    eps: float
+    rows: int
+
+    def tensor(self, ctx: StepContext) -> torch.Tensor:
+        from ..kernels import ops
+        out = ctx.alloc((self.rows, self.scaled.shape[-1]), self.scaled.dtype)
+        ops.scale_rows(out, self.scaled, self.partials, self.eps, self.rows)
+        return out
+
+
+class ResidualSink:
+    """Offered (ctx.sink) to a mixer or feed-forward whose output goes straight into the
+    residual stream and then into `norm`: its last product may add its result to
+    stream.resid itself and leave the rows for that norm (Linear(..., sink=ctx.take_sink())),
+    returning None instead of a tensor. A part that ignores the offer loses nothing."""
+
+    def __init__(self, stream: "ResidualStream", norm: Norm):
+        self.stream = stream
+        self.norm = norm
+
+
 class ResidualStream:
     """The fp32 residual rows of a step plus one branch output not yet added:
     the add is fused into the next norm."""
@@ -221,14 +271,33 @@ class ResidualStream:
         self.resid = resid
         self.rows = rows
         self.pending: torch.Tensor | None = None
+        self.prepared: tuple[Norm, NormedRows] | None = None   # rows already made for that norm
 
     def add(self, delta, ctx: StepContext) -> None:
-        """delta: a tensor [rows, D] or the split sums of a product."""
+        """delta: a tensor [rows, D], the split sums of a product, or None when the
+        producer has added its result through a ResidualSink."""
+        if delta is None:
+            return
+        self.prepared = None
         if self.pending is not None:
             self.materialize(ctx)
         self.pending = delta
 
-    def normed(self, norm: Norm, ctx: StepContext) -> torch.Tensor:
+    def sink_for(self, norm: Norm | None, ctx: StepContext) -> "ResidualSink | None":
+        """A sink for the part that runs next, when `norm` (the norm that will read the stream
+        after it) can be carried and the kernels for that are in use."""
+        if norm is None or self.pending is not None or norm.carried() is None:
+            return None
+        if not ctx.env.fast_kernels or ctx.env.dtype != torch.bfloat16:
+            return None
+        return ResidualSink(self, norm)
+
+    def normed(self, norm: Norm, ctx: StepContext, rows_ok: bool = False):
+        """norm(resid + pending) in the activation dtype. With rows_ok the caller takes
+        NormedRows too (rows a product has left for this norm)."""
+        prepared, self.prepared = self.prepared, None
+        if prepared is not None and prepared[0] is norm and self.pending is None:
+            return prepared[1] if rows_ok else prepared[1].tensor(ctx)
         out = norm.add_norm(self.resid, self.pending, self.rows, ctx)
         self.pending = None
         return out

@@ -1,7 +1,9 @@
 """Arrangement of a layer: pre-norm residual block
     x = x + mixer(norm1(x));  x = x + feed_forward(norm2(x))
 (reference: src/graph_builder.cpp:1195, :1366-1374, :1396, :1443). Each
-residual add is carried as pending and fused into the next norm."""
+residual add is carried as pending and fused into the next norm, or, with few
+rows, done by the last product of the mixer / feed-forward, which then also prepares
+the rows of the norm that follows (parts.base.ResidualSink)."""
 from __future__ import annotations
 
 from .base import (Block, BuildEnv, LayerCache, PartSpec, ResidualStream, StepContext,
@@ -36,7 +38,14 @@ class PreNormBlock(Block):
             c.bind(tensors)
 
     def forward(self, stream: ResidualStream, ctx: StepContext, cache: LayerCache) -> None:
-        n = stream.normed(self.mixer_norm, ctx)
-        stream.add(self.mixer.forward(n, ctx, cache), ctx)
-        n = stream.normed(self.ff_norm, ctx)
-        stream.add(self.feed_forward.forward(n, ctx), ctx)
+        after = ctx.next_norm                  # reads the stream once this block is done
+        n = stream.normed(self.mixer_norm, ctx, self.mixer.accepts_normed_rows)
+        ctx.sink = stream.sink_for(self.ff_norm, ctx)
+        delta = self.mixer.forward(n, ctx, cache)
+        ctx.sink = None
+        stream.add(delta, ctx)
+        n = stream.normed(self.ff_norm, ctx, self.feed_forward.accepts_normed_rows)
+        ctx.sink = stream.sink_for(after, ctx)
+        delta = self.feed_forward.forward(n, ctx)
+        ctx.sink = None
+        stream.add(delta, ctx)

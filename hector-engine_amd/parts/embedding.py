@@ -37,6 +37,8 @@ class TokenEmbedding(Part):
 
 @register_part("head", "linear_head")
 class LinearHead(Part):
+    accepts_normed_rows = True
+
     def __init__(self, params: dict, prefix: str, env: BuildEnv):
         super().__init__(prefix, env)
         self.vocab = param(params, "vocab_size", int)

@@ -16,13 +16,19 @@ when a caller says `allow_split` and SPLIT_TO_CONSUMER is on, handed over as a
 :class:`SplitSum` to a kernel that adds the slices while it reads (the fused norm,
 the q/k/v kernel). That hand-over is off: with few rows the reading kernel has one
 workgroup per row and adding the slices there is slower than the small kernel.
+
+The block-split kernel also carries an RMS norm across a pair of products, so that a
+step of few rows has no norm kernels: given a :class:`ResidualSink` it adds its result
+to the residual rows itself and leaves r * gain and the sums of r^2 for the norm that
+follows (:class:`NormedRows`); given NormedRows as input it applies the owed row scale
+to its sums. Any other path turns NormedRows into a tensor first and ignores the sink.
 """
 from __future__ import annotations
 
 import torch
 
 from ..kernels import ops
-from .base import StepContext
+from .base import NormedRows, ResidualSink, StepContext
 
 
 class SplitSum:
@@ -66,14 +72,36 @@ class Linear:
         self.out_features, self.in_features = weight.shape
         self._splits: dict[int, int] = {}
 
-    def __call__(self, x: torch.Tensor, rows: int, ctx: StepContext, *, use_bias: bool = True,
+    def _blocksplit_rows(self, rows: int, ctx: StepContext, act: torch.dtype) -> bool:
+        """Whether the block-split kernel runs this product."""
+        N, K = self.weight.shape
+        return (self.weight.dtype == torch.bfloat16 and act == torch.bfloat16
+                and ctx.env.fast_kernels and K % 8 == 0
+                and 0 < rows <= (ops.BLOCKSPLIT_MAX_M if K >= LONG_K else 16))
+
+    def __call__(self, x, rows: int, ctx: StepContext, *, use_bias: bool = True,
                  out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None,
-                 allow_split: bool = False):
+                 allow_split: bool = False, sink: ResidualSink | None = None):
+        """x: a tensor or NormedRows. With a sink the result may go into the residual
+        stream directly; the call then returns None."""
         w = self.weight
         N, K = w.shape
         bias = self.bias if use_bias else None
-        act = x.dtype
+        act = x.scaled.dtype if isinstance(x, NormedRows) else x.dtype
         out_dtype = out_dtype or act
+        if self._blocksplit_rows(rows, ctx, act):
+            if sink is not None and out is None and out_dtype == act and rows <= 16 \
+                    and sink.stream.rows == rows and sink.stream.resid.shape[-1] == N:
+                return self._into_residual(x, bias, rows, ctx, sink)
+            if out is None:
+                out = ctx.alloc((rows, N), out_dtype)
+            if isinstance(x, NormedRows):
+                ops.gemm_blocksplit(out, x.scaled, w, bias, rows, row_scale=(x.partials, x.eps))
+            else:
+                ops.gemm_blocksplit(out, x, w, bias, rows)
+            return out
+        if isinstance(x, NormedRows):
+            x = x.tensor(ctx)
         if rows == 0:
             return out if out is not None else ctx.alloc((0, N), out_dtype)
         if w.dtype == torch.float32:
@@ -116,6 +144,17 @@ class Linear:
             torch.mm(x[:rows], w.t(), out=out[:rows])
         return out
 
+    def _into_residual(self, x, bias, rows, ctx, sink: ResidualSink):
+        N, K = self.weight.shape
+        gain, eps = sink.norm.carried()
+        xg = ctx.alloc((rows, N), torch.bfloat16)
+        sq = ctx.alloc((rows, ops.gemm_blocksplit_blocks(rows, N, K)), torch.float32)
+        scale = (x.partials, x.eps) if isinstance(x, NormedRows) else None
+        ops.gemm_blocksplit(None, x.scaled if scale else x, self.weight, bias, rows, row_scale=scale,
+                            residual=(sink.stream.resid, gain, xg, sq))
+        sink.stream.prepared = (sink.norm, NormedRows(xg, sq, eps, rows))
+        return None
+
     def _skinny(self, x, bias, rows, ctx, out, out_dtype, allow_split):
         N, K = self.weight.shape
         if rows <= 16 or (rows <= ops.BLOCKSPLIT_MAX_M and K >= LONG_K):
@@ -140,12 +179,17 @@ class Linear:
             return s
         return s.materialize(ctx, out_dtype, out)
 
-    def gated_silu(self, x: torch.Tensor, rows: int, ctx: StepContext, out: torch.Tensor) -> bool:
+    def gated_silu(self, x, rows: int, ctx: StepContext, out: torch.Tensor) -> bool:
         """out[rows, N/2] = silu(gate) * up in one kernel, for a weight whose rows
-        interleave gate and up in blocks of 16. False when that kernel does not apply."""
+        interleave gate and up in blocks of 16. x: a tensor or NormedRows. False when that
+        kernel does not apply."""
         w = self.weight
-        if not (ctx.env.fast_kernels and w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
+        act = x.scaled.dtype if isinstance(x, NormedRows) else x.dtype
+        if not (ctx.env.fast_kernels and w.dtype == torch.bfloat16 and act == torch.bfloat16
                 and 0 < rows <= 16 and w.shape[1] % 8 == 0 and w.shape[0] % 32 == 0):
             return False
-        ops.gemm_blocksplit(out, x, w, None, rows, gated=True)
+        if isinstance(x, NormedRows):
+            ops.gemm_blocksplit(out, x.scaled, w, None, rows, gated=True, row_scale=(x.partials, x.eps))
+        else:
+            ops.gemm_blocksplit(out, x, w, None, rows, gated=True)
         return True

@@ -17,6 +17,8 @@ _ROW_CHUNK = 8192
 
 @register_part("feed_forward", "gated_mlp")
 class GatedMLP(FeedForward):
+    accepts_normed_rows = True
+
     def __init__(self, params: dict, prefix: str, env: BuildEnv):
         super().__init__(prefix, env)
         self.hidden = param(params, "hidden_size", int)
@@ -65,7 +67,9 @@ class GatedMLP(FeedForward):
                     ops.silu_mul(h, gu.partial, rows, self.interleaved, gu.splits)
                 else:
                     ops.silu_mul(h, gu, rows, self.interleaved)
-            return self.down(h, rows, ctx, allow_split=True)
+            return self.down(h, rows, ctx, allow_split=True, sink=ctx.take_sink())
+        if not isinstance(x, torch.Tensor):
+            x = x.tensor(ctx)
         out = ctx.alloc((rows, self.hidden))
         for r0 in range(0, rows, _ROW_CHUNK):
             n = min(_ROW_CHUNK, rows - r0)

@@ -25,6 +25,9 @@ class RMSNorm(Norm):
     def bind(self, tensors):
         self.weight = tensors[self.prefix + "weight"]
 
+    def carried(self):
+        return self.weight, self.eps
+
     def add_norm(self, resid, delta, rows, ctx: StepContext, want_out: bool = True):
         out = ctx.alloc((rows, self.size)) if want_out else None
         if isinstance(delta, SplitSum):      # the K slices of a product: added while read

@@ -284,6 +284,80 @@ def test_gemm_blocksplit_gated_epilogue(ops, M, I, K, nw):
     assert (out.cpu().double() - ref).abs().max().item() <= 2 ** -8 * ref.abs().max().item() + 1e-6
 
 
+@pytest.mark.parametrize("M", [1, 8, 16])
+@pytest.mark.parametrize("D,K,N2,eps", [(80, 136, 301, 3e-6), (3584, 520, 160, 1e-6), (1000, 18944, 64, 1e-5)])
+@pytest.mark.parametrize("gain_dtype", [torch.bfloat16, torch.float32])
+def test_gemm_blocksplit_carries_the_norm(ops, M, D, K, N2, eps, gain_dtype):
+    """A product adds its result to the residual rows and leaves r * gain and the sums of
+    r^2; the next product (plain, gated) applies the owed scale: together they equal
+    add + RMS norm + product of the plain implementation, without a norm kernel."""
+    if K == 18944 and (M == 8 or gain_dtype == torch.float32):
+        pytest.skip("long K at two row counts, one gain dtype")
+    x = rnd(M, K, seed=100).to(torch.bfloat16)
+    w1 = rnd(D, K, seed=101, scale=0.05).to(torch.bfloat16)
+    b1 = rnd(D, seed=102).to(torch.bfloat16)
+    r0 = rnd(M + 1, D, seed=103, scale=3.0)
+    gain = (1 + 0.1 * rnd(D, seed=104)).to(gain_dtype)
+    blocks = ops.gemm_blocksplit_blocks(M, D, K)
+    assert blocks >= (D + 31) // 32
+    resid = dev(r0.clone())
+    xg = torch.zeros(M, D, dtype=torch.bfloat16, device="cuda")
+    sq = torch.full((M, blocks), float("nan"), device="cuda")
+    ops.gemm_blocksplit(None, dev(x), dev(w1), dev(b1), M, residual=(resid, dev(gain), xg, sq))
+    r1 = r0[:M].double() + x.double() @ w1.double().T + b1.double()
+    got_r = resid.cpu()
+    assert torch.equal(got_r[M], r0[M])                                   # the row after the last is untouched
+    assert (got_r[:M].double() - r1).abs().max().item() <= 1e-4 * r1.abs().max().item()
+    want_xg = (got_r[:M] * gain.float()).to(torch.bfloat16)
+    assert (xg.cpu().float() - want_xg.float()).abs().max().item() <= 2 ** -7 * want_xg.float().abs().max().item()
+    assert torch.allclose(sq.cpu().double().sum(1), (got_r[:M].double() ** 2).sum(1), rtol=1e-5)
+    # the consumer: scale applied to the sums, then bias
+    normed = P.rmsnorm(got_r[:M].double(), gain.double(), eps)
+    w2 = rnd(N2, D, seed=105, scale=0.05).to(torch.bfloat16)
+    b2 = rnd(N2, seed=106).to(torch.bfloat16)
+    out = torch.empty(M, N2, dtype=torch.float32, device="cuda")
+    ops.gemm_blocksplit(out, xg, dev(w2), dev(b2), M, row_scale=(sq, eps))
+    ref = normed @ w2.double().T + b2.double()
+    assert (out.cpu().double() - ref).abs().max().item() <= 2 ** -7 * ref.abs().max().item()
+    # gated consumer
+    I = N2 // 32 * 16
+    if I:
+        g, u = w2[:I], rnd(I, D, seed=107, scale=0.05).to(torch.bfloat16)
+        wi = torch.stack([g.view(I // 16, 16, D), u.view(I // 16, 16, D)], 1).reshape(2 * I, D).contiguous()
+        h = torch.empty(M, I, dtype=torch.bfloat16, device="cuda")
+        ops.gemm_blocksplit(h, xg, dev(wi), None, M, gated=True, row_scale=(sq, eps))
+        ref = P.silu(normed @ g.double().T) * (normed @ u.double().T)
+        assert (h.cpu().double() - ref).abs().max().item() <= 2 ** -6 * ref.abs().max().item() + 1e-6
+    # and as a tensor for anything that is not such a product
+    t = torch.empty(M, D, dtype=torch.bfloat16, device="cuda")
+    ops.scale_rows(t, xg, sq, eps, M)
+    assert (t.cpu().double() - normed).abs().max().item() <= 2 ** -6 * normed.abs().max().item()
+    # a chain: the consumer is itself a producer (row scale and residual epilogue together)
+    resid2 = dev(r0.clone())
+    w3 = rnd(D, D, seed=108, scale=0.05).to(torch.bfloat16)
+    blocks3 = ops.gemm_blocksplit_blocks(M, D, D)
+    xg2 = torch.zeros(M, D, dtype=torch.bfloat16, device="cuda")
+    sq2 = torch.zeros(M, blocks3, device="cuda")
+    ops.gemm_blocksplit(None, xg, dev(w3), None, M, row_scale=(sq, eps), residual=(resid2, dev(gain), xg2, sq2))
+    r2 = r0[:M].double() + normed @ w3.double().T
+    assert (resid2.cpu()[:M].double() - r2).abs().max().item() <= 2 ** -7 * r2.abs().max().item()
+    assert torch.allclose(sq2.cpu().double().sum(1), (resid2.cpu()[:M].double() ** 2).sum(1), rtol=1e-5)
+
+
+def test_gemm_blocksplit_residual_epilogue_checks_its_buffers(ops):
+    from hector_engine_amd.kernels.lib import KernelLibraryError
+    M, D, K = 4, 64, 64
+    x = torch.zeros(M, K, dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(D, K, dtype=torch.bfloat16, device="cuda")
+    resid = torch.zeros(M, D, device="cuda")
+    gain = torch.ones(D, device="cuda")
+    xg = torch.zeros(M, D, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(KernelLibraryError, match="partial sums per row"):
+        ops.gemm_blocksplit(None, x, w, None, M, residual=(resid, gain, xg, torch.zeros(M, 1, device="cuda")))
+    with pytest.raises(ValueError):
+        ops.gemm_blocksplit(None, x, w, None, M, gated=True, residual=(resid, gain, xg, torch.zeros(M, 4, device="cuda")))
+
+
 def test_gemm_skinny_refuses_bad_sizes(ops):
     from hector_engine_amd.kernels.lib import KernelLibraryError
     a = torch.zeros(2, 20, dtype=torch.bfloat16, device="cuda")
