@@ -184,13 +184,21 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
   if (to_resid && threadIdx.x < OUT_TILES * 64)
     bs_load_resid<MT>(fu, threadIdx.x, n0, M, N, res0, gain0);
 
-  // two steps of 64 U k values per turn; a step past k_end loads nothing and adds zeros
+  // two steps of 64 U k values per turn; a step past k_end loads nothing and adds zeros.
+  // The turns of a wavefront start at a point of its slice that differs from workgroup to
+  // workgroup and wrap around: workgroups that run in step then read addresses that do not
+  // all sit at the same offset of their (equally spaced) weight rows.
   BsFrags<MT, R, U> f0, f1;
-  bs_load<MT, R, U>(f0, wp, xp, k_begin, lg, k_end);
-  for (int k = k_begin; k < k_end; k += 128 * U) {
+  constexpr int TURN = 128 * U;
+  const int turns = k_end > k_begin ? (k_end - k_begin + TURN - 1) / TURN : 0;
+  int k = turns > 0 ? k_begin + (int)((blockIdx.x * 3u) % (unsigned)turns) * TURN : k_begin;
+  bs_load<MT, R, U>(f0, wp, xp, k, lg, k_end);
+  for (int j = 0; j < turns; ++j) {
     bs_load<MT, R, U>(f1, wp, xp, k + 64 * U, lg, k_end);
     bs_multiply<MT, R, U>(f0, acc);
-    bs_load<MT, R, U>(f0, wp, xp, k + 128 * U, lg, k_end);
+    k += TURN;
+    if (k >= k_end) k = k_begin;
+    if (j + 1 < turns) bs_load<MT, R, U>(f0, wp, xp, k, lg, k_end);
     bs_multiply<MT, R, U>(f1, acc);
   }
 
@@ -307,18 +315,20 @@ static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int
   p.MT = (M + 15) / 16;
   int r, u, nw;
   if (N >= 65536) {                 // output head
-    if (p.MT == 1 && M <= 4) r = 1, u = 2, nw = 16;
-    else if (p.MT == 1) r = 2, u = 4, nw = 8;
-    else r = 2, u = 2, nw = 2;
+    if (M <= 8) r = 2, u = 1, nw = 8;
+    else if (p.MT == 1) r = 4, u = 2, nw = 4;
+    else r = 2, u = 2, nw = 4;
   } else if (K >= 8192) {           // long K (down projection)
-    if (p.MT == 1) r = 1, u = 2, nw = 8;
-    else r = 1, u = 1, nw = 8;
+    r = 1, u = 1, nw = p.MT == 1 ? 8 : 4;
   } else if (N >= 16384) {          // wide N (gate||up)
-    r = 2, u = 1, nw = p.MT == 1 ? 8 : 4;
+    r = 2, u = 1, nw = 8;
+    if (p.MT == 2) u = 2, nw = 4;
   } else {                          // small products (q||k||v, o)
-    r = 1, u = 1, nw = p.MT == 1 ? 16 : 8;
+    r = N >= 4096 ? 2 : 1;
+    u = p.MT == 1 ? 4 : 1;
+    nw = 8;
   }
-  if (gated) r = 2, u = u > 2 ? 2 : u;
+  if (gated && (r & 1)) r = 2;
   p.R = R > 0 ? R : r;
   p.U = U > 0 ? U : u;
   if (NW <= 0) {
@@ -354,7 +364,7 @@ static int dispatch_blocksplit(const BlockSplitPlan& p, void* C, const void* X, 
   if (!GATED) {
     BS(1, 1, 1) BS(1, 1, 2) BS(1, 1, 4) BS(2, 1, 1) BS(2, 1, 2)
   }
-  BS(1, 2, 1) BS(1, 2, 2) BS(1, 2, 4) BS(2, 2, 1) BS(2, 2, 2)
+  BS(1, 2, 1) BS(1, 2, 2) BS(1, 2, 4) BS(2, 2, 1) BS(2, 2, 2) BS(1, 4, 1) BS(1, 4, 2)
 #undef BS
   he_set_error("he_gemm_blocksplit_bf16: no kernel for MT=%d R=%d U=%d", p.MT, p.R, p.U);
   return -1;
@@ -392,7 +402,7 @@ extern "C" int he_gemm_blocksplit_fused_bf16(void* C, const void* A, const void*
   const BlockSplitPlan p = blocksplit_plan(M, N, K, gated, R, U, NW);
   HE_REQUIRE(p.NW >= 1 && p.NW <= 16, "he_gemm_blocksplit_bf16: %d wavefronts outside [1, 16]",
              p.NW);
-  HE_REQUIRE(!gated || p.R == 2, "he_gemm_blocksplit_bf16: the gated epilogue needs R = 2");
+  HE_REQUIRE(!gated || (p.R & 1) == 0, "he_gemm_blocksplit_bf16: the gated epilogue needs an even R");
   const int blocks = (N + 16 * p.R - 1) / (16 * p.R);
   if (resid != nullptr) {
     HE_REQUIRE(!gated && gain != nullptr && xg != nullptr && sq_out != nullptr,
