@@ -54,6 +54,8 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=FULL_LAYERS)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points")
+    ap.add_argument("--no-tune", action="store_true",
+                    help="leave the library's default kernels for the tall matrix products")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
@@ -69,7 +71,7 @@ def main() -> int:
     max_batch = args.batch if args.no_points else max(args.batch, 64)
     t_load = time.perf_counter()
     engine = he.Engine(config=config, seed=0, dtype="bfloat16", max_tokens=max_batch * CONTEXT,
-                       max_slots=max_batch, max_seq_len=CONTEXT)
+                       max_slots=max_batch, max_seq_len=CONTEXT, tune_library=not args.no_tune)
     sampler = he.Sampler(he.SamplingConfig.deterministic(), engine.device)
     torch.cuda.synchronize()
     load_s = time.perf_counter() - t_load
@@ -156,6 +158,7 @@ def main() -> int:
             "rope_theta": SHAPE["rope_theta"], "rms_norm_eps": SHAPE["rms_norm_eps"],
             "global_batch": args.batch, "seq_len": CONTEXT, "prompt_len": PROMPT,
             "parallelism": "single GPU", "sampling": "greedy", "load_s": round(load_s, 1),
+            "library_gemm_autotuned": not args.no_tune,
         },
         "prefill": {"value": round(PROMPT / prefill_s, 1), "tokens": PROMPT,
                     "ms": round(prefill_s * 1e3, 3),

@@ -58,6 +58,9 @@ def parse_args(argv: list[str]):
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--stop-ids", default=None, help="comma-separated stop token ids")
     ap.add_argument("--no-graph", action="store_true", help="run one-token steps without HIP graphs")
+    ap.add_argument("--tune-gemm", action="store_true",
+                    help="let the library's autotuner choose the kernels of tall matrix products (a second or so "
+                         "per new shape)")
     ap.add_argument("rest", nargs="*")
     ns = ap.parse_args(argv)
     rest = list(ns.rest)
@@ -102,7 +105,7 @@ def main(argv: list[str] | None = None) -> int:
     pages = max(1, len(prompts)) * ((ctx + 63) // 64)
     start = time.perf_counter()
     engine = he.Engine(model, dtype=ns.dtype, max_tokens=pages * 64, max_slots=max(1, len(prompts)),
-                       max_seq_len=ctx, use_graphs=not ns.no_graph)
+                       max_seq_len=ctx, use_graphs=not ns.no_graph, tune_library=ns.tune_gemm)
     print(f"Model: {model}  ({config.architecture}, {ns.dtype})  loaded in "
           f"{(time.perf_counter() - start) * 1e3:.0f} ms")
     t0 = time.perf_counter()

@@ -22,6 +22,7 @@ from ..cache.paged import PagedCache
 from ..cache.pages import CacheError, CacheFull  # noqa: F401
 from ..config.base import ModelConfig
 from ..kernels import lib as kernel_lib
+from ..kernels import library_tuning
 from ..parts.base import BuildEnv, StepContext
 from ..registry import build_model, load_config
 from ..weights.loader import load_tensors
@@ -79,7 +80,10 @@ class Engine:
     def __init__(self, model_dir: str | None = None, *, config: ModelConfig | None = None,
                  seed: int | None = None, dtype: str = "bfloat16", max_tokens: int = 8192,
                  max_slots: int | None = None, max_seq_len: int | None = None,
-                 device: str = "cuda:0", fast_kernels: bool = True, use_graphs: bool = True):
+                 device: str = "cuda:0", fast_kernels: bool = True, use_graphs: bool = True,
+                 tune_library: bool = False):
+        """tune_library: let the library's autotuner choose the kernel of each tall bfloat16
+        matrix product the first time its shape is seen (kernels/library_tuning.py)."""
         if dtype not in _DTYPES:
             raise ValueError(f"dtype must be one of {sorted(_DTYPES)}, got {dtype!r}")
         if not torch.cuda.is_available():
@@ -93,6 +97,8 @@ class Engine:
             # reduced-precision mode could slip in through torch either
             torch.backends.cuda.matmul.allow_tf32 = False
         self.env = BuildEnv(self.device, self.dtype, fast_kernels)
+        if tune_library and self.dtype == torch.bfloat16:
+            library_tuning.enable()
         if model_dir is not None:
             self.config = load_config(model_dir)
         elif config is not None:
@@ -272,7 +278,7 @@ class Engine:
             bucket.pool.frozen = True
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
+            with library_tuning.no_new_tuning(), torch.cuda.graph(graph):
                 bucket.pool.reset()
                 bucket.logits = self.model.forward(bucket.views["tokens"], ctx, self.caches,
                                                    bucket.views["want_rows"], size)

@@ -1,0 +1,56 @@
+"""The library matrix product's own autotuner (torch's TunableOp over hipBLASLt / rocBLAS).
+
+Tall products (more rows than the hand-written kernels take) go to the library, as the
+reference sends every product to its BLAS library (kernels/matmul_cublas.cu:240-277).
+The library's default choice of kernel is not always its best on MI355X: at the
+Qwen2.5-7B shapes its tuner finds kernels 17-27 % faster for the 2048-row down and
+gate||up products and 20 % faster for gate||up at 64 rows. Tuning runs the first time a
+shape (rows, N, K) is seen and takes a second or so per shape, so it is meant for
+workloads whose shapes repeat (decode buckets, fixed prompt chunks); it is off unless
+asked for. Results are kept in a file and read again by the next process.
+"""
+from __future__ import annotations
+
+import contextlib
+import os
+import tempfile
+
+import torch
+
+_enabled = False
+
+
+def results_path() -> str:
+    folder = os.path.join(tempfile.gettempdir(), f"hector-engine_amd-{os.getuid()}")
+    os.makedirs(folder, exist_ok=True)
+    return os.path.join(folder, "library_gemm_tuning.csv")
+
+
+def enable(max_seconds_per_shape: int = 30, max_iterations: int = 10) -> None:
+    global _enabled
+    t = torch.cuda.tunable
+    t.set_filename(results_path())
+    t.enable(True)
+    t.tuning_enable(True)
+    t.set_max_tuning_duration(max_seconds_per_shape)
+    t.set_max_tuning_iterations(max_iterations)
+    _enabled = True
+
+
+def enabled() -> bool:
+    return _enabled
+
+
+@contextlib.contextmanager
+def no_new_tuning():
+    """Inside: tuned choices are used, but no shape is tuned (graph capture cannot hold the
+    tuner's timing runs)."""
+    if not _enabled:
+        yield
+        return
+    t = torch.cuda.tunable
+    t.tuning_enable(False)
+    try:
+        yield
+    finally:
+        t.tuning_enable(True)
