@@ -90,18 +90,176 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 }
 
 // ------------------------------------------------------------------ prefill, K/V through LDS
-// grid (ceil(max_q_len / 128), H, num_seqs), 512 threads. The workgroup takes 128
-// consecutive queries of one sequence and head, wave w the 16 queries 16w..16w+15. The
-// keys are walked a page (64 keys) at a time: the page's K and V^T are copied once into
-// LDS, already in the order the MFMA operands are read (one operand of all 64 lanes is
-// one contiguous KiB, so the reads have no bank conflicts), every wave builds its
-// operands from there, and the next page is already on its way into registers while the
-// current one is used. Head sizes up to 128.
-#define PF_WAVES 8
-#define PF_QUERIES (16 * PF_WAVES)
+// grid (ceil(max_q_len / 128), H, num_seqs), 256 threads. The workgroup takes 128
+// consecutive queries of one sequence and head, wavefront w the 32 queries 32w..32w+31 as
+// two tiles. The keys are walked a page (64 keys) at a time: the page's K and V^T are copied
+// once into LDS, already in the order the MFMA operands are read (one operand of all 64
+// lanes is one contiguous KiB, so the reads have no bank conflicts), and every operand a
+// wavefront reads from LDS feeds two MFMAs, one per tile - with one tile a wavefront the LDS
+// reads (32 KiB a page and wavefront), not the matrix cores, set the pace. The page in LDS
+// is double-buffered: the next page is written into the other buffer while this one is
+// used, one barrier a page; the page after that is on its way into registers meanwhile.
+// Head sizes up to 128. The staging arrays are native vectors: arrays of the uint4 struct
+// are not kept in registers by the compiler (it moves them to LDS or scratch).
+#define PF2_WAVES 4
+#define PF2_QUERIES (32 * PF2_WAVES)
+
+// Online softmax of one tile's scores of a step of 32 keys (see attend_frag); returns P^T
+// as the B operand of the value product.
+template <int NT, bool MASK>
+__device__ __forceinline__ bf16x8 softmax_step(AttnState<NT>& st, const floatx4* s, int key_base,
+                                               int lo, int hi, float scale_log2, int lg) {
+  float p[2][4];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float v = s[t][r] * scale_log2;
+      if (MASK) {
+        const int key = key_base + 8 * lg + 4 * t + r;
+        v = (key >= lo && key <= hi) ? v : -INFINITY;
+      }
+      p[t][r] = v;
+      mx = fmaxf(mx, v);
+    }
+  mx = fmaxf(mx, __shfl_xor(mx, 16, HE_WAVE));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, HE_WAVE));
+  const float m_new = fmaxf(st.m, mx);
+  const bool moved = __builtin_amdgcn_ballot_w64(m_new != st.m) != 0;   // wave-uniform
+  const float m_use = m_new == -INFINITY ? 0.f : m_new;
+  float sum = 0.f;
+  uint32_t packed[4];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int r = 0; r < 4; r += 2) {
+      const float e0 = __builtin_amdgcn_exp2f(p[t][r] - m_use);
+      const float e1 = __builtin_amdgcn_exp2f(p[t][r + 1] - m_use);
+      sum += e0 + e1;
+      packed[2 * t + (r >> 1)] = pack2_bf16(e0, e1);
+    }
+  if (moved) {
+    const float alpha = __builtin_amdgcn_exp2f(st.m - m_use);
+    st.l = st.l * alpha + sum;
+    st.m = m_new;
+#pragma unroll
+    for (int dt = 0; dt < NT; ++dt) st.o[dt] *= alpha;
+  } else {
+    st.l += sum;
+  }
+  return __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
+}
+
+typedef uint32_t pf2_vec __attribute__((ext_vector_type(4)));   // 16 bytes, a native vector
+
+// A page of K and of V^T of one kv head, global memory -> registers (16-byte chunks, one
+// per thread and turn) -> LDS in operand order.
 template <int NT>
-__global__ __launch_bounds__(64 * PF_WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void
-attention_prefill_lds_kernel(
+struct Pf2 {
+  static constexpr int HD = 16 * NT;
+  static constexpr int KS = (HD + 31) / 32;
+  static constexpr int CHUNKS = HE_PAGE_TOKENS * HD / 8;
+  static constexpr int THREADS = 64 * PF2_WAVES;
+  static constexpr int PER_THREAD = (CHUNKS + THREADS - 1) / THREADS;
+};
+
+template <int NT>
+__device__ __forceinline__ void pf2_fetch(pf2_vec (&kreg)[Pf2<NT>::PER_THREAD],
+                                          pf2_vec (&vreg)[Pf2<NT>::PER_THREAD],
+                                          const uint16_t* __restrict__ kp,
+                                          const uint16_t* __restrict__ vp, int page, int num_pages,
+                                          int64_t page_stride) {
+  if (page < 0 || page >= num_pages) page = 0;   // never for an admitted batch
+#pragma unroll
+  for (int j = 0; j < Pf2<NT>::PER_THREAD; ++j) {
+    const int c = threadIdx.x + Pf2<NT>::THREADS * j;
+    if (c < Pf2<NT>::CHUNKS) {
+      kreg[j] = *reinterpret_cast<const pf2_vec*>(kp + (int64_t)page * page_stride + 8 * c);
+      vreg[j] = *reinterpret_cast<const pf2_vec*>(vp + (int64_t)page * page_stride + 8 * c);
+    }
+  }
+}
+
+template <int NT>
+__device__ __forceinline__ void pf2_stage(const pf2_vec (&kreg)[Pf2<NT>::PER_THREAD],
+                                          const pf2_vec (&vreg)[Pf2<NT>::PER_THREAD], pf2_vec* k_lds,
+                                          pf2_vec* v_lds) {
+  constexpr int HD = Pf2<NT>::HD, KS = Pf2<NT>::KS;
+#pragma unroll
+  for (int j = 0; j < Pf2<NT>::PER_THREAD; ++j) {
+    const int c = threadIdx.x + Pf2<NT>::THREADS * j;
+    if (c < Pf2<NT>::CHUNKS) {
+      // K chunk: key krow, dims 8*kcol..+8 -> operand (half, tile, k step) and its lane
+      const int krow = c / (HD / 8), kcol = c % (HD / 8);
+      const int kl = krow & 31;
+      const int klane = 16 * (kcol & 3) + (((kl >> 3) << 2) | (kl & 3));
+      k_lds[(((krow >> 5) * 2 + ((kl >> 2) & 1)) * KS + (kcol >> 2)) * 64 + klane] = kreg[j];
+      // V^T chunk: dim vrow, keys 8*vcol..+8 -> operand (half, dim tile) and its lane
+      const int vrow = c / (HE_PAGE_TOKENS / 8), vcol = c % (HE_PAGE_TOKENS / 8);
+      v_lds[((vcol >> 2) * NT + (vrow >> 4)) * 64 + 16 * (vcol & 3) + (vrow & 15)] = vreg[j];
+    }
+  }
+}
+
+// One tile of 16 queries (a query per column) of such a wavefront.
+template <int NT>
+struct PairTile {
+  static constexpr int HD = 16 * NT;
+  static constexpr int KS = (HD + 31) / 32;
+  bf16x8 qf[KS];
+  AttnState<NT> st;
+  int qi, hi, lo, clear_lo, clear_hi;
+  bool ok;
+
+  __device__ __forceinline__ void init(const uint16_t* __restrict__ q, int row0, int q_len,
+                                       int start, int qt, int H, int h, int window, int lr,
+                                       int lg) {
+    qi = qt + lr;
+    ok = qi < q_len;
+    const int pos = start + qi;
+    hi = ok ? pos : -1;
+    lo = (window > 0 && ok) ? max(0, pos + 1 - window) : 0;
+    load_q<NT>(qf, q + ((int64_t)(row0 + min(qi, q_len - 1)) * H + h) * HD, ok, lg);
+#pragma unroll
+    for (int dt = 0; dt < NT; ++dt) st.o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    st.m = -INFINITY;
+    st.l = 0.f;
+    // keys every query of a full tile sees: from its last query's window start to its first
+    // query's position
+    const int tlast = start + min(qt + 15, q_len - 1);
+    clear_lo = window > 0 ? max(0, tlast + 1 - window) : 0;
+    clear_hi = qt + 15 < q_len ? start + qt : -1;
+  }
+
+  __device__ __forceinline__ bf16x8 softmax(const floatx4* s, int key_base, float scale_log2,
+                                            int lg) {
+    if (key_base >= clear_lo && key_base + 31 <= clear_hi)
+      return softmax_step<NT, false>(st, s, key_base, lo, hi, scale_log2, lg);
+    return softmax_step<NT, true>(st, s, key_base, lo, hi, scale_log2, lg);
+  }
+
+  __device__ __forceinline__ void store(uint16_t* __restrict__ out, int row0, int H, int h, int lr,
+                                        int lg) {
+    float l = st.l;
+    l += __shfl_xor(l, 16, HE_WAVE);
+    l += __shfl_xor(l, 32, HE_WAVE);
+    if (!ok) return;
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    uint16_t* orow = out + ((int64_t)(row0 + qi) * H + h) * HD;
+#pragma unroll
+    for (int dt = 0; dt < NT; ++dt) {
+      uint2 w;
+      w.x = pack2_bf16(st.o[dt][0] * inv, st.o[dt][1] * inv);
+      w.y = pack2_bf16(st.o[dt][2] * inv, st.o[dt][3] * inv);
+      *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * lg) = w;
+    }
+  }
+};
+
+template <int NT>
+__global__ __launch_bounds__(64 * PF2_WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void
+attention_prefill_pair_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q,
     const uint16_t* __restrict__ kpool, const uint16_t* __restrict__ vpool,
     const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_slot,
@@ -110,11 +268,12 @@ attention_prefill_lds_kernel(
   constexpr int HD = 16 * NT;
   constexpr int KS = (HD + 31) / 32;
   constexpr int CHUNKS = HE_PAGE_TOKENS * HD / 8;   // 16-byte chunks of one page of K (or V^T)
-  constexpr int THREADS = 64 * PF_WAVES;
+  constexpr int THREADS = 64 * PF2_WAVES;
   constexpr int PER_THREAD = (CHUNKS + THREADS - 1) / THREADS;
-  // operand-ordered: k_lds[((hb*2 + t)*KS + ks)*64 + lane], v_lds[(hb*NT + dt)*64 + lane]
-  __shared__ uint4 k_lds[2 * 2 * KS * 64];
-  __shared__ uint4 v_lds[2 * NT * 64];
+  constexpr int K_OPS = 2 * 2 * KS * 64, V_OPS = 2 * NT * 64;   // uint4 per buffer
+  // operand-ordered: k[((hb*2 + t)*KS + ks)*64 + lane], v[(hb*NT + dt)*64 + lane]
+  __shared__ pf2_vec k_lds[2][K_OPS];
+  __shared__ pf2_vec v_lds[2][V_OPS];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int lr = lane & 15, lg = lane >> 4;
@@ -123,8 +282,13 @@ attention_prefill_lds_kernel(
   if (slot < 0) return;
   const int row0 = cu_seqlens[seq];
   const int q_len = cu_seqlens[seq + 1] - row0;
-  // long workgroups first: the last queries of a sequence have the most keys
-  const int qb = PF_QUERIES * (gridDim.x - 1 - blockIdx.x);
+  // Long workgroups first: the last queries of a sequence have the most keys. Workgroups
+  // are handed to the compute units in rounds of 256 (one per unit); every other round runs
+  // from short to long, so that a unit that got a long one in one round gets a short one in
+  // the next - with two resident per unit, the pairs then do equal work.
+  const unsigned linear = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+  const int qslot = ((linear >> 8) & 1) ? (int)blockIdx.x : (int)(gridDim.x - 1 - blockIdx.x);
+  const int qb = PF2_QUERIES * qslot;
   if (qb >= q_len) return;
   const int start = seq_start[seq];
   const int kvh = h / (H / KVH);
@@ -133,110 +297,64 @@ attention_prefill_lds_kernel(
   const uint16_t* kp = kpool + (int64_t)kvh * (HE_PAGE_TOKENS * HD);
   const uint16_t* vp = vpool + (int64_t)kvh * (HE_PAGE_TOKENS * HD);
 
-  const int qw = qb + 16 * wave;                 // this wave's 16 queries
+  const int qw = qb + 32 * wave;                 // this wave's 32 queries: tiles qw and qw + 16
   const bool wave_ok = qw < q_len;
-  const int qi = qw + lr;
-  const bool q_ok = qi < q_len;
-  const int pos = start + qi;
-  const int hi = q_ok ? pos : -1;
-  const int lo = (window > 0 && q_ok) ? max(0, pos + 1 - window) : 0;
-  bf16x8 qf[KS];
-  load_q<NT>(qf, q + ((int64_t)(row0 + min(qi, q_len - 1)) * H + h) * HD, q_ok, lg);
-  AttnState<NT> st;
-#pragma unroll
-  for (int dt = 0; dt < NT; ++dt) st.o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
-  st.m = -INFINITY;
-  st.l = 0.f;
-  const int wlast = start + min(qw + 15, q_len - 1);            // last position this wave sees
+  PairTile<NT> t0, t1;
+  t0.init(q, row0, q_len, start, qw, H, h, window, lr, lg);
+  t1.init(q, row0, q_len, start, qw + 16, H, h, window, lr, lg);
+  const int wlast = start + min(qw + 31, q_len - 1);            // last position this wave sees
   const int wfirst = window > 0 ? max(0, start + qw + 1 - window) : 0;
-  // keys every query of a full tile sees: from the last query's window start to the first
-  // query's position
-  const int clear_lo = window > 0 ? max(0, wlast + 1 - window) : 0;
-  const int clear_hi = qw + 15 < q_len ? start + qw : -1;
   const float scale_log2 = scale * 1.4426950408889634f;
 
-  const int blk_last = start + min(qb + PF_QUERIES - 1, q_len - 1);
+  const int blk_last = start + min(qb + PF2_QUERIES - 1, q_len - 1);
   const int blk_first = window > 0 ? max(0, start + qb + 1 - window) : 0;
   const int pb0 = blk_first >> HE_PAGE_SHIFT, pb1 = blk_last >> HE_PAGE_SHIFT;
 
-  uint4 kreg[PER_THREAD], vreg[PER_THREAD];
-  int page = pt[pb0];
-  if (page < 0 || page >= num_pages) page = 0;   // never for an admitted batch
-#pragma unroll
-  for (int j = 0; j < PER_THREAD; ++j) {
-    const int c = threadIdx.x + THREADS * j;
-    if (c < CHUNKS) {
-      kreg[j] = *reinterpret_cast<const uint4*>(kp + (int64_t)page * page_stride + 8 * c);
-      vreg[j] = *reinterpret_cast<const uint4*>(vp + (int64_t)page * page_stride + 8 * c);
-    }
-  }
+  pf2_vec kreg[PER_THREAD], vreg[PER_THREAD];
+  pf2_fetch<NT>(kreg, vreg, kp, vp, pt[pb0], num_pages, page_stride);
+  pf2_stage<NT>(kreg, vreg, k_lds[0], v_lds[0]);
+  if (pb0 < pb1) pf2_fetch<NT>(kreg, vreg, kp, vp, pt[pb0 + 1], num_pages, page_stride);
+  __syncthreads();
   for (int pb = pb0; pb <= pb1; ++pb) {
-    __syncthreads();   // everyone is done with the page in LDS
+    const int buf = (pb - pb0) & 1;
+    if (pb < pb1) {
+      // everyone left the other buffer before the last barrier
+      pf2_stage<NT>(kreg, vreg, k_lds[buf ^ 1], v_lds[buf ^ 1]);
+      if (pb + 1 < pb1) pf2_fetch<NT>(kreg, vreg, kp, vp, pt[pb + 2], num_pages, page_stride);
+    }
+    const int page_lo = pb << HE_PAGE_SHIFT;
+    if (wave_ok && page_lo <= wlast && page_lo + HE_PAGE_TOKENS - 1 >= wfirst) {
 #pragma unroll
-    for (int j = 0; j < PER_THREAD; ++j) {
-      const int c = threadIdx.x + THREADS * j;
-      if (c < CHUNKS) {
-        // K chunk: key krow, dims 8*kcol..+8 -> operand (half, tile, k step) and its lane
-        const int krow = c / (HD / 8), kcol = c % (HD / 8);
-        const int kl = krow & 31;
-        const int klane = 16 * (kcol & 3) + (((kl >> 3) << 2) | (kl & 3));
-        k_lds[(((krow >> 5) * 2 + ((kl >> 2) & 1)) * KS + (kcol >> 2)) * 64 + klane] = kreg[j];
-        // V^T chunk: dim vrow, keys 8*vcol..+8 -> operand (half, dim tile) and its lane
-        const int vrow = c / (HE_PAGE_TOKENS / 8), vcol = c % (HE_PAGE_TOKENS / 8);
-        v_lds[((vcol >> 2) * NT + (vrow >> 4)) * 64 + 16 * (vcol & 3) + (vrow & 15)] = vreg[j];
+      for (int hb = 0; hb < 2; ++hb) {
+        const int key_base = page_lo + 32 * hb;
+        if (key_base > wlast || key_base + 31 < wfirst) continue;
+        floatx4 s0[2], s1[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) s0[t] = s1[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            pf2_vec v = {0u, 0u, 0u, 0u};
+            if (32 * ks + 8 * lg < HD) v = k_lds[buf][((hb * 2 + t) * KS + ks) * 64 + lane];
+            const bf16x8 kf = __builtin_bit_cast(bf16x8, v);
+            s0[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, t0.qf[ks], s0[t], 0, 0, 0);
+            s1[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, t1.qf[ks], s1[t], 0, 0, 0);
+          }
+        const bf16x8 p0 = t0.softmax(s0, key_base, scale_log2, lg);
+        const bf16x8 p1 = t1.softmax(s1, key_base, scale_log2, lg);
+#pragma unroll
+        for (int dt = 0; dt < NT; ++dt) {
+          const bf16x8 vf = __builtin_bit_cast(bf16x8, v_lds[buf][(hb * NT + dt) * 64 + lane]);
+          t0.st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p0, t0.st.o[dt], 0, 0, 0);
+          t1.st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p1, t1.st.o[dt], 0, 0, 0);
+        }
       }
     }
     __syncthreads();
-    if (pb < pb1) {   // the next page is fetched while this one is used
-      page = pt[pb + 1];
-      if (page < 0 || page >= num_pages) page = 0;
-#pragma unroll
-      for (int j = 0; j < PER_THREAD; ++j) {
-        const int c = threadIdx.x + THREADS * j;
-        if (c < CHUNKS) {
-          kreg[j] = *reinterpret_cast<const uint4*>(kp + (int64_t)page * page_stride + 8 * c);
-          vreg[j] = *reinterpret_cast<const uint4*>(vp + (int64_t)page * page_stride + 8 * c);
-        }
-      }
-    }
-    const int page_lo = pb << HE_PAGE_SHIFT;
-    if (!wave_ok || page_lo > wlast || page_lo + HE_PAGE_TOKENS - 1 < wfirst) continue;
-#pragma unroll
-    for (int hb = 0; hb < 2; ++hb) {
-      const int key_base = page_lo + 32 * hb;
-      if (key_base > wlast || key_base + 31 < wfirst) continue;
-      KVFrag<NT> f;
-      f.ok = 1;
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          uint4 v = make_uint4(0, 0, 0, 0);
-          if (32 * ks + 8 * lg < HD) v = k_lds[((hb * 2 + t) * KS + ks) * 64 + lane];
-          f.k[t][ks] = __builtin_bit_cast(bf16x8, v);
-        }
-#pragma unroll
-      for (int dt = 0; dt < NT; ++dt)
-        f.v[dt] = __builtin_bit_cast(bf16x8, v_lds[(hb * NT + dt) * 64 + lane]);
-      if (key_base >= clear_lo && key_base + 31 <= clear_hi)
-        attend_frag<NT, false>(st, qf, f, key_base, lo, hi, scale_log2, lg);
-      else
-        attend_frag<NT, true>(st, qf, f, key_base, lo, hi, scale_log2, lg);
-    }
   }
-  float l = st.l;
-  l += __shfl_xor(l, 16, HE_WAVE);
-  l += __shfl_xor(l, 32, HE_WAVE);
-  if (!q_ok) return;
-  const float inv = l > 0.f ? 1.f / l : 0.f;
-  uint16_t* orow = out + ((int64_t)(row0 + qi) * H + h) * HD;
-#pragma unroll
-  for (int dt = 0; dt < NT; ++dt) {
-    uint2 w;
-    w.x = pack2_bf16(st.o[dt][0] * inv, st.o[dt][1] * inv);
-    w.y = pack2_bf16(st.o[dt][2] * inv, st.o[dt][3] * inv);
-    *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * lg) = w;
-  }
+  t0.store(out, row0, H, h, lr, lg);
+  t1.store(out, row0, H, h, lr, lg);
 }
 
 // ------------------------------------------------------------------ decode
@@ -492,7 +610,7 @@ extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* k
     dim3 grid128((max_q_len + 127) / 128, H, num_seqs);
 #define PREFILL_LDS(NTV)                                                                        \
   case NTV:                                                                                     \
-    attention_prefill_lds_kernel<NTV><<<grid128, 64 * PF_WAVES, 0, s>>>(                                  \
+    attention_prefill_pair_kernel<NTV><<<grid128, 64 * PF2_WAVES, 0, s>>>(                      \
         (uint16_t*)out, (const uint16_t*)q, (const uint16_t*)kpool, (const uint16_t*)vpool,     \
         (const int32_t*)cu_seqlens, (const int32_t*)seq_slot, (const int32_t*)seq_start,        \
         (const int32_t*)page_table, max_blocks, num_pages, H, KVH, window, scale);              \
