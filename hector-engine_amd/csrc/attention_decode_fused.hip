@@ -155,8 +155,7 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
                             scale * 1.4426950408889634f, lr, lg);
   }
   float l = st.l;
-  l += __shfl_xor(l, 16, HE_WAVE);
-  l += __shfl_xor(l, 32, HE_WAVE);
+  l = xor32_sum(xor16_sum(l));
 
   // ---- join the slices through LDS, in wavefront order
   float* lds_o = lds;
@@ -255,6 +254,7 @@ extern "C" int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_
                                               void* stream) {
   HE_REQUIRE(rows >= 0 && H > 0 && KVH > 0 && hd > 0 && max_keys > 0,
              "he_attention_decode_fused_bf16: bad sizes");
+  HE_REQUIRE(scale > 0.f, "he_attention_decode_fused_bf16: the score scale must be positive");
   HE_REQUIRE(he_attention_decode_fused_ok(H, KVH, hd, rotary_dim),
              "he_attention_decode_fused_bf16: sizes H=%d KVH=%d head_dim=%d rotary_dim=%d are not "
              "taken (head_dim 64 or 128, rotated whole)", H, KVH, hd, rotary_dim);

@@ -75,8 +75,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
                    (last_pos & ~31) + 32, lo, hi, clear_lo, clear_hi, scale * 1.4426950408889634f,
                    lr, lg);
   float l = st.l;
-  l += __shfl_xor(l, 16, HE_WAVE);
-  l += __shfl_xor(l, 32, HE_WAVE);
+  l = xor32_sum(xor16_sum(l));
   if (!q_ok) return;
   const float inv = l > 0.f ? 1.f / l : 0.f;
   uint16_t* orow = out + ((int64_t)(row0 + qi) * H + h) * HD;
@@ -109,13 +108,15 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 template <int NT, bool MASK>
 __device__ __forceinline__ bf16x8 softmax_step(AttnState<NT>& st, const floatx4* s, int key_base,
                                                int lo, int hi, float scale_log2, int lg) {
+  // raw scores (masked ones at -inf), their maximum, then p = 2^(raw * scale - m) with the
+  // scale folded into the subtraction (scale > 0, so the maximum commutes with it)
   float p[2][4];
   float mx = -INFINITY;
 #pragma unroll
   for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      float v = s[t][r] * scale_log2;
+      float v = s[t][r];
       if (MASK) {
         const int key = key_base + 8 * lg + 4 * t + r;
         v = (key >= lo && key <= hi) ? v : -INFINITY;
@@ -123,9 +124,10 @@ __device__ __forceinline__ bf16x8 softmax_step(AttnState<NT>& st, const floatx4*
       p[t][r] = v;
       mx = fmaxf(mx, v);
     }
-  mx = fmaxf(mx, __shfl_xor(mx, 16, HE_WAVE));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, HE_WAVE));
-  const float m_new = fmaxf(st.m, mx);
+  mx = xor32_max(xor16_max(mx)) * scale_log2;
+  // the reference point follows the maximum only when that has grown by more than
+  // 2^HE_SOFTMAX_SLACK: p stays below that factor, and the accumulators are rarely rescaled
+  const float m_new = mx > st.m + HE_SOFTMAX_SLACK ? mx : st.m;
   const bool moved = __builtin_amdgcn_ballot_w64(m_new != st.m) != 0;   // wave-uniform
   const float m_use = m_new == -INFINITY ? 0.f : m_new;
   float sum = 0.f;
@@ -134,8 +136,8 @@ __device__ __forceinline__ bf16x8 softmax_step(AttnState<NT>& st, const floatx4*
   for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int r = 0; r < 4; r += 2) {
-      const float e0 = __builtin_amdgcn_exp2f(p[t][r] - m_use);
-      const float e1 = __builtin_amdgcn_exp2f(p[t][r + 1] - m_use);
+      const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(p[t][r], scale_log2, -m_use));
+      const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(p[t][r + 1], scale_log2, -m_use));
       sum += e0 + e1;
       packed[2 * t + (r >> 1)] = pack2_bf16(e0, e1);
     }
@@ -164,6 +166,9 @@ struct Pf2 {
   static constexpr int PER_THREAD = (CHUNKS + THREADS - 1) / THREADS;
 };
 
+__device__ __forceinline__ int pf2_kx(int ks, int a) { return ((ks & 3) << 2) | a; }
+__device__ __forceinline__ int pf2_vx(int hb, int a) { return (hb << 3) | (a << 1); }
+
 template <int NT>
 __device__ __forceinline__ void pf2_fetch(pf2_vec (&kreg)[Pf2<NT>::PER_THREAD],
                                           pf2_vec (&vreg)[Pf2<NT>::PER_THREAD],
@@ -181,23 +186,42 @@ __device__ __forceinline__ void pf2_fetch(pf2_vec (&kreg)[Pf2<NT>::PER_THREAD],
   }
 }
 
+// Where the chunks of this thread go in LDS. An operand (64 lanes x 16 bytes) is one KiB;
+// inside it, lane 16a + c sits at slot 16a + (c ^ x), x chosen per operand and a so that the
+// 16 chunks that neighbouring threads store at once (one key row, or two rows of V^T) fall
+// into 16 different 16-byte columns of the 256-byte bank row, as the 16 lanes of one read do.
+// Without it the stores of a wavefront hit 4 columns (K) or 2 (V^T) and serialise.
 template <int NT>
-__device__ __forceinline__ void pf2_stage(const pf2_vec (&kreg)[Pf2<NT>::PER_THREAD],
-                                          const pf2_vec (&vreg)[Pf2<NT>::PER_THREAD], pf2_vec* k_lds,
-                                          pf2_vec* v_lds) {
+__device__ __forceinline__ void pf2_slots(int (&kdst)[Pf2<NT>::PER_THREAD],
+                                          int (&vdst)[Pf2<NT>::PER_THREAD]) {
   constexpr int HD = Pf2<NT>::HD, KS = Pf2<NT>::KS;
 #pragma unroll
   for (int j = 0; j < Pf2<NT>::PER_THREAD; ++j) {
     const int c = threadIdx.x + Pf2<NT>::THREADS * j;
+    // K chunk: key krow, dims 8*kcol..+8 -> operand (half, tile, k step), lane 16a + cc
+    const int krow = c / (HD / 8), kcol = c % (HD / 8);
+    const int kl = krow & 31;
+    const int ks = kcol >> 2, a = kcol & 3, cc = ((kl >> 3) << 2) | (kl & 3);
+    kdst[j] = (((krow >> 5) * 2 + ((kl >> 2) & 1)) * KS + ks) * 64 + 16 * a + (cc ^ pf2_kx(ks, a));
+    // V^T chunk: dim vrow, keys 8*vcol..+8 -> operand (half, dim tile), lane 16a + cc
+    const int vrow = c / (HE_PAGE_TOKENS / 8), vcol = c % (HE_PAGE_TOKENS / 8);
+    const int hb = vcol >> 2, va = vcol & 3;
+    vdst[j] = (hb * NT + (vrow >> 4)) * 64 + 16 * va + ((vrow & 15) ^ pf2_vx(hb, va));
+  }
+}
+
+template <int NT>
+__device__ __forceinline__ void pf2_stage(const pf2_vec (&kreg)[Pf2<NT>::PER_THREAD],
+                                          const pf2_vec (&vreg)[Pf2<NT>::PER_THREAD],
+                                          const int (&kdst)[Pf2<NT>::PER_THREAD],
+                                          const int (&vdst)[Pf2<NT>::PER_THREAD], pf2_vec* k_lds,
+                                          pf2_vec* v_lds) {
+#pragma unroll
+  for (int j = 0; j < Pf2<NT>::PER_THREAD; ++j) {
+    const int c = threadIdx.x + Pf2<NT>::THREADS * j;
     if (c < Pf2<NT>::CHUNKS) {
-      // K chunk: key krow, dims 8*kcol..+8 -> operand (half, tile, k step) and its lane
-      const int krow = c / (HD / 8), kcol = c % (HD / 8);
-      const int kl = krow & 31;
-      const int klane = 16 * (kcol & 3) + (((kl >> 3) << 2) | (kl & 3));
-      k_lds[(((krow >> 5) * 2 + ((kl >> 2) & 1)) * KS + (kcol >> 2)) * 64 + klane] = kreg[j];
-      // V^T chunk: dim vrow, keys 8*vcol..+8 -> operand (half, dim tile) and its lane
-      const int vrow = c / (HE_PAGE_TOKENS / 8), vcol = c % (HE_PAGE_TOKENS / 8);
-      v_lds[((vcol >> 2) * NT + (vrow >> 4)) * 64 + 16 * (vcol & 3) + (vrow & 15)] = vreg[j];
+      k_lds[kdst[j]] = kreg[j];
+      v_lds[vdst[j]] = vreg[j];
     }
   }
 }
@@ -210,13 +234,21 @@ struct PairTile {
   bf16x8 qf[KS];
   AttnState<NT> st;
   int qi, hi, lo, clear_lo, clear_hi;
+  int first, last;   // positions any query of the tile sees; first > last: no tile here
   bool ok;
 
+  // whether the 32 keys from key_base on hold a key some query of the tile sees
+  __device__ __forceinline__ bool active(int key_base) const {
+    return key_base <= last && key_base + 31 >= first;
+  }
+
   __device__ __forceinline__ void init(const uint16_t* __restrict__ q, int row0, int q_len,
-                                       int start, int qt, int H, int h, int window, int lr,
-                                       int lg) {
+                                       int start, int qt, bool valid, int H, int h, int window,
+                                       int lr, int lg) {
     qi = qt + lr;
-    ok = qi < q_len;
+    ok = valid && qi < q_len;
+    last = valid ? start + min(qt + 15, q_len - 1) : -1;
+    first = !valid ? 0x7fffffff : (window > 0 ? max(0, start + qt + 1 - window) : 0);
     const int pos = start + qi;
     hi = ok ? pos : -1;
     lo = (window > 0 && ok) ? max(0, pos + 1 - window) : 0;
@@ -242,8 +274,7 @@ struct PairTile {
   __device__ __forceinline__ void store(uint16_t* __restrict__ out, int row0, int H, int h, int lr,
                                         int lg) {
     float l = st.l;
-    l += __shfl_xor(l, 16, HE_WAVE);
-    l += __shfl_xor(l, 32, HE_WAVE);
+    l = xor32_sum(xor16_sum(l));
     if (!ok) return;
     const float inv = l > 0.f ? 1.f / l : 0.f;
     uint16_t* orow = out + ((int64_t)(row0 + qi) * H + h) * HD;
@@ -257,6 +288,46 @@ struct PairTile {
   }
 };
 
+// One step of 32 keys (half hb of the page in LDS) for the tiles that see keys in it. With
+// both, every operand read from LDS feeds two MFMAs.
+template <int NT, bool D0, bool D1>
+__device__ __forceinline__ void pf2_step(PairTile<NT>& t0, PairTile<NT>& t1, const pf2_vec* k_lds,
+                                         const pf2_vec* v_lds, int hb, int key_base,
+                                         float scale_log2, int lr, int lg) {
+  constexpr int HD = 16 * NT;
+  constexpr int KS = (HD + 31) / 32;
+  floatx4 s0[2], s1[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) s0[t] = s1[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      pf2_vec v = {0u, 0u, 0u, 0u};
+      if (32 * ks + 8 * lg < HD)
+        v = k_lds[((hb * 2 + t) * KS + ks) * 64 + 16 * lg + (lr ^ pf2_kx(ks, lg))];
+      const bf16x8 kf = __builtin_bit_cast(bf16x8, v);
+      if (D0) s0[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, t0.qf[ks], s0[t], 0, 0, 0);
+      if (D1) s1[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, t1.qf[ks], s1[t], 0, 0, 0);
+    }
+  bf16x8 p0, p1;
+  if (D0) p0 = t0.softmax(s0, key_base, scale_log2, lg);
+  if (D1) p1 = t1.softmax(s1, key_base, scale_log2, lg);
+#pragma unroll
+  for (int dt = 0; dt < NT; ++dt) {
+    const bf16x8 vf = __builtin_bit_cast(
+        bf16x8, v_lds[(hb * NT + dt) * 64 + 16 * lg + (lr ^ pf2_vx(hb, lg))]);
+    if (D0) t0.st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p0, t0.st.o[dt], 0, 0, 0);
+    if (D1) t1.st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p1, t1.st.o[dt], 0, 0, 0);
+  }
+}
+
+// The query tiles (16 queries) of a sequence are paired from both ends: tile a with tile
+// T - 1 - a. Under the causal mask an early tile sees few keys and a late one many; a pair
+// sees the same number of keys whatever a is, so every wavefront (one pair) and every
+// workgroup (four pairs) does the same work and none waits for a longest one. Where both
+// tiles of a pair see keys of a step the LDS operands are shared; the late tile walks the
+// rest alone.
 template <int NT>
 __global__ __launch_bounds__(64 * PF2_WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 attention_prefill_pair_kernel(
@@ -267,11 +338,9 @@ attention_prefill_pair_kernel(
     int num_pages, int H, int KVH, int window, float scale) {
   constexpr int HD = 16 * NT;
   constexpr int KS = (HD + 31) / 32;
-  constexpr int CHUNKS = HE_PAGE_TOKENS * HD / 8;   // 16-byte chunks of one page of K (or V^T)
-  constexpr int THREADS = 64 * PF2_WAVES;
-  constexpr int PER_THREAD = (CHUNKS + THREADS - 1) / THREADS;
-  constexpr int K_OPS = 2 * 2 * KS * 64, V_OPS = 2 * NT * 64;   // uint4 per buffer
-  // operand-ordered: k[((hb*2 + t)*KS + ks)*64 + lane], v[(hb*NT + dt)*64 + lane]
+  constexpr int PER_THREAD = Pf2<NT>::PER_THREAD;
+  constexpr int K_OPS = 2 * 2 * KS * 64, V_OPS = 2 * NT * 64;   // 16-byte slots per buffer
+  // operand-ordered: k[((hb*2 + t)*KS + ks)*64 + slot(lane)], v[(hb*NT + dt)*64 + slot(lane)]
   __shared__ pf2_vec k_lds[2][K_OPS];
   __shared__ pf2_vec v_lds[2][V_OPS];
 
@@ -282,14 +351,10 @@ attention_prefill_pair_kernel(
   if (slot < 0) return;
   const int row0 = cu_seqlens[seq];
   const int q_len = cu_seqlens[seq + 1] - row0;
-  // Long workgroups first: the last queries of a sequence have the most keys. Workgroups
-  // are handed to the compute units in rounds of 256 (one per unit); every other round runs
-  // from short to long, so that a unit that got a long one in one round gets a short one in
-  // the next - with two resident per unit, the pairs then do equal work.
-  const unsigned linear = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
-  const int qslot = ((linear >> 8) & 1) ? (int)blockIdx.x : (int)(gridDim.x - 1 - blockIdx.x);
-  const int qb = PF2_QUERIES * qslot;
-  if (qb >= q_len) return;
+  const int tiles = (q_len + 15) >> 4;
+  const int pairs = (tiles + 1) >> 1;
+  const int pair0 = PF2_WAVES * blockIdx.x;      // the workgroup's first pair: its earliest and latest tile
+  if (pair0 >= pairs) return;
   const int start = seq_start[seq];
   const int kvh = h / (H / KVH);
   const int32_t* pt = page_table + (int64_t)slot * max_blocks;
@@ -297,59 +362,42 @@ attention_prefill_pair_kernel(
   const uint16_t* kp = kpool + (int64_t)kvh * (HE_PAGE_TOKENS * HD);
   const uint16_t* vp = vpool + (int64_t)kvh * (HE_PAGE_TOKENS * HD);
 
-  const int qw = qb + 32 * wave;                 // this wave's 32 queries: tiles qw and qw + 16
-  const bool wave_ok = qw < q_len;
+  const int pair = pair0 + wave;
+  const int ta = pair, tb = tiles - 1 - pair;    // ta <= tb while pair < pairs
   PairTile<NT> t0, t1;
-  t0.init(q, row0, q_len, start, qw, H, h, window, lr, lg);
-  t1.init(q, row0, q_len, start, qw + 16, H, h, window, lr, lg);
-  const int wlast = start + min(qw + 31, q_len - 1);            // last position this wave sees
-  const int wfirst = window > 0 ? max(0, start + qw + 1 - window) : 0;
+  t0.init(q, row0, q_len, start, 16 * ta, pair < pairs, H, h, window, lr, lg);
+  t1.init(q, row0, q_len, start, 16 * tb, pair < pairs && tb > ta, H, h, window, lr, lg);
   const float scale_log2 = scale * 1.4426950408889634f;
 
-  const int blk_last = start + min(qb + PF2_QUERIES - 1, q_len - 1);
-  const int blk_first = window > 0 ? max(0, start + qb + 1 - window) : 0;
+  // pages from the first key the earliest tile sees to the last key of the latest tile
+  const int blk_last = start + min(16 * (tiles - 1 - pair0) + 15, q_len - 1);
+  const int blk_first = window > 0 ? max(0, start + 16 * pair0 + 1 - window) : 0;
   const int pb0 = blk_first >> HE_PAGE_SHIFT, pb1 = blk_last >> HE_PAGE_SHIFT;
 
   pf2_vec kreg[PER_THREAD], vreg[PER_THREAD];
+  int kdst[PER_THREAD], vdst[PER_THREAD];
+  pf2_slots<NT>(kdst, vdst);
   pf2_fetch<NT>(kreg, vreg, kp, vp, pt[pb0], num_pages, page_stride);
-  pf2_stage<NT>(kreg, vreg, k_lds[0], v_lds[0]);
+  pf2_stage<NT>(kreg, vreg, kdst, vdst, k_lds[0], v_lds[0]);
   if (pb0 < pb1) pf2_fetch<NT>(kreg, vreg, kp, vp, pt[pb0 + 1], num_pages, page_stride);
   __syncthreads();
   for (int pb = pb0; pb <= pb1; ++pb) {
     const int buf = (pb - pb0) & 1;
     if (pb < pb1) {
       // everyone left the other buffer before the last barrier
-      pf2_stage<NT>(kreg, vreg, k_lds[buf ^ 1], v_lds[buf ^ 1]);
+      pf2_stage<NT>(kreg, vreg, kdst, vdst, k_lds[buf ^ 1], v_lds[buf ^ 1]);
       if (pb + 1 < pb1) pf2_fetch<NT>(kreg, vreg, kp, vp, pt[pb + 2], num_pages, page_stride);
     }
-    const int page_lo = pb << HE_PAGE_SHIFT;
-    if (wave_ok && page_lo <= wlast && page_lo + HE_PAGE_TOKENS - 1 >= wfirst) {
 #pragma unroll
-      for (int hb = 0; hb < 2; ++hb) {
-        const int key_base = page_lo + 32 * hb;
-        if (key_base > wlast || key_base + 31 < wfirst) continue;
-        floatx4 s0[2], s1[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) s0[t] = s1[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int ks = 0; ks < KS; ++ks) {
-            pf2_vec v = {0u, 0u, 0u, 0u};
-            if (32 * ks + 8 * lg < HD) v = k_lds[buf][((hb * 2 + t) * KS + ks) * 64 + lane];
-            const bf16x8 kf = __builtin_bit_cast(bf16x8, v);
-            s0[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, t0.qf[ks], s0[t], 0, 0, 0);
-            s1[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, t1.qf[ks], s1[t], 0, 0, 0);
-          }
-        const bf16x8 p0 = t0.softmax(s0, key_base, scale_log2, lg);
-        const bf16x8 p1 = t1.softmax(s1, key_base, scale_log2, lg);
-#pragma unroll
-        for (int dt = 0; dt < NT; ++dt) {
-          const bf16x8 vf = __builtin_bit_cast(bf16x8, v_lds[buf][(hb * NT + dt) * 64 + lane]);
-          t0.st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p0, t0.st.o[dt], 0, 0, 0);
-          t1.st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p1, t1.st.o[dt], 0, 0, 0);
-        }
-      }
+    for (int hb = 0; hb < 2; ++hb) {
+      const int key_base = (pb << HE_PAGE_SHIFT) + 32 * hb;
+      const bool a0 = t0.active(key_base), a1 = t1.active(key_base);   // the same in all lanes
+      if (a0 && a1)
+        pf2_step<NT, true, true>(t0, t1, k_lds[buf], v_lds[buf], hb, key_base, scale_log2, lr, lg);
+      else if (a1)
+        pf2_step<NT, false, true>(t0, t1, k_lds[buf], v_lds[buf], hb, key_base, scale_log2, lr, lg);
+      else if (a0)
+        pf2_step<NT, true, false>(t0, t1, k_lds[buf], v_lds[buf], hb, key_base, scale_log2, lr, lg);
     }
     __syncthreads();
   }
@@ -417,8 +465,7 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   attend_range<NT, false>(st, qf, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, kb_begin,
                    (kb_end + 31) & ~31, first, hi, first, hi, scale * 1.4426950408889634f, lr, lg);
   float l = st.l;
-  l += __shfl_xor(l, 16, HE_WAVE);
-  l += __shfl_xor(l, 32, HE_WAVE);
+  l = xor32_sum(xor16_sum(l));
   if (nsplit == 1) {                      // nothing to merge
     if (!h_ok) return;
     const float inv = l > 0.f ? 1.f / l : 0.f;
@@ -544,6 +591,7 @@ extern "C" int he_attention_decode_bf16(void* out, const void* q, const void* kp
                                         int64_t workspace_floats, void* stream) {
   HE_REQUIRE(rows >= 0 && H > 0 && KVH > 0 && hd > 0 && max_keys > 0,
              "he_attention_decode_bf16: bad sizes");
+  HE_REQUIRE(scale > 0.f, "he_attention_decode_bf16: the score scale must be positive");
   HE_REQUIRE(H % KVH == 0, "he_attention_decode_bf16: heads %d not a multiple of kv heads %d", H,
              KVH);
   HE_REQUIRE(hd % 16 == 0 && hd <= 256,
@@ -596,6 +644,7 @@ extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* k
                                          int window, float scale, void* stream) {
   HE_REQUIRE(num_seqs >= 0 && max_q_len >= 0 && H > 0 && KVH > 0 && hd > 0,
              "he_attention_prefill_bf16: bad sizes");
+  HE_REQUIRE(scale > 0.f, "he_attention_prefill_bf16: the score scale must be positive");
   HE_REQUIRE(H % KVH == 0, "he_attention_prefill_bf16: heads %d not a multiple of kv heads %d", H,
              KVH);
   HE_REQUIRE(hd % 16 == 0 && hd <= 256,

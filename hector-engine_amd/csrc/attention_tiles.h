@@ -5,6 +5,12 @@
 #pragma once
 #include "common.h"
 
+// Online softmax keeps, per query, a reference point m (base-2 domain) and sums of
+// 2^(s - m). Any m gives the same quotient; m need only be close enough to the running
+// maximum that 2^(s - m) stays small. Following the maximum exactly makes one of the 16
+// queries of a tile move it in most steps, and every move rescales all accumulators.
+#define HE_SOFTMAX_SLACK 8.0f
+
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
@@ -17,7 +23,7 @@ __device__ __forceinline__ bf16x8 ld8(const uint16_t* p, bool ok) {
 template <int NT>
 struct AttnState {
   floatx4 o[NT];  // O^T[16*dt + 4*lg + i][q], unnormalised
-  float m;        // running maximum of the query of this lane's column
+  float m;        // reference point (near the running maximum) of the query of this lane's column
   float l;        // this lane's share of the running sum
 };
 
@@ -58,8 +64,8 @@ __device__ __forceinline__ void load_frag(KVFrag<NT>& f, const uint16_t* __restr
 // The lane's query sees the keys in [lo, hi]; with MASK false the caller has checked
 // that all 32 keys are visible to every query of the tile. Scores are kept in the
 // base-2 domain: s2 = (q . k) * scale * log2(e), p = 2^(s2 - m), so the exponential is
-// the bare hardware instruction; m is the running maximum of s2. When no query's
-// maximum moves, the rescaling of the accumulators is skipped.
+// the bare hardware instruction; m is the reference point of s2 (see HE_SOFTMAX_SLACK). When
+// no query's reference point moves, the rescaling of the accumulators is skipped.
 template <int NT, bool MASK>
 __device__ __forceinline__ void attend_frag(AttnState<NT>& st, const bf16x8* qf,
                                             const KVFrag<NT>& f, int key_base, int lo, int hi,
@@ -75,13 +81,15 @@ __device__ __forceinline__ void attend_frag(AttnState<NT>& st, const bf16x8* qf,
     for (int ks = 0; ks < KS; ++ks)
       s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k[t][ks], qf[ks], s[t], 0, 0, 0);
   }
+  // raw scores (masked ones at -inf), their maximum, then p = 2^(raw * scale - m) with the
+  // scale folded into the subtraction (scale > 0, so the maximum commutes with it)
   float p[2][4];
   float mx = -INFINITY;
 #pragma unroll
   for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      float v = s[t][r] * scale_log2;
+      float v = s[t][r];
       if (MASK) {
         const int key = key_base + 8 * lg + 4 * t + r;
         v = (key >= lo && key <= hi) ? v : -INFINITY;
@@ -89,9 +97,10 @@ __device__ __forceinline__ void attend_frag(AttnState<NT>& st, const bf16x8* qf,
       p[t][r] = v;
       mx = fmaxf(mx, v);
     }
-  mx = fmaxf(mx, __shfl_xor(mx, 16, HE_WAVE));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, HE_WAVE));
-  const float m_new = fmaxf(st.m, mx);
+  mx = xor32_max(xor16_max(mx)) * scale_log2;
+  // the reference point follows the maximum only when that has grown by more than
+  // 2^HE_SOFTMAX_SLACK: p stays below that factor, and the accumulators are rarely rescaled
+  const float m_new = mx > st.m + HE_SOFTMAX_SLACK ? mx : st.m;
   const bool moved = __builtin_amdgcn_ballot_w64(m_new != st.m) != 0;   // wave-uniform
   const float m_use = m_new == -INFINITY ? 0.f : m_new;
   float sum = 0.f;
@@ -100,8 +109,8 @@ __device__ __forceinline__ void attend_frag(AttnState<NT>& st, const bf16x8* qf,
   for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int r = 0; r < 4; r += 2) {
-      const float e0 = __builtin_amdgcn_exp2f(p[t][r] - m_use);
-      const float e1 = __builtin_amdgcn_exp2f(p[t][r + 1] - m_use);
+      const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(p[t][r], scale_log2, -m_use));
+      const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(p[t][r + 1], scale_log2, -m_use));
       sum += e0 + e1;
       packed[2 * t + (r >> 1)] = pack2_bf16(e0, e1);
     }

@@ -80,6 +80,36 @@ __device__ __forceinline__ void sincos_angle(float a, float* sn, float* cs) {
   *cs = (float)(((q + 1) & 2) ? -cv : cv);
 }
 
+// Exchange across the halves (32 lanes) or across neighbouring rows of 16 lanes with the
+// gfx950 lane-swap instructions: a vector-ALU move, where __shfl_xor goes through the LDS
+// crossbar with five instructions of address arithmetic. Both lanes of a pair get the
+// same operands, so sums are bit-identical in both.
+__device__ __forceinline__ float max_plain(float a, float b) {   // operands are never NaN here
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ float xor32_max(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return max_plain(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float xor16_max(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  return max_plain(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float xor32_sum(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float xor16_sum(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int off = HE_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, HE_WAVE);

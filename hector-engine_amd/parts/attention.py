@@ -44,7 +44,7 @@ class Attention(Mixer):
         self.q_only: Linear | None = None
         self.o_proj: Linear | None = None
         self.fast = env.dtype == torch.bfloat16 and getattr(env, "fast_kernels", True) \
-            and self.hd % 16 == 0 and self.hd <= 256
+            and self.hd % 16 == 0 and self.hd <= 256 and self.scale > 0   # else the plain kernel
 
     def children(self):
         return [self.position]
