@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 10
+#define HE_ABI_VERSION 11
 
 #ifdef __cplusplus
 extern "C" {
@@ -115,8 +115,9 @@ int he_attention_prefill_bf16(void* out, const void* q, const void* kpool, const
                               void* stream);
 
 // ---- sampling ------------------------------------------------------------
+int64_t he_argmax_workspace_bytes(int rows, int V);
 int he_argmax_rows(void* out_i32, const void* logits_f32, int rows, int V, int64_t row_stride,
-                   void* stream);
+                   void* workspace, int64_t workspace_bytes, void* stream);
 int he_apply_penalties(void* logits_f32, int rows, int V, int64_t row_stride, const void* ids,
                        const void* counts, const void* offsets, float rep, float freq, float pres,
                        void* stream);

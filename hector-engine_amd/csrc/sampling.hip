@@ -19,29 +19,29 @@
 #define SAMP_FIXED_ONE 1099511627776.0f  // 2^40
 
 // ---------------------------------------------------------------- argmax
-__global__ __launch_bounds__(SAMP_THREADS) void argmax_rows_kernel(int32_t* __restrict__ out,
-                                                                   const float* __restrict__ logits,
-                                                                   int V, int64_t stride) {
-  __shared__ float sval[SAMP_THREADS / HE_WAVE];
-  __shared__ int sidx[SAMP_THREADS / HE_WAVE];
-  const float* x = logits + blockIdx.x * stride;
-  float best = -INFINITY;
-  int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) {
-    const float v = x[i];
-    if (v > best || (bi == 0x7fffffff && v == best)) {  // strict: first maximum wins
-      best = v;
-      bi = i;
-    }
+// The lowest index among the maxima of each row. A row is cut into parts of ARGMAX_PART
+// elements, one workgroup each, so that a long vocabulary is read by many compute units at
+// once; a second small launch takes the best of a row's parts (with one part the first
+// launch writes the result itself).
+#define ARGMAX_PART 8192
+#define ARGMAX_THREADS 256
+
+__device__ __forceinline__ void argmax_take(float& best, int& bi, float v, int i) {
+  if (v > best || (v == best && i < bi)) {
+    best = v;
+    bi = i;
   }
+}
+
+// Reduces (best, bi) over the workgroup; valid in thread 0.
+__device__ __forceinline__ void argmax_block(float& best, int& bi) {
+  __shared__ float sval[ARGMAX_THREADS / HE_WAVE];
+  __shared__ int sidx[ARGMAX_THREADS / HE_WAVE];
 #pragma unroll
   for (int off = HE_WAVE / 2; off > 0; off >>= 1) {
     const float ov = __shfl_xor(best, off, HE_WAVE);
     const int oi = __shfl_xor(bi, off, HE_WAVE);
-    if (ov > best || (ov == best && oi < bi)) {
-      best = ov;
-      bi = oi;
-    }
+    argmax_take(best, bi, ov, oi);
   }
   const int lane = threadIdx.x & (HE_WAVE - 1), wave = threadIdx.x >> 6;
   if (lane == 0) {
@@ -49,26 +49,89 @@ __global__ __launch_bounds__(SAMP_THREADS) void argmax_rows_kernel(int32_t* __re
     sidx[wave] = bi;
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    const int nw = blockDim.x >> 6;
-    for (int w = 1; w < nw; ++w) {
-      if (sval[w] > best || (sval[w] == best && sidx[w] < bi)) {
-        best = sval[w];
-        bi = sidx[w];
+  if (threadIdx.x == 0)
+    for (int w = 1; w < (int)(blockDim.x >> 6); ++w) argmax_take(best, bi, sval[w], sidx[w]);
+}
+
+// grid (parts, rows)
+__global__ __launch_bounds__(ARGMAX_THREADS) void argmax_parts_kernel(
+    int32_t* __restrict__ out, float* __restrict__ part_val, int32_t* __restrict__ part_idx,
+    const float* __restrict__ logits, int V, int64_t stride) {
+  const float* x = logits + blockIdx.y * stride;
+  const int lo = blockIdx.x * ARGMAX_PART, hi = min(V, lo + ARGMAX_PART);
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  const bool vec = ((stride & 3) == 0) && ((((uintptr_t)logits) & 15) == 0);
+  if (vec) {
+    for (int i = lo + 4 * threadIdx.x; i < hi; i += 4 * ARGMAX_THREADS) {
+      if (i + 4 <= hi) {
+        const float4 v = *reinterpret_cast<const float4*>(x + i);
+        argmax_take(best, bi, v.x, i);
+        argmax_take(best, bi, v.y, i + 1);
+        argmax_take(best, bi, v.z, i + 2);
+        argmax_take(best, bi, v.w, i + 3);
+      } else {
+        for (int j = i; j < hi; ++j) argmax_take(best, bi, x[j], j);
       }
     }
-    out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+  } else {
+    for (int i = lo + threadIdx.x; i < hi; i += ARGMAX_THREADS) argmax_take(best, bi, x[i], i);
+  }
+  argmax_block(best, bi);
+  if (threadIdx.x == 0) {
+    if (gridDim.x == 1) {
+      out[blockIdx.y] = bi == 0x7fffffff ? 0 : bi;   // a row of NaN only
+    } else {
+      part_val[blockIdx.y * gridDim.x + blockIdx.x] = best;
+      part_idx[blockIdx.y * gridDim.x + blockIdx.x] = bi;
+    }
   }
 }
 
+// grid rows, one wavefront
+__global__ __launch_bounds__(HE_WAVE) void argmax_join_kernel(int32_t* __restrict__ out,
+                                                              const float* __restrict__ part_val,
+                                                              const int32_t* __restrict__ part_idx,
+                                                              int parts) {
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int p = threadIdx.x; p < parts; p += HE_WAVE)
+    argmax_take(best, bi, part_val[blockIdx.x * parts + p], part_idx[blockIdx.x * parts + p]);
+#pragma unroll
+  for (int off = HE_WAVE / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(best, off, HE_WAVE);
+    const int oi = __shfl_xor(bi, off, HE_WAVE);
+    argmax_take(best, bi, ov, oi);
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+}
+
+extern "C" int64_t he_argmax_workspace_bytes(int rows, int V) {
+  if (rows <= 0 || V <= ARGMAX_PART) return 0;
+  return (int64_t)rows * ((V + ARGMAX_PART - 1) / ARGMAX_PART) * 8;
+}
+
 extern "C" int he_argmax_rows(void* out_i32, const void* logits_f32, int rows, int V,
-                              int64_t row_stride, void* stream) {
+                              int64_t row_stride, void* workspace, int64_t workspace_bytes,
+                              void* stream) {
   HE_REQUIRE(rows >= 0 && V > 0 && row_stride >= V, "he_argmax_rows: bad sizes rows=%d V=%d", rows,
              V);
+  HE_REQUIRE(rows <= 65535, "he_argmax_rows: %d rows above 65535", rows);
   if (rows == 0) return 0;
-  argmax_rows_kernel<<<rows, SAMP_THREADS, 0, (hipStream_t)stream>>>(
-      (int32_t*)out_i32, (const float*)logits_f32, V, row_stride);
-  return he_check_launch("he_argmax_rows");
+  const int parts = (V + ARGMAX_PART - 1) / ARGMAX_PART;
+  const int64_t need = he_argmax_workspace_bytes(rows, V);
+  HE_REQUIRE(need == 0 || (workspace != nullptr && workspace_bytes >= need),
+             "he_argmax_rows: workspace of %lld bytes, need %lld", (long long)workspace_bytes,
+             (long long)need);
+  float* part_val = (float*)workspace;
+  int32_t* part_idx = (int32_t*)workspace + (int64_t)rows * parts;
+  hipStream_t s = (hipStream_t)stream;
+  argmax_parts_kernel<<<dim3(parts, rows), ARGMAX_THREADS, 0, s>>>(
+      (int32_t*)out_i32, part_val, part_idx, (const float*)logits_f32, V, row_stride);
+  int rc = he_check_launch("he_argmax_rows");
+  if (rc || parts == 1) return rc;
+  argmax_join_kernel<<<rows, HE_WAVE, 0, s>>>((int32_t*)out_i32, part_val, part_idx, parts);
+  return he_check_launch("he_argmax_rows join");
 }
 
 // ---------------------------------------------------------------- penalties

@@ -468,7 +468,9 @@ def argmax_rows(out_i32, logits, rows: int) -> None:
     if logits.numel() < rows * V or out_i32.numel() < rows:
         raise ValueError("argmax_rows: buffers smaller than the row count")
     L = _lib.load()
-    _lib.check(L.he_argmax_rows(out_i32.data_ptr(), logits.data_ptr(), rows, V, V, _stream()))
+    need = int(L.he_argmax_workspace_bytes(rows, V))
+    ws = torch.empty(need, dtype=torch.uint8, device=logits.device) if need else None
+    _lib.check(L.he_argmax_rows(out_i32.data_ptr(), logits.data_ptr(), rows, V, V, _ptr(ws), need, _stream()))
 
 
 def apply_penalties(logits, rows: int, ids, counts, offsets, rep: float, freq: float,

@@ -637,6 +637,22 @@ def test_argmax_lowest_index_on_ties(ops):
     assert out.tolist() == [P.argmax_lowest(r) for r in x]
 
 
+@pytest.mark.parametrize("V", [8192, 8193, 30001, 152064])
+def test_argmax_over_parts(ops, V):
+    """Long rows are cut across workgroups: ties across a cut, a maximum at either end, at
+    a cut and in the last (short) part; a width that is no multiple of 4."""
+    x = rnd(6, V, seed=61)
+    x[0, 8191] = x[0, V - 1] = 30.0               # tie across parts: the lower index
+    x[1, V - 1] = 40.0
+    x[2, 0] = 40.0
+    x[3, :] = -3.0                                # all equal
+    x[4, min(V - 1, 8192)] = x[4, 5000] = 35.0
+    out = torch.empty(6, dtype=torch.int32, device="cuda")
+    ops.argmax_rows(out, dev(x), 6)
+    assert out.tolist() == [P.argmax_lowest(r) for r in x]
+    assert out.tolist()[:5] == [8191, V - 1, 0, 0, 5000]
+
+
 def test_penalties(ops):
     V = 50
     x = rnd(2, V, seed=61)
