@@ -201,25 +201,47 @@ struct SampShared {
   float m;
 };
 
+// Exact (integer) sum over the workgroup: wavefronts first, then their 16 sums in order.
 __device__ u64 block_sum_u64(u64 v, SampShared& sh) {
-  __syncthreads();
-  sh.red[threadIdx.x] = v;
-  __syncthreads();
-  for (int s = SAMP_THREADS / 2; s > 0; s >>= 1) {
-    if ((int)threadIdx.x < s) sh.red[threadIdx.x] += sh.red[threadIdx.x + s];
-    __syncthreads();
+#pragma unroll
+  for (int off = HE_WAVE / 2; off > 0; off >>= 1) {
+    const uint32_t lo = __shfl_xor((uint32_t)v, off, HE_WAVE);
+    const uint32_t hi = __shfl_xor((uint32_t)(v >> 32), off, HE_WAVE);
+    v += ((u64)hi << 32) | lo;
   }
-  const u64 r = sh.red[0];
+  __syncthreads();
+  if ((threadIdx.x & (HE_WAVE - 1)) == 0) sh.red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  u64 r = 0;
+  for (int w = 0; w < SAMP_THREADS / HE_WAVE; ++w) r += sh.red[w];
   __syncthreads();
   return r;
 }
 
-template <bool MASS>
-__device__ u64 set_total(const float* x, int V, float m, float inv_temp, Cut cut,
-                         SampShared& sh) {
+// Where the elements come from: the whole row in global memory, or a list in LDS of the
+// row's largest elements (value and index), in no particular order.
+struct RowSource {
+  const float* x;
+  int n;
+  __device__ __forceinline__ bool valid(int) const { return true; }
+  __device__ __forceinline__ float value(int i) const { return clean(x[i]); }
+  __device__ __forceinline__ int index(int i) const { return i; }
+};
+struct ListSource {   // n slots; a slot with index -1 is empty
+  const float* v;
+  const int* idx;
+  int n;
+  __device__ __forceinline__ bool valid(int i) const { return idx[i] >= 0; }
+  __device__ __forceinline__ float value(int i) const { return v[i]; }
+  __device__ __forceinline__ int index(int i) const { return idx[i]; }
+};
+
+template <bool MASS, typename Source>
+__device__ u64 set_total(const Source& src, float m, float inv_temp, Cut cut, SampShared& sh) {
   u64 local = 0;
-  for (int i = threadIdx.x; i < V; i += SAMP_THREADS) {
-    const float v = clean(x[i]);
+  for (int i = threadIdx.x; i < src.n; i += SAMP_THREADS) {
+    if (!src.valid(i)) continue;
+    const float v = src.value(i);
     const uint32_t k = ordered_key(v);
     if (cut.any && k <= cut.key) continue;
     local += MASS ? fixed_mass(v, m, inv_temp) : 1ull;
@@ -229,11 +251,33 @@ __device__ u64 set_total(const float* x, int V, float m, float inv_temp, Cut cut
   return block_sum_u64(local, sh);
 }
 
+// Adds every lane's pending (bin, run) to the histogram. Lanes of a wavefront that hold the
+// same bin - all of them in the passes over the upper key bytes - are summed first and one
+// lane adds the sum: a thousand 64-bit LDS atomics on one address take tens of microseconds.
+__device__ __forceinline__ void flush_runs(u64* hist, int bin, u64 run) {
+  const int lane = threadIdx.x & (HE_WAVE - 1);
+  unsigned long long pending = __builtin_amdgcn_ballot_w64(bin >= 0);
+  while (pending) {
+    const int leader = __builtin_ctzll(pending);
+    const int lb = __shfl(bin, leader, HE_WAVE);
+    const bool same = bin == lb;
+    u64 v = same ? run : 0ull;
+#pragma unroll
+    for (int off = HE_WAVE / 2; off > 0; off >>= 1) {
+      const uint32_t lo = __shfl_xor((uint32_t)v, off, HE_WAVE);
+      const uint32_t hi = __shfl_xor((uint32_t)(v >> 32), off, HE_WAVE);
+      v += ((u64)hi << 32) | lo;
+    }
+    if (lane == leader) atomicAdd(&hist[lb], v);
+    pending &= ~__builtin_amdgcn_ballot_w64(same);
+  }
+}
+
 // Finds, in descending order inside `cut`, the element at which the cumulative
 // count (MASS = false) or mass (MASS = true) first reaches t (t >= 1), and
 // returns the set of everything up to and including it.
-template <bool MASS>
-__device__ Cut descend(const float* x, int V, float m, float inv_temp, Cut cut, u64 t,
+template <bool MASS, typename Source>
+__device__ Cut descend(const Source& src, float m, float inv_temp, Cut cut, u64 t,
                        SampShared& sh) {
   uint32_t prefix = 0;
   for (int pass = 0; pass < 4; ++pass) {
@@ -243,8 +287,9 @@ __device__ Cut descend(const float* x, int V, float m, float inv_temp, Cut cut, 
     __syncthreads();
     int cur = -1;
     u64 run = 0;
-    for (int i = threadIdx.x; i < V; i += SAMP_THREADS) {
-      const float v = clean(x[i]);
+    for (int i = threadIdx.x; i < src.n; i += SAMP_THREADS) {
+      if (!src.valid(i)) continue;
+      const float v = src.value(i);
       const uint32_t k = ordered_key(v);
       if (pass > 0 && (k >> (shift + 8)) != (prefix >> (shift + 8))) continue;
       if (cut.any && k <= cut.key) continue;
@@ -256,34 +301,57 @@ __device__ Cut descend(const float* x, int V, float m, float inv_temp, Cut cut, 
       }
       run += MASS ? fixed_mass(v, m, inv_temp) : 1ull;
     }
-    if (cur >= 0) atomicAdd(&sh.hist[cur], run);
+    flush_runs(sh.hist, cur, run);
     if (threadIdx.x == 0 && cut.any && cut.ties > 0 &&
         (pass == 0 || (cut.key >> (shift + 8)) == (prefix >> (shift + 8)))) {
       const u64 w = MASS ? fixed_mass(key_to_float(cut.key), m, inv_temp) : 1ull;
       atomicAdd(&sh.hist[(cut.key >> shift) & 255], w * (u64)cut.ties);
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-      u64 acc = 0;
-      int found = -1, last = -1;
-      for (int b = 255; b >= 0; --b) {
-        const u64 hb = sh.hist[b];
-        if (hb == 0) continue;
-        last = b;
-        if (acc < t && t <= acc + hb) {
-          found = b;
-          break;
+    if (threadIdx.x < HE_WAVE) {
+      // Walk the bins from 255 down to the one in which the running total reaches t: lane l
+      // owns bins 4l..4l+3, a suffix sum over the lanes gives what lies above each, one lane
+      // finds the crossing among its four.
+      const int lane = threadIdx.x;
+      u64 h[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) h[j] = sh.hist[4 * lane + j];
+      const u64 mine = (h[0] + h[1]) + (h[2] + h[3]);
+      u64 incl = mine;
+#pragma unroll
+      for (int off = 1; off < HE_WAVE; off <<= 1) {
+        const uint32_t lo = __shfl_down((uint32_t)incl, off, HE_WAVE);
+        const uint32_t hi = __shfl_down((uint32_t)(incl >> 32), off, HE_WAVE);
+        if (lane + off < HE_WAVE) incl += ((u64)hi << 32) | lo;
+      }
+      const u64 above = incl - mine;
+      const bool has = mine > 0 && above < t && t <= above + mine;
+      const unsigned long long crossing = __builtin_amdgcn_ballot_w64(has);
+      const unsigned long long filled = __builtin_amdgcn_ballot_w64(mine > 0);
+      if (crossing) {
+        if (has) {
+          u64 acc = above;
+          for (int j = 3; j >= 0; --j) {
+            if (h[j] == 0) continue;
+            if (acc < t && t <= acc + h[j]) {
+              sh.prefix = prefix | ((uint32_t)(4 * lane + j) << shift);
+              sh.t = t - acc;
+              break;
+            }
+            acc += h[j];
+          }
         }
-        acc += hb;
+      } else if (filled) {   // t beyond the total: end at the last (lowest) element
+        if (lane == __builtin_ctzll(filled)) {
+          int j = 0;
+          while (h[j] == 0) ++j;
+          sh.prefix = prefix | ((uint32_t)(4 * lane + j) << shift);
+          sh.t = h[j];
+        }
+      } else if (lane == 0) {
+        sh.prefix = prefix;
+        sh.t = 1;
       }
-      if (found < 0) {  // t beyond the total: end at the last element
-        found = last < 0 ? 0 : last;
-        t = last < 0 ? 1 : sh.hist[found];
-      } else {
-        t -= acc;
-      }
-      sh.prefix = prefix | ((uint32_t)found << shift);
-      sh.t = t;
     }
     __syncthreads();
     prefix = sh.prefix;
@@ -299,52 +367,9 @@ __device__ Cut descend(const float* x, int V, float m, float inv_temp, Cut cut, 
   return r;
 }
 
-__global__ __launch_bounds__(SAMP_THREADS) void sample_rows_kernel(
-    int32_t* __restrict__ out, const float* __restrict__ logits, int V, int64_t stride,
-    const uint32_t* __restrict__ uniforms, float inv_temp, int top_k, float top_p) {
-  __shared__ SampShared sh;
-  __shared__ int s_counts[SAMP_THREADS];
-  const float* x = logits + blockIdx.x * stride;
-
-  // row maximum
-  float best = -INFINITY;
-  for (int i = threadIdx.x; i < V; i += SAMP_THREADS) best = fmaxf(best, clean(x[i]));
-  best = wave_max(best);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) sh.red[threadIdx.x >> 6] = (u64)__float_as_uint(best);
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    float mm = -INFINITY;
-    for (int w = 0; w < SAMP_THREADS / HE_WAVE; ++w)
-      mm = fmaxf(mm, __uint_as_float((uint32_t)sh.red[w]));
-    sh.m = mm;
-  }
-  __syncthreads();
-  const float m = sh.m;
-  if (!(m > -INFINITY)) {  // nothing finite: fall back to index 0
-    if (threadIdx.x == 0) out[blockIdx.x] = 0;
-    return;
-  }
-
-  Cut cut;
-  cut.any = 0;
-  cut.key = 0;
-  cut.ties = 0;
-  if (top_k > 0 && top_k < V) cut = descend<false>(x, V, m, inv_temp, cut, (u64)top_k, sh);
-  u64 Z = set_total<true>(x, V, m, inv_temp, cut, sh);
-  if (top_p > 0.f && top_p < 1.f) {
-    u64 target = (u64)ceil((double)top_p * (double)Z);
-    if (target < 1) target = 1;
-    if (target > Z) target = Z;
-    cut = descend<true>(x, V, m, inv_temp, cut, target, sh);
-    Z = set_total<true>(x, V, m, inv_temp, cut, sh);
-  }
-  // r = floor(u * Z / 2^32), Z < 2^58
-  const u64 u = (u64)uniforms[blockIdx.x];
-  const u64 r = u * (Z >> 32) + ((u * (Z & 0xffffffffull)) >> 32);
-  const Cut pick = descend<true>(x, V, m, inv_temp, cut, r + 1, sh);
-
-  // the pick.ties-th element (by ascending index) whose key equals pick.key
+// The index of the pick.ties-th element, by ascending index, whose key equals pick.key.
+__device__ int pick_index_row(const float* x, int V, Cut pick, int* s_counts) {
+  __shared__ int s_res;
   const int chunk = (V + SAMP_THREADS - 1) / SAMP_THREADS;
   const int b = threadIdx.x * chunk;
   const int e = min(V, b + chunk);
@@ -367,8 +392,219 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_rows_kernel(
         acc += s_counts[th];
       }
     }
-    out[blockIdx.x] = res < 0 ? 0 : res;
+    s_res = res < 0 ? 0 : res;
   }
+  __syncthreads();
+  return s_res;
+}
+
+// The same on a list, for a small rank: the lowest index among the equal keys, then the
+// next one, ... `ties` times. Returns -1 when the rank is not small (the caller then walks
+// the row).
+#define SAMP_PICK_ROUNDS 16
+__device__ int pick_index_list(const ListSource& src, Cut pick, SampShared& sh) {
+  if (pick.ties > SAMP_PICK_ROUNDS) return -1;
+  int after = -1;
+  for (uint32_t round = 0; round < pick.ties; ++round) {
+    int best = 0x7fffffff;
+    for (int i = threadIdx.x; i < src.n; i += SAMP_THREADS) {
+      const int id = src.idx[i];
+      if (id > after && id < best && ordered_key(src.v[i]) == pick.key) best = id;
+    }
+#pragma unroll
+    for (int off = HE_WAVE / 2; off > 0; off >>= 1) best = min(best, __shfl_xor(best, off, HE_WAVE));
+    __syncthreads();
+    if ((threadIdx.x & (HE_WAVE - 1)) == 0) sh.red[threadIdx.x >> 6] = (u64)(uint32_t)best;
+    __syncthreads();
+    for (int w = 0; w < SAMP_THREADS / HE_WAVE; ++w) best = min(best, (int)(uint32_t)sh.red[w]);
+    __syncthreads();
+    if (best == 0x7fffffff) return 0;   // fewer equal keys than the rank: not for a consistent pick
+    after = best;
+  }
+  return after;
+}
+
+// top-k, top-p and the draw on one source. rest: mass of the row's elements that are not
+// in the source (they all come after every element of the source in descending order).
+// Returns false when the answer needs elements outside the source (rest > 0 only).
+template <typename Source>
+__device__ bool choose(const Source& src, float m, float inv_temp, int top_k, float top_p, int V,
+                       u64 u, u64 rest, SampShared& sh, Cut* pick_out) {
+  Cut cut;
+  cut.any = 0;
+  cut.key = 0;
+  cut.ties = 0;
+  if (top_k > 0 && top_k < V) {
+    if ((u64)top_k > set_total<false>(src, m, inv_temp, cut, sh)) return false;
+    cut = descend<false>(src, m, inv_temp, cut, (u64)top_k, sh);
+    rest = 0;   // the set is inside the source
+  }
+  u64 inside = set_total<true>(src, m, inv_temp, cut, sh);
+  u64 Z = inside + rest;
+  if (top_p > 0.f && top_p < 1.f) {
+    u64 target = (u64)ceil((double)top_p * (double)Z);
+    if (target < 1) target = 1;
+    if (target > Z) target = Z;
+    if (target > inside) return false;
+    cut = descend<true>(src, m, inv_temp, cut, target, sh);
+    inside = set_total<true>(src, m, inv_temp, cut, sh);
+    Z = inside;
+  }
+  // r = floor(u * Z / 2^32), Z < 2^58
+  const u64 r = u * (Z >> 32) + ((u * (Z & 0xffffffffull)) >> 32);
+  if (r + 1 > inside) return false;
+  *pick_out = descend<true>(src, m, inv_temp, cut, r + 1, sh);
+  return true;
+}
+
+// One workgroup per row. Two passes over the row: (1) its maximum; (2) its largest
+// elements - all whose key is at least a threshold - go into a list in LDS, and the mass
+// of all others is summed. The threshold is the value that a strided sample of the row
+// puts at the rank which aims at SAMP_AIM list elements (the list holds twice that; a row
+// no longer than the list goes in whole). top-k, top-p and the draw then run on the list.
+// When they need more than the list holds (a top-k beyond it, a nucleus or a draw that
+// reaches into the rest, a list that overflowed) the same steps run on the whole row
+// instead, many passes over it: rare, and the result is the same either way.
+#define SAMP_LIST 6144
+#define SAMP_AIM 3072
+#define SAMP_SAMPLE 4096
+
+__global__ __launch_bounds__(SAMP_THREADS) void sample_rows_kernel(
+    int32_t* __restrict__ out, const float* __restrict__ logits, int V, int64_t stride,
+    const uint32_t* __restrict__ uniforms, float inv_temp, int top_k, float top_p) {
+  __shared__ SampShared sh;
+  __shared__ int s_counts[SAMP_THREADS];
+  __shared__ float list_v[SAMP_LIST];
+  __shared__ int list_i[SAMP_LIST];
+  __shared__ int list_n;
+  const float* x = logits + blockIdx.x * stride;
+
+  // pass 1: row maximum
+  float best = -INFINITY;
+  if (((stride & 3) == 0) && ((((uintptr_t)logits) & 15) == 0)) {
+    const int V4 = V & ~3;
+    for (int i = 4 * threadIdx.x; i < V4; i += 4 * SAMP_THREADS) {
+      const float4 v = *reinterpret_cast<const float4*>(x + i);
+      best = fmaxf(fmaxf(best, clean(v.x)), fmaxf(clean(v.y), fmaxf(clean(v.z), clean(v.w))));
+    }
+    for (int i = V4 + threadIdx.x; i < V; i += SAMP_THREADS) best = fmaxf(best, clean(x[i]));
+  } else {
+    for (int i = threadIdx.x; i < V; i += SAMP_THREADS) best = fmaxf(best, clean(x[i]));
+  }
+  best = wave_max(best);
+  if (threadIdx.x == 0) list_n = 0;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) sh.red[threadIdx.x >> 6] = (u64)__float_as_uint(best);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float mm = -INFINITY;
+    for (int w = 0; w < SAMP_THREADS / HE_WAVE; ++w)
+      mm = fmaxf(mm, __uint_as_float((uint32_t)sh.red[w]));
+    sh.m = mm;
+  }
+  __syncthreads();
+  const float m = sh.m;
+  if (!(m > -INFINITY)) {  // nothing finite: fall back to index 0
+    if (threadIdx.x == 0) out[blockIdx.x] = 0;
+    return;
+  }
+  const u64 u = (u64)uniforms[blockIdx.x];
+  Cut pick;
+
+  // the threshold key of the list
+  uint32_t threshold = 0;
+  if (V > SAMP_LIST) {
+    const int n = SAMP_SAMPLE;
+    for (int j = threadIdx.x; j < n; j += SAMP_THREADS) {
+      list_v[j] = clean(x[(int)(((int64_t)j * V) / n)]);
+      list_i[j] = j;
+    }
+    __syncthreads();
+    ListSource sample;
+    sample.v = list_v;
+    sample.idx = list_i;
+    sample.n = n;
+    Cut none;
+    none.any = 0;
+    none.key = 0;
+    none.ties = 0;
+    const u64 rank = ((u64)n * SAMP_AIM + V - 1) / V + 1;
+    threshold = descend<false>(sample, m, inv_temp, none, rank, sh).key;
+    __syncthreads();
+  }
+
+  // pass 2: the list and the mass of the rest. Every wavefront fills a segment of its own;
+  // the slot of an element follows from the ballot of the lanes that append in this turn, so
+  // the wavefronts neither wait for one another nor for a counter in memory.
+  constexpr int SEGMENT = SAMP_LIST / (SAMP_THREADS / HE_WAVE);
+  for (int i = threadIdx.x; i < SAMP_LIST; i += SAMP_THREADS) list_i[i] = -1;
+  if (threadIdx.x == 0) list_n = 0;   // becomes 1 when a segment overflows
+  __syncthreads();
+  const int lane = threadIdx.x & (HE_WAVE - 1), wave = threadIdx.x >> 6;
+  int filled = 0;                     // the same in all lanes of the wavefront
+  u64 rest_local = 0;
+  auto take = [&](float raw, int i, bool in_range) {
+    const float v = clean(raw);
+    const bool mine = in_range && ordered_key(v) >= threshold;
+    const unsigned long long appenders = __builtin_amdgcn_ballot_w64(mine);
+    if (mine) {
+      const int at = filled + __builtin_popcountll(appenders & ((1ull << lane) - 1ull));
+      if (at < SEGMENT) {
+        list_v[wave * SEGMENT + at] = v;
+        list_i[wave * SEGMENT + at] = i;
+      }
+    } else if (in_range) {
+      rest_local += fixed_mass(v, m, inv_temp);
+    }
+    filled += __builtin_popcountll(appenders);
+  };
+  if (V > SAMP_LIST && ((stride & 3) == 0) && ((((uintptr_t)logits) & 15) == 0)) {
+    // 16 bytes a load, the next one on its way while this one is looked at; all lanes of a
+    // wavefront make the same number of turns
+    const int V4 = V & ~3;
+    const int turns = (V4 + 4 * SAMP_THREADS - 1) / (4 * SAMP_THREADS);
+    int i = 4 * threadIdx.x;
+    float4 cur = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (i < V4) cur = *reinterpret_cast<const float4*>(x + i);
+    for (int t = 0; t < turns; ++t) {
+      const int nx = i + 4 * SAMP_THREADS;
+      float4 nxt = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (nx < V4) nxt = *reinterpret_cast<const float4*>(x + nx);
+      const bool in = i < V4;
+      take(cur.x, i, in);
+      take(cur.y, i + 1, in);
+      take(cur.z, i + 2, in);
+      take(cur.w, i + 3, in);
+      cur = nxt;
+      i = nx;
+    }
+    const int j = V4 + threadIdx.x;
+    take(j < V ? x[j] : 0.f, j, j < V);   // at most three elements are left
+  } else {
+    const int turns = (V + SAMP_THREADS - 1) / SAMP_THREADS;
+    for (int t = 0; t < turns; ++t) {
+      const int i = threadIdx.x + t * SAMP_THREADS;
+      take(i < V ? x[i] : 0.f, i, i < V);
+    }
+  }
+  if (lane == 0 && filled > SEGMENT) list_n = 1;
+  const u64 rest = block_sum_u64(rest_local, sh);   // its barriers also publish list_n
+  ListSource list;
+  list.v = list_v;
+  list.idx = list_i;
+  list.n = SAMP_LIST;
+  if (list_n == 0 && choose(list, m, inv_temp, top_k, top_p, V, u, rest, sh, &pick)) {
+    int res = pick_index_list(list, pick, sh);
+    if (res < 0) res = pick_index_row(x, V, pick, s_counts);
+    if (threadIdx.x == 0) out[blockIdx.x] = res;
+    return;
+  }
+  RowSource row;
+  row.x = x;
+  row.n = V;
+  choose(row, m, inv_temp, top_k, top_p, V, u, 0, sh, &pick);
+  const int res = pick_index_row(x, V, pick, s_counts);
+  if (threadIdx.x == 0) out[blockIdx.x] = res;
 }
 
 extern "C" int he_sample_rows(void* out_i32, const void* logits_f32, int rows, int V,

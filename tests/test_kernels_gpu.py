@@ -691,6 +691,40 @@ def test_sample_rows_equals_plain(ops, V, temperature, top_k, top_p):
         assert got == [P.argmax_lowest(r) for r in x]
 
 
+@pytest.mark.parametrize("case", ["top_k beyond the list", "all equal", "ties at the threshold", "two values",
+                                  "deep nucleus"])
+def test_sample_rows_list_and_whole_row_agree(ops, case):
+    """The kernel works on a list of the row's largest elements and falls back to the whole row
+    when that is not enough; both must give the plain implementation's token."""
+    V = 40000
+    x = rnd(4, V, seed=63, scale=2.0)
+    temperature, top_k, top_p = 0.9, 0, 1.0
+    if case == "top_k beyond the list":
+        top_k = 9000
+    elif case == "all equal":
+        x[:] = 1.5
+    elif case == "ties at the threshold":
+        x = torch.round(x * 2) / 2                 # a few dozen distinct values, thousands of ties each
+        top_k = 500
+    elif case == "two values":
+        x[:] = -4.0
+        x[:, ::7] = 3.0
+        top_p = 0.5
+    elif case == "deep nucleus":
+        top_p = 0.9999
+        temperature = 3.0                          # flat: the nucleus reaches far beyond the list
+    us = [0, 2 ** 32 - 1, 123456789, 3000000000]
+    u = torch.tensor(us, dtype=torch.int64).to(torch.uint32)
+    out = torch.empty(4, dtype=torch.int32, device="cuda")
+    ops.sample_rows(out, dev(x), 4, dev(u), temperature, top_k, top_p)
+    got = out.tolist()
+    want = [P.sample(x[r], temperature, top_k, top_p, us[r]) for r in range(4)]
+    for r in range(4):
+        if got[r] != want[r]:                      # a last-bit difference of exp(): neighbours in the order
+            order = torch.argsort(-x[r].double(), stable=True).tolist()
+            assert abs(order.index(got[r]) - order.index(want[r])) == 1, (case, r, got[r], want[r])
+
+
 def test_sample_frequencies(ops):
     """Empirical frequencies follow softmax(logits / T) on a small vocabulary."""
     V, n = 8, 20000
