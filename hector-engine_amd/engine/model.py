@@ -83,7 +83,9 @@ class DecoderModel:
                 ctx.next_norm = getattr(self.blocks[self.schedule[e + 1].layer], "mixer_norm", None)
             else:
                 ctx.next_norm = self.final_norm if (ctx.want_all and n_want == rows) else None
+            ctx.scratch.begin_layer()
             self.blocks[entry.layer].forward(stream, ctx, caches[e])
+        ctx.scratch.end_layers()
         ctx.next_norm = None
         if n_want == 0:
             stream.materialize(ctx)

@@ -73,8 +73,10 @@ class GatedMLP(FeedForward):
         out = ctx.alloc((rows, self.hidden))
         for r0 in range(0, rows, _ROW_CHUNK):
             n = min(_ROW_CHUNK, rows - r0)
+            turn = ctx.scratch.mark()
             h = ctx.alloc((n, self.inter))
             gu = self.gate_up(x[r0:r0 + n], n, ctx)
             ops.silu_mul(h, gu, n, self.interleaved)
             self.down(h, n, ctx, out=out[r0:r0 + n])
+            ctx.scratch.release(turn)       # the next turn reuses h and gate||up
         return out

@@ -299,3 +299,28 @@ def test_a_reused_slot_holds_nothing_of_its_past(engines, plain_models):
     eng.release(s2)
     assert torch.equal(first, again)
     close(again, plain_logits(plain_models, "B", short), "float32")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_step_of_thousands_of_rows(model_dirs, plain_models, dtype):
+    """24 prompts of 400 tokens in one step: more rows than the feed-forward holds at once (it
+    then works in turns and gives their temporaries back), layers that take the activation
+    arenas in turn, and the decode step after it."""
+    import hector_engine_amd as he
+    name = "C"
+    vocab = plain_models[name][0]["vocab_size"]
+    eng = he.Engine(model_dirs[name], dtype=dtype, max_tokens=24 * 448, max_slots=24, max_seq_len=448)
+    prompts = [rand_ids(vocab, 400 - (i % 3), 300 + i) for i in range(24)]
+    slots = [eng.acquire() for _ in prompts]
+    got = eng.step([entry(s, p, [0, len(p) - 1]) for s, p in zip(slots, prompts)])
+    assert sum(len(p) for p in prompts) > 8192
+    for i in (0, 7, 23):
+        want = plain_logits(plain_models, name, prompts[i])
+        close(got[2 * i:2 * i + 2], want[[0, len(prompts[i]) - 1]], dtype)
+    nxt = [int(t) for t in got[1::2].argmax(-1).tolist()]
+    got2 = eng.step([entry(s, [t], [0]) for s, t in zip(slots, nxt)])
+    for i in (0, 23):
+        want = plain_logits(plain_models, name, prompts[i] + [nxt[i]])
+        close(got2[i:i + 1], want[-1:], dtype)
+    for s in slots:
+        eng.release(s)
