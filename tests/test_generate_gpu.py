@@ -124,6 +124,23 @@ def test_command_line(model_dirs, plain_models):
     assert ",".join(map(str, t)) in out.stdout
 
 
+def test_command_line_with_the_library_tuner(model_dirs, tmp_path):
+    """--tune-gemm: tall bfloat16 products go through the library's tuner (its own process, since the
+    tuner is process-wide); the same tokens as without it where the decision is clear."""
+    exe = os.path.join(ROOT, "bin", "hector_generate")
+    prompt = ",".join(str(7 + (i * 37) % 200) for i in range(48))          # 48 rows: a library product
+    env = dict(os.environ, TMPDIR=str(tmp_path))
+    runs = []
+    for extra in ([], ["--tune-gemm"]):
+        out = subprocess.run([sys.executable, exe, model_dirs["A"], prompt, "4", "--dtype", "bfloat16"] + extra,
+                             capture_output=True, text=True, timeout=300, env=env)
+        assert out.returncode == 0, out.stderr
+        runs.append([l for l in out.stdout.splitlines() if l.startswith("[0]")])
+    assert runs[0] and runs[1]
+    first = lambda lines: lines[0].rsplit(": ", 1)[-1].split(",")[0]       # "...(max_tokens): 12,7,..."
+    assert first(runs[0]).isdigit() and first(runs[0]) == first(runs[1])
+
+
 def test_smoke_entry():
     sys.path.insert(0, ROOT)
     import __graft_entry__
