@@ -300,6 +300,43 @@ def toys(fw):
             if k is not None:
                 k.copy_((k.float() * f).to(k.dtype))
 
+    @parts.register_part("feed_forward", "toy_top1_experts")
+    class Top1Experts(parts.FeedForward):
+        """A router picks one of E gated MLPs per token (fp32 logits, the lowest index on ties).
+        Every expert runs on every row and a mask keeps the chosen one: slow and simple, and
+        without a host decision, so one-token steps can still be captured."""
+
+        def __init__(self, params, prefix, env):
+            super().__init__(prefix, env)
+            self.D = parts.param(params, "hidden_size", int)
+            self.I = parts.param(params, "intermediate_size", int)
+            self.E = parts.param(params, "experts", int)
+
+        def tensor_specs(self):
+            specs = {self.prefix + "router.weight": parts.TensorSpec((self.E, self.D))}
+            for e in range(self.E):
+                q = f"{self.prefix}experts.{e}."
+                specs[q + "gate_proj.weight"] = parts.TensorSpec((self.I, self.D))
+                specs[q + "up_proj.weight"] = parts.TensorSpec((self.I, self.D))
+                specs[q + "down_proj.weight"] = parts.TensorSpec((self.D, self.I))
+            return specs
+
+        def bind(self, tensors):
+            self.t = {k[len(self.prefix):]: v for k, v in tensors.items() if k.startswith(self.prefix)}
+
+        def forward(self, x, ctx):
+            rows = ctx.rows
+            xs = x[:rows]
+            chosen = (xs.float() @ self.t["router.weight"].float().T).argmax(-1)
+            out = ctx.alloc((rows, self.D))
+            out.zero_()
+            for e in range(self.E):
+                g = xs @ self.t[f"experts.{e}.gate_proj.weight"].T
+                u = xs @ self.t[f"experts.{e}.up_proj.weight"].T
+                y = (torch.nn.functional.silu(g.float()) * u.float()).to(xs.dtype) @ self.t[f"experts.{e}.down_proj.weight"].T
+                out += y * (chosen == e)[:, None].to(y.dtype)
+            return out
+
     @dataclasses.dataclass
     class ToyConfig(ModelConfig):
         vocab_size: int = 0
@@ -325,11 +362,12 @@ def toys(fw):
             return parts.PartSpec("attention", {"hidden_size": D, "num_heads": 4, "num_kv_heads": 2,
                                                 "head_dim": 16, "qkv_bias": True, "position": pos})
 
-        def block(mixer):
+        def block(mixer, feed_forward=ff):
             return parts.PartSpec("pre_norm", {"mixer_norm": norm, "feed_forward_norm": norm, "mixer": mixer,
-                                               "feed_forward": ff, "names": names})
+                                               "feed_forward": feed_forward, "names": names})
 
         rotary = parts.PartSpec("rotary", {"head_dim": 16, "theta": 1e4})
+        routed = parts.PartSpec("toy_top1_experts", {"hidden_size": D, "intermediate_size": D + 16, "experts": 3})
         if cfg.kind == "state":
             mixers = [attn(rotary), parts.PartSpec("toy_running_mean", {"hidden_size": D}), attn(rotary)]
             schedule = [parts.ScheduleEntry(0), parts.ScheduleEntry(1), parts.ScheduleEntry(2)]
@@ -339,13 +377,18 @@ def toys(fw):
         elif cfg.kind == "twice":
             mixers = [attn(rotary), attn(rotary)]
             schedule = [parts.ScheduleEntry(0), parts.ScheduleEntry(1), parts.ScheduleEntry(1)]
+        elif cfg.kind == "routed":   # the last layer's feed-forward routes each token to one of three experts
+            mixers = [attn(rotary), attn(rotary)]
+            schedule = [parts.ScheduleEntry(0), parts.ScheduleEntry(1)]
         else:   # "shared": the third run reads the keys and values the second run wrote
             mixers = [attn(rotary), attn(rotary)]
             schedule = [parts.ScheduleEntry(0), parts.ScheduleEntry(1), parts.ScheduleEntry(1, cache_from=1)]
         return parts.ModelSpec(
             hidden_size=D, vocab_size=V,
             embedding=parts.PartSpec("token_embedding", {"vocab_size": V, "hidden_size": D}),
-            embedding_prefix="emb.", layers=[parts.LayerSpec(f"layers.{i}.", block(m)) for i, m in enumerate(mixers)],
+            embedding_prefix="emb.",
+            layers=[parts.LayerSpec(f"layers.{i}.", block(m, routed if cfg.kind == "routed" and i == 1 else ff))
+                    for i, m in enumerate(mixers)],
             schedule=schedule, final_norm=norm, final_norm_prefix="norm.",
             head=parts.PartSpec("linear_head", {"vocab_size": V, "hidden_size": D}), head_prefix="head.",
             max_positions=512)
@@ -373,10 +416,20 @@ def toy_plain(w, kind, ids):
             k, v = kv
         return P.linear(P.attention(q, k, v, pos, pos), w[p + "o_proj.weight"]), (k, v)
 
+    margins = []
+
     def ff(l, h):
         p = f"layers.{l}."
-        return h + P.swiglu(P.rmsnorm(h, w[p + "ln2.weight"], 1e-5), w[p + "ff.gate_proj.weight"],
-                            w[p + "ff.up_proj.weight"], w[p + "ff.down_proj.weight"])
+        n2 = P.rmsnorm(h, w[p + "ln2.weight"], 1e-5)
+        if p + "ff.router.weight" in w:      # one expert per token
+            logits = n2 @ w[p + "ff.router.weight"].T
+            top = logits.topk(2, -1).values
+            margins.append((top[:, 0] - top[:, 1]) / logits.abs().max())
+            chosen = [P.argmax_lowest(r) for r in logits]
+            rows = [P.swiglu(n2[i:i + 1], w[f"{p}ff.experts.{e}.gate_proj.weight"], w[f"{p}ff.experts.{e}.up_proj.weight"],
+                             w[f"{p}ff.experts.{e}.down_proj.weight"]) for i, e in enumerate(chosen)]
+            return h + torch.cat(rows)
+        return h + P.swiglu(n2, w[p + "ff.gate_proj.weight"], w[p + "ff.up_proj.weight"], w[p + "ff.down_proj.weight"])
 
     rot = lambda t: P.rope(t, pos, 1e4)
     scale = lambda t: t * (1 + pos.double() / 100)[:, None, None]
@@ -387,6 +440,8 @@ def toy_plain(w, kind, ids):
         runs = [(0, scale, None), (1, same, None)]
     elif kind == "twice":
         runs = [(0, rot, None), (1, rot, None), (1, rot, None)]
+    elif kind == "routed":
+        runs = [(0, rot, None), (1, rot, None)]
     else:
         runs = [(0, rot, None), (1, rot, None), (1, rot, 1)]
     kvs = {}
@@ -397,7 +452,10 @@ def toy_plain(w, kind, ids):
         else:
             a, kvs[e] = attn(l, n, enc, kvs[src] if src is not None else None)
         x = ff(l, x + a)
-    return P.linear(P.rmsnorm(x, w["norm.weight"], 1e-5), w["head.weight"])
+    out = P.linear(P.rmsnorm(x, w["norm.weight"], 1e-5), w["head.weight"])
+    if margins:      # the routed toy: also how clear each token's choice of expert was
+        return out, margins[-1]
+    return out
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -450,6 +508,35 @@ def test_toy_models_build_and_step(fw, toys, tmp_path, kind, dtype):
                     live.remove(i)
         for i in batch:
             close(torch.cat(got[i]), want[i], dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_toy_feed_forward_with_routing(fw, toys, tmp_path, dtype):
+    """A routed feed-forward registered in the test: built, stepped whole and token by token (captured
+    one-token steps included), and fed with plain rows although the mixer before it left its result as
+    rows for the norm (the part does not take those)."""
+    import hector_engine_amd as he
+    from hector_engine_amd.engine.engine import StepEntry
+    cfg = toys(architecture="ToyForCausalLM", vocab_size=97, hidden_size=64, kind="routed")
+    folder = str(tmp_path / "routed")
+    he.write_random_model(cfg, 6, folder)
+    w = {k: v.double() for k, v in P.read_safetensors(os.path.join(folder, "model.safetensors")).items()}
+    eng = he.Engine(folder, dtype=dtype, max_tokens=1024, max_slots=2, max_seq_len=256)
+    assert eng.use_graphs
+    ids = rand_ids(97, 40, 91)
+    want, margin = toy_plain(w, "routed", ids)
+    clear = (margin > (0.0 if dtype == "float32" else 0.05)).nonzero().flatten().tolist()
+    assert len(clear) >= 25
+    s = eng.acquire()
+    close(eng.step([StepEntry(s, ids, clear)]), want[clear], dtype)
+    eng.release(s)
+    s = eng.acquire()
+    got = [eng.step([StepEntry(s, ids[:8], list(range(8)))])]
+    for t in ids[8:]:
+        got.append(eng.step([StepEntry(s, [t], [0])]).clone())
+    close(torch.cat(got)[clear], want[clear], dtype)
+    assert eng.stats["graph_replays"] > 20
+    eng.release(s)
 
 
 def test_bad_schedules_are_refused(fw, toys):
