@@ -206,20 +206,24 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
   }
 }
 
-// Wavefronts per workgroup and workgroups per (sequence, kv head, head tile). Many
-// sequences: one workgroup of 8 wavefronts each, no second launch. Few: 4 wavefronts and
-// enough workgroups to put about 512 on the chip, while a slice keeps 64 keys at max_keys.
+// Wavefronts per workgroup and workgroups per (sequence, kv head, head tile), measured on
+// MI355X at 4 kv heads of 128 from 1 to 64 sequences and 500 to 8000 keys: with 256 or more
+// (sequence, kv head) pairs one workgroup of 8 wavefronts each and no second launch; below,
+// 4 wavefronts and as many workgroups per pair as bring the grid to about 256 (one per
+// compute unit; at 32 sequences that is 41 us against 52 us for one workgroup per pair), at
+// most 16 (32 for contexts beyond 16384), while a slice keeps 64 keys at max_keys.
 static void fused_shape(int rows, int H, int KVH, int hd, int max_keys, int* nw, int* Z) {
   const int G = H / KVH;
   const int gt = G < 16 ? G : 16;
   const int groups = rows * KVH * ((G + 15) / 16);
   int w = (int64_t)8 * gt * (hd + 2) * 4 <= 65536 ? 8 : 4, zz = 1;
-  if (groups < 128) {
+  if (groups < 256) {
     w = 4;
-    zz = (512 + groups - 1) / groups;
+    zz = (256 + groups - 1) / groups;
+    const int cap = max_keys > 16384 ? 32 : 16;
+    if (zz > cap) zz = cap;
     const int most = (max_keys + 4 * FUSED_MIN_CHUNK - 1) / (4 * FUSED_MIN_CHUNK);
     if (zz > most) zz = most;
-    if (zz > 64) zz = 64;
     if (zz < 1) zz = 1;
   }
   *nw = w;
