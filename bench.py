@@ -16,7 +16,7 @@ import time
 
 import numpy as np
 
-# Qwen2.5-7B layer sizes (BASELINE.json configs[2])
+# Qwen2.5-7B layer sizes: the model configuration this benchmark is quoted on
 SHAPE = dict(num_hidden_layers=28, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
              head_dim=128, intermediate_size=18944, vocab_size=152064, rope_theta=1000000.0,
              rms_norm_eps=1e-6, max_position_embeddings=32768, tie_word_embeddings=False)
