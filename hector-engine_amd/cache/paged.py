@@ -20,6 +20,7 @@ import dataclasses
 import torch
 
 from ..parts.base import KVNeed, LayerCache
+from . import layout
 from .pages import PAGE_TOKENS, CacheError, CacheFull, GroupPages, SlotBook, blocks_for  # noqa: F401
 
 
@@ -39,10 +40,10 @@ class _Group:
         self.runs = runs
         # zero-filled once (as the reference's cache is: src/kv_cache.hpp:161-203): a masked
         # key still enters the matrix products with weight 0, so it must never be NaN
-        self.kpool = torch.zeros((len(runs), num_pages, need.kv_heads, PAGE_TOKENS, need.head_dim),
+        # a page of a kv head is kept in the order the attention kernels read it (cache/layout.py)
+        self.kpool = torch.zeros((len(runs), num_pages, need.kv_heads, layout.k_page_elems(need.head_dim)),
                                  dtype=dtype, device=device)
-        # V is transposed inside a page so that 8 consecutive tokens of one dim are contiguous
-        self.vpool = torch.zeros((len(runs), num_pages, need.kv_heads, need.head_dim, PAGE_TOKENS),
+        self.vpool = torch.zeros((len(runs), num_pages, need.kv_heads, layout.v_page_elems(need.head_dim)),
                                  dtype=dtype, device=device)
         self.page_table = torch.full((max_slots, max_blocks), -1, dtype=torch.int32, device=device)
 
@@ -161,4 +162,6 @@ class PagedCache:
 
     def bytes_per_token(self) -> int:
         es = torch.empty((), dtype=self.dtype).element_size()
-        return sum(2 * len(g.runs) * g.need.kv_heads * g.need.head_dim * es for g in self.groups)
+        return sum(len(g.runs) * g.need.kv_heads * es
+                   * (layout.k_page_elems(g.need.head_dim) + layout.v_page_elems(g.need.head_dim)) // PAGE_TOKENS
+                   for g in self.groups)

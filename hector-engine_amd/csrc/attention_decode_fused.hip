@@ -120,8 +120,9 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
       const int off = p & (HE_PAGE_TOKENS - 1);
       const int half = rotary_dim >> 1;
       const int k_col = H * HD + kvh * HD, v_col = (H + KVH) * HD + kvh * HD;
-      uint16_t* krow = kpool + (((int64_t)page * KVH + kvh) * HE_PAGE_TOKENS + off) * HD;
-      uint16_t* vcol = vpool + ((int64_t)page * KVH + kvh) * HD * HE_PAGE_TOKENS + off;
+      // the page in operand order (cache_layout.h)
+      uint16_t* kpage = kpool + ((int64_t)page * KVH + kvh) * he_k_page_elems(HD);
+      uint16_t* vpage = vpool + ((int64_t)page * KVH + kvh) * he_v_page_elems(HD);
       if (lane < half) {                     // half <= 64: one pair per lane
         const int j = lane;
         float x0 = bf16_bits_to_float(qkv_row[k_col + j]);
@@ -130,13 +131,13 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
           x0 += load_param(bias, k_col + j, bias_dtype);
           x1 += load_param(bias, k_col + j + half, bias_dtype);
         }
-        krow[j] = float_to_bf16_bits(x0 * c - x1 * sn);
-        krow[j + half] = float_to_bf16_bits(x0 * sn + x1 * c);
+        kpage[he_k_index(off, j, KS)] = float_to_bf16_bits(x0 * c - x1 * sn);
+        kpage[he_k_index(off, j + half, KS)] = float_to_bf16_bits(x0 * sn + x1 * c);
       }
       for (int d = lane; d < HD; d += 64) {
         float x = bf16_bits_to_float(qkv_row[v_col + d]);
         if (bias) x += load_param(bias, v_col + d, bias_dtype);
-        vcol[(int64_t)d * HE_PAGE_TOKENS] = float_to_bf16_bits(x);
+        vpage[he_v_index(off, d, NT)] = float_to_bf16_bits(x);
       }
     }
     __threadfence_block();   // this wavefront reads the row back below

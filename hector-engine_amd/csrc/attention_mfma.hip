@@ -92,8 +92,9 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 // grid (ceil(max_q_len / 128), H, num_seqs), 256 threads. The workgroup takes 128
 // consecutive queries of one sequence and head, wavefront w the 32 queries 32w..32w+31 as
 // two tiles. The keys are walked a page (64 keys) at a time: the page's K and V^T are copied
-// once into LDS, already in the order the MFMA operands are read (one operand of all 64
-// lanes is one contiguous KiB, so the reads have no bank conflicts), and every operand a
+// once into LDS as the cache holds them, in the order the MFMA operands are read (one
+// operand of all 64 lanes is one contiguous KiB, so the reads have no bank conflicts, and
+// neither have the staging stores), and every operand a
 // wavefront reads from LDS feeds two MFMAs, one per tile - with one tile a wavefront the LDS
 // reads (32 KiB a page and wavefront), not the matrix cores, set the pace. The page in LDS
 // is double-buffered: the next page is written into the other buffer while this one is
@@ -155,74 +156,54 @@ __device__ __forceinline__ bf16x8 softmax_step(AttnState<NT>& st, const floatx4*
 
 typedef uint32_t pf2_vec __attribute__((ext_vector_type(4)));   // 16 bytes, a native vector
 
-// A page of K and of V^T of one kv head, global memory -> registers (16-byte chunks, one
-// per thread and turn) -> LDS in operand order.
+// A page of K and of V^T of one kv head, global memory -> registers -> LDS, 16-byte pieces,
+// one per thread and turn. The cache keeps its pages in operand order (cache_layout.h), so
+// the copy is straight: piece c goes to slot c, neighbouring threads write neighbouring
+// slots, and an operand read (64 lanes x 16 bytes, contiguous) has no bank conflicts.
 template <int NT>
 struct Pf2 {
   static constexpr int HD = 16 * NT;
   static constexpr int KS = (HD + 31) / 32;
-  static constexpr int CHUNKS = HE_PAGE_TOKENS * HD / 8;
   static constexpr int THREADS = 64 * PF2_WAVES;
-  static constexpr int PER_THREAD = (CHUNKS + THREADS - 1) / THREADS;
+  static constexpr int K_PIECES = 2 * 2 * KS * 64, V_PIECES = 2 * NT * 64;
+  static constexpr int K_TURNS = (K_PIECES + THREADS - 1) / THREADS;
+  static constexpr int V_TURNS = (V_PIECES + THREADS - 1) / THREADS;
 };
 
-__device__ __forceinline__ int pf2_kx(int ks, int a) { return ((ks & 3) << 2) | a; }
-__device__ __forceinline__ int pf2_vx(int hb, int a) { return (hb << 3) | (a << 1); }
-
 template <int NT>
-__device__ __forceinline__ void pf2_fetch(pf2_vec (&kreg)[Pf2<NT>::PER_THREAD],
-                                          pf2_vec (&vreg)[Pf2<NT>::PER_THREAD],
+__device__ __forceinline__ void pf2_fetch(pf2_vec (&kreg)[Pf2<NT>::K_TURNS],
+                                          pf2_vec (&vreg)[Pf2<NT>::V_TURNS],
                                           const uint16_t* __restrict__ kp,
                                           const uint16_t* __restrict__ vp, int page, int num_pages,
-                                          int64_t page_stride) {
+                                          int64_t k_stride, int64_t v_stride) {
   if (page < 0 || page >= num_pages) page = 0;   // never for an admitted batch
 #pragma unroll
-  for (int j = 0; j < Pf2<NT>::PER_THREAD; ++j) {
+  for (int j = 0; j < Pf2<NT>::K_TURNS; ++j) {
     const int c = threadIdx.x + Pf2<NT>::THREADS * j;
-    if (c < Pf2<NT>::CHUNKS) {
-      kreg[j] = *reinterpret_cast<const pf2_vec*>(kp + (int64_t)page * page_stride + 8 * c);
-      vreg[j] = *reinterpret_cast<const pf2_vec*>(vp + (int64_t)page * page_stride + 8 * c);
-    }
+    if (c < Pf2<NT>::K_PIECES)
+      kreg[j] = *reinterpret_cast<const pf2_vec*>(kp + (int64_t)page * k_stride + 8 * c);
   }
-}
-
-// Where the chunks of this thread go in LDS. An operand (64 lanes x 16 bytes) is one KiB;
-// inside it, lane 16a + c sits at slot 16a + (c ^ x), x chosen per operand and a so that the
-// 16 chunks that neighbouring threads store at once (one key row, or two rows of V^T) fall
-// into 16 different 16-byte columns of the 256-byte bank row, as the 16 lanes of one read do.
-// Without it the stores of a wavefront hit 4 columns (K) or 2 (V^T) and serialise.
-template <int NT>
-__device__ __forceinline__ void pf2_slots(int (&kdst)[Pf2<NT>::PER_THREAD],
-                                          int (&vdst)[Pf2<NT>::PER_THREAD]) {
-  constexpr int HD = Pf2<NT>::HD, KS = Pf2<NT>::KS;
 #pragma unroll
-  for (int j = 0; j < Pf2<NT>::PER_THREAD; ++j) {
+  for (int j = 0; j < Pf2<NT>::V_TURNS; ++j) {
     const int c = threadIdx.x + Pf2<NT>::THREADS * j;
-    // K chunk: key krow, dims 8*kcol..+8 -> operand (half, tile, k step), lane 16a + cc
-    const int krow = c / (HD / 8), kcol = c % (HD / 8);
-    const int kl = krow & 31;
-    const int ks = kcol >> 2, a = kcol & 3, cc = ((kl >> 3) << 2) | (kl & 3);
-    kdst[j] = (((krow >> 5) * 2 + ((kl >> 2) & 1)) * KS + ks) * 64 + 16 * a + (cc ^ pf2_kx(ks, a));
-    // V^T chunk: dim vrow, keys 8*vcol..+8 -> operand (half, dim tile), lane 16a + cc
-    const int vrow = c / (HE_PAGE_TOKENS / 8), vcol = c % (HE_PAGE_TOKENS / 8);
-    const int hb = vcol >> 2, va = vcol & 3;
-    vdst[j] = (hb * NT + (vrow >> 4)) * 64 + 16 * va + ((vrow & 15) ^ pf2_vx(hb, va));
+    if (c < Pf2<NT>::V_PIECES)
+      vreg[j] = *reinterpret_cast<const pf2_vec*>(vp + (int64_t)page * v_stride + 8 * c);
   }
 }
 
 template <int NT>
-__device__ __forceinline__ void pf2_stage(const pf2_vec (&kreg)[Pf2<NT>::PER_THREAD],
-                                          const pf2_vec (&vreg)[Pf2<NT>::PER_THREAD],
-                                          const int (&kdst)[Pf2<NT>::PER_THREAD],
-                                          const int (&vdst)[Pf2<NT>::PER_THREAD], pf2_vec* k_lds,
+__device__ __forceinline__ void pf2_stage(const pf2_vec (&kreg)[Pf2<NT>::K_TURNS],
+                                          const pf2_vec (&vreg)[Pf2<NT>::V_TURNS], pf2_vec* k_lds,
                                           pf2_vec* v_lds) {
 #pragma unroll
-  for (int j = 0; j < Pf2<NT>::PER_THREAD; ++j) {
+  for (int j = 0; j < Pf2<NT>::K_TURNS; ++j) {
     const int c = threadIdx.x + Pf2<NT>::THREADS * j;
-    if (c < Pf2<NT>::CHUNKS) {
-      k_lds[kdst[j]] = kreg[j];
-      v_lds[vdst[j]] = vreg[j];
-    }
+    if (c < Pf2<NT>::K_PIECES) k_lds[c] = kreg[j];
+  }
+#pragma unroll
+  for (int j = 0; j < Pf2<NT>::V_TURNS; ++j) {
+    const int c = threadIdx.x + Pf2<NT>::THREADS * j;
+    if (c < Pf2<NT>::V_PIECES) v_lds[c] = vreg[j];
   }
 }
 
@@ -304,8 +285,7 @@ __device__ __forceinline__ void pf2_step(PairTile<NT>& t0, PairTile<NT>& t1, con
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       pf2_vec v = {0u, 0u, 0u, 0u};
-      if (32 * ks + 8 * lg < HD)
-        v = k_lds[((hb * 2 + t) * KS + ks) * 64 + 16 * lg + (lr ^ pf2_kx(ks, lg))];
+      if (32 * ks + 8 * lg < HD) v = k_lds[((hb * 2 + t) * KS + ks) * 64 + 16 * lg + lr];
       const bf16x8 kf = __builtin_bit_cast(bf16x8, v);
       if (D0) s0[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, t0.qf[ks], s0[t], 0, 0, 0);
       if (D1) s1[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, t1.qf[ks], s1[t], 0, 0, 0);
@@ -315,8 +295,7 @@ __device__ __forceinline__ void pf2_step(PairTile<NT>& t0, PairTile<NT>& t1, con
   if (D1) p1 = t1.softmax(s1, key_base, scale_log2, lg);
 #pragma unroll
   for (int dt = 0; dt < NT; ++dt) {
-    const bf16x8 vf = __builtin_bit_cast(
-        bf16x8, v_lds[(hb * NT + dt) * 64 + 16 * lg + (lr ^ pf2_vx(hb, lg))]);
+    const bf16x8 vf = __builtin_bit_cast(bf16x8, v_lds[(hb * NT + dt) * 64 + 16 * lg + lr]);
     if (D0) t0.st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p0, t0.st.o[dt], 0, 0, 0);
     if (D1) t1.st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p1, t1.st.o[dt], 0, 0, 0);
   }
@@ -338,11 +317,9 @@ attention_prefill_pair_kernel(
     int num_pages, int H, int KVH, int window, float scale) {
   constexpr int HD = 16 * NT;
   constexpr int KS = (HD + 31) / 32;
-  constexpr int PER_THREAD = Pf2<NT>::PER_THREAD;
-  constexpr int K_OPS = 2 * 2 * KS * 64, V_OPS = 2 * NT * 64;   // 16-byte slots per buffer
-  // operand-ordered: k[((hb*2 + t)*KS + ks)*64 + slot(lane)], v[(hb*NT + dt)*64 + slot(lane)]
-  __shared__ pf2_vec k_lds[2][K_OPS];
-  __shared__ pf2_vec v_lds[2][V_OPS];
+  // a page as the cache holds it: k[((hb*2 + t)*KS + ks)*64 + lane], v[(hb*NT + dt)*64 + lane]
+  __shared__ pf2_vec k_lds[2][Pf2<NT>::K_PIECES];
+  __shared__ pf2_vec v_lds[2][Pf2<NT>::V_PIECES];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int lr = lane & 15, lg = lane >> 4;
@@ -358,9 +335,9 @@ attention_prefill_pair_kernel(
   const int start = seq_start[seq];
   const int kvh = h / (H / KVH);
   const int32_t* pt = page_table + (int64_t)slot * max_blocks;
-  const int64_t page_stride = (int64_t)KVH * (HE_PAGE_TOKENS * HD);
-  const uint16_t* kp = kpool + (int64_t)kvh * (HE_PAGE_TOKENS * HD);
-  const uint16_t* vp = vpool + (int64_t)kvh * (HE_PAGE_TOKENS * HD);
+  const int64_t k_stride = (int64_t)KVH * he_k_page_elems(HD), v_stride = (int64_t)KVH * he_v_page_elems(HD);
+  const uint16_t* kp = kpool + (int64_t)kvh * he_k_page_elems(HD);
+  const uint16_t* vp = vpool + (int64_t)kvh * he_v_page_elems(HD);
 
   const int pair = pair0 + wave;
   const int ta = pair, tb = tiles - 1 - pair;    // ta <= tb while pair < pairs
@@ -374,19 +351,17 @@ attention_prefill_pair_kernel(
   const int blk_first = window > 0 ? max(0, start + 16 * pair0 + 1 - window) : 0;
   const int pb0 = blk_first >> HE_PAGE_SHIFT, pb1 = blk_last >> HE_PAGE_SHIFT;
 
-  pf2_vec kreg[PER_THREAD], vreg[PER_THREAD];
-  int kdst[PER_THREAD], vdst[PER_THREAD];
-  pf2_slots<NT>(kdst, vdst);
-  pf2_fetch<NT>(kreg, vreg, kp, vp, pt[pb0], num_pages, page_stride);
-  pf2_stage<NT>(kreg, vreg, kdst, vdst, k_lds[0], v_lds[0]);
-  if (pb0 < pb1) pf2_fetch<NT>(kreg, vreg, kp, vp, pt[pb0 + 1], num_pages, page_stride);
+  pf2_vec kreg[Pf2<NT>::K_TURNS], vreg[Pf2<NT>::V_TURNS];
+  pf2_fetch<NT>(kreg, vreg, kp, vp, pt[pb0], num_pages, k_stride, v_stride);
+  pf2_stage<NT>(kreg, vreg, k_lds[0], v_lds[0]);
+  if (pb0 < pb1) pf2_fetch<NT>(kreg, vreg, kp, vp, pt[pb0 + 1], num_pages, k_stride, v_stride);
   __syncthreads();
   for (int pb = pb0; pb <= pb1; ++pb) {
     const int buf = (pb - pb0) & 1;
     if (pb < pb1) {
       // everyone left the other buffer before the last barrier
-      pf2_stage<NT>(kreg, vreg, kdst, vdst, k_lds[buf ^ 1], v_lds[buf ^ 1]);
-      if (pb + 1 < pb1) pf2_fetch<NT>(kreg, vreg, kp, vp, pt[pb + 2], num_pages, page_stride);
+      pf2_stage<NT>(kreg, vreg, k_lds[buf ^ 1], v_lds[buf ^ 1]);
+      if (pb + 1 < pb1) pf2_fetch<NT>(kreg, vreg, kp, vp, pt[pb + 2], num_pages, k_stride, v_stride);
     }
 #pragma unroll
     for (int hb = 0; hb < 2; ++hb) {

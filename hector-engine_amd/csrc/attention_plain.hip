@@ -8,7 +8,7 @@
 // For the query at absolute position p: first = window > 0 ? max(0, p+1-window) : 0,
 // s_j = (q . k_j) * scale for j in [first, p], out = sum_j softmax(s)_j v_j,
 // kv head = h / (H / KVH)   (reference: kernels/attention.cu:155-316, :664-773, :60).
-#include "common.h"
+#include "cache_layout.h"
 #include "hector_kernels.h"
 
 #define AP_MAX_PER_LANE 8
@@ -53,14 +53,15 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(
     const int page = pt[j >> HE_PAGE_SHIFT];
     if (page < 0 || page >= num_pages) continue;  // never for an admitted batch
     const int off = j & (HE_PAGE_TOKENS - 1);
-    const int64_t base = (((int64_t)page * KVH + kvh) * HE_PAGE_TOKENS + off) * hd;
-    // V is stored transposed inside a page: [head_dim][tokens]
-    const int64_t vbase = ((int64_t)page * KVH + kvh) * hd * HE_PAGE_TOKENS + off;
+    // the pages are stored in the MFMA kernels' operand order (cache_layout.h)
+    const int64_t base = ((int64_t)page * KVH + kvh) * he_k_page_elems(hd);
+    const int64_t vbase = ((int64_t)page * KVH + kvh) * he_v_page_elems(hd);
+    const int KS = he_k_steps(hd), NT = he_v_tiles(hd);
     float part = 0.f;
 #pragma unroll
     for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
       const int d = lane + i * HE_WAVE;
-      if (i < npl && d < hd) part = fmaf(qv[i], to_float(kpool[base + d]), part);
+      if (i < npl && d < hd) part = fmaf(qv[i], to_float(kpool[base + he_k_index(off, d, KS)]), part);
     }
     const float s = wave_sum(part) * scale;
     const float m_new = fmaxf(m, s);
@@ -70,7 +71,7 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(
 #pragma unroll
     for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
       const int d = lane + i * HE_WAVE;
-      if (i < npl && d < hd) acc[i] = acc[i] * alpha + w * to_float(vpool[vbase + (int64_t)d * HE_PAGE_TOKENS]);
+      if (i < npl && d < hd) acc[i] = acc[i] * alpha + w * to_float(vpool[vbase + he_v_index(off, d, NT)]);
     }
     m = m_new;
   }

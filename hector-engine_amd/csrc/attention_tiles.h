@@ -3,7 +3,7 @@
 // walks a key range one step ahead with its loads. The layout notes are in
 // attention_mfma.hip.
 #pragma once
-#include "common.h"
+#include "cache_layout.h"
 
 // Online softmax keeps, per query, a reference point m (base-2 domain) and sums of
 // 2^(s - m). Any m gives the same quotient; m need only be close enough to the running
@@ -36,28 +36,26 @@ struct KVFrag {
   int ok;   // the page exists (always, for an admitted batch)
 };
 
-// kpool/vpool of this kv head; page: physical page of the 32 keys; koff: 0 or 32.
+// kpool/vpool of this kv head; page: physical page of the 32 keys; koff: 0 or 32. The pages
+// are stored in operand order (cache_layout.h): every load below is one contiguous KiB.
 template <int NT>
 __device__ __forceinline__ void load_frag(KVFrag<NT>& f, const uint16_t* __restrict__ kpool,
                                           const uint16_t* __restrict__ vpool, int page,
-                                          int num_pages, int64_t page_stride, int koff, int lr,
-                                          int lg) {
+                                          int num_pages, int64_t k_page_stride,
+                                          int64_t v_page_stride, int koff, int lr, int lg) {
   constexpr int HD = 16 * NT;
   constexpr int KS = (HD + 31) / 32;
   f.ok = page >= 0 && page < num_pages;
-  const int64_t pbase = (int64_t)(f.ok ? page : 0) * page_stride;
-  const uint16_t* kpage = kpool + pbase;
-  const uint16_t* vpage = vpool + pbase;
+  const int lane = 16 * lg + lr, h = koff >> 5;
+  const uint16_t* kpage = kpool + (int64_t)(f.ok ? page : 0) * k_page_stride + ((h * 2) * KS * 64 + lane) * 8;
+  const uint16_t* vpage = vpool + (int64_t)(f.ok ? page : 0) * v_page_stride + (h * NT * 64 + lane) * 8;
 #pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    const int key_local = 8 * (lr >> 2) + 4 * t + (lr & 3);
-    const uint16_t* krow = kpage + (koff + key_local) * HD + 8 * lg;
+  for (int t = 0; t < 2; ++t)
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) f.k[t][ks] = ld8(krow + 32 * ks, 32 * ks + 8 * lg < HD);
-  }
+    for (int ks = 0; ks < KS; ++ks)
+      f.k[t][ks] = ld8(kpage + (t * KS + ks) * 512, 32 * ks + 8 * lg < HD);
 #pragma unroll
-  for (int dt = 0; dt < NT; ++dt)
-    f.v[dt] = ld8(vpage + (16 * dt + lr) * HE_PAGE_TOKENS + koff + 8 * lg, true);
+  for (int dt = 0; dt < NT; ++dt) f.v[dt] = ld8(vpage + dt * 512, true);
 }
 
 // One step of 32 keys starting at absolute position key_base (a multiple of 32).
@@ -143,14 +141,14 @@ __device__ __forceinline__ void attend_range(AttnState<NT>& st, const bf16x8* qf
                                              int clear_hi, float scale_log2, int lr, int lg) {
   constexpr int HD = 16 * NT;
   if (kb_begin >= kb_end) return;
-  const int64_t page_stride = (int64_t)KVH * (HE_PAGE_TOKENS * HD);
-  const uint16_t* kp = kpool + (int64_t)kvh * (HE_PAGE_TOKENS * HD);
-  const uint16_t* vp = vpool + (int64_t)kvh * (HE_PAGE_TOKENS * HD);
+  const int64_t k_stride = (int64_t)KVH * he_k_page_elems(HD), v_stride = (int64_t)KVH * he_v_page_elems(HD);
+  const uint16_t* kp = kpool + (int64_t)kvh * he_k_page_elems(HD);
+  const uint16_t* vp = vpool + (int64_t)kvh * he_v_page_elems(HD);
   int block = kb_begin >> HE_PAGE_SHIFT;
   int page = pt[block];
   int page_ahead = pt[min(block + 1, max_blocks - 1)];
   KVFrag<NT> cur, nxt;
-  load_frag<NT>(cur, kp, vp, page, num_pages, page_stride, kb_begin & 32, lr, lg);
+  load_frag<NT>(cur, kp, vp, page, num_pages, k_stride, v_stride, kb_begin & 32, lr, lg);
   for (int kb = kb_begin; kb < kb_end; kb += 32) {
     const int kn = kb + 32;
     if (kn < kb_end) {
@@ -159,7 +157,7 @@ __device__ __forceinline__ void attend_range(AttnState<NT>& st, const bf16x8* qf
         page = page_ahead;
         page_ahead = pt[min(block + 1, max_blocks - 1)];
       }
-      load_frag<NT>(nxt, kp, vp, page, num_pages, page_stride, kn & 32, lr, lg);
+      load_frag<NT>(nxt, kp, vp, page, num_pages, k_stride, v_stride, kn & 32, lr, lg);
     }
     // keys in [clear_lo, clear_hi] are visible to every query of the tile
     if (UNMASKED_STEPS && kb >= clear_lo && kb + 31 <= clear_hi && cur.ok)

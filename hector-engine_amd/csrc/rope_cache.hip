@@ -11,7 +11,7 @@
 //
 // The projected rows may arrive as the fp32 partial sums [splits][rows][width]
 // of a product cut along K; they are added here in the order of the slice index.
-#include "common.h"
+#include "cache_layout.h"
 #include "hector_kernels.h"
 
 #define ROPE_MAX_HALF 256
@@ -89,7 +89,8 @@ __global__ void qkv_rope_cache_kernel(
       const int h = it / per_head;
       const int j = it - h * per_head;
       const int base = h * hd;
-      T* out = kpool + (((int64_t)page * KVH + h) * HE_PAGE_TOKENS + off) * hd;
+      T* out = kpool + ((int64_t)page * KVH + h) * he_k_page_elems(hd);   // the page, in operand order
+      const int KS = he_k_steps(hd);
       if (j < half) {
         float x0 = load_in(in + base + j, splits, split_stride);
         float x1 = load_in(in + base + j + half, splits, split_stride);
@@ -98,13 +99,13 @@ __global__ void qkv_rope_cache_kernel(
           x1 += load_param(k_bias, base + j + half, bias_dtype);
         }
         const float c = cs[0][j], sn = cs[1][j];
-        out[j] = from_float<T>(x0 * c - x1 * sn);
-        out[j + half] = from_float<T>(x0 * sn + x1 * c);
+        out[he_k_index(off, j, KS)] = from_float<T>(x0 * c - x1 * sn);
+        out[he_k_index(off, j + half, KS)] = from_float<T>(x0 * sn + x1 * c);
       } else {
         const int d = rotary_dim + (j - half);
         float x = load_in(in + base + d, splits, split_stride);
         if (k_bias) x += load_param(k_bias, base + d, bias_dtype);
-        out[d] = from_float<T>(x);
+        out[he_k_index(off, d, KS)] = from_float<T>(x);
       }
     }
   }
@@ -116,8 +117,8 @@ __global__ void qkv_rope_cache_kernel(
       const int d = it - h * hd;
       float x = load_in(in + it, splits, split_stride);
       if (v_bias) x += load_param(v_bias, it, bias_dtype);
-      // V is stored transposed inside a page: [head_dim][tokens]
-      vpool[(((int64_t)page * KVH + h) * hd + d) * HE_PAGE_TOKENS + off] = from_float<T>(x);
+      vpool[((int64_t)page * KVH + h) * he_v_page_elems(hd) + he_v_index(off, d, he_v_tiles(hd))] =
+          from_float<T>(x);
     }
   }
 }
@@ -180,13 +181,16 @@ __global__ __launch_bounds__(256) void qkv_rope_cache_vec_kernel(
       const int g = idx - h * per_head;
       const uint16_t* in = (is_q ? q_in : k_in) + row * in_stride + h * hd;
       const uint16_t* bias = is_q ? q_bias : k_bias;
+      // where the eight elements from dim d on go: the q row, or the cache page in operand order
       uint16_t* out;
+      const int KS = he_k_steps(hd);
       if (is_q) {
         out = q_out + row * (int64_t)H * hd + h * hd;
       } else {
         if (!cache_ok) continue;
-        out = kpool + (((int64_t)page * KVH + h) * HE_PAGE_TOKENS + off) * hd;
+        out = kpool + ((int64_t)page * KVH + h) * he_k_page_elems(hd);
       }
+      auto at = [&](int d) { return out + (is_q ? d : he_k_index(off, d, KS)); };
       float x0[8], x1[8], b0[8], b1[8];
       if (g < rot8) {
         const int j = 8 * g;
@@ -205,8 +209,8 @@ __global__ __launch_bounds__(256) void qkv_rope_cache_vec_kernel(
           y0[i] = a0 * c - a1 * sn;
           y1[i] = a0 * sn + a1 * c;
         }
-        *reinterpret_cast<uint4*>(out + j) = pack8(y0);
-        *reinterpret_cast<uint4*>(out + j + half) = pack8(y1);
+        *reinterpret_cast<uint4*>(at(j)) = pack8(y0);
+        *reinterpret_cast<uint4*>(at(j + half)) = pack8(y1);
       } else {
         const int d = rotary_dim + 8 * (g - rot8);
         unpack8(*reinterpret_cast<const uint4*>(in + d), x0);
@@ -215,7 +219,7 @@ __global__ __launch_bounds__(256) void qkv_rope_cache_vec_kernel(
 #pragma unroll
           for (int i = 0; i < 8; ++i) x0[i] += b0[i];
         }
-        *reinterpret_cast<uint4*>(out + d) = pack8(x0);
+        *reinterpret_cast<uint4*>(at(d)) = pack8(x0);
       }
     } else {
       if (!cache_ok) continue;
@@ -228,10 +232,10 @@ __global__ __launch_bounds__(256) void qkv_rope_cache_vec_kernel(
 #pragma unroll
         for (int i = 0; i < 8; ++i) x[i] += b[i];
       }
-      // V is stored transposed inside a page: [head_dim][tokens]
-      uint16_t* out = vpool + (((int64_t)page * KVH + h) * hd + d) * HE_PAGE_TOKENS + off;
+      uint16_t* out = vpool + ((int64_t)page * KVH + h) * he_v_page_elems(hd);
+      const int NT = he_v_tiles(hd);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) out[i * HE_PAGE_TOKENS] = float_to_bf16_bits(x[i]);
+      for (int i = 0; i < 8; ++i) out[he_v_index(off, d + i, NT)] = float_to_bf16_bits(x[i]);
     }
   }
 }

@@ -5,6 +5,7 @@ from __future__ import annotations
 
 import torch
 
+from ..cache import layout
 from . import lib as _lib
 
 F32, BF16 = 0, 1
@@ -327,8 +328,8 @@ def qkv_rope_cache(q_out, kpool, vpool, qkv, q_cols: int, kv_cols: int, bias, po
     k_in = v_in = None
     max_blocks = num_pages = 0
     if write_kv:
-        _need(kpool, "kpool", q_out.dtype, (None, KVH, PAGE_TOKENS, hd))
-        _need(vpool, "vpool", q_out.dtype, (None, KVH, hd, PAGE_TOKENS))
+        _need(kpool, "kpool", q_out.dtype, (None, KVH, layout.k_page_elems(hd)))
+        _need(vpool, "vpool", q_out.dtype, (None, KVH, layout.v_page_elems(hd)))
         _need(page_table, "page_table", torch.int32)
         num_pages = kpool.shape[0]
         max_blocks = page_table.shape[1]
@@ -358,8 +359,8 @@ def qkv_rope_cache(q_out, kpool, vpool, qkv, q_cols: int, kv_cols: int, bias, po
 def _check_attention(out, q, kpool, vpool, page_table, rows, H, KVH, hd):
     _need(q, "q")
     _need(out, "out", q.dtype)
-    _need(kpool, "kpool", q.dtype, (None, KVH, PAGE_TOKENS, hd))
-    _need(vpool, "vpool", q.dtype, (None, KVH, hd, PAGE_TOKENS))
+    _need(kpool, "kpool", q.dtype, (None, KVH, layout.k_page_elems(hd)))
+    _need(vpool, "vpool", q.dtype, (None, KVH, layout.v_page_elems(hd)))
     _need(page_table, "page_table", torch.int32)
     if page_table.dim() != 2:
         raise ValueError("attention: page_table must be [slots, blocks]")
@@ -423,8 +424,8 @@ def attention_decode_fused(out, qkv, bias, kpool, vpool, positions, row_seq, seq
     _need(out, "out", torch.bfloat16)
     if qkv.dim() != 2 or qkv.shape[1] != width or qkv.shape[0] < rows or out.numel() < rows * H * hd:
         raise ValueError("attention_decode_fused: qkv/out do not match the head sizes and row count")
-    _need(kpool, "kpool", torch.bfloat16, (None, KVH, PAGE_TOKENS, hd))
-    _need(vpool, "vpool", torch.bfloat16, (None, KVH, hd, PAGE_TOKENS))
+    _need(kpool, "kpool", torch.bfloat16, (None, KVH, layout.k_page_elems(hd)))
+    _need(vpool, "vpool", torch.bfloat16, (None, KVH, layout.v_page_elems(hd)))
     _need(page_table, "page_table", torch.int32)
     for name, t in (("positions", positions), ("row_seq", row_seq), ("seq_slot", seq_slot)):
         _need(t, name, torch.int32)

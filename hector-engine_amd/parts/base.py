@@ -132,7 +132,7 @@ class StepContext:
 class LayerCache:
     """The cache as one run of a layer sees it."""
 
-    kpool: torch.Tensor | None        # [pages, kv_heads, 64, head_dim]
+    kpool: torch.Tensor | None        # [pages, kv_heads, elements of a page] in the kernels' operand order (cache/layout.py)
     vpool: torch.Tensor | None
     page_table: torch.Tensor | None   # int32 [slots, blocks] of the layer's group
     writes: bool                      # False: the keys/values are another run's

@@ -382,9 +382,48 @@ def paged_setup(lengths, KVH, hd, dtype, seed, extra_pages=3):
     for s, nb in zip(slots, blocks):
         for b in range(nb):
             table[s, b] = next(it)
-    kpool = torch.zeros(num_pages, KVH, PAGE, hd, dtype=dtype)
-    vpool = torch.zeros(num_pages, KVH, hd, PAGE, dtype=dtype)
+    kpool = torch.zeros(num_pages, KVH, 64 * 32 * ((hd + 31) // 32), dtype=dtype)
+    vpool = torch.zeros(num_pages, KVH, 64 * 16 * ((hd + 15) // 16), dtype=dtype)
     return slots, table, kpool, vpool
+
+
+_maps = {}
+
+
+def page_maps(hd):
+    """Where element (token, dim) of a page lies, written out from the layout's description
+    (operand order): K [half][key tile][k step][lane][8], V [half][dim tile][lane][8] with
+    lane = 16 lg + lr; K: key = 32 h + 8 (lr // 4) + 4 t + lr % 4, dim = 32 ks + 8 lg + e;
+    V: dim = 16 dt + lr, key = 32 h + 8 lg + e. Returns index tensors [64, hd]."""
+    if hd not in _maps:
+        KS, NT = (hd + 31) // 32, (hd + 15) // 16
+        km = torch.full((PAGE, hd), -1, dtype=torch.long)
+        vm = torch.full((PAGE, hd), -1, dtype=torch.long)
+        for h in range(2):
+            for lane in range(64):
+                lr, lg = lane % 16, lane // 16
+                for e in range(8):
+                    for t in range(2):
+                        for ks in range(KS):
+                            key, dim = 32 * h + 8 * (lr // 4) + 4 * t + lr % 4, 32 * ks + 8 * lg + e
+                            if dim < hd:
+                                km[key, dim] = ((((h * 2 + t) * KS + ks) * 64) + lane) * 8 + e
+                    for dt in range(NT):
+                        key, dim = 32 * h + 8 * lg + e, 16 * dt + lr
+                        if dim < hd:
+                            vm[key, dim] = ((h * NT + dt) * 64 + lane) * 8 + e
+        assert (km >= 0).all() and (vm >= 0).all() and km.unique().numel() == PAGE * hd
+        _maps[hd] = (km, vm)
+    return _maps[hd]
+
+
+def cached_k(kpool, page, token, hd):
+    """[KVH, hd] of one token of a page."""
+    return kpool[page][:, page_maps(hd)[0][token]]
+
+
+def cached_v(vpool, page, token, hd):
+    return vpool[page][:, page_maps(hd)[1][token]]
 
 
 def fill_cache(table, slots, kpool, vpool, ks, vs):
@@ -392,8 +431,10 @@ def fill_cache(table, slots, kpool, vpool, ks, vs):
         for b in range((k.shape[0] + PAGE - 1) // PAGE):
             page = table[s, b].item()
             kb, vb = k[b * PAGE:(b + 1) * PAGE], v[b * PAGE:(b + 1) * PAGE]
-            kpool[page, :, :kb.shape[0], :] = kb.transpose(0, 1)
-            vpool[page, :, :, :vb.shape[0]] = vb.permute(1, 2, 0)
+            km, vm = page_maps(kb.shape[-1])
+            n = kb.shape[0]
+            kpool[page][:, km[:n].reshape(-1)] = kb.transpose(0, 1).reshape(kb.shape[1], -1)
+            vpool[page][:, vm[:n].reshape(-1)] = vb.transpose(0, 1).reshape(vb.shape[1], -1)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -433,8 +474,8 @@ def test_qkv_rope_cache(ops, dtype, H, KVH, hd, rot):
     for r in range(rows):
         s = slots[row_seq[r]]
         page = table[s, pos[r] // PAGE].item()
-        assert torch.allclose(kp[page, :, pos[r] % PAGE, :].double(), k[r], rtol=tol, atol=tol * 4)
-        assert torch.allclose(vp[page, :, :, pos[r] % PAGE].double(), v[r], rtol=tol, atol=tol * 4)
+        assert torch.allclose(cached_k(kp, page, pos[r] % PAGE, hd).double(), k[r], rtol=tol, atol=tol * 4)
+        assert torch.allclose(cached_v(vp, page, pos[r] % PAGE, hd).double(), v[r], rtol=tol, atol=tol * 4)
     # nothing else in the pools was touched
     assert (kp != 0).sum().item() <= rows * KVH * hd
 
@@ -569,9 +610,9 @@ def test_attention_decode_fused(ops, H, KVH, hd, window, write_kv, copies):
             v_new = x[s, (H + KVH) * hd:].reshape(1, KVH, hd)
             k_new, v_new = k_new.to(torch.bfloat16), v_new.to(torch.bfloat16)
             page = table[slots[s], (n - 1) // PAGE].item()
-            assert torch.allclose(kp[page, :, (n - 1) % PAGE, :].double(), k_new[0].double(),
+            assert torch.allclose(cached_k(kp, page, (n - 1) % PAGE, hd).double(), k_new[0].double(),
                                   rtol=2 ** -7, atol=2 ** -7), s
-            assert torch.allclose(vp[page, :, :, (n - 1) % PAGE].double(), v_new[0].double(),
+            assert torch.allclose(cached_v(vp, page, (n - 1) % PAGE, hd).double(), v_new[0].double(),
                                   rtol=2 ** -7, atol=2 ** -7), s
             k_all, v_all = torch.cat([k_all, k_new.double()]), torch.cat([v_all, v_new.double()])
         want = P.attention(q, k_all, v_all, pos, torch.arange(n), window).reshape(-1)
