@@ -523,7 +523,7 @@ def attention_case(ops, kind, dtype, H, KVH, hd, window, lengths, q_lens, seed, 
     return got, want
 
 
-ATT_SHAPES = [(6, 3, 48), (4, 1, 64), (28, 4, 128), (5, 5, 16), (2, 1, 80)]
+ATT_SHAPES = [(6, 3, 48), (4, 1, 64), (28, 4, 128), (5, 5, 16), (2, 1, 80), (4, 2, 192), (2, 1, 256)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
