@@ -2,7 +2,10 @@
 """Decode throughput of the Qwen2.5-7B shape (bf16, random weights, synthetic
 token ids) on one MI355X, with prefill and roofline figures on the same line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--shape 7b|32b|72b]
+
+The default is the 7B shape; --shape runs the same measurement at the layer sizes of
+Qwen2.5-32B (context 8192) or Qwen2-72B (context 4096).
 
 A step is one decode step of the whole batch: the engine's step function (HIP
 graph replay) plus greedy sampling and the copy of the chosen ids to the host.
@@ -16,12 +19,17 @@ import time
 
 import numpy as np
 
-# Qwen2.5-7B layer sizes: the model configuration this benchmark is quoted on
-SHAPE = dict(num_hidden_layers=28, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
-             head_dim=128, intermediate_size=18944, vocab_size=152064, rope_theta=1000000.0,
-             rms_norm_eps=1e-6, max_position_embeddings=32768, tie_word_embeddings=False)
-FULL_LAYERS = 28
-CONTEXT = 8192
+# layer sizes; the benchmark is quoted on the first (Qwen2.5-7B)
+_COMMON = dict(head_dim=128, vocab_size=152064, rope_theta=1000000.0, rms_norm_eps=1e-6,
+               max_position_embeddings=32768, tie_word_embeddings=False)
+SHAPES = {
+    "7b": ("Qwen2.5-7B shape", 8192, dict(_COMMON, num_hidden_layers=28, hidden_size=3584, num_attention_heads=28,
+                                          num_key_value_heads=4, intermediate_size=18944)),
+    "32b": ("Qwen2.5-32B shape", 8192, dict(_COMMON, num_hidden_layers=64, hidden_size=5120, num_attention_heads=40,
+                                            num_key_value_heads=8, intermediate_size=27648)),
+    "72b": ("Qwen2-72B shape", 4096, dict(_COMMON, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64,
+                                          num_key_value_heads=8, intermediate_size=29568)),
+}
 PROMPT = 2048
 HBM_PEAK_GBS = 8000.0
 BF16_PEAK_FLOPS = 2.5e15
@@ -52,7 +60,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0 = all)")
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="7b")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points")
     ap.add_argument("--no-tune", action="store_true",
                     help="leave the library's default kernels for the tall matrix products")
@@ -60,12 +69,21 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    MODEL, CONTEXT, SHAPE = SHAPES[args.shape]
+    FULL_LAYERS = SHAPE["num_hidden_layers"]
+    args.layers = args.layers or FULL_LAYERS
 
     import torch
     import hector_engine_amd as he
     from hector_engine_amd.config.qwen2 import Qwen2Config
     from hector_engine_amd.engine.engine import StepEntry
 
+    t_start = time.perf_counter()
+
+    def progress(what):
+        print(f"[bench {time.perf_counter() - t_start:6.1f}s] {what}", file=sys.stderr, flush=True)
+
+    progress(f"{MODEL}: random weights, {args.layers} layers")
     cfg_dict = dict(SHAPE, num_hidden_layers=args.layers, architectures=["Qwen2ForCausalLM"])
     config = Qwen2Config.from_dict(cfg_dict)
     max_batch = args.batch if args.no_points else max(args.batch, 64)
@@ -112,6 +130,7 @@ def main() -> int:
         return dt / steps, avg_len
 
     # ---- prefill of one 2,048-token prompt (second run timed; the first warms the library GEMMs)
+    progress(f"weights ready; prefill of {PROMPT} tokens")
     slot = engine.acquire()
     p = prompts(1)[0]
     engine.step([StepEntry(slot, p, [PROMPT - 1])])
@@ -126,6 +145,7 @@ def main() -> int:
     flops = prefill_flops(SHAPE, args.layers, PROMPT)
 
     # ---- decode at the headline batch
+    progress(f"decode at batch {args.batch}")
     step_s, avg_len = decode_run(args.batch, args.steps, args.warmup)
     wbytes = weight_bytes(SHAPE, args.layers)
     step_bytes = wbytes + args.batch * avg_len * kv_bytes_per_token(SHAPE, args.layers)
@@ -134,11 +154,12 @@ def main() -> int:
     points = {}
     if not args.no_points:
         for b in (1, 64):
+            progress(f"decode at batch {b}")
             s, _ = decode_run(b, max(8, args.steps // 2), max(3, args.warmup // 2))
             points[f"decode_b{b}"] = round(b / s, 1)
 
     line = {
-        "metric": "decode tok/s @ bs 8, Qwen2.5-7B shape bf16, context 8192, prompts 2048",
+        "metric": f"decode tok/s @ bs {args.batch}, {MODEL} bf16, context {CONTEXT}, prompts {PROMPT}",
         "value": round(args.batch / step_s, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -151,7 +172,7 @@ def main() -> int:
         "dtype": "bf16",
         "data": "synthetic token ids (uniform), random N(0, 0.02) weights",
         "config": {
-            "model": "Qwen2.5-7B shape", "layers": args.layers, "layers_full": FULL_LAYERS,
+            "model": MODEL, "layers": args.layers, "layers_full": FULL_LAYERS,
             "hidden_size": SHAPE["hidden_size"], "heads": SHAPE["num_attention_heads"],
             "kv_heads": SHAPE["num_key_value_heads"], "head_dim": SHAPE["head_dim"],
             "intermediate_size": SHAPE["intermediate_size"], "vocab_size": SHAPE["vocab_size"],

@@ -308,8 +308,8 @@ struct BlockSplitPlan {
   int MT, R, U, NW, kslice;
 };
 
-// Tilings measured on MI355X (graph-timed sweeps over R, U and NW at the Qwen2.5-7B
-// shapes). The rule depends on the sizes only, so a product always runs the same way.
+// Tilings measured on MI355X (graph-timed sweeps over R, U and NW at the Qwen2.5-7B, Qwen2.5-32B
+// and Qwen2-72B shapes). The rule depends on the sizes only, so a product always runs the same way.
 static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int U, int NW) {
   BlockSplitPlan p;
   p.MT = (M + 15) / 16;
@@ -318,11 +318,25 @@ static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int
     if (M <= 8) r = 2, u = 1, nw = 8;
     else if (p.MT == 1) r = 4, u = 2, nw = 4;
     else r = 2, u = 2, nw = 4;
-  } else if (K >= 8192) {           // long K (down projection)
-    r = 1, u = 1, nw = p.MT == 1 ? 8 : 4;
+  } else if (K >= 8192) {           // long K
+    const int groups = (N + 31) / 32, last_round = groups % 256;   // with two tiles a workgroup
+    if (N < 4096) {                 // few weight rows: one tile a workgroup, or the chip is not filled
+      r = 1, u = 1, nw = p.MT == 1 ? 8 : 4;
+    } else if (p.MT == 2) {
+      r = 2, u = 2, nw = 4;
+    } else if (M > 8 && N >= 10240) {
+      r = 4, u = 2, nw = 4;         // the activation rows are read half as often
+    } else if (groups < 256) {
+      r = 2, u = 1, nw = 8;         // under one workgroup a compute unit: more wavefronts each
+    } else if (groups < 1024 && last_round > 0 && last_round <= 128) {
+      r = 1, u = 2, nw = 8;         // the last round of workgroups would fill under half of the chip
+    } else {
+      r = 2, u = 4, nw = 4;
+    }
   } else if (N >= 16384) {          // wide N (gate||up)
     r = 2, u = 1, nw = 8;
     if (p.MT == 2) u = 2, nw = 4;
+    else if (M > 8 && K >= 5120) r = 4;
   } else {                          // small products (q||k||v, o)
     r = N >= 4096 ? 2 : 1;
     u = p.MT == 1 ? 4 : 1;
