@@ -323,14 +323,22 @@ attention_prefill_pair_kernel(
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int lr = lane & 15, lg = lane >> 4;
-  const int seq = blockIdx.z, h = blockIdx.y;
+  // Workgroups go to the eight XCDs in turn, and each XCD has an L2 of its own. The work is
+  // numbered so that an XCD gets a contiguous range of (head, sequence, query tiles): its
+  // workgroups then read the pages of one or two kv heads, not of all, and its L2 holds them.
+  const int total = gridDim.x * gridDim.y * gridDim.z;
+  const int launched = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  const int xcd = launched & 7, share = total >> 3, extra = total & 7;
+  const int work = xcd * share + min(xcd, extra) + (launched >> 3);
+  const int tile_x = work % gridDim.x;
+  const int seq = (work / gridDim.x) % gridDim.z, h = work / (gridDim.x * gridDim.z);
   const int slot = seq_slot[seq];
   if (slot < 0) return;
   const int row0 = cu_seqlens[seq];
   const int q_len = cu_seqlens[seq + 1] - row0;
   const int tiles = (q_len + 15) >> 4;
   const int pairs = (tiles + 1) >> 1;
-  const int pair0 = PF2_WAVES * blockIdx.x;      // the workgroup's first pair: its earliest and latest tile
+  const int pair0 = PF2_WAVES * tile_x;          // the workgroup's first pair: its earliest and latest tile
   if (pair0 >= pairs) return;
   const int start = seq_start[seq];
   const int kvh = h / (H / KVH);

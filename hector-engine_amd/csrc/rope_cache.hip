@@ -142,22 +142,109 @@ __device__ __forceinline__ uint4 pack8(const float* f) {
   return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
-__global__ __launch_bounds__(256) void qkv_rope_cache_vec_kernel(
+// grid: one workgroup per row for q and k (blockIdx.x < rows), then one per 8 rows for v.
+// V lies transposed in a page (8 keys of one dim are 16 contiguous bytes), so the v values of
+// a run of tokens that share such a group are gathered dim by dim and stored together: 16
+// bytes a store when the run is a whole group (a prompt), 2 bytes a token otherwise.
+__global__ __launch_bounds__(1024) void qkv_rope_cache_vec_kernel(
     uint16_t* __restrict__ q_out, uint16_t* __restrict__ kpool, uint16_t* __restrict__ vpool,
     const uint16_t* __restrict__ q_in, const uint16_t* __restrict__ k_in,
     const uint16_t* __restrict__ v_in, int64_t in_stride, const uint16_t* __restrict__ q_bias,
     const uint16_t* __restrict__ k_bias, const uint16_t* __restrict__ v_bias,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
     const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ page_table, int max_blocks,
-    int num_pages, const float* __restrict__ inv_freq, int rotary_dim, int H, int KVH, int hd) {
+    int num_pages, const float* __restrict__ inv_freq, int rotary_dim, int rows, int H, int KVH,
+    int hd) {
   __shared__ float cs[2][ROPE_MAX_HALF];
+  if ((int)blockIdx.x >= rows) {
+    // ---- v: the runs of tokens that begin in rows [r0, r0 + 8)
+    const int r0 = 8 * ((int)blockIdx.x - rows);
+    const int NT = he_v_tiles(hd);
+    for (int r = r0; r < min(r0 + 8, rows); ++r) {
+      const int seq = row_seq[r];
+      if (seq < 0) continue;
+      const int pos = positions[r];
+      const bool begins = (pos & 7) == 0 || r == 0 || row_seq[r - 1] != seq || positions[r - 1] != pos - 1;
+      if (!begins) continue;
+      int n = 1;   // tokens of the run: the same sequence, consecutive positions, one group of 8 keys
+      while (n < 8 - (pos & 7) && r + n < rows && row_seq[r + n] == seq && positions[r + n] == pos + n) ++n;
+      const int page = page_table[(int64_t)seq_slot[seq] * max_blocks + (pos >> HE_PAGE_SHIFT)];
+      if (page < 0 || page >= num_pages) continue;
+      const int off = pos & (HE_PAGE_TOKENS - 1);
+      for (int e = threadIdx.x; e < KVH * hd; e += blockDim.x) {
+        const int h = e / hd, d = e - h * hd;
+        const float b = v_bias ? bf16_bits_to_float(v_bias[e]) : 0.f;
+        uint16_t vals[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          vals[i] = 0;
+          if (i < n) {
+            const uint16_t x = v_in[(int64_t)(r + i) * in_stride + e];
+            vals[i] = v_bias ? float_to_bf16_bits(bf16_bits_to_float(x) + b) : x;
+          }
+        }
+        uint16_t* out = vpool + ((int64_t)page * KVH + h) * he_v_page_elems(hd) + he_v_index(off, d, NT);
+        if (n == 8) {
+          *reinterpret_cast<uint4*>(out) =
+              make_uint4(vals[0] | ((uint32_t)vals[1] << 16), vals[2] | ((uint32_t)vals[3] << 16),
+                         vals[4] | ((uint32_t)vals[5] << 16), vals[6] | ((uint32_t)vals[7] << 16));
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            if (i < n) out[i] = vals[i];
+        }
+      }
+    }
+    return;
+  }
+  // ---- q and k of one row
   const int64_t row = blockIdx.x;
   const int seq = row_seq[row];
-  const int pos = positions[row];
   if (seq < 0) return;  // padding row
+  const int half = rotary_dim >> 1;
+  const int rot8 = half >> 3;                 // groups of 8 pairs per head
+  const int pass8 = (hd - rotary_dim) >> 3;   // groups of 8 pass-through dims per head
+  const int per_head = rot8 + pass8;
+  const int q_items = H * per_head;
+  const int items = q_items + (k_in ? KVH * per_head : 0);
+  // an item: eight pairs (j.., j + half..) of one head, or eight pass-through dims from d on
+  struct Item {
+    const uint16_t* in;
+    const uint16_t* bias;
+    int h, j;
+    bool is_q, rotated;
+  };
+  auto item = [&](int it) {
+    Item im;
+    im.is_q = it < q_items;
+    const int idx = im.is_q ? it : it - q_items;
+    im.h = idx / per_head;
+    const int g = idx - im.h * per_head;
+    im.rotated = g < rot8;
+    im.j = im.rotated ? 8 * g : rotary_dim + 8 * (g - rot8);
+    im.in = (im.is_q ? q_in : k_in) + row * in_stride + im.h * hd;
+    const uint16_t* bias = im.is_q ? q_bias : k_bias;
+    im.bias = bias ? bias + im.h * hd : nullptr;
+    return im;
+  };
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  auto load = [&](const Item& im, uint4 (&raw)[4]) {
+    raw[0] = *reinterpret_cast<const uint4*>(im.in + im.j);
+    raw[1] = im.rotated ? *reinterpret_cast<const uint4*>(im.in + im.j + half) : zero;
+    raw[2] = im.bias ? *reinterpret_cast<const uint4*>(im.bias + im.j) : zero;
+    raw[3] = im.bias && im.rotated ? *reinterpret_cast<const uint4*>(im.bias + im.j + half) : zero;
+  };
+  // the loads of a thread's first item are on their way while the angles are computed
+  Item first;
+  uint4 first_raw[4];
+  const bool has_first = (int)threadIdx.x < items;
+  if (has_first) {
+    first = item(threadIdx.x);
+    load(first, first_raw);
+  }
+  const int pos = positions[row];
   int page = -1;
   if (k_in != nullptr) page = page_table[(int64_t)seq_slot[seq] * max_blocks + (pos >> HE_PAGE_SHIFT)];
-  const int half = rotary_dim >> 1;
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
     float sn, c;
     sincos_angle((float)pos * inv_freq[i], &sn, &c);
@@ -165,78 +252,51 @@ __global__ __launch_bounds__(256) void qkv_rope_cache_vec_kernel(
     cs[1][i] = sn;
   }
   __syncthreads();
-  const int rot8 = half >> 3;                 // groups of 8 pairs per head
-  const int pass8 = (hd - rotary_dim) >> 3;   // groups of 8 pass-through dims per head
-  const int per_head = rot8 + pass8;
-  const int q_items = H * per_head;
-  const int k_items = k_in ? KVH * per_head : 0;
-  const int v_items = k_in ? (KVH * hd) >> 3 : 0;
   const bool cache_ok = page >= 0 && page < num_pages;
   const int off = pos & (HE_PAGE_TOKENS - 1);
-  for (int it = threadIdx.x; it < q_items + k_items + v_items; it += blockDim.x) {
-    if (it < q_items + k_items) {
-      const bool is_q = it < q_items;
-      const int idx = is_q ? it : it - q_items;
-      const int h = idx / per_head;
-      const int g = idx - h * per_head;
-      const uint16_t* in = (is_q ? q_in : k_in) + row * in_stride + h * hd;
-      const uint16_t* bias = is_q ? q_bias : k_bias;
-      // where the eight elements from dim d on go: the q row, or the cache page in operand order
-      uint16_t* out;
-      const int KS = he_k_steps(hd);
-      if (is_q) {
-        out = q_out + row * (int64_t)H * hd + h * hd;
-      } else {
-        if (!cache_ok) continue;
-        out = kpool + ((int64_t)page * KVH + h) * he_k_page_elems(hd);
-      }
-      auto at = [&](int d) { return out + (is_q ? d : he_k_index(off, d, KS)); };
-      float x0[8], x1[8], b0[8], b1[8];
-      if (g < rot8) {
-        const int j = 8 * g;
-        unpack8(*reinterpret_cast<const uint4*>(in + j), x0);
-        unpack8(*reinterpret_cast<const uint4*>(in + j + half), x1);
-        if (bias) {
-          unpack8(*reinterpret_cast<const uint4*>(bias + h * hd + j), b0);
-          unpack8(*reinterpret_cast<const uint4*>(bias + h * hd + j + half), b1);
-        }
-        float y0[8], y1[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const float a0 = bias ? x0[i] + b0[i] : x0[i];
-          const float a1 = bias ? x1[i] + b1[i] : x1[i];
-          const float c = cs[0][j + i], sn = cs[1][j + i];
-          y0[i] = a0 * c - a1 * sn;
-          y1[i] = a0 * sn + a1 * c;
-        }
-        *reinterpret_cast<uint4*>(at(j)) = pack8(y0);
-        *reinterpret_cast<uint4*>(at(j + half)) = pack8(y1);
-      } else {
-        const int d = rotary_dim + 8 * (g - rot8);
-        unpack8(*reinterpret_cast<const uint4*>(in + d), x0);
-        if (bias) {
-          unpack8(*reinterpret_cast<const uint4*>(bias + h * hd + d), b0);
-#pragma unroll
-          for (int i = 0; i < 8; ++i) x0[i] += b0[i];
-        }
-        *reinterpret_cast<uint4*>(at(d)) = pack8(x0);
-      }
+  const int KS = he_k_steps(hd);
+  auto finish = [&](const Item& im, const uint4 (&raw)[4]) {
+    // where the eight elements from dim d on go: the q row, or the cache page in operand order
+    uint16_t* out;
+    if (im.is_q) {
+      out = q_out + row * (int64_t)H * hd + im.h * hd;
     } else {
-      if (!cache_ok) continue;
-      const int e = 8 * (it - q_items - k_items);   // element of the v row
-      const int h = e / hd, d = e - h * hd;
-      float x[8], b[8];
-      unpack8(*reinterpret_cast<const uint4*>(v_in + row * in_stride + e), x);
-      if (v_bias) {
-        unpack8(*reinterpret_cast<const uint4*>(v_bias + e), b);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) x[i] += b[i];
-      }
-      uint16_t* out = vpool + ((int64_t)page * KVH + h) * he_v_page_elems(hd);
-      const int NT = he_v_tiles(hd);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) out[he_v_index(off, d + i, NT)] = float_to_bf16_bits(x[i]);
+      if (!cache_ok) return;
+      out = kpool + ((int64_t)page * KVH + im.h) * he_k_page_elems(hd);
     }
+    auto at = [&](int d) { return out + (im.is_q ? d : he_k_index(off, d, KS)); };
+    float x0[8], x1[8], b0[8], b1[8];
+    unpack8(raw[0], x0);
+    unpack8(raw[2], b0);
+    if (im.rotated) {
+      unpack8(raw[1], x1);
+      unpack8(raw[3], b1);
+      float y0[8], y1[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float a0 = x0[i] + b0[i], a1 = x1[i] + b1[i];
+        const float c = cs[0][im.j + i], sn = cs[1][im.j + i];
+        y0[i] = a0 * c - a1 * sn;
+        y1[i] = a0 * sn + a1 * c;
+      }
+      *reinterpret_cast<uint4*>(at(im.j)) = pack8(y0);
+      *reinterpret_cast<uint4*>(at(im.j + half)) = pack8(y1);
+    } else {
+      if (im.bias) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x0[i] += b0[i];
+        *reinterpret_cast<uint4*>(at(im.j)) = pack8(x0);
+      } else {
+        *reinterpret_cast<uint4*>(at(im.j)) = raw[0];
+      }
+    }
+  };
+  if (has_first) finish(first, first_raw);
+  for (int it = threadIdx.x + blockDim.x; it < items; it += blockDim.x) {
+    const Item im = item(it);
+    uint4 raw[4];
+    load(im, raw);
+    finish(im, raw);
   }
 }
 
@@ -278,12 +338,15 @@ extern "C" int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const vo
                         ((uintptr_t)q_bias) | ((uintptr_t)k_bias) | ((uintptr_t)v_bias) |
                         ((uintptr_t)q_out) | ((uintptr_t)kpool)) & 15) == 0;
   if (vec_ok) {
-    qkv_rope_cache_vec_kernel<<<rows, threads, 0, s>>>(
+    const int items = (H + (k_in ? KVH : 0)) * ((rotary_dim >> 4) + ((hd - rotary_dim) >> 3));
+    const int vec_threads = min(1024, max(64, (items + 63) / 64 * 64));
+    const int v_blocks = k_in ? (rows + 7) / 8 : 0;
+    qkv_rope_cache_vec_kernel<<<rows + v_blocks, vec_threads, 0, s>>>(
         (uint16_t*)q_out, (uint16_t*)kpool, (uint16_t*)vpool, (const uint16_t*)q_in,
         (const uint16_t*)k_in, (const uint16_t*)v_in, in_stride, (const uint16_t*)q_bias,
         (const uint16_t*)k_bias, (const uint16_t*)v_bias, (const int32_t*)positions,
         (const int32_t*)row_seq, (const int32_t*)seq_slot, (const int32_t*)page_table, max_blocks,
-        num_pages, (const float*)inv_freq, rotary_dim, H, KVH, hd);
+        num_pages, (const float*)inv_freq, rotary_dim, rows, H, KVH, hd);
   } else if (in_splits > 0) {  // the input rows are fp32 partial sums
     if (dtype == HE_BF16)
       ROPE_LAUNCH(bf16_t, float);
