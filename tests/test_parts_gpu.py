@@ -224,7 +224,7 @@ def test_embedding_and_heads(fw, dtype):
         out = head.forward(x.cuda(), 4, ctx)
         assert out.dtype == torch.float32
         assert torch.allclose(out.cpu().double(), x.double() @ wt.double().T, rtol=1e-4, atol=1e-4)
-    # 100 wanted rows go through in chunks of 64
+    # 100 wanted rows: more than the MFMA kernels take at once (under bfloat16 the library writes the fp32 results)
     ctx = make_ctx(fw, env, [100], [0], [0])
     x = rnd(100, 80, seed=4).to(dtype)
     out = own.forward(x.cuda(), 100, ctx)
