@@ -115,13 +115,24 @@ struct BsFusion {
 
 // The residual values and gains of output item (tile, lane) of a non-gated product:
 // row m = 16 t + lane % 16, columns n0 + 16 r + 4 (lane / 16) .. + 4.
+// With few rows the 16 columns of the activation tile hold each row several times: column c
+// is row c >> spread (spread 2 up to 4 rows, 1 up to 8), so that the four lanes the memory
+// pipeline takes together read one or two rows, not four (1-4 % of a product's time). The
+// first column of a row owns its outputs.
+template <int MT>
+__device__ __forceinline__ int bs_spread(int M) {
+  return MT == 1 ? (M <= 4 ? 2 : (M <= 8 ? 1 : 0)) : 0;
+}
+
 template <int MT>
 __device__ __forceinline__ void bs_load_resid(const BsFusion& fu, int item, int n0, int M, int N,
                                               float res[4], float gain[4]) {
+  const int spread = bs_spread<MT>(M);
   const int ot = item >> 6, ol = item & 63;
-  const int m = 16 * (ot % MT) + (ol & 15);
+  const int col = 16 * (ot % MT) + (ol & 15);
+  const int m = col >> spread;
   const int n = n0 + 16 * (ot / MT) + 4 * (ol >> 4);
-  const int valid = m < M ? max(0, min(4, N - n)) : 0;
+  const int valid = (m < M && (m << spread) == col) ? max(0, min(4, N - n)) : 0;
   if (valid == 4 && (N & 3) == 0) {
     const float4 r4 = *reinterpret_cast<const float4*>(fu.resid + (int64_t)m * N + n);
     res[0] = r4.x, res[1] = r4.y, res[2] = r4.z, res[3] = r4.w;
@@ -146,13 +157,14 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
   const int k_begin = wave * kslice;
   const int k_end = min(K, k_begin + kslice);
   const int lr = lane & 15, lg = lane >> 4;
+  const int spread = bs_spread<MT>(M);
 
   const uint16_t* wp[R];
   const uint16_t* xp[MT];
 #pragma unroll
   for (int r = 0; r < R; ++r) wp[r] = W + (int64_t)min(n0 + 16 * r + lr, N - 1) * K + lg * 16;
 #pragma unroll
-  for (int t = 0; t < MT; ++t) xp[t] = X + (int64_t)min(16 * t + lr, M - 1) * K + lg * 16;
+  for (int t = 0; t < MT; ++t) xp[t] = X + (int64_t)min((16 * t + lr) >> spread, M - 1) * K + lg * 16;
 
   floatx4 acc[R][MT];
 #pragma unroll
@@ -239,7 +251,8 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
     const int olr = ol & 15, olg = ol >> 4;
     const int t = ot % MT;
     const int r = GATED ? 2 * (ot / MT) : ot / MT;
-    const int m = 16 * t + olr;
+    const int col = 16 * t + olr, m = col >> spread;
+    const bool owner = m < M && (m << spread) == col;
     float4 s = make_float4(0.f, 0.f, 0.f, 0.f), s2 = s;
     for (int w = 0; w < nw; ++w) {
       const float4 v = tiles[(w * (R * MT) + r * MT + t) * 64 + ol];
@@ -255,7 +268,7 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
       const float up[4] = {s2.x, s2.y, s2.z, s2.w};
       const int NO = N >> 1;
       const int n = (n0 >> 1) + 8 * r + 4 * olg;
-      const int valid = m < M ? min(4, NO - n) : 0;
+      const int valid = owner ? min(4, NO - n) : 0;
       if (valid <= 0) continue;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -265,7 +278,7 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
       bs_store4<TC>(C + (int64_t)m * NO + n, v, (NO & 3) == 0, valid);
     } else {
       const int n = n0 + 16 * r + 4 * olg;
-      const int valid = m < M ? max(0, min(4, N - n)) : 0;
+      const int valid = owner ? max(0, min(4, N - n)) : 0;
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] *= rs;
       if (bias != nullptr)
@@ -298,7 +311,8 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
     const int m = threadIdx.x;
     if (m < M && m < 16 * MT) {
       float sq = 0.f;
-      for (int r = 0; r < R; ++r) sq += row_sq[r * MT + m / 16][m % 16];
+      const int col = m << spread;
+      for (int r = 0; r < R; ++r) sq += row_sq[r * MT + col / 16][col % 16];
       fu.sq_out[(int64_t)m * gridDim.x + blockIdx.x] = sq;
     }
   }
