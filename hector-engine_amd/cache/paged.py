@@ -122,6 +122,11 @@ class PagedCache:
             if need > g.pool.available:
                 raise CacheFull(f"the step needs {need} more pages of {PAGE_TOKENS} tokens per "
                                 f"group, {g.pool.available} are free")
+        if need == 0:       # most one-token steps: every new position already has its page
+            for s, n in growth:
+                if n < self.book.length[s]:
+                    raise CacheError(f"slot {s}: cannot shrink from {self.book.length[s]} to {n}")
+            return
         added = []
         for s, n in growth:
             added += self.book.reserve(s, n)

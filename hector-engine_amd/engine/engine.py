@@ -128,6 +128,7 @@ class Engine:
         self._pinned = [torch.empty(1 << 16, dtype=torch.int32).pin_memory() for _ in range(4)]
         self._pinned_events: list[torch.cuda.Event | None] = [None] * 4
         self._pinned_next = 0
+        self._iota_cache = np.arange(64, dtype=np.int32)
         self.stats = {"steps": 0, "graph_replays": 0, "graph_captures": 0, "eager_steps": 0}
 
     # -- slots ----------------------------------------------------------------
@@ -164,8 +165,12 @@ class Engine:
             if start + n > self.cache.max_seq_len:
                 raise StepError(f"slot {e.slot}: {start} cached + {n} new tokens exceed the "
                                 f"longest sequence {self.cache.max_seq_len}")
-            toks = np.asarray(e.tokens, dtype=np.int64)
-            if toks.ndim != 1 or toks.min() < 0 or toks.max() >= self.vocab_size:
+            if n == 1 and type(e.tokens[0]) is int:     # the common one-token step, without numpy
+                in_range = 0 <= e.tokens[0] < self.vocab_size
+            else:
+                toks = np.asarray(e.tokens, dtype=np.int64)
+                in_range = toks.ndim == 1 and toks.min() >= 0 and toks.max() < self.vocab_size
+            if not in_range:
                 raise StepError(f"slot {e.slot}: token ids must lie in [0, {self.vocab_size})")
             for w in e.want:
                 if not 0 <= int(w) < n:
@@ -202,6 +207,23 @@ class Engine:
         v["positions"][:] = 0
         v["seq_slot"][:] = -1
         v["seq_start"][:] = 0
+        if len(entries) == meta.offsets["tokens"][1] or all(len(e.tokens) == 1 for e in entries):
+            # one token a sequence: whole columns at once
+            k = len(entries)
+            starts = [self.cache.length(e.slot) for e in entries]
+            v["tokens"][:k] = [e.tokens[0] for e in entries]
+            v["positions"][:k] = starts
+            v["seq_start"][:k] = starts
+            v["seq_slot"][:k] = [e.slot for e in entries]
+            v["row_seq"][:k] = self._iota(k)
+            v["cu_seqlens"][:k] = self._iota(k)
+            v["cu_seqlens"][k:] = k
+            nw = 0
+            for row, e in enumerate(entries):
+                for w in e.want:
+                    v["want_rows"][nw] = row + int(w)
+                    nw += 1
+            return host, i, nw
         row = 0
         nw = 0
         for s, e in enumerate(entries):
@@ -219,6 +241,11 @@ class Engine:
             row += n
         v["cu_seqlens"][len(entries):] = row
         return host, i, nw
+
+    def _iota(self, n: int) -> np.ndarray:
+        if n > self._iota_cache.size:
+            self._iota_cache = np.arange(1 << (n - 1).bit_length(), dtype=np.int32)
+        return self._iota_cache[:n]
 
     def _upload(self, host, index: int, dev: torch.Tensor) -> None:
         dev.copy_(host, non_blocking=True)
