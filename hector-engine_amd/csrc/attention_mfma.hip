@@ -624,9 +624,15 @@ extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* k
                                          const void* seq_slot, const void* seq_start,
                                          const void* page_table, int max_blocks, int num_pages,
                                          int num_seqs, int max_q_len, int H, int KVH, int hd,
-                                         int window, float scale, void* stream) {
+                                         int window, float scale, int tiles_per_wave,
+                                         void* stream) {
   HE_REQUIRE(num_seqs >= 0 && max_q_len >= 0 && H > 0 && KVH > 0 && hd > 0,
              "he_attention_prefill_bf16: bad sizes");
+  HE_REQUIRE(tiles_per_wave >= 0 && tiles_per_wave <= 2,
+             "he_attention_prefill_bf16: %d query tiles a wavefront (0 = the library's choice, 1, 2)",
+             tiles_per_wave);
+  HE_REQUIRE(tiles_per_wave < 2 || hd <= 128,
+             "he_attention_prefill_bf16: %d tiles a wavefront need head_dim %d <= 128", tiles_per_wave, hd);
   HE_REQUIRE(scale > 0.f, "he_attention_prefill_bf16: the score scale must be positive");
   HE_REQUIRE(H % KVH == 0, "he_attention_prefill_bf16: heads %d not a multiple of kv heads %d", H,
              KVH);
@@ -638,7 +644,8 @@ extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* k
              "he_attention_prefill_bf16: buffers must be 16-byte aligned");
   if (num_seqs == 0 || max_q_len == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  if (hd <= 128 && max_q_len > 16) {   // K/V pages shared through LDS by 128 queries
+  if (tiles_per_wave == 0) tiles_per_wave = (hd > 128 || max_q_len <= 16) ? 1 : 2;
+  if (tiles_per_wave == 2) {   // K/V pages shared through LDS by 128 queries
     dim3 grid128((max_q_len + 127) / 128, H, num_seqs);
 #define PREFILL_LDS(NTV)                                                                        \
   case NTV:                                                                                     \

@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 11
+#define HE_ABI_VERSION 12
 
 #ifdef __cplusplus
 extern "C" {
@@ -112,7 +112,7 @@ int he_attention_prefill_bf16(void* out, const void* q, const void* kpool, const
                               const void* cu_seqlens, const void* seq_slot, const void* seq_start,
                               const void* page_table, int max_blocks, int num_pages, int num_seqs,
                               int max_q_len, int H, int KVH, int hd, int window, float scale,
-                              void* stream);
+                              int tiles_per_wave, void* stream);
 
 // ---- sampling ------------------------------------------------------------
 int64_t he_argmax_workspace_bytes(int rows, int V);

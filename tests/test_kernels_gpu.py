@@ -480,7 +480,7 @@ def test_qkv_rope_cache(ops, dtype, H, KVH, hd, rot):
     assert (kp != 0).sum().item() <= rows * KVH * hd
 
 
-def attention_case(ops, kind, dtype, H, KVH, hd, window, lengths, q_lens, seed, pad=0):
+def attention_case(ops, kind, dtype, H, KVH, hd, window, lengths, q_lens, seed, pad=0, tiles=0):
     """Runs one attention kernel over a crafted cache; returns (got, want) lists per sequence."""
     B = len(lengths)
     slots, table, kpool, vpool = paged_setup(lengths, KVH, hd, dtype, seed)
@@ -510,7 +510,7 @@ def attention_case(ops, kind, dtype, H, KVH, hd, window, lengths, q_lens, seed, 
                              dev(table), rows + pad, H, KVH, hd, window, scale, max_keys, ws)
     else:
         ops.attention_prefill(out, dev(q), *args, dev(cu), dev(seq_slot), dev(seq_start), dev(table),
-                              B, max(q_lens), rows, H, KVH, hd, window, scale)
+                              B, max(q_lens), rows, H, KVH, hd, window, scale, tiles_per_wave=tiles)
     got, want = [], []
     r = 0
     for i, (n, m) in enumerate(zip(lengths, q_lens)):
@@ -547,10 +547,31 @@ def test_attention_decode(ops, H, KVH, hd, window):
 
 @pytest.mark.parametrize("H,KVH,hd", ATT_SHAPES)
 @pytest.mark.parametrize("window", [0, 70])
-def test_attention_prefill(ops, H, KVH, hd, window):
-    # whole prompts, a continuation (200 cached + 37 new) and a single token
+@pytest.mark.parametrize("tiles", [0, 1, 2])
+def test_attention_prefill(ops, H, KVH, hd, window, tiles):
+    """Each of the prompt kernels (1 or 2 query tiles a wavefront; 0 = the library's choice):
+    whole prompts, a continuation (200 cached + 37 new) and a single token."""
+    if tiles >= 2 and hd > 128:
+        from hector_engine_amd.kernels.lib import KernelLibraryError
+        with pytest.raises(KernelLibraryError, match="head_dim"):
+            attention_case(ops, "prefill", torch.bfloat16, H, KVH, hd, window, [150], [150], 42, tiles=tiles)
+        return
     got, want = attention_case(ops, "prefill", torch.bfloat16, H, KVH, hd, window,
-                               [150, 237, 3, 66], [150, 37, 3, 1], 42)
+                               [150, 237, 3, 66], [150, 37, 3, 1], 42, tiles=tiles)
+    for g, w in zip(got, want):
+        assert torch.allclose(g, w, rtol=2 ** -6, atol=2 ** -6)
+
+
+@pytest.mark.parametrize("H,KVH,hd", [(4, 1, 64), (7, 1, 128), (3, 3, 48)])
+@pytest.mark.parametrize("window", [0, 70, 300])
+@pytest.mark.parametrize("tiles", [1, 2])
+def test_attention_prefill_of_many_tiles(ops, H, KVH, hd, window, tiles):
+    """Prompts of several workgroups' worth of query tiles: an even and an odd number of tiles, a
+    last tile that is not full, a continuation whose first position is no multiple of 32 (its tiles'
+    diagonals then fall into different steps of 32 keys), and a prompt short enough that the pairs
+    from both ends meet inside one workgroup."""
+    got, want = attention_case(ops, "prefill", torch.bfloat16, H, KVH, hd, window,
+                               [1024, 713, 530, 48, 272], [1024, 713, 330, 48, 17], 43, tiles=tiles)
     for g, w in zip(got, want):
         assert torch.allclose(g, w, rtol=2 ** -6, atol=2 ** -6)
 
