@@ -1,21 +1,24 @@
 """The linear layer all parts share: y[M,N] = x[M,K] . W[N,K]^T (+ bias).
 
 Which kernel runs is decided by precision and row count:
-  float32                 -> the plain FMA kernel (fixed summation order per element)
-  bfloat16, M <= 64       -> the hand-written MFMA kernel that streams each weight once
-  bfloat16, M  > 64       -> the library matrix product (the reference calls its
-                             BLAS library here: kernels/matmul_cublas.cu:240-277)
-A weight that was stored in 32-bit stays 32-bit; under bfloat16 activations it
-runs through the float32 kernel.
-
-Up to 16 rows (and up to 32 when K is long) the block-split kernel runs: K is cut
-inside the workgroup, one launch gives the finished result. From 33 to 64 rows the
-library is faster on MI355X except for long K, where the wavefront kernel with K
-cut across workgroups wins; its fp32 partial sums are added by a small kernel, or,
-when a caller says `allow_split` and SPLIT_TO_CONSUMER is on, handed over as a
-:class:`SplitSum` to a kernel that adds the slices while it reads (the fused norm,
-the q/k/v kernel). That hand-over is off: with few rows the reading kernel has one
-workgroup per row and adding the slices there is slower than the small kernel.
+  float32 weights          -> the plain FMA kernel (fixed summation order per element);
+                              a weight that was stored in 32-bit stays 32-bit and runs
+                              through it also under bfloat16 activations
+  bfloat16, M <= 16        -> the block-split MFMA kernel: K is cut inside the workgroup,
+                              one launch gives the finished result
+  bfloat16, 17 <= M <= 64  -> the library, except for long K (>= 8192) while the library's
+                              tuner is off (its default kernels do not cut K): then the
+                              block-split kernel up to 32 rows and, up to 64, the wavefront
+                              kernel with K cut across workgroups
+  bfloat16, M > 64         -> the library matrix product (the reference calls its BLAS
+                              library for every product: kernels/matmul_cublas.cu:240-277)
+  fp32 results (logits)    -> the MFMA kernels up to 32 rows, above that the library,
+                              which writes fp32 from bf16 operands
+The wavefront kernel's fp32 partial sums are added by a small kernel, or, when a caller
+says `allow_split` and SPLIT_TO_CONSUMER is on, handed over as a :class:`SplitSum` to a
+kernel that adds the slices while it reads (the fused norm, the q/k/v kernel). That
+hand-over is off: with few rows the reading kernel has one workgroup per row and adding
+the slices there is slower than the small kernel.
 
 The block-split kernel also carries an RMS norm across a pair of products, so that a
 step of few rows has no norm kernels: given a :class:`ResidualSink` it adds its result
