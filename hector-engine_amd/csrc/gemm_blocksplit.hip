@@ -125,15 +125,15 @@ __device__ __forceinline__ int bs_spread(int M) {
 }
 
 template <int MT>
-__device__ __forceinline__ void bs_load_resid(const BsFusion& fu, int item, int n0, int M, int N,
-                                              float res[4], float gain[4]) {
+__device__ __forceinline__ void bs_load_resid(const BsFusion& fu, int item, int n0, int n_end, int M,
+                                              int N, float res[4], float gain[4]) {
   const int spread = bs_spread<MT>(M);
   const int ot = item >> 6, ol = item & 63;
   const int col = 16 * (ot % MT) + (ol & 15);
   const int m = col >> spread;
   const int n = n0 + 16 * (ot / MT) + 4 * (ol >> 4);
-  const int valid = (m < M && (m << spread) == col) ? max(0, min(4, N - n)) : 0;
-  if (valid == 4 && (N & 3) == 0) {
+  const int valid = (m < M && (m << spread) == col) ? max(0, min(4, n_end - n)) : 0;
+  if (valid == 4 && ((N | n0) & 3) == 0) {
     const float4 r4 = *reinterpret_cast<const float4*>(fu.resid + (int64_t)m * N + n);
     res[0] = r4.x, res[1] = r4.y, res[2] = r4.z, res[3] = r4.w;
   } else {
@@ -146,14 +146,17 @@ __device__ __forceinline__ void bs_load_resid(const BsFusion& fu, int item, int 
 template <int MT, int R, int U, bool GATED, typename TC>
 __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_kernel(
     TC* __restrict__ C, const uint16_t* __restrict__ X, const uint16_t* __restrict__ W,
-    const void* __restrict__ bias, int bias_dtype, int M, int N, int K, int kslice, BsFusion fu) {
+    const void* __restrict__ bias, int bias_dtype, int M, int N, int K, int kslice, int rows_per_block,
+    BsFusion fu) {
   extern __shared__ float4 tiles[];   // [NW][R*MT][64]
   __shared__ float row_scale[16 * MT];
   __shared__ float row_sq[R * MT][16];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
-  const int n0 = blockIdx.x * 16 * R;
+  // the workgroup's weight rows [n0, n_end): at most 16 R, fewer when the rows are dealt out evenly
+  const int n0 = blockIdx.x * rows_per_block;
+  const int n_end = min(N, n0 + rows_per_block);
   const int k_begin = wave * kslice;
   const int k_end = min(K, k_begin + kslice);
   const int lr = lane & 15, lg = lane >> 4;
@@ -162,7 +165,7 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
   const uint16_t* wp[R];
   const uint16_t* xp[MT];
 #pragma unroll
-  for (int r = 0; r < R; ++r) wp[r] = W + (int64_t)min(n0 + 16 * r + lr, N - 1) * K + lg * 16;
+  for (int r = 0; r < R; ++r) wp[r] = W + (int64_t)min(n0 + 16 * r + lr, n_end - 1) * K + lg * 16;
 #pragma unroll
   for (int t = 0; t < MT; ++t) xp[t] = X + (int64_t)min((16 * t + lr) >> spread, M - 1) * K + lg * 16;
 
@@ -194,7 +197,7 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
   }
   float res0[4] = {0.f, 0.f, 0.f, 0.f}, gain0[4] = {0.f, 0.f, 0.f, 0.f};
   if (to_resid && threadIdx.x < OUT_TILES * 64)
-    bs_load_resid<MT>(fu, threadIdx.x, n0, M, N, res0, gain0);
+    bs_load_resid<MT>(fu, threadIdx.x, n0, n_end, M, N, res0, gain0);
 
   // two steps of 64 U k values per turn; a step past k_end loads nothing and adds zeros.
   // The turns of a wavefront start at a point of its slice that differs from workgroup to
@@ -278,16 +281,16 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
       bs_store4<TC>(C + (int64_t)m * NO + n, v, (NO & 3) == 0, valid);
     } else {
       const int n = n0 + 16 * r + 4 * olg;
-      const int valid = owner ? max(0, min(4, N - n)) : 0;
+      const int valid = owner ? max(0, min(4, n_end - n)) : 0;
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] *= rs;
       if (bias != nullptr)
         for (int i = 0; i < valid; ++i) v[i] += load_param(bias, n + i, bias_dtype);
       if (!to_resid) {
-        if (valid > 0) bs_store4<TC>(C + (int64_t)m * N + n, v, (N & 3) == 0, valid);
+        if (valid > 0) bs_store4<TC>(C + (int64_t)m * N + n, v, ((N | n0) & 3) == 0, valid);
         continue;
       }
-      if (item != threadIdx.x) bs_load_resid<MT>(fu, item, n0, M, N, res0, gain0);
+      if (item != threadIdx.x) bs_load_resid<MT>(fu, item, n0, n_end, M, N, res0, gain0);
       float sq = 0.f, x[4], xgv[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -297,8 +300,8 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
       }
       if (valid > 0) {
         const int64_t at = (int64_t)m * N + n;
-        bs_store4<float>(fu.resid + at, x, (N & 3) == 0, valid);
-        bs_store4<bf16_t>(reinterpret_cast<bf16_t*>(fu.xg) + at, xgv, (N & 3) == 0, valid);
+        bs_store4<float>(fu.resid + at, x, ((N | n0) & 3) == 0, valid);
+        bs_store4<bf16_t>(reinterpret_cast<bf16_t*>(fu.xg) + at, xgv, ((N | n0) & 3) == 0, valid);
       }
       // the four lane groups hold the row's other columns of this tile
       sq += __shfl_xor(sq, 16, HE_WAVE);
@@ -320,6 +323,7 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
 
 struct BlockSplitPlan {
   int MT, R, U, NW, kslice;
+  int rows_per_block;   // weight rows of a workgroup, at most 16 R
 };
 
 // Tilings measured on MI355X (graph-timed sweeps over R, U and NW at the Qwen2.5-7B, Qwen2.5-32B
@@ -357,6 +361,16 @@ static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int
     nw = 8;
   }
   if (gated && (r & 1)) r = 2;
+  // Weight rows are dealt out evenly over the 256 compute units (or twice, three times ... 256
+  // workgroups, at most 32 rows each) rather than in whole tiles of 16: 4608 rows as 256
+  // workgroups of 18 rows instead of 144 of 32. The last tile of such a workgroup is partly
+  // empty. (Not with the gated epilogue, whose rows come in blocks of 32.)
+  int rows = 0;
+  if (!gated && R <= 0 && r <= 2 && N >= 2048 && N < 65536) {
+    const int rounds = (N + 256 * 32 - 1) / (256 * 32);
+    rows = (N + 256 * rounds - 1) / (256 * rounds);
+    r = rows > 16 ? 2 : 1;
+  }
   p.R = R > 0 ? R : r;
   p.U = U > 0 ? U : u;
   if (NW <= 0) {
@@ -367,6 +381,7 @@ static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int
   p.NW = NW;
   int ks = (K + NW - 1) / NW;
   p.kslice = (ks + 63) / 64 * 64;
+  p.rows_per_block = rows > 0 ? rows : 16 * p.R;
   return p;
 }
 
@@ -374,10 +389,11 @@ template <int MT, int R, int U, bool GATED, typename TC>
 static void launch_blocksplit(const BlockSplitPlan& p, void* C, const void* X, const void* W,
                               const void* bias, int bias_dtype, int M, int N, int K,
                               const BsFusion& fu, hipStream_t s) {
-  const int blocks = (N + 16 * R - 1) / (16 * R);
+  const int blocks = (N + p.rows_per_block - 1) / p.rows_per_block;
   const size_t lds = (size_t)p.NW * R * MT * 64 * sizeof(float4);
   gemm_blocksplit_kernel<MT, R, U, GATED, TC><<<blocks, 64 * p.NW, lds, s>>>(
-      (TC*)C, (const uint16_t*)X, (const uint16_t*)W, bias, bias_dtype, M, N, K, p.kslice, fu);
+      (TC*)C, (const uint16_t*)X, (const uint16_t*)W, bias, bias_dtype, M, N, K, p.kslice,
+      p.rows_per_block, fu);
 }
 
 template <bool GATED, typename TC>
@@ -402,7 +418,7 @@ static int dispatch_blocksplit(const BlockSplitPlan& p, void* C, const void* X, 
 extern "C" int he_gemm_blocksplit_blocks(int M, int N, int K) {
   if (M <= 0 || M > HE_BLOCKSPLIT_MAX_M || N <= 0 || K <= 0) return 0;
   const BlockSplitPlan p = blocksplit_plan(M, N, K, 0, 0, 0, 0);
-  return (N + 16 * p.R - 1) / (16 * p.R);
+  return (N + p.rows_per_block - 1) / p.rows_per_block;
 }
 
 // R, U, NW <= 0 choose the heuristic tiling (NW wavefronts = K slices per workgroup).
@@ -431,7 +447,7 @@ extern "C" int he_gemm_blocksplit_fused_bf16(void* C, const void* A, const void*
   HE_REQUIRE(p.NW >= 1 && p.NW <= 16, "he_gemm_blocksplit_bf16: %d wavefronts outside [1, 16]",
              p.NW);
   HE_REQUIRE(!gated || (p.R & 1) == 0, "he_gemm_blocksplit_bf16: the gated epilogue needs an even R");
-  const int blocks = (N + 16 * p.R - 1) / (16 * p.R);
+  const int blocks = (N + p.rows_per_block - 1) / p.rows_per_block;
   if (resid != nullptr) {
     HE_REQUIRE(!gated && gain != nullptr && xg != nullptr && sq_out != nullptr,
                "he_gemm_blocksplit_bf16: the residual epilogue needs gain, xg and sq_out, and no gate");

@@ -245,7 +245,7 @@ def test_gemm_skinny_gated_epilogue(ops, M, I, K):
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 20, 32])
-@pytest.mark.parametrize("N,K", [(301, 136), (1000, 1544), (37, 4104), (4608, 3584)])
+@pytest.mark.parametrize("N,K", [(301, 136), (1000, 1544), (37, 4104), (4608, 3584), (2051, 264)])
 @pytest.mark.parametrize("plan", [(0, 0, 0), (1, 1, 1), (2, 2, 4), (1, 2, 16), (2, 1, 8)])
 def test_gemm_blocksplit(ops, M, N, K, plan):
     """K cut inside the workgroup: every tiling gives the product, twice the same bits."""
@@ -285,7 +285,8 @@ def test_gemm_blocksplit_gated_epilogue(ops, M, I, K, nw):
 
 
 @pytest.mark.parametrize("M", [1, 8, 16])
-@pytest.mark.parametrize("D,K,N2,eps", [(80, 136, 301, 3e-6), (3584, 520, 160, 1e-6), (1000, 18944, 64, 1e-5)])
+@pytest.mark.parametrize("D,K,N2,eps", [(80, 136, 301, 3e-6), (3584, 520, 160, 1e-6), (1000, 18944, 64, 1e-5),
+                                        (2312, 264, 64, 1e-6)])
 @pytest.mark.parametrize("gain_dtype", [torch.bfloat16, torch.float32])
 def test_gemm_blocksplit_carries_the_norm(ops, M, D, K, N2, eps, gain_dtype):
     """A product adds its result to the residual rows and leaves r * gain and the sums of
