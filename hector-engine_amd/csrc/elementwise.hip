@@ -89,9 +89,9 @@ extern "C" int he_residual_add(void* resid_f32, const void* delta, int64_t n, in
 
 // out[r, i] = silu(gate[r, i]) * up[r, i] with x = [rows, 2I],
 // silu(z) = z / (1 + exp(-z)) in fp32 (reference: kernels/activations.cu:19-21,183-198).
-// Column layout of x: gate then up (x[r, i], x[r, I + i]); or, interleaved in
-// blocks of 16 as the fused gate||up weight of the MFMA path lays its rows out:
-// gate i at column 32*(i/16) + i%16, its up 16 columns later.
+// Column layout of x: gate then up (x[r, i], x[r, I + i]); or interleaved, as the
+// fused gate||up weight of the MFMA path lays its rows out: gate i at column 2i,
+// its up at 2i + 1.
 // With splits > 0, x is the fp32 K slices [splits][rows][2I] of the gate||up product,
 // added here in the order of the slice index.
 template <typename T, typename TI>
@@ -104,8 +104,8 @@ __global__ void silu_mul_kernel(T* __restrict__ out, const TI* __restrict__ x, i
   for (; i < n; i += stride) {
     const int64_t r = i / I;
     const int c = (int)(i - r * I);
-    const int gc = interleaved ? 32 * (c >> 4) + (c & 15) : c;
-    const int uc = interleaved ? gc + 16 : I + c;
+    const int gc = interleaved ? 2 * c : c;
+    const int uc = interleaved ? gc + 1 : I + c;
     const TI* row = x + r * 2 * (int64_t)I;
     float g = to_float(row[gc]), u = to_float(row[uc]);
     for (int s = 1; s < splits; ++s) {
@@ -117,8 +117,8 @@ __global__ void silu_mul_kernel(T* __restrict__ out, const TI* __restrict__ x, i
   }
 }
 
-// bf16, eight outputs per thread. Both layouts keep eight consecutive gates (and their
-// ups) contiguous when I is a multiple of 8 (16 for the interleaved one).
+// bf16, eight outputs per thread, I a multiple of 8: eight consecutive gates and their ups are
+// two runs of 16 bytes, or, interleaved, one run of 32 bytes of (gate, up) pairs.
 __global__ void silu_mul_vec_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ x,
                                     int64_t rows, int I, int interleaved) {
   const int64_t n8 = rows * (int64_t)(I >> 3);
@@ -128,18 +128,28 @@ __global__ void silu_mul_vec_kernel(uint16_t* __restrict__ out, const uint16_t* 
   for (; i < n8; i += stride) {
     const int64_t r = i / per_row;
     const int c = (int)(i - r * per_row) << 3;
-    const int gc = interleaved ? 32 * (c >> 4) + (c & 15) : c;
-    const int uc = interleaved ? gc + 16 : I + c;
     const uint16_t* row = x + r * 2 * (int64_t)I;
-    const uint4 g4 = *reinterpret_cast<const uint4*>(row + gc);
-    const uint4 u4 = *reinterpret_cast<const uint4*>(row + uc);
-    const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
     uint32_t o[4];
+    if (interleaved) {
+      const uint4 a = *reinterpret_cast<const uint4*>(row + 2 * c);
+      const uint4 b = *reinterpret_cast<const uint4*>(row + 2 * c + 8);
+      const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};   // (gate, up) a word
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
-      const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
-      o[j] = pack2_bf16(g0 / (1.f + expf(-g0)) * u0, g1 / (1.f + expf(-g1)) * u1);
+      for (int j = 0; j < 4; ++j) {
+        const float g0 = __uint_as_float(w[2 * j] << 16), u0 = __uint_as_float(w[2 * j] & 0xffff0000u);
+        const float g1 = __uint_as_float(w[2 * j + 1] << 16), u1 = __uint_as_float(w[2 * j + 1] & 0xffff0000u);
+        o[j] = pack2_bf16(g0 / (1.f + expf(-g0)) * u0, g1 / (1.f + expf(-g1)) * u1);
+      }
+    } else {
+      const uint4 g4 = *reinterpret_cast<const uint4*>(row + c);
+      const uint4 u4 = *reinterpret_cast<const uint4*>(row + I + c);
+      const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
+        const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
+        o[j] = pack2_bf16(g0 / (1.f + expf(-g0)) * u0, g1 / (1.f + expf(-g1)) * u1);
+      }
     }
     *reinterpret_cast<uint4*>(out + r * (int64_t)I + c) = make_uint4(o[0], o[1], o[2], o[3]);
   }
@@ -148,8 +158,6 @@ __global__ void silu_mul_vec_kernel(uint16_t* __restrict__ out, const uint16_t* 
 extern "C" int he_silu_mul(void* out, const void* gate_up, int rows, int I, int interleaved,
                            int splits, int dtype, void* stream) {
   HE_REQUIRE(rows >= 0 && I > 0, "he_silu_mul: bad sizes rows=%d I=%d", rows, I);
-  HE_REQUIRE(!interleaved || (I & 15) == 0,
-             "he_silu_mul: interleaved layout needs I=%d a multiple of 16", I);
   HE_REQUIRE(splits >= 0 && splits <= 64, "he_silu_mul: bad slice count %d", splits);
   HE_REQUIRE(dtype == HE_BF16 || dtype == HE_F32, "he_silu_mul: unknown dtype %d", dtype);
   if (rows == 0) return 0;
@@ -157,7 +165,7 @@ extern "C" int he_silu_mul(void* out, const void* gate_up, int rows, int I, int 
   int64_t blocks = (n + 255) / 256;
   if (blocks > 65535 * 4) blocks = 65535 * 4;
   hipStream_t s = (hipStream_t)stream;
-  if (splits == 0 && dtype == HE_BF16 && (I & (interleaved ? 15 : 7)) == 0 &&
+  if (splits == 0 && dtype == HE_BF16 && (I & 7) == 0 &&
       ((((uintptr_t)out) | ((uintptr_t)gate_up)) & 15) == 0) {
     const int64_t n8 = n >> 3;
     int64_t vb = (n8 + 255) / 256;

@@ -9,10 +9,10 @@
 // With 16 wavefronts a product as small as 3584 x 3584 still puts 3584
 // wavefronts on the chip.
 //
-// Gated epilogue: the weight interleaves gate and up rows in blocks of 16, the
-// two row tiles of a workgroup (R = 2) are a gate block and its up block, and the
-// output is silu(gate) * up, [M, N/2] (reference: kernels/activations.cu:183-198
-// as a kernel of its own).
+// Gated epilogue: the weight alternates gate and up rows (gate i at row 2i, its up at
+// 2i + 1), so the four neighbouring weight rows whose sums a thread holds are two
+// (gate, up) pairs, and the output is silu(gate) * up, [M, N/2] (reference:
+// kernels/activations.cu:183-198 as a kernel of its own).
 //
 // Two more epilogues carry an RMS norm across a pair of products without a kernel of
 // its own (reference: kernels/fused_add_rmsnorm.cu:47-81 as a separate kernel):
@@ -52,6 +52,27 @@ __device__ __forceinline__ void bs_store4<bf16_t>(bf16_t* p, const float v[4], b
     w.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
     w.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
     *reinterpret_cast<uint2*>(p) = w;
+  } else {
+    for (int i = 0; i < valid; ++i) p[i].v = float_to_bf16_bits(v[i]);
+  }
+}
+
+template <typename TC>
+__device__ __forceinline__ void bs_store2(TC* p, const float v[2], bool vec, int valid);
+template <>
+__device__ __forceinline__ void bs_store2<float>(float* p, const float v[2], bool vec, int valid) {
+  if (vec && valid == 2) {
+    *reinterpret_cast<float2*>(p) = make_float2(v[0], v[1]);
+  } else {
+    for (int i = 0; i < valid; ++i) p[i] = v[i];
+  }
+}
+template <>
+__device__ __forceinline__ void bs_store2<bf16_t>(bf16_t* p, const float v[2], bool vec,
+                                                  int valid) {
+  if (vec && valid == 2) {
+    *reinterpret_cast<uint32_t*>(p) =
+        (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
   } else {
     for (int i = 0; i < valid; ++i) p[i].v = float_to_bf16_bits(v[i]);
   }
@@ -179,7 +200,7 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
   // latency is not added at the end: the partial sums of squares of the input rows
   // (wavefront w takes the rows w and w + nw; lanes hold strided partials) and, for the
   // residual epilogue, the residual values and gains of this thread's first outputs.
-  constexpr int OUT_TILES = GATED ? (R / 2) * MT : R * MT;
+  constexpr int OUT_TILES = R * MT;
   const bool scaled = fu.scale_partials != nullptr;
   const bool to_resid = !GATED && fu.resid != nullptr;
   const bool scale_early = scaled && fu.scale_count <= 256 && M <= 2 * nw;
@@ -253,32 +274,29 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
     const int ot = item >> 6, ol = item & 63;
     const int olr = ol & 15, olg = ol >> 4;
     const int t = ot % MT;
-    const int r = GATED ? 2 * (ot / MT) : ot / MT;
+    const int r = ot / MT;
     const int col = 16 * t + olr, m = col >> spread;
     const bool owner = m < M && (m << spread) == col;
-    float4 s = make_float4(0.f, 0.f, 0.f, 0.f), s2 = s;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int w = 0; w < nw; ++w) {
       const float4 v = tiles[(w * (R * MT) + r * MT + t) * 64 + ol];
       s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
-      if (GATED) {
-        const float4 u2 = tiles[(w * (R * MT) + (r + 1) * MT + t) * 64 + ol];
-        s2.x += u2.x; s2.y += u2.y; s2.z += u2.z; s2.w += u2.w;
-      }
     }
     float v[4] = {s.x, s.y, s.z, s.w};
     const float rs = (scaled && m < M) ? row_scale[m] : 1.f;
     if (GATED) {
-      const float up[4] = {s2.x, s2.y, s2.z, s2.w};
+      // the thread's four weight rows are two (gate, up) pairs: two outputs
       const int NO = N >> 1;
-      const int n = (n0 >> 1) + 8 * r + 4 * olg;
-      const int valid = owner ? min(4, NO - n) : 0;
+      const int n = n0 + 16 * r + 4 * olg;
+      const int valid = owner ? max(0, min(4, n_end - n)) >> 1 : 0;
       if (valid <= 0) continue;
+      float y[2];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float g = v[i] * rs;
-        v[i] = g / (1.f + expf(-g)) * (up[i] * rs);
+      for (int i = 0; i < 2; ++i) {
+        const float g = v[2 * i] * rs;
+        y[i] = g / (1.f + expf(-g)) * (v[2 * i + 1] * rs);
       }
-      bs_store4<TC>(C + (int64_t)m * NO + n, v, (NO & 3) == 0, valid);
+      bs_store2<TC>(C + (int64_t)m * NO + (n >> 1), y, ((NO | (n0 >> 1)) & 1) == 0, valid);
     } else {
       const int n = n0 + 16 * r + 4 * olg;
       const int valid = owner ? max(0, min(4, n_end - n)) : 0;
@@ -360,15 +378,15 @@ static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int
     u = p.MT == 1 ? 4 : 1;
     nw = 8;
   }
-  if (gated && (r & 1)) r = 2;
   // Weight rows are dealt out evenly over the 256 compute units (or twice, three times ... 256
   // workgroups, at most 32 rows each) rather than in whole tiles of 16: 4608 rows as 256
-  // workgroups of 18 rows instead of 144 of 32. The last tile of such a workgroup is partly
-  // empty. (Not with the gated epilogue, whose rows come in blocks of 32.)
+  // workgroups of 18 rows instead of 144 of 32, the 37888 rows of gate||up as 1280 of 30
+  // instead of 1184 of 32 (4.6 a compute unit). The last tile of such a workgroup is partly
+  // empty. A workgroup's rows are an even number, so a gate stays with its up.
   int rows = 0;
-  if (!gated && R <= 0 && r <= 2 && N >= 2048 && N < 65536) {
+  if (R <= 0 && r <= 2 && N >= 2048 && N < 65536) {
     const int rounds = (N + 256 * 32 - 1) / (256 * 32);
-    rows = (N + 256 * rounds - 1) / (256 * rounds);
+    rows = ((N + 256 * rounds - 1) / (256 * rounds) + 1) & ~1;
     r = rows > 16 ? 2 : 1;
   }
   p.R = R > 0 ? R : r;
@@ -405,9 +423,7 @@ static int dispatch_blocksplit(const BlockSplitPlan& p, void* C, const void* X, 
     launch_blocksplit<MT_, R_, U_, GATED, TC>(p, C, X, W, bias, bias_dtype, M, N, K, fu, s); \
     return 0;                                                                        \
   }
-  if (!GATED) {
-    BS(1, 1, 1) BS(1, 1, 2) BS(1, 1, 4) BS(2, 1, 1) BS(2, 1, 2)
-  }
+  BS(1, 1, 1) BS(1, 1, 2) BS(1, 1, 4) BS(2, 1, 1) BS(2, 1, 2)
   BS(1, 2, 1) BS(1, 2, 2) BS(1, 2, 4) BS(2, 2, 1) BS(2, 2, 2) BS(1, 4, 1) BS(1, 4, 2)
 #undef BS
   he_set_error("he_gemm_blocksplit_bf16: no kernel for MT=%d R=%d U=%d", p.MT, p.R, p.U);
@@ -438,15 +454,13 @@ extern "C" int he_gemm_blocksplit_fused_bf16(void* C, const void* A, const void*
   HE_REQUIRE(out_dtype == HE_BF16 || out_dtype == HE_F32, "he_gemm_blocksplit_bf16: bad out dtype");
   HE_REQUIRE((((uintptr_t)A | (uintptr_t)W) & 15) == 0,
              "he_gemm_blocksplit_bf16: operands must be 16-byte aligned");
-  HE_REQUIRE(!gated || ((N & 31) == 0 && bias == nullptr),
-             "he_gemm_blocksplit_bf16: the gated epilogue needs N=%d a multiple of 32 and no bias",
-             N);
+  HE_REQUIRE(!gated || ((N & 1) == 0 && bias == nullptr),
+             "he_gemm_blocksplit_bf16: the gated epilogue needs an even N=%d and no bias", N);
   HE_REQUIRE(scale_partials == nullptr || scale_count > 0,
              "he_gemm_blocksplit_bf16: row scale without partial sums");
   const BlockSplitPlan p = blocksplit_plan(M, N, K, gated, R, U, NW);
   HE_REQUIRE(p.NW >= 1 && p.NW <= 16, "he_gemm_blocksplit_bf16: %d wavefronts outside [1, 16]",
              p.NW);
-  HE_REQUIRE(!gated || (p.R & 1) == 0, "he_gemm_blocksplit_bf16: the gated epilogue needs an even R");
   const int blocks = (N + p.rows_per_block - 1) / p.rows_per_block;
   if (resid != nullptr) {
     HE_REQUIRE(!gated && gain != nullptr && xg != nullptr && sq_out != nullptr,

@@ -23,10 +23,7 @@
 // floating-point atomics and no device-wide fences: a fence that makes one
 // XCD's writes visible to another costs more than the product itself.
 //
-// Epilogues: bias; or, for a weight whose rows interleave gate and up in blocks
-// of 16 (rows 32j..32j+15 gate, 32j+16..32j+31 the matching up rows), the gated
-// activation silu(gate) * up written as [M, N/2] (reference:
-// kernels/activations.cu:183-198 runs it as a kernel of its own).
+// Epilogue: bias.
 #include "common.h"
 #include "hector_kernels.h"
 
@@ -62,16 +59,12 @@ static void finish_plan(SkinnyPlan& p, int N, int K, int splits_wanted) {
 // Tilings measured on MI355X (graph-timed sweeps over R, U and the slice count at
 // the Qwen2.5-7B shapes); the rule depends on the sizes only, so a product always
 // runs the same way.
-static SkinnyPlan skinny_plan(int M, int N, int K, int gated) {
+static SkinnyPlan skinny_plan(int M, int N, int K) {
   SkinnyPlan p;
   p.MT = (M + 15) / 16;
   if (p.MT >= 3) p.MT = 4;
   int splits;
-  if (gated) {
-    p.R = p.MT == 4 ? 4 : 2;
-    p.U = 1;
-    splits = 1;
-  } else if (N >= 65536) {          // output head: plenty of row tiles, one slice
+  if (N >= 65536) {          // output head: plenty of row tiles, one slice
     p.R = p.MT == 4 ? 4 : 2;
     p.U = p.MT == 1 && M <= 8 ? 4 : (p.MT == 4 ? 1 : 2);
     splits = 1;
@@ -120,7 +113,7 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, const float v[4], bool
   }
 }
 
-template <int MT, int R, int U, bool GATED, typename TC>
+template <int MT, int R, int U, typename TC>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(
     TC* __restrict__ C, float* __restrict__ partial, const uint16_t* __restrict__ X, const uint16_t* __restrict__ W,
     const void* __restrict__ bias, int bias_dtype, int M, int N, int K, int ntiles, int splits,
@@ -197,29 +190,6 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(
     return;
   }
 
-  if (GATED) {
-    // rows of tile pair (2j, 2j+1) are gate and up of the outputs 16j..16j+15
-    const int NO = N >> 1;
-#pragma unroll
-    for (int r = 0; r < R; r += 2) {
-      const int n = (n0 >> 1) + 8 * r + 4 * lg;   // output column of acc[r][.][0]
-      const int valid = min(4, NO - n);
-      if (valid <= 0) continue;
-#pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        const int m = 16 * t + lr;
-        if (m >= M) continue;
-        float v[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float g = acc[r][t][i], u = acc[r + (R > 1 ? 1 : 0)][t][i];
-          v[i] = g / (1.f + __expf(-g)) * u;
-        }
-        store4<TC>(C + (int64_t)m * NO + n, v, (NO & 3) == 0, valid);
-      }
-    }
-    return;
-  }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int n = n0 + 16 * r + 4 * lg;
@@ -271,28 +241,26 @@ extern "C" int he_splitk_reduce(void* C, const void* partial_f32, const void* bi
   return he_check_launch("he_splitk_reduce");
 }
 
-template <int MT, int R, int U, bool GATED, typename TC>
+template <int MT, int R, int U, typename TC>
 static void launch_skinny(const SkinnyPlan& p, void* C, float* partial, const void* X,
                           const void* W, const void* bias, int bias_dtype, int M, int N, int K,
                           hipStream_t s) {
   const int waves = p.ntiles * p.splits;
-  gemm_skinny_kernel<MT, R, U, GATED, TC><<<(waves + 3) / 4, 256, 0, s>>>(
+  gemm_skinny_kernel<MT, R, U, TC><<<(waves + 3) / 4, 256, 0, s>>>(
       (TC*)C, partial, (const uint16_t*)X, (const uint16_t*)W, bias, bias_dtype, M, N, K, p.ntiles,
       p.splits, p.kslice);
 }
 
-template <bool GATED, typename TC>
+template <typename TC>
 static int dispatch_skinny(const SkinnyPlan& p, void* C, float* partial, const void* X,
                            const void* W, const void* bias, int bias_dtype, int M, int N, int K,
                            hipStream_t s) {
 #define SK(MT_, R_, U_)                                                                 \
   if (p.MT == MT_ && p.R == R_ && p.U == U_) {                                          \
-    launch_skinny<MT_, R_, U_, GATED, TC>(p, C, partial, X, W, bias, bias_dtype, M, N, K, s); \
+    launch_skinny<MT_, R_, U_, TC>(p, C, partial, X, W, bias, bias_dtype, M, N, K, s); \
     return 0;                                                                           \
   }
-  if (!GATED) {
-    SK(1, 1, 1) SK(1, 1, 2) SK(1, 1, 4)
-  }
+  SK(1, 1, 1) SK(1, 1, 2) SK(1, 1, 4)
   SK(1, 2, 1) SK(1, 2, 2) SK(1, 2, 4) SK(2, 2, 1) SK(2, 2, 2) SK(4, 4, 1) SK(4, 2, 1) SK(4, 2, 2)
   SK(1, 4, 1) SK(1, 4, 2) SK(2, 4, 1) SK(2, 4, 2)
 #undef SK
@@ -301,7 +269,7 @@ static int dispatch_skinny(const SkinnyPlan& p, void* C, float* partial, const v
 }
 
 static int check_skinny(const void* A, const void* W, const void* bias, int M, int N, int K,
-                        int out_dtype, int gated) {
+                        int out_dtype) {
   HE_REQUIRE(M > 0 && M <= HE_SKINNY_MAX_M, "he_gemm_skinny_bf16: M=%d outside [1, %d]", M,
              HE_SKINNY_MAX_M);
   HE_REQUIRE(N > 0 && K > 0, "he_gemm_skinny_bf16: bad sizes N=%d K=%d", N, K);
@@ -309,15 +277,13 @@ static int check_skinny(const void* A, const void* W, const void* bias, int M, i
   HE_REQUIRE(out_dtype == HE_BF16 || out_dtype == HE_F32, "he_gemm_skinny_bf16: bad out dtype");
   HE_REQUIRE((((uintptr_t)A | (uintptr_t)W) & 15) == 0,
              "he_gemm_skinny_bf16: operands must be 16-byte aligned");
-  HE_REQUIRE(!gated || ((N & 31) == 0 && bias == nullptr),
-             "he_gemm_skinny_bf16: the gated epilogue needs N=%d a multiple of 32 and no bias", N);
   return 0;
 }
 
 // Number of K slices the heuristic cuts this product into (1 = none).
 extern "C" int he_gemm_skinny_splits(int M, int N, int K) {
   if (M <= 0 || N <= 0 || K <= 0) return 1;
-  return skinny_plan(M, N, K, 0).splits;
+  return skinny_plan(M, N, K).splits;
 }
 
 // R, U <= 0: the heuristic tiling. splits <= 0: the heuristic's slice count.
@@ -325,33 +291,26 @@ extern "C" int he_gemm_skinny_splits(int M, int N, int K) {
 // [slices][M][N] fp32 sums; *splits_used tells how many slices were written.
 extern "C" int he_gemm_skinny_bf16(void* C, void* partial_f32, int64_t partial_floats,
                                    const void* A, const void* W, const void* bias, int M, int N,
-                                   int K, int out_dtype, int bias_dtype, int gated, int R, int U,
+                                   int K, int out_dtype, int bias_dtype, int R, int U,
                                    int splits, int* splits_used, void* stream) {
-  if (int rc = check_skinny(A, W, bias, M, N, K, out_dtype, gated)) return rc;
-  SkinnyPlan p = skinny_plan(M, N, K, gated);
+  if (int rc = check_skinny(A, W, bias, M, N, K, out_dtype)) return rc;
+  SkinnyPlan p = skinny_plan(M, N, K);
   if (R > 0) p.R = R;
   if (U > 0) p.U = U;
-  if (R > 0 || U > 0 || splits > 0) finish_plan(p, N, K, gated ? 1 : splits);
+  if (R > 0 || U > 0 || splits > 0) finish_plan(p, N, K, splits);
   const int64_t need = p.splits > 1 ? (int64_t)p.splits * M * N : 0;
   HE_REQUIRE(partial_floats >= need && (need == 0 || partial_f32 != nullptr),
              "he_gemm_skinny_bf16: room for %lld partial sums, need %lld",
              (long long)partial_floats, (long long)need);
   HE_REQUIRE(need == 0 || (((uintptr_t)partial_f32) & 15) == 0,
              "he_gemm_skinny_bf16: the partial sums must be 16-byte aligned");
-  HE_REQUIRE(!gated || (p.splits == 1 && p.R >= 2),
-             "he_gemm_skinny_bf16: the gated epilogue needs one K slice and row-tile pairs");
   if (splits_used) *splits_used = p.splits;
   hipStream_t s = (hipStream_t)stream;
   float* partial = (float*)partial_f32;
   int rc;
-  if (gated)
-    rc = out_dtype == HE_BF16
-             ? dispatch_skinny<true, bf16_t>(p, C, partial, A, W, bias, bias_dtype, M, N, K, s)
-             : dispatch_skinny<true, float>(p, C, partial, A, W, bias, bias_dtype, M, N, K, s);
-  else
-    rc = out_dtype == HE_BF16
-             ? dispatch_skinny<false, bf16_t>(p, C, partial, A, W, bias, bias_dtype, M, N, K, s)
-             : dispatch_skinny<false, float>(p, C, partial, A, W, bias, bias_dtype, M, N, K, s);
+  rc = out_dtype == HE_BF16
+           ? dispatch_skinny<bf16_t>(p, C, partial, A, W, bias, bias_dtype, M, N, K, s)
+           : dispatch_skinny<float>(p, C, partial, A, W, bias, bias_dtype, M, N, K, s);
   if (rc) return rc;
   return he_check_launch("he_gemm_skinny_bf16");
 }

@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 12
+#define HE_ABI_VERSION 13
 
 #ifdef __cplusplus
 extern "C" {
@@ -42,14 +42,12 @@ int he_gemm_plain(void* C, const void* A, const void* W, const void* bias, int M
                   int bias_dtype, void* stream);
 // bf16 MFMA product for M <= HE_SKINNY_MAX_M rows: every weight element is read once.
 #define HE_SKINNY_MAX_M 64
-// gated: W's rows interleave gate and up in blocks of 16 and C is [M, N/2] = silu(gate) * up.
 // R, U, splits <= 0 choose the heuristic tiling. When K is cut into more than one slice, C is
 // not written: partial_f32 receives fp32 [slices][M][N] (bias not added) and *splits_used says
 // how many; the reader adds them in index order (he_splitk_reduce, he_add_rmsnorm, he_qkv_rope_cache).
 int he_gemm_skinny_bf16(void* C, void* partial_f32, int64_t partial_floats, const void* A,
                         const void* W, const void* bias, int M, int N, int K, int out_dtype,
-                        int bias_dtype, int gated, int R, int U, int splits, int* splits_used,
-                        void* stream);
+                        int bias_dtype, int R, int U, int splits, int* splits_used, void* stream);
 int he_gemm_skinny_splits(int M, int N, int K);
 // bf16 MFMA product for M <= HE_BLOCKSPLIT_MAX_M with K cut inside the workgroup (NW
 // wavefronts, one slice each, added in LDS): complete in one launch.

@@ -16,7 +16,7 @@ _lib = None
 
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 
-EXPECTED_ABI = 12
+EXPECTED_ABI = 13
 
 c_int, c_i64, c_f32, c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
@@ -33,7 +33,7 @@ _SIGNATURES = {
     "he_gemm_plain": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_i64, c_i64, c_i64,
                       c_int, c_int, c_int, c_ptr],
     "he_gemm_skinny_bf16": [c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int,
-                            c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(c_int), c_ptr],
+                            c_int, c_int, c_int, c_int, ctypes.POINTER(c_int), c_ptr],
     "he_gemm_skinny_splits": [c_int, c_int, c_int],
     "he_gemm_blocksplit_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_int,
                                 c_int, c_int, c_int, c_ptr],

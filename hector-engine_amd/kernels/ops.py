@@ -164,16 +164,14 @@ def gemm_skinny_splits(M: int, N: int, K: int) -> int:
     return int(_lib.load().he_gemm_skinny_splits(M, N, K))
 
 
-def gemm_skinny(out, partial, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0),
-                out_dtype=None) -> int:
+def gemm_skinny(out, partial, a, w, bias, M: int, plan=(0, 0, 0), out_dtype=None) -> int:
     """bf16 MFMA product for M <= 64. plan = (R, U, splits), zeros for the heuristic.
-    With one K slice `out` (bf16 or fp32) is written, with bias or, gated, as
-    [M, N/2] = silu(gate) * up for a weight that interleaves gate and up rows in blocks
-    of 16. With more slices `partial` (fp32, room for [slices, M, N]) is written
-    instead, without bias. Returns the number of slices."""
+    With one K slice `out` (bf16 or fp32) is written, with bias. With more slices
+    `partial` (fp32, room for [slices, M, N]) is written instead, without bias. Returns
+    the number of slices."""
     import ctypes
     N, K = w.shape
-    NO = N // 2 if gated else N
+    NO = N
     _need(a, "a", torch.bfloat16)
     _need(w, "w", torch.bfloat16)
     if M > SKINNY_MAX_M:
@@ -197,7 +195,7 @@ def gemm_skinny(out, partial, a, w, bias, M: int, gated: bool = False, plan=(0, 
         raise ValueError("gemm_skinny: neither an output nor room for partial sums")
     _lib.check(L.he_gemm_skinny_bf16(_ptr(out), _ptr(partial), pfloats, a.data_ptr(), w.data_ptr(),
                                      _ptr(bias), M, N, K, dtype_code(out_dtype or torch.bfloat16),
-                                     dtype_code(bias.dtype) if bias is not None else F32, int(gated),
+                                     dtype_code(bias.dtype) if bias is not None else F32,
                                      int(plan[0]), int(plan[1]), int(plan[2]), ctypes.byref(used),
                                      _stream()))
     if used.value == 1 and out is None:
@@ -217,7 +215,8 @@ def gemm_blocksplit(out, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0)
                     row_scale=None, residual=None) -> None:
     """bf16 MFMA product for M <= 32 with K cut inside the workgroup; one launch, complete
     result (bf16 or fp32), with bias or, gated, as [M, N/2] = silu(gate) * up for a weight
-    that interleaves gate and up rows in blocks of 16. plan = (R, U, NW), zeros = heuristic.
+    that alternates gate and up rows (gate i at row 2i, its up at 2i + 1). plan = (R, U, NW),
+    zeros = heuristic.
 
     row_scale = (partials fp32 [M, count], eps): the rows of `a` are r * gain of an RMS norm
     whose 1/sqrt(mean(r^2) + eps) is applied to the sums here (mean over K).

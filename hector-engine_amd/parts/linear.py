@@ -193,12 +193,12 @@ class Linear:
 
     def gated_silu(self, x, rows: int, ctx: StepContext, out: torch.Tensor) -> bool:
         """out[rows, N/2] = silu(gate) * up in one kernel, for a weight whose rows
-        interleave gate and up in blocks of 16. x: a tensor or NormedRows. False when that
+        alternate gate and up (gate i at row 2i, its up at 2i + 1). x: a tensor or NormedRows. False when that
         kernel does not apply."""
         w = self.weight
         act = x.scaled.dtype if isinstance(x, NormedRows) else x.dtype
         if not (ctx.env.fast_kernels and w.dtype == torch.bfloat16 and act == torch.bfloat16
-                and 0 < rows <= 16 and w.shape[1] % 8 == 0 and w.shape[0] % 32 == 0):
+                and 0 < rows <= 16 and w.shape[1] % 8 == 0 and w.shape[0] % 2 == 0):
             return False
         if isinstance(x, NormedRows):
             ops.gemm_blocksplit(out, x.scaled, w, None, rows, gated=True, row_scale=(x.partials, x.eps))

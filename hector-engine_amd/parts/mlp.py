@@ -26,7 +26,6 @@ class GatedMLP(FeedForward):
         act = param(params, "activation", str, "silu")
         if act not in ("silu", "swish"):
             raise ValueError(f"gated_mlp: unsupported activation '{act}'")
-        self.interleaved = False
         self.gate_up: Linear | None = None
         self.down: Linear | None = None
 
@@ -43,16 +42,10 @@ class GatedMLP(FeedForward):
         g, u = tensors.pop(p + "gate_proj.weight"), tensors.pop(p + "up_proj.weight")
         if g.dtype != u.dtype:
             raise TypeError(f"{p}gate_proj and up_proj are stored in different dtypes")
-        if self.inter % 16 == 0:
-            # rows interleaved in blocks of 16 (gate block j, then up block j): the tile pair
-            # of one MFMA wavefront then holds a gate and its up, and the gated activation
-            # is the product's epilogue
-            I, D = g.shape
-            w = torch.stack([g.view(I // 16, 16, D), u.view(I // 16, 16, D)], 1).reshape(2 * I, D)
-            self.interleaved = True
-        else:
-            w = torch.cat([g, u], 0)
-            self.interleaved = False
+        # gate and up rows alternate (gate i at row 2i, its up at 2i + 1): the four neighbouring
+        # rows whose sums a thread of the MFMA product holds are then two (gate, up) pairs, and
+        # the gated activation is that product's epilogue
+        w = torch.stack([g, u], 1).reshape(2 * g.shape[0], g.shape[1])
         self.gate_up = Linear(w.contiguous())
         del g, u, w
         self.down = Linear(tensors[p + "down_proj.weight"])
@@ -61,12 +54,12 @@ class GatedMLP(FeedForward):
         rows = ctx.rows
         if rows <= _ROW_CHUNK:
             h = ctx.alloc((rows, self.inter))
-            if not (self.interleaved and self.gate_up.gated_silu(x, rows, ctx, h)):
+            if not self.gate_up.gated_silu(x, rows, ctx, h):
                 gu = self.gate_up(x, rows, ctx, allow_split=True)
                 if isinstance(gu, SplitSum):     # K slices: the activation kernel adds them while it reads
-                    ops.silu_mul(h, gu.partial, rows, self.interleaved, gu.splits)
+                    ops.silu_mul(h, gu.partial, rows, True, gu.splits)
                 else:
-                    ops.silu_mul(h, gu, rows, self.interleaved)
+                    ops.silu_mul(h, gu, rows, True)
             return self.down(h, rows, ctx, allow_split=True, sink=ctx.take_sink())
         if not isinstance(x, torch.Tensor):
             x = x.tensor(ctx)
@@ -76,7 +69,7 @@ class GatedMLP(FeedForward):
             turn = ctx.scratch.mark()
             h = ctx.alloc((n, self.inter))
             gu = self.gate_up(x[r0:r0 + n], n, ctx)
-            ops.silu_mul(h, gu, n, self.interleaved)
+            ops.silu_mul(h, gu, n, True)
             self.down(h, n, ctx, out=out[r0:r0 + n])
             ctx.scratch.release(turn)       # the next turn reuses h and gate||up
         return out

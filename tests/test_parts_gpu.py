@@ -103,7 +103,7 @@ def test_rotary_part(fw):
 
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("rows", [5, 100])
-@pytest.mark.parametrize("inter", [136, 160])          # 160: gate and up interleaved in blocks of 16
+@pytest.mark.parametrize("inter", [136, 160, 37])
 def test_gated_mlp_part(fw, dtype, rows, inter):
     env = env_for(fw, dtype)
     mlp = fw.parts.build_part("feed_forward", fw.parts.PartSpec(
@@ -113,7 +113,6 @@ def test_gated_mlp_part(fw, dtype, rows, inter):
         "m.gate_proj.weight": (inter, 80), "m.up_proj.weight": (inter, 80), "m.down_proj.weight": (80, inter)}
     w = {k: rnd(*v.shape, seed=i, scale=0.1).to(dtype) for i, (k, v) in enumerate(specs.items())}
     mlp.bind({k: v.cuda() for k, v in w.items()})
-    assert mlp.interleaved == (inter % 16 == 0)
     ctx = make_ctx(fw, env, [rows], [0], [0])
     x = rnd(rows, 80, seed=9).to(dtype)
     out = as_tensor(mlp.forward(x.cuda(), ctx), ctx)
