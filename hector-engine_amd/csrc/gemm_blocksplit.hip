@@ -34,24 +34,30 @@ __device__ __forceinline__ bf16x8 bs_load8(const uint16_t* p, bool ok) {
   return __builtin_bit_cast(bf16x8, v);
 }
 
+// Four neighbouring outputs. align: how many elements the address is a multiple of (4, 2 or 1).
 template <typename TC>
-__device__ __forceinline__ void bs_store4(TC* p, const float v[4], bool vec, int valid);
+__device__ __forceinline__ void bs_store4(TC* p, const float v[4], int align, int valid);
 template <>
-__device__ __forceinline__ void bs_store4<float>(float* p, const float v[4], bool vec, int valid) {
-  if (vec && valid == 4) {
+__device__ __forceinline__ void bs_store4<float>(float* p, const float v[4], int align, int valid) {
+  if (align >= 4 && valid == 4) {
     *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  } else if (align >= 2 && valid == 4) {
+    *reinterpret_cast<float2*>(p) = make_float2(v[0], v[1]);
+    *reinterpret_cast<float2*>(p + 2) = make_float2(v[2], v[3]);
   } else {
     for (int i = 0; i < valid; ++i) p[i] = v[i];
   }
 }
 template <>
-__device__ __forceinline__ void bs_store4<bf16_t>(bf16_t* p, const float v[4], bool vec,
+__device__ __forceinline__ void bs_store4<bf16_t>(bf16_t* p, const float v[4], int align,
                                                   int valid) {
-  if (vec && valid == 4) {
-    uint2 w;
-    w.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
-    w.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
-    *reinterpret_cast<uint2*>(p) = w;
+  const uint32_t lo = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+  const uint32_t hi = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+  if (align >= 4 && valid == 4) {
+    *reinterpret_cast<uint2*>(p) = make_uint2(lo, hi);
+  } else if (align >= 2 && valid == 4) {
+    *reinterpret_cast<uint32_t*>(p) = lo;
+    *reinterpret_cast<uint32_t*>(p + 2) = hi;
   } else {
     for (int i = 0; i < valid; ++i) p[i].v = float_to_bf16_bits(v[i]);
   }
@@ -157,6 +163,10 @@ __device__ __forceinline__ void bs_load_resid(const BsFusion& fu, int item, int 
   if (valid == 4 && ((N | n0) & 3) == 0) {
     const float4 r4 = *reinterpret_cast<const float4*>(fu.resid + (int64_t)m * N + n);
     res[0] = r4.x, res[1] = r4.y, res[2] = r4.z, res[3] = r4.w;
+  } else if (valid == 4 && ((N | n0) & 1) == 0) {
+    const float2 a = *reinterpret_cast<const float2*>(fu.resid + (int64_t)m * N + n);
+    const float2 b = *reinterpret_cast<const float2*>(fu.resid + (int64_t)m * N + n + 2);
+    res[0] = a.x, res[1] = a.y, res[2] = b.x, res[3] = b.y;
   } else {
     for (int i = 0; i < 4; ++i) res[i] = i < valid ? fu.resid[(int64_t)m * N + n + i] : 0.f;
   }
@@ -201,6 +211,7 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
   // (wavefront w takes the rows w and w + nw; lanes hold strided partials) and, for the
   // residual epilogue, the residual values and gains of this thread's first outputs.
   constexpr int OUT_TILES = R * MT;
+  const int out_align = ((N | n0) & 3) == 0 ? 4 : (((N | n0) & 1) == 0 ? 2 : 1);
   const bool scaled = fu.scale_partials != nullptr;
   const bool to_resid = !GATED && fu.resid != nullptr;
   const bool scale_early = scaled && fu.scale_count <= 256 && M <= 2 * nw;
@@ -305,7 +316,7 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
       if (bias != nullptr)
         for (int i = 0; i < valid; ++i) v[i] += load_param(bias, n + i, bias_dtype);
       if (!to_resid) {
-        if (valid > 0) bs_store4<TC>(C + (int64_t)m * N + n, v, ((N | n0) & 3) == 0, valid);
+        if (valid > 0) bs_store4<TC>(C + (int64_t)m * N + n, v, out_align, valid);
         continue;
       }
       if (item != threadIdx.x) bs_load_resid<MT>(fu, item, n0, n_end, M, N, res0, gain0);
@@ -318,8 +329,8 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
       }
       if (valid > 0) {
         const int64_t at = (int64_t)m * N + n;
-        bs_store4<float>(fu.resid + at, x, ((N | n0) & 3) == 0, valid);
-        bs_store4<bf16_t>(reinterpret_cast<bf16_t*>(fu.xg) + at, xgv, ((N | n0) & 3) == 0, valid);
+        bs_store4<float>(fu.resid + at, x, out_align, valid);
+        bs_store4<bf16_t>(reinterpret_cast<bf16_t*>(fu.xg) + at, xgv, out_align, valid);
       }
       // the four lane groups hold the row's other columns of this tile
       sq += __shfl_xor(sq, 16, HE_WAVE);
@@ -382,7 +393,8 @@ static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int
   // workgroups, at most 32 rows each) rather than in whole tiles of 16: 4608 rows as 256
   // workgroups of 18 rows instead of 144 of 32, the 37888 rows of gate||up as 1280 of 30
   // instead of 1184 of 32 (4.6 a compute unit). The last tile of such a workgroup is partly
-  // empty. A workgroup's rows are an even number, so a gate stays with its up.
+  // empty. A workgroup's rows are an even number: a gate stays with its up, and outputs can be
+  // stored in pairs.
   int rows = 0;
   if (R <= 0 && r <= 2 && N >= 2048 && N < 65536) {
     const int rounds = (N + 256 * 32 - 1) / (256 * 32);

@@ -242,6 +242,32 @@ def alternate_rows(g, u):
     return torch.stack([g, u], 1).reshape(2 * g.shape[0], g.shape[1]).contiguous()
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 20, 32])
+@pytest.mark.parametrize("N,K", [(301, 136), (1000, 1544), (37, 4104), (4608, 3584), (2051, 264)])
+@pytest.mark.parametrize("plan", [(0, 0, 0), (1, 1, 1), (2, 2, 4), (1, 2, 16), (2, 1, 8)])
+def test_gemm_blocksplit(ops, M, N, K, plan):
+    """K cut inside the workgroup: every tiling gives the product, twice the same bits."""
+    if (N, K) == (4608, 3584) and (M not in (1, 32) or plan[2] not in (0, 16)):
+        pytest.skip("large shape at two row counts and two tilings only")
+    if M > 16 and plan[1] == 4:
+        pytest.skip("not instantiated")
+    a = rnd(M, K, seed=90).to(torch.bfloat16)
+    w = rnd(N, K, seed=91, scale=0.05).to(torch.bfloat16)
+    b = rnd(N, seed=92).to(torch.bfloat16)
+    ref = a.double() @ w.double().T + b.double()
+    outs = []
+    for _ in range(2):
+        out = torch.empty(M, N, dtype=torch.float32, device="cuda")
+        ops.gemm_blocksplit(out, dev(a), dev(w), dev(b), M, plan=plan)
+        outs.append(out.cpu())
+    assert torch.equal(outs[0], outs[1])
+    assert (outs[0].double() - ref).abs().max().item() <= 1e-4 * ref.abs().max().item()
+    out16 = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    ops.gemm_blocksplit(out16, dev(a), dev(w), None, M, plan=plan)
+    ref0 = a.double() @ w.double().T
+    assert (out16.cpu().double() - ref0).abs().max().item() <= 2 ** -8 * ref0.abs().max().item() + 1e-6
+
+
 @pytest.mark.parametrize("M", [1, 8, 20, 32])
 @pytest.mark.parametrize("I,K", [(160, 64), (1008, 520), (37, 136), (1515, 264)])
 @pytest.mark.parametrize("plan", [(0, 0, 0), (1, 0, 1), (2, 0, 8)])
