@@ -24,33 +24,48 @@
 #define FUSED_MIN_CHUNK 64
 
 // q of the group's heads as B operand, from the un-biased projection row: lane (lr =
-// head column, lg) holds dims 32ks + 8lg .. +8 of head lr for every k step ks. The partner
-// of dim d < half is d + half = the same lane's element in k step ks + half/32. sn, c: the
-// sine and cosine of angle `lane` (lanes below half), fetched from the lane that holds them.
+// head column, lg) holds dims 32ks + 8lg .. +8 of head lr for every k step ks. In two parts,
+// so that the loads can be issued before anything else and the rotation done while the first
+// keys are on their way: the biased values, then the rotation. The partner of dim d < half is
+// d + half = the same lane's element in k step ks + half/32. sn, c: the sine and cosine of
+// angle `lane` (lanes below half), fetched from the lane that holds them.
 template <int NT>
-__device__ __forceinline__ void load_q_rotated(bf16x8* qf, const uint16_t* qrow,
-                                               const void* bias, int bias_dtype, int bias_off,
-                                               bool valid, int lg, float sn, float c) {
-  constexpr int HD = 16 * NT;
-  constexpr int KS = HD / 32;
-  constexpr int HS = KS / 2;   // k steps per half of the head
-  float x[KS][8];
+__device__ __forceinline__ void load_q_biased(float (&x)[NT / 2][8], const uint16_t* qrow,
+                                              const void* bias, int bias_dtype, int bias_off,
+                                              bool valid, int lg) {
+  constexpr int KS = NT / 2;
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
     const int d0 = 32 * ks + 8 * lg;
-    const bool ok = valid && d0 < HD;
     uint4 raw = make_uint4(0, 0, 0, 0);
-    if (ok) raw = *reinterpret_cast<const uint4*>(qrow + d0);
+    if (valid) raw = *reinterpret_cast<const uint4*>(qrow + d0);
     const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       x[ks][2 * j] = __uint_as_float(w[j] << 16);
       x[ks][2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
     }
-    if (ok && bias != nullptr)
+    if (valid && bias != nullptr) {
+      if (bias_dtype == HE_BF16 && (((uintptr_t)bias) & 15) == 0) {   // the eight values in one load
+        const uint4 b4 = *reinterpret_cast<const uint4*>((const uint16_t*)bias + bias_off + d0);
+        const uint32_t bw[4] = {b4.x, b4.y, b4.z, b4.w};
 #pragma unroll
-      for (int j = 0; j < 8; ++j) x[ks][j] += load_param(bias, bias_off + d0 + j, bias_dtype);
+        for (int j = 0; j < 4; ++j) {
+          x[ks][2 * j] += __uint_as_float(bw[j] << 16);
+          x[ks][2 * j + 1] += __uint_as_float(bw[j] & 0xffff0000u);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[ks][j] += load_param(bias, bias_off + d0 + j, bias_dtype);
+      }
+    }
   }
+}
+
+template <int NT>
+__device__ __forceinline__ void rotate_q(bf16x8* qf, float (&x)[NT / 2][8], int lg, float sn, float c) {
+  constexpr int KS = NT / 2;
+  constexpr int HS = KS / 2;   // k steps per half of the head
 #pragma unroll
   for (int ks = 0; ks < HS; ++ks)
 #pragma unroll
@@ -89,6 +104,11 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
   const int GT = min(16, G - 16 * ht);     // heads of this tile
   const bool h_ok = lr < GT;
   const int h = kvh * G + 16 * ht + min(lr, GT - 1);
+  // loads that need nothing but the row: issued first, used last
+  const uint16_t* qkv_row = qkv + (int64_t)row * qkv_stride;
+  float qx[NT / 2][8];
+  load_q_biased<NT>(qx, qkv_row + (int64_t)h * HD, bias, bias_dtype, h * HD, h_ok, lg);
+  const float freq = lane < HD / 2 ? inv_freq[lane] : 0.f;
   const int seq = row_seq[row];
   const int Z = gridDim.z, z = blockIdx.z;
   if (seq < 0) {                           // padding row: zeros (from the merge kernel if there is one)
@@ -108,13 +128,18 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
   const int kb_begin = span_lo + (z * nw + wave) * chunk;
   const int kb_end = min(kb_begin + chunk, n_keys);
   const int32_t* pt = page_table + (int64_t)slot * max_blocks;
-  const uint16_t* qkv_row = qkv + (int64_t)row * qkv_stride;
   const bool has_keys = kb_begin < kb_end;   // uniform in the wavefront
+  // the first keys and values are asked for before the angles are computed and q is rotated -
+  // unless this wavefront writes the new key into that very step
+  const bool writes = write_kv && p >= kb_begin && p < kb_end;
+  const bool early = has_keys && !(writes && p < kb_begin + 32);
+  AttendCursor<NT> cursor;
+  if (early) attend_start<NT>(cursor, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, kb_begin, lr, lg);
   float sn = 0.f, c = 1.f;                   // lane j < HD / 2: angle j of position p
-  if (has_keys && lane < HD / 2) sincos_angle((float)p * inv_freq[lane], &sn, &c);
+  if (has_keys && lane < HD / 2) sincos_angle((float)p * freq, &sn, &c);
 
   // ---- the new key and value go into the cache, written by the wavefront that reads them
-  if (write_kv && p >= kb_begin && p < kb_end) {
+  if (writes) {
     const int page = pt[p >> HE_PAGE_SHIFT];
     if (page >= 0 && page < num_pages) {
       const int off = p & (HE_PAGE_TOKENS - 1);
@@ -150,10 +175,10 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
   st.l = 0.f;
   if (has_keys) {
     bf16x8 qf[KS];
-    load_q_rotated<NT>(qf, qkv_row + (int64_t)h * HD, bias, bias_dtype, h * HD, h_ok, lg, sn, c);
-    attend_range<NT, false>(st, qf, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, kb_begin,
-                            (kb_end + 31) & ~31, first, p, first, p,
-                            scale * 1.4426950408889634f, lr, lg);
+    rotate_q<NT>(qf, qx, lg, sn, c);
+    if (!early) attend_start<NT>(cursor, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, kb_begin, lr, lg);
+    attend_walk<NT, false>(st, qf, cursor, pt, max_blocks, num_pages, kb_begin, (kb_end + 31) & ~31,
+                           first, p, first, p, scale * 1.4426950408889634f, lr, lg);
   }
   float l = st.l;
   l = xor32_sum(xor16_sum(l));

@@ -131,6 +131,65 @@ __device__ __forceinline__ void attend_frag(AttnState<NT>& st, const bf16x8* qf,
 // Runs the steps kb = kb_begin, kb_begin + 32, ... < kb_end (all multiples of 32) of one
 // (sequence, kv head) against the state, one step ahead with its loads and one page
 // ahead with its page-table entry.
+// Where a walk over the keys stands: the page of the current step, the entry of the page
+// after it, and the fragments of the step to come, already on their way.
+template <int NT>
+struct AttendCursor {
+  const uint16_t* kp;
+  const uint16_t* vp;
+  int64_t k_stride, v_stride;
+  int block, page, page_ahead;
+  KVFrag<NT> cur;
+};
+
+// Starts the walk at key kb_begin (a multiple of 32): reads the page-table entries and issues
+// the loads of the first step. A caller with other work to do (a query to load and rotate)
+// does it between this and attend_walk, while the fragments are on their way.
+template <int NT>
+__device__ __forceinline__ void attend_start(AttendCursor<NT>& c, const uint16_t* __restrict__ kpool,
+                                             const uint16_t* __restrict__ vpool,
+                                             const int32_t* __restrict__ pt, int max_blocks,
+                                             int num_pages, int KVH, int kvh, int kb_begin, int lr,
+                                             int lg) {
+  constexpr int HD = 16 * NT;
+  c.k_stride = (int64_t)KVH * he_k_page_elems(HD);
+  c.v_stride = (int64_t)KVH * he_v_page_elems(HD);
+  c.kp = kpool + (int64_t)kvh * he_k_page_elems(HD);
+  c.vp = vpool + (int64_t)kvh * he_v_page_elems(HD);
+  c.block = kb_begin >> HE_PAGE_SHIFT;
+  c.page = pt[c.block];
+  c.page_ahead = pt[min(c.block + 1, max_blocks - 1)];
+  load_frag<NT>(c.cur, c.kp, c.vp, c.page, num_pages, c.k_stride, c.v_stride, kb_begin & 32, lr, lg);
+}
+
+// Runs the keys [kb_begin, kb_end) (multiples of 32) of one (sequence, kv head) against the
+// state, one step ahead with its loads and one page ahead with its page-table entry.
+template <int NT, bool UNMASKED_STEPS>
+__device__ __forceinline__ void attend_walk(AttnState<NT>& st, const bf16x8* qf, AttendCursor<NT>& c,
+                                            const int32_t* __restrict__ pt, int max_blocks,
+                                            int num_pages, int kb_begin, int kb_end, int lo, int hi,
+                                            int clear_lo, int clear_hi, float scale_log2, int lr,
+                                            int lg) {
+  KVFrag<NT> nxt;
+  for (int kb = kb_begin; kb < kb_end; kb += 32) {
+    const int kn = kb + 32;
+    if (kn < kb_end) {
+      if ((kn & 32) == 0) {   // the next step starts a new page
+        ++c.block;
+        c.page = c.page_ahead;
+        c.page_ahead = pt[min(c.block + 1, max_blocks - 1)];
+      }
+      load_frag<NT>(nxt, c.kp, c.vp, c.page, num_pages, c.k_stride, c.v_stride, kn & 32, lr, lg);
+    }
+    // keys in [clear_lo, clear_hi] are visible to every query of the tile
+    if (UNMASKED_STEPS && kb >= clear_lo && kb + 31 <= clear_hi && c.cur.ok)
+      attend_frag<NT, false>(st, qf, c.cur, kb, lo, hi, scale_log2, lg);
+    else
+      attend_frag<NT, true>(st, qf, c.cur, kb, lo, hi, scale_log2, lg);
+    c.cur = nxt;
+  }
+}
+
 template <int NT, bool UNMASKED_STEPS>
 __device__ __forceinline__ void attend_range(AttnState<NT>& st, const bf16x8* qf,
                                              const uint16_t* __restrict__ kpool,
@@ -139,33 +198,11 @@ __device__ __forceinline__ void attend_range(AttnState<NT>& st, const bf16x8* qf
                                              int num_pages, int KVH, int kvh, int kb_begin,
                                              int kb_end, int lo, int hi, int clear_lo,
                                              int clear_hi, float scale_log2, int lr, int lg) {
-  constexpr int HD = 16 * NT;
   if (kb_begin >= kb_end) return;
-  const int64_t k_stride = (int64_t)KVH * he_k_page_elems(HD), v_stride = (int64_t)KVH * he_v_page_elems(HD);
-  const uint16_t* kp = kpool + (int64_t)kvh * he_k_page_elems(HD);
-  const uint16_t* vp = vpool + (int64_t)kvh * he_v_page_elems(HD);
-  int block = kb_begin >> HE_PAGE_SHIFT;
-  int page = pt[block];
-  int page_ahead = pt[min(block + 1, max_blocks - 1)];
-  KVFrag<NT> cur, nxt;
-  load_frag<NT>(cur, kp, vp, page, num_pages, k_stride, v_stride, kb_begin & 32, lr, lg);
-  for (int kb = kb_begin; kb < kb_end; kb += 32) {
-    const int kn = kb + 32;
-    if (kn < kb_end) {
-      if ((kn & 32) == 0) {   // the next step starts a new page
-        ++block;
-        page = page_ahead;
-        page_ahead = pt[min(block + 1, max_blocks - 1)];
-      }
-      load_frag<NT>(nxt, kp, vp, page, num_pages, k_stride, v_stride, kn & 32, lr, lg);
-    }
-    // keys in [clear_lo, clear_hi] are visible to every query of the tile
-    if (UNMASKED_STEPS && kb >= clear_lo && kb + 31 <= clear_hi && cur.ok)
-      attend_frag<NT, false>(st, qf, cur, kb, lo, hi, scale_log2, lg);
-    else
-      attend_frag<NT, true>(st, qf, cur, kb, lo, hi, scale_log2, lg);
-    cur = nxt;
-  }
+  AttendCursor<NT> c;
+  attend_start<NT>(c, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, kb_begin, lr, lg);
+  attend_walk<NT, UNMASKED_STEPS>(st, qf, c, pt, max_blocks, num_pages, kb_begin, kb_end, lo, hi,
+                                  clear_lo, clear_hi, scale_log2, lr, lg);
 }
 
 template <int NT>
