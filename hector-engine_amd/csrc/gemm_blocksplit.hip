@@ -1,6 +1,7 @@
 // bf16 matrix product for few rows (M <= 32) with K cut inside the workgroup:
 // C[M,N] = X[M,K] * W[N,K]^T (+ bias), or the gated activation of a gate||up
-// weight. One workgroup owns 16*R weight rows; its NW wavefronts take one K slice
+// weight. One workgroup owns up to 16*R weight rows (the rows are dealt out evenly over the
+// compute units, see blocksplit_plan); its NW wavefronts take one K slice
 // each (operands straight from global memory into the MFMA registers, as in
 // gemm_skinny.hip, whose operand layout this kernel shares), leave their fp32
 // tiles in LDS, and the workgroup adds the slices in wavefront order and writes
