@@ -146,12 +146,21 @@ class Engine:
         return self.cache.max_seq_len
 
     # -- the step function -------------------------------------------------------
-    def step(self, entries: list[StepEntry]) -> torch.Tensor | None:
+    def step(self, entries: list[StepEntry], device_tokens: torch.Tensor | None = None) -> torch.Tensor | None:
         """Runs the entries' tokens as one batch. Returns fp32 logits
         [number of wanted places, vocab] in the order of the entries and of their
-        `want`, or None if nothing is wanted. The tensor is valid until the next step."""
+        `want`, or None if nothing is wanted. The tensor is valid until the next step.
+
+        device_tokens: int32 [len(entries)] on the device, for a step of one token a sequence:
+        the tokens to run, in place of the entries' own (which only have to be valid ids). A
+        sampler's ids go from one step into the next this way without a trip to the host, so
+        several steps can be queued before the host reads any of them."""
         if not entries:
             raise StepError("a step needs at least one entry")
+        if device_tokens is not None:
+            if device_tokens.dtype != torch.int32 or device_tokens.device != self.device \
+                    or device_tokens.numel() != len(entries) or any(len(e.tokens) != 1 for e in entries):
+                raise StepError("device_tokens: int32 on the engine's device, one for each entry of one token")
         seen = set()
         growth = []
         for e in entries:
@@ -181,9 +190,9 @@ class Engine:
         every_wanted = all(list(e.want) == [0] for e in entries)
         self.stats["steps"] += 1
         if self.use_graphs and all_single and every_wanted and len(entries) <= GRAPH_MAX_BUCKET:
-            logits = self._graph_step(entries)
+            logits = self._graph_step(entries, device_tokens)
         else:
-            logits = self._eager_step(entries, all_single)
+            logits = self._eager_step(entries, all_single, device_tokens)
         self.cache.commit(growth)
         return logits
 
@@ -260,7 +269,7 @@ class Engine:
                            max_q_len=max_q_len, max_keys=self.cache.max_seq_len,
                            all_single=all_single, env=self.env, scratch=pool)
 
-    def _eager_step(self, entries, all_single: bool):
+    def _eager_step(self, entries, all_single: bool, device_tokens=None):
         rows = sum(len(e.tokens) for e in entries)
         wants = sum(len(e.want) for e in entries)
         meta = _Meta(rows, len(entries), wants)
@@ -269,6 +278,8 @@ class Engine:
         dev = self.scratch.alloc((meta.total,), torch.int32)
         self._upload(host, idx, dev)
         views = meta.views(dev)
+        if device_tokens is not None:
+            views["tokens"][:len(entries)].copy_(device_tokens)
         ctx = self._context(views, rows, len(entries), max(len(e.tokens) for e in entries),
                             all_single, self.scratch)
         ctx.host = {"q_lens": [len(e.tokens) for e in entries],
@@ -279,7 +290,7 @@ class Engine:
         self.stats["eager_steps"] += 1
         return self.model.forward(views["tokens"], ctx, self.caches, views["want_rows"], nw)
 
-    def _graph_step(self, entries):
+    def _graph_step(self, entries, device_tokens=None):
         n = len(entries)
         size = 1 << (n - 1).bit_length()
         bucket = self._buckets.get(size)
@@ -290,6 +301,8 @@ class Engine:
         host, idx, _ = self._pack(padded, bucket.meta, size, size)
         host.numpy()[bucket.meta.offsets["want_rows"][0]:][:size] = np.arange(size, dtype=np.int32)
         self._upload(host, idx, bucket.dev)
+        if device_tokens is not None:
+            bucket.views["tokens"][:n].copy_(device_tokens)
         bucket.uses += 1
         if bucket.graph is None:
             ctx = self._context(bucket.views, size, size, 1, True, bucket.pool)

@@ -66,14 +66,26 @@ def after_token(token: int, generated: int, max_new_tokens: int, length: int, ma
     return True, None
 
 
+RUN_OF_STEPS = 8
+
+
 def generate(engine, prompts: list[list[int]], *, max_new_tokens: int = 100, sampling=None,
              stop_ids=(), include_stop: bool = False, batch_size: int | None = None,
-             cancel: Callable[[], bool] | None = None, sample_fn=None) -> list[GenerationResult]:
-    """Generates for every prompt; returns results in the order of `prompts`."""
+             cancel: Callable[[], bool] | None = None, sample_fn=None,
+             run_of_steps: int = RUN_OF_STEPS) -> list[GenerationResult]:
+    """Generates for every prompt; returns results in the order of `prompts`.
+
+    run_of_steps: with the library's own sampler and no penalties, up to so many one-token
+    steps are queued at a time: each step's ids go into the next on the device and the host
+    reads them once per run. The tokens are the same as step by step; a sequence that ends
+    inside a run keeps its slot until the run ends, and `cancel` is asked between runs."""
     from ..sampling import Sampler, SamplingConfig
+    sampler = None
     if sample_fn is None:
         sampler = Sampler(sampling or SamplingConfig.deterministic(), engine.device)
         sample_fn = sampler.sample
+        if sampler.config.has_penalties or run_of_steps <= 1:
+            sampler = None          # penalties need each token on the host before the next
     stop_ids = frozenset(int(s) for s in stop_ids)
     results: list[GenerationResult | None] = [None] * len(prompts)
     pending = [(i, len(p)) for i, p in enumerate(prompts)]
@@ -92,12 +104,37 @@ def generate(engine, prompts: list[list[int]], *, max_new_tokens: int = 100, sam
                 raise RuntimeError("the cache holds other sequences and no request fits beside them")
             continue
         _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, include_stop,
-                   cancel, sample_fn)
+                   cancel, sample_fn, sampler, run_of_steps)
     return results
 
 
+def steps_in_run(generated: list[int], lengths: list[int], max_new_tokens: int, max_seq_len: int,
+                 run_of_steps: int) -> int:
+    """How many one-token steps can be queued for sequences that have `generated` tokens (the
+    one to feed included) and `lengths` cached tokens, so that none passes max_new_tokens or
+    runs out of room whatever it samples: every step feeds one token and samples one."""
+    room = min(max_seq_len - n for n in lengths)            # tokens that can still be fed
+    budget = min(max_new_tokens - g for g in generated)     # tokens that may still be sampled
+    return max(1, min(run_of_steps, room, budget))
+
+
+def _run_of_steps(engine, sampler, slots: list[int], tokens: list[int], seqs: list[int],
+                  steps: list[int], count: int) -> list[list[int]]:
+    """Feeds `tokens` and queues `count` steps; returns the sampled ids of each, [count][rows]."""
+    uniforms = None if sampler.config.is_greedy else sampler.uniforms_device(seqs, steps, count)
+    ids, device_ids = [], None
+    for j in range(count):
+        entries = [StepEntry(s, [t], [0]) for s, t in zip(slots, tokens)]
+        logits = engine.step(entries, device_tokens=device_ids)
+        device_ids = sampler.sample_device(logits, seqs, [t + j for t in steps],
+                                           uniforms=None if uniforms is None else uniforms[j])
+        ids.append(device_ids)
+    import torch
+    return torch.stack(ids).tolist()          # the one wait of the run
+
+
 def _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, include_stop, cancel,
-               sample_fn) -> None:
+               sample_fn, sampler=None, run_of_steps: int = 1) -> None:
     slots = {i: engine.acquire() for i in admitted}
     out: dict[int, list[int]] = {i: [] for i in admitted}
     t0 = time.perf_counter()
@@ -131,8 +168,33 @@ def _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, inc
             active = [i for i, _ in feed]
             if not active:
                 break
-            logits = engine.step([StepEntry(slots[i], [tok], [0]) for i, tok in feed])
-            tokens = sample_fn(logits, active, [len(out[i]) for i in active], [out[i] for i in active])
+            count = 1 if sampler is None else steps_in_run(
+                [len(out[i]) for i in active], [engine.length(slots[i]) for i in active],
+                max_new_tokens, engine.max_seq_len, run_of_steps)
+            if count == 1:
+                logits = engine.step([StepEntry(slots[i], [tok], [0]) for i, tok in feed])
+                tokens = sample_fn(logits, active, [len(out[i]) for i in active], [out[i] for i in active])
+                continue
+            run = _run_of_steps(engine, sampler, [slots[i] for i in active], [tok for _, tok in feed],
+                                active, [len(out[i]) for i in active], count)
+            # all but the last step of the run are decided here, as the loop above decides one;
+            # a sequence that ends inside the run drops the rest of its ids
+            ended: set[int] = set()
+            for j in range(count - 1):
+                for col, i in enumerate(active):
+                    if i in ended:
+                        continue
+                    tok = run[j][col]
+                    keep, reason = after_token(tok, len(out[i]), max_new_tokens,
+                                               engine.length(slots[i]) - (count - 1 - j),
+                                               engine.max_seq_len, stop_ids)
+                    if keep or include_stop:
+                        out[i].append(tok)
+                    if reason is not None:
+                        finish(i, reason)
+                        ended.add(i)
+            tokens = [run[count - 1][col] for col, i in enumerate(active) if i not in ended]
+            active = [i for i in active if i not in ended]
     finally:
         for i in list(slots):
             engine.release(slots.pop(i))

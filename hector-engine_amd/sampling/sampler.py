@@ -92,6 +92,21 @@ class Sampler:
         """logits: fp32 [rows, vocab] on the device; sequences[r] and steps[r] key
         the row's random draw; contexts[r] are the row's generated tokens so far.
         Returns the chosen ids (one device-to-host copy, which synchronises)."""
+        return self.sample_device(logits, sequences, steps, contexts).tolist()
+
+    def uniforms_device(self, sequences: list[int], steps: list[int], count: int) -> torch.Tensor:
+        """The random draws of `count` successive steps of these rows (steps[r], steps[r] + 1, ...)
+        on the device, int32 bits [count, rows]: one upload for a run of steps."""
+        cfg = self.config
+        u = np.array([[uniform_u32(cfg.seed, s, t + j) for s, t in zip(sequences, steps)]
+                      for j in range(count)], dtype=np.uint32)
+        return torch.from_numpy(u.view(np.int32)).to(self.device)
+
+    def sample_device(self, logits: torch.Tensor, sequences: list[int], steps: list[int],
+                      contexts: list[list[int]] | None = None,
+                      uniforms: torch.Tensor | None = None) -> torch.Tensor:
+        """The same, the ids left on the device (int32 [rows]). With `uniforms` (a row of
+        uniforms_device) and no penalties nothing is copied or waited for."""
         cfg = self.config
         rows, V = logits.shape
         if cfg.has_penalties and contexts is not None and any(contexts):
@@ -112,7 +127,7 @@ class Sampler:
         if cfg.is_greedy:
             ops.argmax_rows(out, logits, rows)
         else:
-            u = np.array([uniform_u32(cfg.seed, s, t) for s, t in zip(sequences, steps)], dtype=np.uint32)
-            ud = torch.from_numpy(u.view(np.int32)).to(self.device)
-            ops.sample_rows(out, logits, rows, ud, cfg.temperature, cfg.top_k, cfg.top_p)
-        return out.tolist()
+            if uniforms is None:
+                uniforms = self.uniforms_device(sequences, steps, 1)[0]
+            ops.sample_rows(out, logits, rows, uniforms, cfg.temperature, cfg.top_k, cfg.top_p)
+        return out

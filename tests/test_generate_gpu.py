@@ -87,6 +87,43 @@ def test_stop_tokens_and_early_finishers(he, model_dirs, plain_models):
     assert eng.cache.free_pages == eng.cache.num_pages and eng.cache.book.slots.available == eng.cache.max_slots
 
 
+@pytest.mark.parametrize("kw", [dict(), dict(temperature=0.9, top_k=20, seed=5)])
+def test_runs_of_queued_steps_give_the_same_tokens(he, model_dirs, plain_models, kw):
+    """Steps queued several at a time (ids handed from step to step on the device) against one
+    step at a time: budgets that are no multiple of the run, a stop token inside a run, a
+    sequence whose cache room ends inside one."""
+    cfg, w = plain_models["B"]
+    prompts = prompts_for(cfg, [3, 7, 17, 30, 50], 500)
+    sampling = he.SamplingConfig(temperature=0.0, **kw) if not kw else he.SamplingConfig(**kw)
+    eng = he.Engine(model_dirs["B"], dtype="float32", max_tokens=2048, max_seq_len=64)
+    one = he.generate(eng, prompts, max_new_tokens=21, sampling=sampling, run_of_steps=1)
+    stop = {one[1].tokens[9], one[2].tokens[2]}
+    for budget, stops in ((21, ()), (13, stop), (40, stop)):
+        a = he.generate(eng, prompts, max_new_tokens=budget, sampling=sampling, stop_ids=stops, run_of_steps=1)
+        for run in (2, 8, 32):
+            b = he.generate(eng, prompts, max_new_tokens=budget, sampling=sampling, stop_ids=stops, run_of_steps=run)
+            assert [(r.tokens, r.finish_reason) for r in a] == [(r.tokens, r.finish_reason) for r in b]
+        assert eng.cache.free_pages == eng.cache.num_pages
+    assert {r.finish_reason for r in a} >= {"eos", "stop"}          # budget 40: the long prompts fill their room
+
+
+def test_a_step_takes_its_tokens_from_the_device(he, model_dirs):
+    from hector_engine_amd.engine.engine import StepEntry, StepError
+    eng = he.Engine(model_dirs["A"], dtype="bfloat16", max_tokens=1024, max_seq_len=128)
+    slots = [eng.acquire() for _ in range(3)]
+    eng.step([StepEntry(s, [5, 6, 7 + s], [2]) for s in slots])
+    toks = [11, 12, 13]
+    for use_graph in (False, True, True):       # the first one-token step of a batch size runs eagerly
+        want = eng.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)]).clone()
+        for s in slots:                          # the same step again, its tokens given on the device
+            eng.cache.book.length[s] -= 1
+        ids = torch.tensor(toks, dtype=torch.int32, device=eng.device)
+        got = eng.step([StepEntry(s, [0], [0]) for s in slots], device_tokens=ids)
+        assert torch.equal(got, want)
+    with pytest.raises(StepError, match="device_tokens"):
+        eng.step([StepEntry(slots[0], [1, 2], [1])], device_tokens=ids[:1])
+
+
 def test_penalties(he, model_dirs, plain_models):
     cfg, w = plain_models["A"]
     p = prompts_for(cfg, [9], 400)[0]

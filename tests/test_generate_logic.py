@@ -5,7 +5,7 @@ import pytest
 
 import hector_engine_amd  # noqa: F401
 from hector_engine_amd.cache import GroupPages, SlotBook
-from hector_engine_amd.engine.generate import after_token, generate, plan_batch
+from hector_engine_amd.engine.generate import after_token, generate, plan_batch, steps_in_run
 
 V = 50
 
@@ -157,3 +157,14 @@ def test_slots_are_released_when_a_step_fails():
     with pytest.raises(RuntimeError, match="sampler failed"):
         generate(eng, [[1, 2], [3]], max_new_tokens=3, sample_fn=boom)
     assert eng.cache.book.slots.available == 3 and eng.cache.free_pages == 16
+
+
+def test_steps_in_run():
+    """How many steps may be queued before the host sees a token: never past the token budget of
+    any sequence, never past the room in its cache, at least one."""
+    assert steps_in_run([1, 1], [10, 20], 100, 256, 8) == 8
+    assert steps_in_run([1, 95], [10, 20], 100, 256, 8) == 5          # 5 more tokens may be sampled
+    assert steps_in_run([1, 1], [10, 253], 100, 256, 8) == 3          # 3 more tokens can be fed
+    assert steps_in_run([99], [10], 100, 256, 8) == 1
+    assert steps_in_run([3], [256], 100, 256, 8) == 1                 # the loop ends such a sequence before
+    assert steps_in_run([1], [10], 100, 256, 1) == 1
