@@ -171,7 +171,14 @@ __device__ __forceinline__ void bs_load_resid(const BsFusion& fu, int item, int 
   } else {
     for (int i = 0; i < 4; ++i) res[i] = i < valid ? fu.resid[(int64_t)m * N + n + i] : 0.f;
   }
-  for (int i = 0; i < 4; ++i) gain[i] = i < valid ? load_param(fu.gain, n + i, fu.gain_dtype) : 0.f;
+  if (valid == 4 && fu.gain_dtype == HE_BF16 && (n & 1) == 0 && (((uintptr_t)fu.gain) & 3) == 0) {
+    const uint32_t* g = reinterpret_cast<const uint32_t*>((const uint16_t*)fu.gain + n);
+    const uint32_t a = g[0], b = g[1];
+    gain[0] = __uint_as_float(a << 16), gain[1] = __uint_as_float(a & 0xffff0000u);
+    gain[2] = __uint_as_float(b << 16), gain[3] = __uint_as_float(b & 0xffff0000u);
+  } else {
+    for (int i = 0; i < 4; ++i) gain[i] = i < valid ? load_param(fu.gain, n + i, fu.gain_dtype) : 0.f;
+  }
 }
 
 // grid: one workgroup per 16*R weight rows; block: 64 * NW threads.
@@ -210,7 +217,8 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
   // Loads the epilogue needs are issued here, ahead of the weight stream, so that their
   // latency is not added at the end: the partial sums of squares of the input rows
   // (wavefront w takes the rows w and w + nw; lanes hold strided partials) and, for the
-  // residual epilogue, the residual values and gains of this thread's first outputs.
+  // residual epilogue (a little further down, behind the first weight loads), the residual
+  // values and gains of this thread's first outputs.
   constexpr int OUT_TILES = R * MT;
   const int out_align = ((N | n0) & 3) == 0 ? 4 : (((N | n0) & 1) == 0 ? 2 : 1);
   const bool scaled = fu.scale_partials != nullptr;
@@ -229,8 +237,6 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
     }
   }
   float res0[4] = {0.f, 0.f, 0.f, 0.f}, gain0[4] = {0.f, 0.f, 0.f, 0.f};
-  if (to_resid && threadIdx.x < OUT_TILES * 64)
-    bs_load_resid<MT>(fu, threadIdx.x, n0, n_end, M, N, res0, gain0);
 
   // two steps of 64 U k values per turn; a step past k_end loads nothing and adds zeros.
   // The turns of a wavefront start at a point of its slice that differs from workgroup to
@@ -241,6 +247,8 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
   const int turns = k_end > k_begin ? (k_end - k_begin + TURN - 1) / TURN : 0;
   int k = turns > 0 ? k_begin + (int)((blockIdx.x * 3u) % (unsigned)turns) * TURN : k_begin;
   bs_load<MT, R, U>(f0, wp, xp, k, lg, k_end);
+  if (to_resid && threadIdx.x < OUT_TILES * 64)   // behind the first weights, ahead of the rest
+    bs_load_resid<MT>(fu, threadIdx.x, n0, n_end, M, N, res0, gain0);
   for (int j = 0; j < turns; ++j) {
     bs_load<MT, R, U>(f1, wp, xp, k + 64 * U, lg, k_end);
     bs_multiply<MT, R, U>(f0, acc);
