@@ -385,7 +385,8 @@ static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int
     } else if (groups < 256) {
       r = 2, u = 1, nw = 8;         // under one workgroup a compute unit: more wavefronts each
     } else if (groups < 1024 && last_round > 0 && last_round <= 128) {
-      r = 1, u = 2, nw = 8;         // the last round of workgroups would fill under half of the chip
+      r = 1, u = 1, nw = 8;         // the last round of whole tiles would fill under half of the chip:
+                                    // the rows are dealt out below, 20 a workgroup for 10240
     } else {
       r = 2, u = 4, nw = 4;
     }
