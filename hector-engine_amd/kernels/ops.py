@@ -79,7 +79,8 @@ def residual_add(resid_f32, delta, rows: int) -> None:
 
 def silu_mul(out, gate_up, rows: int, interleaved: bool = False, splits: int = 0) -> None:
     """out[rows, I] = silu(gate) * up. gate_up: [rows, 2I] in out's dtype, or with
-    splits > 0 the fp32 K slices [splits, rows, 2I] of the product."""
+    splits > 0 the fp32 K slices [splits, rows, 2I] of the product. Its columns are all
+    gates then all ups, or, interleaved, gate i in column 2i and its up in 2i + 1."""
     I = out.shape[-1]
     _need(out, "out")
     _need(gate_up, "gate_up", torch.float32 if splits > 0 else out.dtype)
