@@ -16,6 +16,8 @@ import dataclasses
 import time
 from typing import Callable
 
+import torch
+
 from ..cache.pages import PAGE_TOKENS, blocks_for
 from .engine import StepEntry
 
@@ -129,7 +131,6 @@ def _run_of_steps(engine, sampler, slots: list[int], tokens: list[int], seqs: li
         device_ids = sampler.sample_device(logits, seqs, [t + j for t in steps],
                                            uniforms=None if uniforms is None else uniforms[j])
         ids.append(device_ids)
-    import torch
     return torch.stack(ids).tolist()          # the one wait of the run
 
 
@@ -150,21 +151,22 @@ def _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, inc
                                           (time.perf_counter() - t1) * 1e3)
             engine.release(slots.pop(i))     # the slot goes back at once
 
+        def decide(i, tok, length) -> bool:
+            """Records a sampled token of request i whose cache held `length` tokens when it was
+            sampled; True if the sequence goes on (the token is then to be fed)."""
+            keep, reason = after_token(tok, len(out[i]), max_new_tokens, length, engine.max_seq_len, stop_ids)
+            if keep or include_stop:
+                out[i].append(tok)
+            if reason is not None:
+                finish(i, reason)
+            return reason is None
+
         while active:
             if cancel is not None and cancel():
                 for i in active:
                     finish(i, "cancelled")
                 break
-            feed = []
-            for i, tok in zip(active, tokens):
-                keep, reason = after_token(tok, len(out[i]), max_new_tokens, engine.length(slots[i]),
-                                           engine.max_seq_len, stop_ids)
-                if keep or include_stop:
-                    out[i].append(tok)
-                if reason is not None:
-                    finish(i, reason)
-                else:
-                    feed.append((i, tok))
+            feed = [(i, tok) for i, tok in zip(active, tokens) if decide(i, tok, engine.length(slots[i]))]
             active = [i for i, _ in feed]
             if not active:
                 break
@@ -177,24 +179,15 @@ def _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, inc
                 continue
             run = _run_of_steps(engine, sampler, [slots[i] for i in active], [tok for _, tok in feed],
                                 active, [len(out[i]) for i in active], count)
-            # all but the last step of the run are decided here, as the loop above decides one;
-            # a sequence that ends inside the run drops the rest of its ids
-            ended: set[int] = set()
+            # all but the last step of the run are decided here, each with the cache length of its
+            # moment; a sequence that ends inside the run drops the rest of its ids
+            going = dict.fromkeys(active, True)
             for j in range(count - 1):
                 for col, i in enumerate(active):
-                    if i in ended:
-                        continue
-                    tok = run[j][col]
-                    keep, reason = after_token(tok, len(out[i]), max_new_tokens,
-                                               engine.length(slots[i]) - (count - 1 - j),
-                                               engine.max_seq_len, stop_ids)
-                    if keep or include_stop:
-                        out[i].append(tok)
-                    if reason is not None:
-                        finish(i, reason)
-                        ended.add(i)
-            tokens = [run[count - 1][col] for col, i in enumerate(active) if i not in ended]
-            active = [i for i in active if i not in ended]
+                    if going[i]:
+                        going[i] = decide(i, run[j][col], engine.length(slots[i]) - (count - 1 - j))
+            tokens = [run[count - 1][col] for col, i in enumerate(active) if going[i]]
+            active = [i for i in active if going[i]]
     finally:
         for i in list(slots):
             engine.release(slots.pop(i))
