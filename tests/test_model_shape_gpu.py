@@ -89,3 +89,17 @@ def test_seven_b_layer_sizes(engines):
             clear = (t2[:, 0] - t2[:, 1]) > 0.03 * scale
             assert torch.equal(got.argmax(-1)[clear], ref.argmax(-1)[clear])
     assert e16.stats["graph_replays"] > 0
+
+
+def test_queued_steps_at_seven_b_layer_sizes(engines):
+    """Runs of 8 queued one-token steps (ids handed on the device, HIP graph replays back to back)
+    give the tokens of one step at a time, greedy and sampled, at the sizes of the benchmark."""
+    import hector_engine_amd as he
+    eng = engines("bfloat16")
+    prompts = [rand_ids(152064, n, 700 + n) for n in (40, 9, 21, 33, 5)]
+    for sampling in (he.SamplingConfig.deterministic(), he.SamplingConfig(temperature=0.9, top_k=50, seed=11)):
+        one = he.generate(eng, prompts, max_new_tokens=27, sampling=sampling, run_of_steps=1)
+        many = he.generate(eng, prompts, max_new_tokens=27, sampling=sampling, run_of_steps=8)
+        assert [r.tokens for r in one] == [r.tokens for r in many]
+        assert all(len(r.tokens) == 27 for r in many)
+    assert eng.cache.free_pages == eng.cache.num_pages
