@@ -216,7 +216,7 @@ class Engine:
         v["positions"][:] = 0
         v["seq_slot"][:] = -1
         v["seq_start"][:] = 0
-        if len(entries) == meta.offsets["tokens"][1] or all(len(e.tokens) == 1 for e in entries):
+        if all(len(e.tokens) == 1 for e in entries):
             # one token a sequence: whole columns at once
             k = len(entries)
             starts = [self.cache.length(e.slot) for e in entries]
