@@ -91,7 +91,7 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
     const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ page_table, int max_blocks,
     int num_pages, const float* __restrict__ inv_freq, int rotary_dim, int H, int KVH,
-    int head_tiles, int window, float scale, int write_kv) {
+    int head_tiles, int window, float scale, int write_kv, int out_pieces) {
   constexpr int HD = 16 * NT;
   constexpr int KS = (HD + 31) / 32;
   extern __shared__ __attribute__((aligned(16))) float lds[];   // [NW][GT][HD] O, then [NW][GT][2] (m, l)
@@ -111,10 +111,15 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
   const float freq = lane < HD / 2 ? inv_freq[lane] : 0.f;
   const int seq = row_seq[row];
   const int Z = gridDim.z, z = blockIdx.z;
+  // where dims d.. of head (column) hg of this tile go: row-major [rows, H HD], or piece-major
+  // (16-byte pieces [H HD / 8][rows][8])
+  auto out_at = [&](int hg, int d) {
+    const int64_t c = (int64_t)(kvh * G + 16 * ht + hg) * HD + d;
+    return out_pieces ? out + ((c >> 3) * gridDim.y + row) * 8 + (c & 7) : out + (int64_t)row * H * HD + c;
+  };
   if (seq < 0) {                           // padding row: zeros (from the merge kernel if there is one)
     if (Z == 1)
-      for (int i = threadIdx.x; i < GT * HD; i += blockDim.x)
-        out[((int64_t)row * H + kvh * G + 16 * ht) * HD + i] = 0;
+      for (int i = threadIdx.x; i < GT * HD; i += blockDim.x) *out_at(i / HD, i % HD) = 0;
     return;
   }
   const int slot = seq_slot[seq];
@@ -221,7 +226,7 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
       uint2 w2;
       w2.x = pack2_bf16(acc.x * inv, acc.y * inv);
       w2.y = pack2_bf16(acc.z * inv, acc.w * inv);
-      *reinterpret_cast<uint2*>(out + head * HD + d) = w2;
+      *reinterpret_cast<uint2*>(out_at(hg, d)) = w2;
     } else {                               // a part without keys stores (-inf, 0, zeros)
       *reinterpret_cast<float4*>(ws_o + (head * Z + z) * HD + d) = acc;
       if (d == 0) {
@@ -280,8 +285,8 @@ extern "C" int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_
                                               int num_pages, const void* inv_freq, int rotary_dim,
                                               int rows, int H, int KVH, int hd, int window,
                                               float scale, int max_keys, int write_kv,
-                                              void* workspace_f32, int64_t workspace_floats,
-                                              void* stream) {
+                                              int out_pieces, void* workspace_f32,
+                                              int64_t workspace_floats, void* stream) {
   HE_REQUIRE(rows >= 0 && H > 0 && KVH > 0 && hd > 0 && max_keys > 0,
              "he_attention_decode_fused_bf16: bad sizes");
   HE_REQUIRE(scale > 0.f, "he_attention_decode_fused_bf16: the score scale must be positive");
@@ -317,7 +322,8 @@ extern "C" int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_
         (uint16_t*)kpool,                                                                       \
         (uint16_t*)vpool, (const int32_t*)positions, (const int32_t*)row_seq,                   \
         (const int32_t*)seq_slot, (const int32_t*)page_table, max_blocks, num_pages,            \
-        (const float*)inv_freq, rotary_dim, H, KVH, head_tiles, window, scale, write_kv);       \
+        (const float*)inv_freq, rotary_dim, H, KVH, head_tiles, window, scale, write_kv,        \
+        out_pieces);                                                                            \
     break;
   switch (hd / 16) {
     FUSED(4) FUSED(8)
@@ -327,5 +333,5 @@ extern "C" int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_
 #undef FUSED
   const int rc = he_check_launch("he_attention_decode_fused_bf16");
   if (rc || Z == 1) return rc;
-  return he_attention_merge_parts(out, ws_o, ws_ml, row_seq, rows, H, hd, Z, stream);
+  return he_attention_merge_parts(out, ws_o, ws_ml, row_seq, rows, H, hd, Z, out_pieces, stream);
 }

@@ -481,14 +481,19 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
 __global__ __launch_bounds__(256) void attention_merge_kernel(
     uint16_t* __restrict__ out, const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq, int H, int HD,
-    int nsplit, int window, int all_parts) {
+    int nsplit, int window, int all_parts, int out_pieces) {
   __shared__ float wgt[64];
   __shared__ float part[4][256];
   const int h = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int64_t row = blockIdx.y;
-  uint16_t* orow = out + (row * H + h) * (int64_t)HD;
+  // where dim d of this row and head goes: row-major [rows, H HD], or piece-major (16-byte
+  // pieces [H HD / 8][rows][8], the layout the next product reads best at up to 16 rows)
+  auto at = [&](int d) {
+    const int64_t c = (int64_t)h * HD + d;
+    return out_pieces ? out + ((c >> 3) * gridDim.y + row) * 8 + (c & 7) : out + row * H * (int64_t)HD + c;
+  };
   if (row_seq[row] < 0) {
-    for (int d = threadIdx.x; d < HD; d += 256) orow[d] = 0;
+    for (int d = threadIdx.x; d < HD; d += 256) *at(d) = 0;
     return;
   }
   int active = nsplit;                     // all_parts: every part was stored, empty ones as (-inf, 0, 0)
@@ -523,7 +528,7 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(
     if (d < HD) {
       const float acc = ((part[0][threadIdx.x] + part[1][threadIdx.x]) + part[2][threadIdx.x]) +
                         part[3][threadIdx.x];
-      orow[d] = float_to_bf16_bits(acc * inv);
+      *at(d) = float_to_bf16_bits(acc * inv);
     }
     __syncthreads();
   }
@@ -606,16 +611,16 @@ extern "C" int he_attention_decode_bf16(void* out, const void* q, const void* kp
   if (rc || nsplit == 1) return rc;
   attention_merge_kernel<<<dim3(H, rows), 256, 0, s>>>(
       (uint16_t*)out, ws_o, ws_ml, (const int32_t*)positions, (const int32_t*)row_seq, H, hd,
-      nsplit, window, 0);
+      nsplit, window, 0, 0);
   return he_check_launch("he_attention_decode_bf16 merge");
 }
 
 // Joins parts [rows][H][parts] of (O fp32 [hd], then (m, l) pairs) that were all stored.
 int he_attention_merge_parts(void* out, const float* ws_o, const float* ws_ml, const void* row_seq,
-                             int rows, int H, int hd, int parts, void* stream) {
+                             int rows, int H, int hd, int parts, int out_pieces, void* stream) {
   HE_REQUIRE(parts >= 1 && parts <= 64, "he_attention_merge_parts: %d parts, at most 64", parts);
   attention_merge_kernel<<<dim3(H, rows), 256, 0, (hipStream_t)stream>>>(
-      (uint16_t*)out, ws_o, ws_ml, nullptr, (const int32_t*)row_seq, H, hd, parts, 0, 1);
+      (uint16_t*)out, ws_o, ws_ml, nullptr, (const int32_t*)row_seq, H, hd, parts, 0, 1, out_pieces);
   return he_check_launch("he_attention_merge_parts");
 }
 

@@ -143,7 +143,7 @@ void he_set_error(const char* fmt, ...);
 int he_check_launch(const char* what);
 // attention_mfma.hip: joins attention parts that were all stored (used by the fused one-token kernel)
 int he_attention_merge_parts(void* out, const float* ws_o, const float* ws_ml, const void* row_seq,
-                             int rows, int H, int hd, int parts, void* stream);
+                             int rows, int H, int hd, int parts, int out_pieces, void* stream);
 
 #define HE_REQUIRE(cond, ...)      \
   do {                             \

@@ -23,6 +23,13 @@
 //   row scale: the consumer of xg adds the partials of a row in a fixed order,
 //     s[m] = 1 / sqrt(sum / dim + eps), and multiplies its sums by s[m] before bias or
 //     gate: W (r g s) = s W (r g). The norm's statistics stay fp32.
+//
+// Activations between two such products may lie piece-major instead of row-major: a [M, D]
+// bf16 tensor as 16-byte pieces [D / 8][M][8], element (m, d) at ((d / 8) M + m) 8 + d % 8.
+// The 16 lanes of an activation operand load then read 16 neighbouring pieces (two lines)
+// instead of 16 rows (16 lines): the cost of the activation rows, which grows with their
+// number (gate||up 48 us at 1 row, 50 at 8, 59 at 16), all but goes (49 and 55 us). The
+// producing epilogue writes the layout, the consuming product reads it (x_pieces / out_pieces).
 #include "common.h"
 #include "hector_kernels.h"
 
@@ -85,6 +92,29 @@ __device__ __forceinline__ void bs_store2<bf16_t>(bf16_t* p, const float v[2], b
   }
 }
 
+// `count` (2 or 4) neighbouring columns of row m from column `col` on, into a piece-major
+// [M, D] bf16 tensor; `valid` of them exist.
+__device__ __forceinline__ void bs_store_pieces(uint16_t* base, int M, int m, int col, const float* v,
+                                                int count, int valid) {
+  auto at = [&](int c) { return base + ((int64_t)(c >> 3) * M + m) * 8 + (c & 7); };
+  if (valid == count && (col & 1) == 0) {        // pairs never straddle a piece
+    const uint32_t lo = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+    if (count == 2) {
+      *reinterpret_cast<uint32_t*>(at(col)) = lo;
+      return;
+    }
+    const uint32_t hi = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+    if ((col & 3) == 0) {
+      *reinterpret_cast<uint2*>(at(col)) = make_uint2(lo, hi);
+    } else {
+      *reinterpret_cast<uint32_t*>(at(col)) = lo;
+      *reinterpret_cast<uint32_t*>(at(col + 2)) = hi;
+    }
+    return;
+  }
+  for (int i = 0; i < valid; ++i) *at(col + i) = float_to_bf16_bits(v[i]);
+}
+
 // Registers hold the operands of two steps (the loads of the next step are issued before
 // the products of this one), 16 U (R + MT) of them; above 4 tile pairs the workgroup is
 // limited to 8 wavefronts so that each may use 256 registers.
@@ -95,9 +125,9 @@ struct BsFrags {
   bf16x8 a[U][R][2], b[U][MT][2];
 };
 
-template <int MT, int R, int U>
+template <int MT, int R, int U, bool PIECES>
 __device__ __forceinline__ void bs_load(BsFrags<MT, R, U>& f, const uint16_t* const* wp,
-                                        const uint16_t* const* xp, int k, int lg, int k_end) {
+                                        const uint16_t* const* xp, int k, int lg, int k_end, int M) {
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const int kk = k + 64 * u + lg * 16;   // this lane's 16 k values of the step
@@ -109,8 +139,13 @@ __device__ __forceinline__ void bs_load(BsFrags<MT, R, U>& f, const uint16_t* co
     }
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-      f.b[u][t][0] = bs_load8(xp[t] + k + 64 * u, ok0);
-      f.b[u][t][1] = bs_load8(xp[t] + k + 64 * u + 8, ok1);
+      if (PIECES) {   // piece-major X: the piece of 8 k values from kk on lies at kk M (+ 8 row)
+        f.b[u][t][0] = bs_load8(xp[t] + (k + 64 * u) * M, ok0);
+        f.b[u][t][1] = bs_load8(xp[t] + (k + 64 * u + 8) * M, ok1);
+      } else {
+        f.b[u][t][0] = bs_load8(xp[t] + k + 64 * u, ok0);
+        f.b[u][t][1] = bs_load8(xp[t] + k + 64 * u + 8, ok1);
+      }
     }
   }
 }
@@ -139,6 +174,7 @@ struct BsFusion {
   int gain_dtype;
   uint16_t* xg;                  // [M][N] bf16 out: resid * gain
   float* sq_out;                 // [M][gridDim.x] out: sum of resid^2 over this workgroup's columns
+  int out_pieces;                // the bf16 output (C, or xg) is written piece-major
 };
 
 // The residual values and gains of output item (tile, lane) of a non-gated product:
@@ -182,7 +218,7 @@ __device__ __forceinline__ void bs_load_resid(const BsFusion& fu, int item, int 
 }
 
 // grid: one workgroup per 16*R weight rows; block: 64 * NW threads.
-template <int MT, int R, int U, bool GATED, typename TC>
+template <int MT, int R, int U, bool GATED, bool PIECES, typename TC>
 __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_kernel(
     TC* __restrict__ C, const uint16_t* __restrict__ X, const uint16_t* __restrict__ W,
     const void* __restrict__ bias, int bias_dtype, int M, int N, int K, int kslice, int rows_per_block,
@@ -206,7 +242,9 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
 #pragma unroll
   for (int r = 0; r < R; ++r) wp[r] = W + (int64_t)min(n0 + 16 * r + lr, n_end - 1) * K + lg * 16;
 #pragma unroll
-  for (int t = 0; t < MT; ++t) xp[t] = X + (int64_t)min((16 * t + lr) >> spread, M - 1) * K + lg * 16;
+  for (int t = 0; t < MT; ++t)
+    xp[t] = PIECES ? X + (2 * lg * M + min((16 * t + lr) >> spread, M - 1)) * 8
+                   : X + (int64_t)min((16 * t + lr) >> spread, M - 1) * K + lg * 16;
 
   floatx4 acc[R][MT];
 #pragma unroll
@@ -246,15 +284,15 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
   constexpr int TURN = 128 * U;
   const int turns = k_end > k_begin ? (k_end - k_begin + TURN - 1) / TURN : 0;
   int k = turns > 0 ? k_begin + (int)((blockIdx.x * 3u) % (unsigned)turns) * TURN : k_begin;
-  bs_load<MT, R, U>(f0, wp, xp, k, lg, k_end);
+  bs_load<MT, R, U, PIECES>(f0, wp, xp, k, lg, k_end, M);
   if (to_resid && threadIdx.x < OUT_TILES * 64)   // behind the first weights, ahead of the rest
     bs_load_resid<MT>(fu, threadIdx.x, n0, n_end, M, N, res0, gain0);
   for (int j = 0; j < turns; ++j) {
-    bs_load<MT, R, U>(f1, wp, xp, k + 64 * U, lg, k_end);
+    bs_load<MT, R, U, PIECES>(f1, wp, xp, k + 64 * U, lg, k_end, M);
     bs_multiply<MT, R, U>(f0, acc);
     k += TURN;
     if (k >= k_end) k = k_begin;
-    if (j + 1 < turns) bs_load<MT, R, U>(f0, wp, xp, k, lg, k_end);
+    if (j + 1 < turns) bs_load<MT, R, U, PIECES>(f0, wp, xp, k, lg, k_end, M);
     bs_multiply<MT, R, U>(f1, acc);
   }
 
@@ -316,7 +354,10 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
         const float g = v[2 * i] * rs;
         y[i] = g / (1.f + expf(-g)) * (v[2 * i + 1] * rs);
       }
-      bs_store2<TC>(C + (int64_t)m * NO + (n >> 1), y, ((NO | (n0 >> 1)) & 1) == 0, valid);
+      if (fu.out_pieces)
+        bs_store_pieces(reinterpret_cast<uint16_t*>(C), M, m, n >> 1, y, 2, valid);
+      else
+        bs_store2<TC>(C + (int64_t)m * NO + (n >> 1), y, ((NO | (n0 >> 1)) & 1) == 0, valid);
     } else {
       const int n = n0 + 16 * r + 4 * olg;
       const int valid = owner ? max(0, min(4, n_end - n)) : 0;
@@ -325,7 +366,12 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
       if (bias != nullptr)
         for (int i = 0; i < valid; ++i) v[i] += load_param(bias, n + i, bias_dtype);
       if (!to_resid) {
-        if (valid > 0) bs_store4<TC>(C + (int64_t)m * N + n, v, out_align, valid);
+        if (valid > 0) {
+          if (fu.out_pieces)
+            bs_store_pieces(reinterpret_cast<uint16_t*>(C), M, m, n, v, 4, valid);
+          else
+            bs_store4<TC>(C + (int64_t)m * N + n, v, out_align, valid);
+        }
         continue;
       }
       if (item != threadIdx.x) bs_load_resid<MT>(fu, item, n0, n_end, M, N, res0, gain0);
@@ -339,7 +385,10 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
       if (valid > 0) {
         const int64_t at = (int64_t)m * N + n;
         bs_store4<float>(fu.resid + at, x, out_align, valid);
-        bs_store4<bf16_t>(reinterpret_cast<bf16_t*>(fu.xg) + at, xgv, out_align, valid);
+        if (fu.out_pieces)
+          bs_store_pieces(fu.xg, M, m, n, xgv, 4, valid);
+        else
+          bs_store4<bf16_t>(reinterpret_cast<bf16_t*>(fu.xg) + at, xgv, out_align, valid);
       }
       // the four lane groups hold the row's other columns of this tile
       sq += __shfl_xor(sq, 16, HE_WAVE);
@@ -428,10 +477,18 @@ static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int
 template <int MT, int R, int U, bool GATED, typename TC>
 static void launch_blocksplit(const BlockSplitPlan& p, void* C, const void* X, const void* W,
                               const void* bias, int bias_dtype, int M, int N, int K,
-                              const BsFusion& fu, hipStream_t s) {
+                              const BsFusion& fu, bool x_pieces, hipStream_t s) {
   const int blocks = (N + p.rows_per_block - 1) / p.rows_per_block;
   const size_t lds = (size_t)p.NW * R * MT * 64 * sizeof(float4);
-  gemm_blocksplit_kernel<MT, R, U, GATED, TC><<<blocks, 64 * p.NW, lds, s>>>(
+  if constexpr (MT == 1) {   // piece-major activations are for up to 16 rows
+    if (x_pieces) {
+      gemm_blocksplit_kernel<MT, R, U, GATED, true, TC><<<blocks, 64 * p.NW, lds, s>>>(
+          (TC*)C, (const uint16_t*)X, (const uint16_t*)W, bias, bias_dtype, M, N, K, p.kslice,
+          p.rows_per_block, fu);
+      return;
+    }
+  }
+  gemm_blocksplit_kernel<MT, R, U, GATED, false, TC><<<blocks, 64 * p.NW, lds, s>>>(
       (TC*)C, (const uint16_t*)X, (const uint16_t*)W, bias, bias_dtype, M, N, K, p.kslice,
       p.rows_per_block, fu);
 }
@@ -439,10 +496,10 @@ static void launch_blocksplit(const BlockSplitPlan& p, void* C, const void* X, c
 template <bool GATED, typename TC>
 static int dispatch_blocksplit(const BlockSplitPlan& p, void* C, const void* X, const void* W,
                                const void* bias, int bias_dtype, int M, int N, int K,
-                               const BsFusion& fu, hipStream_t s) {
+                               const BsFusion& fu, bool x_pieces, hipStream_t s) {
 #define BS(MT_, R_, U_)                                                              \
   if (p.MT == MT_ && p.R == R_ && p.U == U_) {                                       \
-    launch_blocksplit<MT_, R_, U_, GATED, TC>(p, C, X, W, bias, bias_dtype, M, N, K, fu, s); \
+    launch_blocksplit<MT_, R_, U_, GATED, TC>(p, C, X, W, bias, bias_dtype, M, N, K, fu, x_pieces, s); \
     return 0;                                                                        \
   }
   BS(1, 1, 1) BS(1, 1, 2) BS(1, 1, 4) BS(2, 1, 1) BS(2, 1, 2)
@@ -468,7 +525,8 @@ extern "C" int he_gemm_blocksplit_fused_bf16(void* C, const void* A, const void*
                                              const void* scale_partials, int scale_count,
                                              float scale_eps, void* resid, const void* gain,
                                              int gain_dtype, void* xg, void* sq_out,
-                                             int sq_count, void* stream) {
+                                             int sq_count, int x_pieces, int out_pieces,
+                                             void* stream) {
   HE_REQUIRE(M > 0 && M <= HE_BLOCKSPLIT_MAX_M, "he_gemm_blocksplit_bf16: M=%d outside [1, %d]", M,
              HE_BLOCKSPLIT_MAX_M);
   HE_REQUIRE(N > 0 && K > 0, "he_gemm_blocksplit_bf16: bad sizes N=%d K=%d", N, K);
@@ -480,6 +538,10 @@ extern "C" int he_gemm_blocksplit_fused_bf16(void* C, const void* A, const void*
              "he_gemm_blocksplit_bf16: the gated epilogue needs an even N=%d and no bias", N);
   HE_REQUIRE(scale_partials == nullptr || scale_count > 0,
              "he_gemm_blocksplit_bf16: row scale without partial sums");
+  HE_REQUIRE(!(x_pieces || out_pieces) || M <= 16,
+             "he_gemm_blocksplit_bf16: piece-major activations are for up to 16 rows, not %d", M);
+  HE_REQUIRE(!out_pieces || ((resid != nullptr || out_dtype == HE_BF16) && ((gated ? N / 2 : N) & 7) == 0),
+             "he_gemm_blocksplit_bf16: a piece-major output is bf16 and a multiple of 8 wide");
   const BlockSplitPlan p = blocksplit_plan(M, N, K, gated, R, U, NW);
   HE_REQUIRE(p.NW >= 1 && p.NW <= 16, "he_gemm_blocksplit_bf16: %d wavefronts outside [1, 16]",
              p.NW);
@@ -504,16 +566,17 @@ extern "C" int he_gemm_blocksplit_fused_bf16(void* C, const void* A, const void*
   fu.gain_dtype = gain_dtype;
   fu.xg = (uint16_t*)xg;
   fu.sq_out = (float*)sq_out;
+  fu.out_pieces = out_pieces;
   hipStream_t s = (hipStream_t)stream;
   int rc;
   if (gated)
     rc = out_dtype == HE_BF16
-             ? dispatch_blocksplit<true, bf16_t>(p, C, A, W, bias, bias_dtype, M, N, K, fu, s)
-             : dispatch_blocksplit<true, float>(p, C, A, W, bias, bias_dtype, M, N, K, fu, s);
+             ? dispatch_blocksplit<true, bf16_t>(p, C, A, W, bias, bias_dtype, M, N, K, fu, x_pieces != 0, s)
+             : dispatch_blocksplit<true, float>(p, C, A, W, bias, bias_dtype, M, N, K, fu, x_pieces != 0, s);
   else
     rc = out_dtype == HE_BF16
-             ? dispatch_blocksplit<false, bf16_t>(p, C, A, W, bias, bias_dtype, M, N, K, fu, s)
-             : dispatch_blocksplit<false, float>(p, C, A, W, bias, bias_dtype, M, N, K, fu, s);
+             ? dispatch_blocksplit<false, bf16_t>(p, C, A, W, bias, bias_dtype, M, N, K, fu, x_pieces != 0, s)
+             : dispatch_blocksplit<false, float>(p, C, A, W, bias, bias_dtype, M, N, K, fu, x_pieces != 0, s);
   if (rc) return rc;
   return he_check_launch("he_gemm_blocksplit_bf16");
 }
@@ -523,5 +586,5 @@ extern "C" int he_gemm_blocksplit_bf16(void* C, const void* A, const void* W, co
                                        int gated, int R, int U, int NW, void* stream) {
   return he_gemm_blocksplit_fused_bf16(C, A, W, bias, M, N, K, out_dtype, bias_dtype, gated, R, U,
                                        NW, nullptr, 0, 0.f, nullptr, nullptr, HE_F32, nullptr,
-                                       nullptr, 0, stream);
+                                       nullptr, 0, 0, 0, stream);
 }

@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 13
+#define HE_ABI_VERSION 14
 
 #ifdef __cplusplus
 extern "C" {
@@ -59,15 +59,19 @@ int he_gemm_blocksplit_bf16(void* C, const void* A, const void* W, const void* b
 // epilogue (resid[M,N] fp32 += result in place, xg[M,N] bf16 = resid * gain, sq_out[M, sq_count]
 // = sums of resid^2 per workgroup, sq_count = he_gemm_blocksplit_blocks). scale_partials != null:
 // the rows of A are such xg rows; the result is scaled by 1/sqrt(sum(partials)/K + eps) per row.
+// x_pieces / out_pieces (M <= 16): A, or the bf16 output (C, or xg), lies piece-major: a [M, D] tensor as
+// 16-byte pieces [D / 8][M][8], element (m, d) at ((d / 8) M + m) 8 + d % 8.
 int he_gemm_blocksplit_blocks(int M, int N, int K);
 int he_gemm_blocksplit_fused_bf16(void* C, const void* A, const void* W, const void* bias, int M,
                                   int N, int K, int out_dtype, int bias_dtype, int gated, int R,
                                   int U, int NW, const void* scale_partials, int scale_count,
                                   float scale_eps, void* resid, const void* gain, int gain_dtype,
-                                  void* xg, void* sq_out, int sq_count, void* stream);
-// out = x / sqrt(sum(partials of the row)/D + eps): such xg rows as a normalised tensor.
+                                  void* xg, void* sq_out, int sq_count, int x_pieces, int out_pieces,
+                                  void* stream);
+// out = x / sqrt(sum(partials of the row)/D + eps): such xg rows as a normalised tensor
+// (row-major; x_pieces: x lies piece-major for exactly `rows` rows).
 int he_scale_rows_bf16(void* out, const void* x, const void* partials, int count, int rows, int D,
-                       float eps, void* stream);
+                       float eps, int x_pieces, void* stream);
 int he_splitk_reduce(void* C, const void* partial_f32, const void* bias, int M, int N, int splits,
                      int out_dtype, int bias_dtype, void* stream);
 
@@ -95,7 +99,8 @@ int64_t he_attention_decode_workspace_floats(int rows, int H, int KVH, int hd, i
 // bf16, one query row per sequence, one launch for bias + rotary + cache write + attention +
 // merge (a second launch joins the parts where few sequences are cut across workgroups).
 // qkv: the un-biased projection rows [rows, (H + 2 KVH) hd]. he_attention_decode_fused_ok: 1
-// when the sizes are taken (head_dim 64 or 128, rotated whole).
+// when the sizes are taken (head_dim 64 or 128, rotated whole). out_pieces: out lies piece-major
+// (as he_gemm_blocksplit_fused_bf16 reads it with x_pieces).
 int he_attention_decode_fused_ok(int H, int KVH, int hd, int rotary_dim);
 int64_t he_attention_decode_fused_workspace_floats(int rows, int H, int KVH, int hd, int max_keys);
 int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_t qkv_stride, const void* bias,
@@ -104,7 +109,8 @@ int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_t qkv_strid
                                    const void* page_table, int max_blocks, int num_pages,
                                    const void* inv_freq, int rotary_dim, int rows, int H, int KVH,
                                    int hd, int window, float scale, int max_keys, int write_kv,
-                                   void* workspace_f32, int64_t workspace_floats, void* stream);
+                                   int out_pieces, void* workspace_f32, int64_t workspace_floats,
+                                   void* stream);
 // bf16, prompt steps: tiles of queries of one sequence against its cache rows.
 int he_attention_prefill_bf16(void* out, const void* q, const void* kpool, const void* vpool,
                               const void* cu_seqlens, const void* seq_slot, const void* seq_start,

@@ -281,8 +281,10 @@ extern "C" int he_rmsnorm_rows(void* out, const void* x, const void* weight, int
 // Rows x = r * gain whose scale is still owed: out = x / sqrt(sum(partials of the row) / D + eps).
 // The partial sums of squares (one per workgroup of the product that made the rows) are
 // added as that product's consumers add them: lanes over strided partials, then the wavefront.
+// x_pieces: x lies piece-major, 16-byte pieces [D / 8][rows][8]; out is row-major either way.
 __global__ void scale_rows_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ x,
-                                  const float* __restrict__ partials, int count, int D, float eps) {
+                                  const float* __restrict__ partials, int count, int D, float eps,
+                                  int x_pieces) {
   __shared__ float inv_s;
   const int64_t row = blockIdx.x;
   if (threadIdx.x < 64) {
@@ -293,16 +295,19 @@ __global__ void scale_rows_kernel(uint16_t* __restrict__ out, const uint16_t* __
   }
   __syncthreads();
   const float inv = inv_s;
-  for (int i = threadIdx.x; i < D; i += blockDim.x)
-    out[row * D + i] = float_to_bf16_bits(bf16_bits_to_float(x[row * D + i]) * inv);
+  for (int i = threadIdx.x; i < D; i += blockDim.x) {
+    const int64_t at = x_pieces ? ((int64_t)(i >> 3) * gridDim.x + row) * 8 + (i & 7) : row * D + i;
+    out[row * D + i] = float_to_bf16_bits(bf16_bits_to_float(x[at]) * inv);
+  }
 }
 
 extern "C" int he_scale_rows_bf16(void* out, const void* x, const void* partials, int count,
-                                  int rows, int D, float eps, void* stream) {
+                                  int rows, int D, float eps, int x_pieces, void* stream) {
   HE_REQUIRE(rows >= 0 && D > 0 && count > 0, "he_scale_rows_bf16: bad sizes rows=%d D=%d count=%d",
              rows, D, count);
+  HE_REQUIRE(!x_pieces || D % 8 == 0, "he_scale_rows_bf16: piece-major rows of width %d, not a multiple of 8", D);
   if (rows == 0) return 0;
   scale_rows_kernel<<<rows, norm_threads(D), 0, (hipStream_t)stream>>>(
-      (uint16_t*)out, (const uint16_t*)x, (const float*)partials, count, D, eps);
+      (uint16_t*)out, (const uint16_t*)x, (const float*)partials, count, D, eps, x_pieces);
   return he_check_launch("he_scale_rows_bf16");
 }

@@ -207,13 +207,26 @@ def gemm_skinny(out, partial, a, w, bias, M: int, plan=(0, 0, 0), out_dtype=None
 BLOCKSPLIT_MAX_M = 32
 
 
+PIECES_MAX_M = 16
+
+
+def pieces_shape(M: int, D: int) -> tuple[int, int, int]:
+    """Shape of a piece-major [M, D] bf16 tensor: 16-byte pieces of 8 columns, the M pieces of
+    one column group next to each other: element (m, d) at [d // 8, m, d % 8]. The block-split
+    product reads its rows best this way (a wavefront's load of 16 rows x 16 bytes touches two
+    cache lines, not sixteen), and writes them so for the next one; at most PIECES_MAX_M rows."""
+    if D % 8 != 0 or not 0 < M <= PIECES_MAX_M:
+        raise ValueError(f"piece-major rows: D={D} must be a multiple of 8 and 0 < M={M} <= {PIECES_MAX_M}")
+    return (D // 8, M, 8)
+
+
 def gemm_blocksplit_blocks(M: int, N: int, K: int) -> int:
     """Partial sums of squares per row that the residual epilogue of this product gives."""
     return int(_lib.load().he_gemm_blocksplit_blocks(M, N, K))
 
 
 def gemm_blocksplit(out, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0), *,
-                    row_scale=None, residual=None) -> None:
+                    row_scale=None, residual=None, x_pieces: bool = False, out_pieces: bool = False) -> None:
     """bf16 MFMA product for M <= 32 with K cut inside the workgroup; one launch, complete
     result (bf16 or fp32), with bias or, gated, as [M, N/2] = silu(gate) * up for a weight
     that alternates gate and up rows (gate i at row 2i, its up at 2i + 1). plan = (R, U, NW),
@@ -223,18 +236,24 @@ def gemm_blocksplit(out, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0)
     whose 1/sqrt(mean(r^2) + eps) is applied to the sums here (mean over K).
     residual = (resid fp32 [M, N], gain [N], xg bf16 [M, N], sq fp32 [M, blocks]): instead of
     writing `out` (None), resid += result in place, xg = resid * gain, sq = the sums of resid^2
-    per workgroup (blocks = gemm_blocksplit_blocks(M, N, K))."""
+    per workgroup (blocks = gemm_blocksplit_blocks(M, N, K)).
+    x_pieces: `a` is piece-major, shaped pieces_shape(M, K). out_pieces: the bf16 output (`out`,
+    or xg of the residual epilogue) is written piece-major, shaped pieces_shape(M, its width)."""
     N, K = w.shape
     NO = N // 2 if gated else N
     _need(a, "a", torch.bfloat16)
     _need(w, "w", torch.bfloat16)
     if M > BLOCKSPLIT_MAX_M:
         raise ValueError(f"gemm_blocksplit: M={M} above {BLOCKSPLIT_MAX_M}")
-    if a.shape[-1] != K or a.numel() < M * K:
+    if x_pieces:
+        _need(a, "a", shape=pieces_shape(M, K))
+    elif a.shape[-1] != K or a.numel() < M * K:
         raise ValueError(f"gemm_blocksplit: shapes a{tuple(a.shape)} w{tuple(w.shape)} M={M}")
     if residual is None:
         _need(out, "out")
-        if out.shape[-1] != NO or out.numel() < M * NO:
+        if out_pieces:
+            _need(out, "out", torch.bfloat16, pieces_shape(M, NO))
+        elif out.shape[-1] != NO or out.numel() < M * NO:
             raise ValueError(f"gemm_blocksplit: out{tuple(out.shape)} for M={M} N={NO}")
     elif out is not None or gated or plan != (0, 0, 0):
         raise ValueError("gemm_blocksplit: the residual epilogue writes no `out`, is not gated and plans itself")
@@ -255,8 +274,10 @@ def gemm_blocksplit(out, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0)
         _need(gain, "gain", shape=(N,))
         _need(xg, "xg", torch.bfloat16)
         _need(sq, "sq", torch.float32)
-        if resid.shape[-1] != N or resid.numel() < M * N or xg.shape[-1] != N or xg.numel() < M * N \
-                or sq.dim() != 2 or sq.shape[0] < M:
+        if out_pieces:
+            _need(xg, "xg", shape=pieces_shape(M, N))
+        if resid.shape[-1] != N or resid.numel() < M * N or xg.numel() < M * N \
+                or (not out_pieces and xg.shape[-1] != N) or sq.dim() != 2 or sq.shape[0] < M:
             raise ValueError("gemm_blocksplit: residual buffers do not match [M, N]")
         rp, gp, xp, qp = resid.data_ptr(), gain.data_ptr(), xg.data_ptr(), sq.data_ptr()
         gdt, qc = dtype_code(gain.dtype), sq.shape[1]
@@ -266,20 +287,24 @@ def gemm_blocksplit(out, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0)
         dtype_code(out.dtype) if out is not None else BF16,
         dtype_code(bias.dtype) if bias is not None else F32, int(gated),
         int(plan[0]), int(plan[1]), int(plan[2]), sp, sc, float(se), rp, gp, gdt, xp, qp, qc,
-        _stream()))
+        int(x_pieces), int(out_pieces), _stream()))
 
 
-def scale_rows(out, x, partials, eps: float, rows: int) -> None:
-    """out = x / sqrt(sum(partials of the row) / D + eps) for rows x = r * gain (bf16)."""
-    D = x.shape[-1]
+def scale_rows(out, x, partials, eps: float, rows: int, x_pieces: bool = False) -> None:
+    """out = x / sqrt(sum(partials of the row) / D + eps) for rows x = r * gain (bf16). out is
+    row-major; x_pieces: x is piece-major, shaped pieces_shape(rows, D)."""
+    D = out.shape[-1]
     _need(out, "out", torch.bfloat16)
     _need(x, "x", torch.bfloat16)
     _need(partials, "partials", torch.float32)
-    if out.shape[-1] != D or out.numel() < rows * D or x.numel() < rows * D \
+    if x_pieces:
+        _need(x, "x", shape=pieces_shape(rows, D))
+    if out.numel() < rows * D or x.numel() < rows * D or (not x_pieces and x.shape[-1] != D) \
             or partials.dim() != 2 or partials.shape[0] < rows:
         raise ValueError("scale_rows: buffers do not match [rows, D]")
     _lib.check(_lib.load().he_scale_rows_bf16(out.data_ptr(), x.data_ptr(), partials.data_ptr(),
-                                              partials.shape[1], rows, D, float(eps), _stream()))
+                                              partials.shape[1], rows, D, float(eps), int(x_pieces),
+                                              _stream()))
 
 
 def splitk_reduce(out, partial, bias, M: int, splits: int) -> None:
@@ -415,15 +440,18 @@ def attention_decode_fused_workspace_floats(rows: int, H: int, KVH: int, hd: int
 def attention_decode_fused(out, qkv, bias, kpool, vpool, positions, row_seq, seq_slot, page_table,
                            inv_freq, rotary_dim: int, rows: int, H: int, KVH: int, hd: int,
                            window: int, scale: float, max_keys: int, write_kv: bool,
-                           workspace) -> None:
+                           workspace, out_pieces: bool = False) -> None:
     """One-token steps in one launch: bias, rotation of q and of the new key, cache write,
     attention over the cache, merge. qkv: bf16 [rows, (H + 2 KVH) hd] without bias; q columns
-    alone where the run reads another run's cache (write_kv False)."""
+    alone where the run reads another run's cache (write_kv False). out_pieces: out is written
+    piece-major for exactly `rows` rows (see :func:`to_pieces`)."""
     width = (H + 2 * KVH) * hd if write_kv else H * hd
     _need(qkv, "qkv", torch.bfloat16)
     _need(out, "out", torch.bfloat16)
     if qkv.dim() != 2 or qkv.shape[1] != width or qkv.shape[0] < rows or out.numel() < rows * H * hd:
         raise ValueError("attention_decode_fused: qkv/out do not match the head sizes and row count")
+    if out_pieces:
+        _need(out, "out", shape=pieces_shape(rows, H * hd))
     _need(kpool, "kpool", torch.bfloat16, (None, KVH, layout.k_page_elems(hd)))
     _need(vpool, "vpool", torch.bfloat16, (None, KVH, layout.v_page_elems(hd)))
     _need(page_table, "page_table", torch.int32)
@@ -442,7 +470,7 @@ def attention_decode_fused(out, qkv, bias, kpool, vpool, positions, row_seq, seq
         dtype_code(bias.dtype) if bias is not None else F32, kpool.data_ptr(), vpool.data_ptr(),
         positions.data_ptr(), row_seq.data_ptr(), seq_slot.data_ptr(), page_table.data_ptr(),
         page_table.shape[1], kpool.shape[0], inv_freq.data_ptr(), rotary_dim, rows, H, KVH, hd,
-        window, float(scale), max_keys, int(write_kv), _ptr(workspace),
+        window, float(scale), max_keys, int(write_kv), int(out_pieces), _ptr(workspace),
         workspace.numel() if workspace is not None else 0, _stream()))
 
 

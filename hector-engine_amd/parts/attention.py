@@ -16,7 +16,7 @@ import math
 import torch
 
 from ..kernels import ops
-from .base import (BuildEnv, KVNeed, LayerCache, Mixer, PartSpec, StepContext, TensorSpec,
+from .base import (BuildEnv, KVNeed, LayerCache, Mixer, PartSpec, PieceRows, StepContext, TensorSpec,
                    build_part, param, register_part)
 from .linear import Linear, SplitSum
 
@@ -101,14 +101,16 @@ class Attention(Mixer):
                 and ops.attention_decode_fused_ok(H, KVH, hd, rot[1]):
             # one-token steps: bias, rotation, cache write and attention in one launch
             qkv = proj(x, rows, ctx, use_bias=False)
-            out = ctx.alloc((rows, H * hd))
+            pieces = self.o_proj.reads_pieces(rows, ctx)       # the layout the output product reads best
+            out = ctx.alloc(ops.pieces_shape(rows, H * hd) if pieces else (rows, H * hd))
             floats = ops.attention_decode_fused_workspace_floats(rows, H, KVH, hd, ctx.max_keys)
             ws = ctx.alloc((floats,), torch.float32) if floats else None
             ops.attention_decode_fused(out, qkv, proj.bias, cache.kpool, cache.vpool, ctx.positions,
                                        ctx.row_seq, ctx.seq_slot, cache.page_table, rot[0], rot[1],
                                        rows, H, KVH, hd, self.window, self.scale, ctx.max_keys,
-                                       writes, ws)
-            return self.o_proj(out, rows, ctx, allow_split=True, sink=ctx.take_sink())
+                                       writes, ws, out_pieces=pieces)
+            return self.o_proj(PieceRows(out) if pieces else out, rows, ctx, allow_split=True,
+                               sink=ctx.take_sink())
         # With a rotation (or no encoding) the bias is added inside the fused kernel;
         # any other encoding sees q and k with their bias already added.
         qkv = proj(x, rows, ctx, use_bias=not fused_bias, allow_split=fused_bias)

@@ -238,18 +238,32 @@ class NormedRows:
     activation dtype, and the sum of r^2 of a row as `partials[row, :]` (fp32, added in
     index order by lanes of 64, then across the lanes). norm(r) = scaled / sqrt(sum / dim +
     eps). A product applies the scale to its sums (parts.linear.Linear); tensor() gives the
-    normalised rows to anything else."""
+    normalised rows to anything else. pieces: `scaled` lies piece-major
+    (kernels.ops.pieces_shape(rows, dim))."""
 
     scaled: torch.Tensor
     partials: torch.Tensor
     eps: float
     rows: int
+    pieces: bool = False
+
+    @property
+    def dim(self) -> int:
+        return self.scaled.shape[0] * 8 if self.pieces else self.scaled.shape[-1]
 
     def tensor(self, ctx: StepContext) -> torch.Tensor:
         from ..kernels import ops
-        out = ctx.alloc((self.rows, self.scaled.shape[-1]), self.scaled.dtype)
-        ops.scale_rows(out, self.scaled, self.partials, self.eps, self.rows)
+        out = ctx.alloc((self.rows, self.dim), self.scaled.dtype)
+        ops.scale_rows(out, self.scaled, self.partials, self.eps, self.rows, self.pieces)
         return out
+
+
+@dataclasses.dataclass
+class PieceRows:
+    """bf16 rows handed from one kernel to a product in the piece-major layout
+    (kernels.ops.pieces_shape): only to a Linear that says reads_pieces(rows, ctx)."""
+
+    pieces: torch.Tensor
 
 
 class ResidualSink:

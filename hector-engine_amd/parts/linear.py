@@ -25,13 +25,19 @@ step of few rows has no norm kernels: given a :class:`ResidualSink` it adds its 
 to the residual rows itself and leaves r * gain and the sums of r^2 for the norm that
 follows (:class:`NormedRows`); given NormedRows as input it applies the owed row scale
 to its sums. Any other path turns NormedRows into a tensor first and ignores the sink.
+
+Between block-split products of up to 16 rows the bf16 rows travel piece-major
+(kernels.ops.pieces_shape): the product's operand loads then touch two cache lines instead
+of sixteen (at the Qwen2.5-7B shapes 2 us a layer at 8 rows, 10 us at 16). The rows it
+leaves for the next norm are written so; a producer of its input (attention, the gated
+product) writes so after asking reads_pieces().
 """
 from __future__ import annotations
 
 import torch
 
 from ..kernels import library_tuning, ops
-from .base import NormedRows, ResidualSink, StepContext
+from .base import NormedRows, PieceRows, ResidualSink, StepContext
 
 
 class SplitSum:
@@ -68,6 +74,16 @@ def _library_is_faster(rows: int, N: int, K: int) -> bool:
     return rows > 16 and (K < LONG_K or library_tuning.enabled())
 
 
+def _operand(x):
+    """(activation dtype, the tensor a kernel reads, the owed row scale or None, whether
+    that tensor lies piece-major) of a tensor, NormedRows or PieceRows."""
+    if isinstance(x, NormedRows):
+        return x.scaled.dtype, x.scaled, (x.partials, x.eps), x.pieces
+    if isinstance(x, PieceRows):
+        return x.pieces.dtype, x.pieces, None, True
+    return x.dtype, x, None, False
+
+
 class Linear:
     def __init__(self, weight: torch.Tensor, bias: torch.Tensor | None = None):
         if weight.dim() != 2:
@@ -84,15 +100,19 @@ class Linear:
                 and ctx.env.fast_kernels and K % 8 == 0
                 and 0 < rows <= (16 if _library_is_faster(ops.BLOCKSPLIT_MAX_M, N, K) else ops.BLOCKSPLIT_MAX_M))
 
+    def reads_pieces(self, rows: int, ctx: StepContext) -> bool:
+        """Whether bf16 input rows may come piece-major (PieceRows)."""
+        return rows <= ops.PIECES_MAX_M and self._blocksplit_rows(rows, ctx, torch.bfloat16)
+
     def __call__(self, x, rows: int, ctx: StepContext, *, use_bias: bool = True,
                  out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None,
                  allow_split: bool = False, sink: ResidualSink | None = None):
-        """x: a tensor or NormedRows. With a sink the result may go into the residual
-        stream directly; the call then returns None."""
+        """x: a tensor, NormedRows or PieceRows. With a sink the result may go into the
+        residual stream directly; the call then returns None."""
         w = self.weight
         N, K = w.shape
         bias = self.bias if use_bias else None
-        act = x.scaled.dtype if isinstance(x, NormedRows) else x.dtype
+        act, a, scale, pieces = _operand(x)
         out_dtype = out_dtype or act
         if self._blocksplit_rows(rows, ctx, act):
             if sink is not None and out is None and out_dtype == act and rows <= 16 \
@@ -100,11 +120,10 @@ class Linear:
                 return self._into_residual(x, bias, rows, ctx, sink)
             if out is None:
                 out = ctx.alloc((rows, N), out_dtype)
-            if isinstance(x, NormedRows):
-                ops.gemm_blocksplit(out, x.scaled, w, bias, rows, row_scale=(x.partials, x.eps))
-            else:
-                ops.gemm_blocksplit(out, x, w, bias, rows)
+            ops.gemm_blocksplit(out, a, w, bias, rows, row_scale=scale, x_pieces=pieces)
             return out
+        if isinstance(x, PieceRows):
+            raise TypeError("Linear: piece-major rows for a product that does not read them (ask reads_pieces)")
         if isinstance(x, NormedRows):
             x = x.tensor(ctx)
         if rows == 0:
@@ -159,12 +178,14 @@ class Linear:
     def _into_residual(self, x, bias, rows, ctx, sink: ResidualSink):
         N, K = self.weight.shape
         gain, eps = sink.norm.carried()
-        xg = ctx.alloc((rows, N), torch.bfloat16)
+        out_pieces = N % 8 == 0 and rows <= ops.PIECES_MAX_M
+        xg = ctx.alloc(ops.pieces_shape(rows, N) if out_pieces else (rows, N), torch.bfloat16)
         sq = ctx.alloc((rows, ops.gemm_blocksplit_blocks(rows, N, K)), torch.float32)
-        scale = (x.partials, x.eps) if isinstance(x, NormedRows) else None
-        ops.gemm_blocksplit(None, x.scaled if scale else x, self.weight, bias, rows, row_scale=scale,
-                            residual=(sink.stream.resid, gain, xg, sq))
-        sink.stream.prepared = (sink.norm, NormedRows(xg, sq, eps, rows))
+        _, a, scale, pieces = _operand(x)
+        ops.gemm_blocksplit(None, a, self.weight, bias, rows, row_scale=scale,
+                            residual=(sink.stream.resid, gain, xg, sq), x_pieces=pieces,
+                            out_pieces=out_pieces)
+        sink.stream.prepared = (sink.norm, NormedRows(xg, sq, eps, rows, out_pieces))
         return None
 
     def _skinny(self, x, bias, rows, ctx, out, out_dtype, allow_split):
@@ -191,17 +212,19 @@ class Linear:
             return s
         return s.materialize(ctx, out_dtype, out)
 
-    def gated_silu(self, x, rows: int, ctx: StepContext, out: torch.Tensor) -> bool:
-        """out[rows, N/2] = silu(gate) * up in one kernel, for a weight whose rows
-        alternate gate and up (gate i at row 2i, its up at 2i + 1). x: a tensor or NormedRows. False when that
-        kernel does not apply."""
+    def gated_silu_rows(self, rows: int, ctx: StepContext, act: torch.dtype) -> bool:
+        """Whether gated_silu applies to this many rows of this dtype."""
         w = self.weight
-        act = x.scaled.dtype if isinstance(x, NormedRows) else x.dtype
-        if not (ctx.env.fast_kernels and w.dtype == torch.bfloat16 and act == torch.bfloat16
-                and 0 < rows <= 16 and w.shape[1] % 8 == 0 and w.shape[0] % 2 == 0):
-            return False
-        if isinstance(x, NormedRows):
-            ops.gemm_blocksplit(out, x.scaled, w, None, rows, gated=True, row_scale=(x.partials, x.eps))
-        else:
-            ops.gemm_blocksplit(out, x, w, None, rows, gated=True)
-        return True
+        return (ctx.env.fast_kernels and w.dtype == torch.bfloat16 and act == torch.bfloat16
+                and 0 < rows <= 16 and w.shape[1] % 8 == 0 and w.shape[0] % 2 == 0)
+
+    def gated_silu(self, x, rows: int, ctx: StepContext, out: torch.Tensor,
+                   out_pieces: bool = False) -> None:
+        """out[rows, N/2] = silu(gate) * up in one kernel, for a weight whose rows alternate gate
+        and up (gate i at row 2i, its up at 2i + 1), where gated_silu_rows() says so. x: a tensor,
+        NormedRows or PieceRows; out_pieces: out is shaped and written piece-major."""
+        act, a, scale, pieces = _operand(x)
+        if not self.gated_silu_rows(rows, ctx, act):
+            raise ValueError("Linear.gated_silu: not for these rows (ask gated_silu_rows)")
+        ops.gemm_blocksplit(out, a, self.weight, None, rows, gated=True, row_scale=scale,
+                            x_pieces=pieces, out_pieces=out_pieces)

@@ -345,6 +345,91 @@ def test_gemm_blocksplit_carries_the_norm(ops, M, D, K, N2, eps, gain_dtype):
     assert torch.allclose(sq2.cpu().double().sum(1), (resid2.cpu()[:M].double() ** 2).sum(1), rtol=1e-5)
 
 
+def to_pieces(x):
+    """[M, D] -> piece-major [D / 8, M, 8]: 16-byte pieces, the M pieces of a column group together."""
+    M, D = x.shape
+    return x.reshape(M, D // 8, 8).permute(1, 0, 2).contiguous()
+
+
+def from_pieces(p):
+    return p.permute(1, 0, 2).reshape(p.shape[1], -1).contiguous()
+
+
+@pytest.mark.parametrize("M", [1, 3, 8, 16])
+@pytest.mark.parametrize("N,K", [(264, 136), (3584, 520), (1000, 18944), (2312, 264), (4608, 3584)])
+def test_gemm_blocksplit_piece_major(ops, M, N, K):
+    """Operand rows and bf16 results in the piece-major layout: the same sums in the same
+    order as row-major, so equal bit for bit: plain, gated, with the residual epilogue and
+    the owed row scale, and back to a tensor."""
+    if K == 18944 and M in (3, 8):
+        pytest.skip("long K at two row counts")
+    x = dev(rnd(M, K, seed=110).to(torch.bfloat16))
+    w = dev(rnd(N, K, seed=111, scale=0.05).to(torch.bfloat16))
+    b = dev(rnd(N, seed=112).to(torch.bfloat16))
+    xp = to_pieces(x)
+    assert tuple(xp.shape) == ops.pieces_shape(M, K)
+    want = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    ops.gemm_blocksplit(want, x, w, b, M)
+    ref = x.cpu().double() @ w.cpu().double().T + b.cpu().double()
+    assert (want.cpu().double() - ref).abs().max().item() <= 2 ** -7 * ref.abs().max().item()
+    for xin, op in ((True, False), (False, True), (True, True)):
+        out = torch.full(ops.pieces_shape(M, N) if op else (M, N), 7.0, dtype=torch.bfloat16, device="cuda")
+        ops.gemm_blocksplit(out, xp if xin else x, w, b, M, x_pieces=xin, out_pieces=op)
+        assert torch.equal(from_pieces(out) if op else out, want), (xin, op)
+    out32, want32 = (torch.empty(M, N, device="cuda") for _ in range(2))          # fp32 results stay row-major
+    ops.gemm_blocksplit(want32, x, w, b, M)
+    ops.gemm_blocksplit(out32, xp, w, b, M, x_pieces=True)
+    assert torch.equal(out32, want32)
+    # gated: [M, N / 2]
+    if (N // 2) % 8 == 0:
+        wh, oh = torch.empty(M, N // 2, dtype=torch.bfloat16, device="cuda"), \
+            torch.empty(ops.pieces_shape(M, N // 2), dtype=torch.bfloat16, device="cuda")
+        ops.gemm_blocksplit(wh, x, w, None, M, gated=True)
+        ops.gemm_blocksplit(oh, xp, w, None, M, gated=True, x_pieces=True, out_pieces=True)
+        assert torch.equal(from_pieces(oh), wh)
+    # residual epilogue leaving piece-major rows, read by a product with the owed scale
+    r0 = dev(rnd(M, N, seed=113, scale=3.0))
+    gain = dev((1 + 0.1 * rnd(N, seed=114)).to(torch.bfloat16))
+    blocks = ops.gemm_blocksplit_blocks(M, N, K)
+    res_a, res_b = r0.clone(), r0.clone()
+    xg_a = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    xg_b = torch.empty(ops.pieces_shape(M, N), dtype=torch.bfloat16, device="cuda")
+    sq_a, sq_b = (torch.empty(M, blocks, device="cuda") for _ in range(2))
+    ops.gemm_blocksplit(None, x, w, b, M, residual=(res_a, gain, xg_a, sq_a))
+    ops.gemm_blocksplit(None, xp, w, b, M, residual=(res_b, gain, xg_b, sq_b), x_pieces=True, out_pieces=True)
+    assert torch.equal(res_a, res_b) and torch.equal(sq_a, sq_b) and torch.equal(from_pieces(xg_b), xg_a)
+    w2 = dev(rnd(72, N, seed=115, scale=0.05).to(torch.bfloat16))
+    y_a, y_b = (torch.empty(M, 72, dtype=torch.bfloat16, device="cuda") for _ in range(2))
+    ops.gemm_blocksplit(y_a, xg_a, w2, None, M, row_scale=(sq_a, 1e-6))
+    ops.gemm_blocksplit(y_b, xg_b, w2, None, M, row_scale=(sq_b, 1e-6), x_pieces=True)
+    assert torch.equal(y_a, y_b)
+    t_a, t_b = (torch.empty(M, N, dtype=torch.bfloat16, device="cuda") for _ in range(2))
+    ops.scale_rows(t_a, xg_a, sq_a, 1e-6, M)
+    ops.scale_rows(t_b, xg_b, sq_b, 1e-6, M, x_pieces=True)
+    assert torch.equal(t_a, t_b)
+
+
+def test_piece_major_rows_are_refused_beyond_their_sizes(ops):
+    from hector_engine_amd.kernels.lib import KernelLibraryError
+    with pytest.raises(ValueError, match="piece-major"):
+        ops.pieces_shape(17, 64)
+    with pytest.raises(ValueError, match="piece-major"):
+        ops.pieces_shape(4, 60)
+    M, N, K = 4, 64, 64
+    x = torch.zeros(ops.pieces_shape(M, K), dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(N, K, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError, match="shape"):       # row-major operand where pieces are announced
+        ops.gemm_blocksplit(torch.empty(M, N, dtype=torch.bfloat16, device="cuda"),
+                            torch.zeros(M, K, dtype=torch.bfloat16, device="cuda"), w, None, M, x_pieces=True)
+    with pytest.raises(TypeError):                         # fp32 results are not written piece-major
+        ops.gemm_blocksplit(torch.empty(ops.pieces_shape(M, N), device="cuda"), x, w, None, M,
+                            x_pieces=True, out_pieces=True)
+    w20 = torch.zeros(20, K, dtype=torch.bfloat16, device="cuda")  # gated width 10: no whole pieces
+    with pytest.raises((ValueError, KernelLibraryError)):
+        ops.gemm_blocksplit(torch.empty(M, 10, dtype=torch.bfloat16, device="cuda"), x, w20, None, M,
+                            gated=True, x_pieces=True, out_pieces=True)
+
+
 def test_gemm_blocksplit_residual_epilogue_checks_its_buffers(ops):
     from hector_engine_amd.kernels.lib import KernelLibraryError
     M, D, K = 4, 64, 64
@@ -642,6 +727,12 @@ def test_attention_decode_fused(ops, H, KVH, hd, window, write_kv, copies):
     if write_kv:   # nothing but the new rows was written
         before = dev(kpool).cpu()
         assert (kp != before).sum().item() <= B * KVH * hd
+    if rows <= ops.PIECES_MAX_M:   # the same result piece-major, as the output product reads it
+        out2 = torch.full(ops.pieces_shape(rows, H * hd), 7.0, dtype=torch.bfloat16, device="cuda")
+        ops.attention_decode_fused(out2, dev(qkv_rows), dev(bias), dev(kp), dev(vp), dev(positions),
+                                   dev(row_seq), dev(seq_slot), dev(table), dev(inv), hd, rows, H, KVH,
+                                   hd, window, 1.0 / math.sqrt(hd), 4096, write_kv, ws, out_pieces=True)
+        assert torch.equal(from_pieces(out2).cpu(), out.cpu())
 
 
 def test_attention_decode_fused_refuses_other_sizes(ops):
