@@ -741,6 +741,48 @@ def test_attention_decode_fused_refuses_other_sizes(ops):
     assert not ops.attention_decode_fused_ok(5, 2, 64, 64)
 
 
+@pytest.mark.parametrize("where", ["far", "first_in_window", "last_outside_window"])
+@pytest.mark.parametrize("copies", [1, 130])
+def test_attention_decode_fused_far_key_and_window_edge(ops, where, copies):
+    """The one-token kernel with one old key made to dominate the scores of each kv group's
+    first head: far back among 900 keys it must be the result; as the oldest key of a window it
+    must be the result too; one place further back it must not count at all. Alone (keys cut
+    across workgroups, joined by a second launch) and among many sequences (one workgroup each)."""
+    H, KVH, hd, n, theta = 4, 2, 64, 900, 10000.0
+    window = 0 if where == "far" else 200
+    key = {"far": 17, "first_in_window": n - 200, "last_outside_window": n - 201}[where]
+    B = copies
+    lengths = [n] + [50 + 3 * i for i in range(B - 1)]
+    slots, table, kpool, vpool = paged_setup(lengths, KVH, hd, torch.bfloat16, 77)
+    width = (H + 2 * KVH) * hd
+    qkv = rnd(B, width, seed=120, scale=0.1).to(torch.bfloat16)
+    pos = torch.tensor([m - 1 for m in lengths], dtype=torch.int32)
+    q_rot = P.rope(qkv[0, :H * hd].double().reshape(1, H, hd), torch.tensor([n - 1]), theta, hd)
+    ks = [rnd(m - 1, KVH, hd, seed=121 + i, scale=0.1).to(torch.bfloat16) for i, m in enumerate(lengths)]
+    vs = [rnd(m - 1, KVH, hd, seed=171 + i).to(torch.bfloat16) for i, m in enumerate(lengths)]
+    ks[0][key] = (q_rot[0, ::H // KVH] * 300).to(torch.bfloat16)
+    fill_cache(table, slots, kpool, vpool, ks, vs)
+    floats = ops.attention_decode_fused_workspace_floats(B, H, KVH, hd, 4096)
+    assert (floats > 0) == (copies == 1)
+    ws = torch.empty(floats, device="cuda") if floats else None
+    out = torch.empty(B, H * hd, dtype=torch.bfloat16, device="cuda")
+    ops.attention_decode_fused(out, dev(qkv), None, dev(kpool), dev(vpool), dev(pos),
+                               dev(torch.arange(B, dtype=torch.int32)), dev(torch.tensor(slots, dtype=torch.int32)),
+                               dev(table), dev(P.rope_inv_freq(hd, theta)), hd, B, H, KVH, hd, window,
+                               1.0 / math.sqrt(hd), 4096, True, ws)
+    got = out.cpu().double()[0].reshape(H, hd)
+    x = qkv[0].double()
+    k_new = P.rope(x[H * hd:(H + KVH) * hd].reshape(1, KVH, hd), torch.tensor([n - 1]), theta, hd).to(torch.bfloat16)
+    v_new = x[(H + KVH) * hd:].reshape(1, KVH, hd).to(torch.bfloat16)
+    k_all, v_all = torch.cat([ks[0], k_new]).double(), torch.cat([vs[0], v_new]).double()
+    want = P.attention(q_rot.to(torch.bfloat16).double(), k_all, v_all, torch.tensor([n - 1]), torch.arange(n),
+                       window).reshape(H, hd)
+    assert torch.allclose(got, want, rtol=2 ** -6, atol=2 ** -6)
+    for h in range(0, H, H // KVH):
+        near = torch.allclose(got[h], vs[0][key, h // (H // KVH)].double(), atol=0.05)
+        assert near == (where != "last_outside_window"), (where, h)
+
+
 def test_attention_far_key_stands_out(ops):
     """One far key is made to dominate: a kernel that drops or misplaces it fails."""
     H, KVH, hd, n = 4, 2, 64, 900
