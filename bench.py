@@ -5,7 +5,8 @@ token ids) on one MI355X, with prefill and roofline figures on the same line.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--shape 7b|32b|72b]
 
 The default is the 7B shape; --shape runs the same measurement at the layer sizes of
-Qwen2.5-32B (context 8192) or Qwen2-72B (context 4096).
+Qwen2.5-32B (context 8192, prompts of 512 to 2048 tokens, batches 1 / 8 / 64) or
+Qwen2-72B (context 4096, prompts of 2048 tokens, batches 1 / 8 / 32).
 
 A step is one decode step of the whole batch: the engine's step function (HIP
 graph replay) plus greedy sampling. As in the library's generation loop, 8 steps are
@@ -15,6 +16,7 @@ reads them once per run of 8.
 from __future__ import annotations
 
 import argparse
+import contextlib
 import json
 import sys
 import time
@@ -25,11 +27,12 @@ import numpy as np
 _COMMON = dict(head_dim=128, vocab_size=152064, rope_theta=1000000.0, rms_norm_eps=1e-6,
                max_position_embeddings=32768, tie_word_embeddings=False)
 SHAPES = {
-    "7b": ("Qwen2.5-7B shape", 8192, dict(_COMMON, num_hidden_layers=28, hidden_size=3584, num_attention_heads=28,
+    # name, context per sequence, prompt lengths of the decode batches (lowest, highest), the large batch, sizes
+    "7b": ("Qwen2.5-7B shape", 8192, (2048, 2048), 64, dict(_COMMON, num_hidden_layers=28, hidden_size=3584, num_attention_heads=28,
                                           num_key_value_heads=4, intermediate_size=18944)),
-    "32b": ("Qwen2.5-32B shape", 8192, dict(_COMMON, num_hidden_layers=64, hidden_size=5120, num_attention_heads=40,
+    "32b": ("Qwen2.5-32B shape", 8192, (512, 2048), 64, dict(_COMMON, num_hidden_layers=64, hidden_size=5120, num_attention_heads=40,
                                             num_key_value_heads=8, intermediate_size=27648)),
-    "72b": ("Qwen2-72B shape", 4096, dict(_COMMON, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64,
+    "72b": ("Qwen2-72B shape", 4096, (2048, 2048), 32, dict(_COMMON, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64,
                                           num_key_value_heads=8, intermediate_size=29568)),
 }
 PROMPT = 2048
@@ -65,14 +68,14 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0 = all)")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="7b")
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points")
+    ap.add_argument("--no-points", action="store_true", help="skip the points at batch 1 and at the large batch")
     ap.add_argument("--no-tune", action="store_true",
                     help="leave the library's default kernels for the tall matrix products")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
-    MODEL, CONTEXT, SHAPE = SHAPES[args.shape]
+    MODEL, CONTEXT, (PROMPT_LO, PROMPT_HI), BIG_BATCH, SHAPE = SHAPES[args.shape]
     FULL_LAYERS = SHAPE["num_hidden_layers"]
     args.layers = args.layers or FULL_LAYERS
 
@@ -80,6 +83,7 @@ def main() -> int:
     import hector_engine_amd as he
     from hector_engine_amd.config.qwen2 import Qwen2Config
     from hector_engine_amd.engine.engine import StepEntry
+    from hector_engine_amd.kernels import library_tuning
 
     t_start = time.perf_counter()
 
@@ -89,7 +93,7 @@ def main() -> int:
     progress(f"{MODEL}: random weights, {args.layers} layers")
     cfg_dict = dict(SHAPE, num_hidden_layers=args.layers, architectures=["Qwen2ForCausalLM"])
     config = Qwen2Config.from_dict(cfg_dict)
-    max_batch = args.batch if args.no_points else max(args.batch, 64)
+    max_batch = args.batch if args.no_points else max(args.batch, BIG_BATCH)
     t_load = time.perf_counter()
     engine = he.Engine(config=config, seed=0, dtype="bfloat16", max_tokens=max_batch * CONTEXT,
                        max_slots=max_batch, max_seq_len=CONTEXT, tune_library=not args.no_tune)
@@ -98,21 +102,25 @@ def main() -> int:
     load_s = time.perf_counter() - t_load
     rng = np.random.default_rng(0)
 
-    def prompts(n):
-        return [rng.integers(0, SHAPE["vocab_size"], PROMPT).tolist() for _ in range(n)]
+    def prompts(n, lo=PROMPT, hi=PROMPT):
+        return [rng.integers(0, SHAPE["vocab_size"], int(rng.integers(lo, hi + 1))).tolist() for _ in range(n)]
 
     def prefill(ps, slots):
         """Prompts in groups of 8 sequences a step; returns the first sampled tokens."""
         toks = []
-        for g in range(0, len(ps), 8):
-            entries = [StepEntry(s, p, [len(p) - 1]) for s, p in zip(slots[g:g + 8], ps[g:g + 8])]
-            logits = engine.step(entries)
-            toks += sampler.sample(logits, list(range(len(entries))), [0] * len(entries))
+        # prompts of random lengths give row counts that never come again: not worth the tuner's trials
+        tuning = library_tuning.no_new_tuning() if PROMPT_LO != PROMPT_HI else contextlib.nullcontext()
+        with tuning:
+            for g in range(0, len(ps), 8):
+                entries = [StepEntry(s, p, [len(p) - 1]) for s, p in zip(slots[g:g + 8], ps[g:g + 8])]
+                logits = engine.step(entries)
+                toks += sampler.sample(logits, list(range(len(entries))), [0] * len(entries))
         return toks
 
     def decode_run(batch, steps, warmup):
         slots = [engine.acquire() for _ in range(batch)]
-        toks = prefill(prompts(batch), slots)
+        ps = prompts(batch, PROMPT_LO, PROMPT_HI)
+        toks = prefill(ps, slots)
         seqs = list(range(batch))
 
         def run(toks, count):
@@ -137,7 +145,7 @@ def main() -> int:
         toks = many(toks, steps)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        avg_len = PROMPT + warmup + steps / 2
+        avg_len = sum(len(p) for p in ps) / batch + warmup + steps / 2
         for s in slots:
             engine.release(s)
         return dt / steps, avg_len
@@ -167,13 +175,14 @@ def main() -> int:
 
     points = {}
     if not args.no_points:
-        for b in (1, 64):
+        for b in (1, BIG_BATCH):
             progress(f"decode at batch {b}")
             s, _ = decode_run(b, max(8, args.steps // 2), max(3, args.warmup // 2))
             points[f"decode_b{b}"] = round(b / s, 1)
 
+    PROMPTS = PROMPT_LO if PROMPT_LO == PROMPT_HI else f"{PROMPT_LO}-{PROMPT_HI}"
     line = {
-        "metric": f"decode tok/s @ bs {args.batch}, {MODEL} bf16, context {CONTEXT}, prompts {PROMPT}",
+        "metric": f"decode tok/s @ bs {args.batch}, {MODEL} bf16, context {CONTEXT}, prompts {PROMPTS}",
         "value": round(args.batch / step_s, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -191,7 +200,7 @@ def main() -> int:
             "kv_heads": SHAPE["num_key_value_heads"], "head_dim": SHAPE["head_dim"],
             "intermediate_size": SHAPE["intermediate_size"], "vocab_size": SHAPE["vocab_size"],
             "rope_theta": SHAPE["rope_theta"], "rms_norm_eps": SHAPE["rms_norm_eps"],
-            "global_batch": args.batch, "seq_len": CONTEXT, "prompt_len": PROMPT,
+            "global_batch": args.batch, "seq_len": CONTEXT, "prompt_len": PROMPTS,
             "parallelism": "single GPU", "sampling": "greedy, ids read every 8 steps", "load_s": round(load_s, 1),
             "library_gemm_autotuned": not args.no_tune,
         },
