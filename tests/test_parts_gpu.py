@@ -336,6 +336,63 @@ def toys(fw):
                 out += y * (chosen == e)[:, None].to(y.dtype)
             return out
 
+    @parts.register_part("norm", "toy_centered")
+    class Centered(parts.Norm):
+        """y = (x - mean x) / sqrt(var x + eps) * weight: not of the form a pair of products can
+        carry, so every reader gets plain rows from add_norm."""
+
+        def __init__(self, params, prefix, env):
+            super().__init__(prefix, env)
+            self.size = parts.param(params, "size", int)
+            self.eps = parts.param(params, "eps", float)
+
+        def tensor_specs(self):
+            return {self.prefix + "weight": parts.TensorSpec((self.size,), ("gain", 1.0, 0.1))}
+
+        def bind(self, tensors):
+            self.w = tensors[self.prefix + "weight"].float()
+
+        def add_norm(self, resid, delta, rows, ctx, want_out=True):
+            from hector_engine_amd.parts.linear import as_tensor
+            r = resid[:rows]
+            if delta is not None:
+                r += as_tensor(delta, ctx)[:rows].float()
+            if not want_out:
+                return None
+            c = r - r.mean(-1, keepdim=True)
+            out = ctx.alloc((rows, self.size))
+            out.copy_((c * torch.rsqrt((c * c).mean(-1, keepdim=True) + self.eps) * self.w).to(out.dtype))
+            return out
+
+    @parts.register_part("block", "toy_parallel")
+    class Parallel(parts.Block):
+        """x = x + mixer(norm(x)) + feed_forward(norm(x)): one norm, both branches read it."""
+
+        def __init__(self, params, prefix, env):
+            super().__init__(prefix, env)
+            self.norm = parts.build_part("norm", parts.param(params, "norm", parts.PartSpec), prefix + "ln.", env)
+            self.mixer = parts.build_part("mixer", parts.param(params, "mixer", parts.PartSpec), prefix + "mix.", env)
+            self.feed_forward = parts.build_part("feed_forward", parts.param(params, "feed_forward", parts.PartSpec),
+                                                 prefix + "ff.", env)
+
+        def children(self):
+            return [self.norm, self.mixer, self.feed_forward]
+
+        def tensor_specs(self):
+            specs = {}
+            for c in self.children():
+                specs.update(c.tensor_specs())
+            return specs
+
+        def bind(self, tensors):
+            for c in self.children():
+                c.bind(tensors)
+
+        def forward(self, stream, ctx, cache):
+            n = stream.normed(self.norm, ctx)
+            stream.add(self.mixer.forward(n, ctx, cache), ctx)
+            stream.add(self.feed_forward.forward(n, ctx), ctx)
+
     @dataclasses.dataclass
     class ToyConfig(ModelConfig):
         vocab_size: int = 0
@@ -361,8 +418,8 @@ def toys(fw):
             return parts.PartSpec("attention", {"hidden_size": D, "num_heads": 4, "num_kv_heads": 2,
                                                 "head_dim": 16, "qkv_bias": True, "position": pos})
 
-        def block(mixer, feed_forward=ff):
-            return parts.PartSpec("pre_norm", {"mixer_norm": norm, "feed_forward_norm": norm, "mixer": mixer,
+        def block(mixer, feed_forward=ff, mixer_norm=norm):
+            return parts.PartSpec("pre_norm", {"mixer_norm": mixer_norm, "feed_forward_norm": norm, "mixer": mixer,
                                                "feed_forward": feed_forward, "names": names})
 
         rotary = parts.PartSpec("rotary", {"head_dim": 16, "theta": 1e4})
@@ -382,12 +439,20 @@ def toys(fw):
         else:   # "shared": the third run reads the keys and values the second run wrote
             mixers = [attn(rotary), attn(rotary)]
             schedule = [parts.ScheduleEntry(0), parts.ScheduleEntry(1), parts.ScheduleEntry(1, cache_from=1)]
+        layers = [parts.LayerSpec(f"layers.{i}.", block(m, routed if cfg.kind == "routed" and i == 1 else ff))
+                  for i, m in enumerate(mixers)]
+        if cfg.kind == "parallel":   # another norm and another arrangement: a parallel block between pre-norm blocks
+            centered = parts.PartSpec("toy_centered", {"size": D, "eps": 1e-4})
+            layers = [parts.LayerSpec("layers.0.", block(attn(rotary))),
+                      parts.LayerSpec("layers.1.", parts.PartSpec("toy_parallel", {"norm": centered, "mixer": attn(rotary),
+                                                                                   "feed_forward": ff})),
+                      parts.LayerSpec("layers.2.", block(attn(rotary), mixer_norm=centered))]
+            schedule = [parts.ScheduleEntry(0), parts.ScheduleEntry(1), parts.ScheduleEntry(2)]
         return parts.ModelSpec(
             hidden_size=D, vocab_size=V,
             embedding=parts.PartSpec("token_embedding", {"vocab_size": V, "hidden_size": D}),
             embedding_prefix="emb.",
-            layers=[parts.LayerSpec(f"layers.{i}.", block(m, routed if cfg.kind == "routed" and i == 1 else ff))
-                    for i, m in enumerate(mixers)],
+            layers=layers,
             schedule=schedule, final_norm=norm, final_norm_prefix="norm.",
             head=parts.PartSpec("linear_head", {"vocab_size": V, "hidden_size": D}), head_prefix="head.",
             max_positions=512)
@@ -433,6 +498,19 @@ def toy_plain(w, kind, ids):
     rot = lambda t: P.rope(t, pos, 1e4)
     scale = lambda t: t * (1 + pos.double() / 100)[:, None, None]
     same = lambda t: t
+    if kind == "parallel":
+        def centered(h, g):
+            c = h - h.mean(-1, keepdim=True)
+            return c / torch.sqrt((c * c).mean(-1, keepdim=True) + 1e-4) * g
+
+        def mlp(l, n):
+            p = f"layers.{l}.ff."
+            return P.swiglu(n, w[p + "gate_proj.weight"], w[p + "up_proj.weight"], w[p + "down_proj.weight"])
+        x = ff(0, x + attn(0, P.rmsnorm(x, w["layers.0.ln1.weight"], 1e-5), rot)[0])
+        n = centered(x, w["layers.1.ln.weight"])
+        x = x + attn(1, n, rot)[0] + mlp(1, n)
+        x = ff(2, x + attn(2, centered(x, w["layers.2.ln1.weight"]), rot)[0])
+        return P.linear(P.rmsnorm(x, w["norm.weight"], 1e-5), w["head.weight"])
     if kind == "state":
         runs = [(0, rot, None), (1, "mean", None), (2, rot, None)]
     elif kind == "position":
@@ -458,7 +536,7 @@ def toy_plain(w, kind, ids):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("kind", ["state", "position", "twice", "shared"])
+@pytest.mark.parametrize("kind", ["state", "position", "twice", "shared", "parallel"])
 def test_toy_models_build_and_step(fw, toys, tmp_path, kind, dtype):
     import hector_engine_amd as he
     from hector_engine_amd.engine.engine import StepEntry
