@@ -139,6 +139,26 @@ def test_unequal_batches_early_finishers_and_slot_reuse(engines, plain_models, n
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", NAMES)
+def test_a_batch_of_a_hundred_unequal_requests(engines, plain_models, name, dtype):
+    """A hundred requests of 2 to 60 tokens in one batch: as they end, the one-token steps shrink from
+    a hundred rows through every range of rows that has kernels and graphs of its own (above 64,
+    33 to 64, 17 to 32, up to 16), and every request's logits still equal the plain implementation's."""
+    eng = engines(name, dtype, max_slots=100, max_tokens=100 * 64)
+    vocab = plain_models[name][0]["vocab_size"]
+    g = torch.Generator().manual_seed(5)
+    lengths = torch.randint(2, 61, (100,), generator=g).tolist()
+    lengths[7], lengths[50] = 60, 60            # some last to the end
+    requests = [rand_ids(vocab, n, 300 + i) for i, n in enumerate(lengths)]
+    got, used = run_batches(eng, requests, [100])
+    assert sorted(used) == list(range(100))
+    for i, ids in enumerate(requests):
+        close(got[i], plain_logits(plain_models, name, ids), dtype)
+    assert eng.cache.book.slots.available == 100 and eng.cache.free_pages == eng.cache.num_pages
+    eng.cache.book.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
 def test_long_decoding(engines, plain_models, name, dtype):
     """Five prompt tokens, then 250 single-token steps: page boundaries at 64, 128 and 192
     are crossed, and configuration C's window of 70 slides and gives pages back."""
