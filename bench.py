@@ -3,6 +3,7 @@
 token ids) on one MI355X, with prefill and roofline figures on the same line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--shape 7b|32b|72b]
+                    [--context C] [--prompt P]
 
 The default is the 7B shape; --shape runs the same measurement at the layer sizes of
 Qwen2.5-32B (context 8192, prompts of 512 to 2048 tokens, batches 1 / 8 / 64) or
@@ -68,6 +69,9 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0 = all)")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="7b")
+    ap.add_argument("--context", type=int, default=0, help="another context length per sequence than the shape's")
+    ap.add_argument("--prompt", type=int, default=0,
+                    help="another prompt length of the decode batches (the prefill figure stays at 2048 tokens)")
     ap.add_argument("--no-points", action="store_true", help="skip the points at batch 1 and at the large batch")
     ap.add_argument("--no-tune", action="store_true",
                     help="leave the library's default kernels for the tall matrix products")
@@ -76,6 +80,13 @@ def main() -> int:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
     MODEL, CONTEXT, (PROMPT_LO, PROMPT_HI), BIG_BATCH, SHAPE = SHAPES[args.shape]
+    CONTEXT = args.context or CONTEXT
+    if args.prompt:
+        PROMPT_LO = PROMPT_HI = args.prompt
+    if max(PROMPT, PROMPT_HI) + args.warmup + args.steps > CONTEXT:
+        print(f"bench.py: prompts of {max(PROMPT, PROMPT_HI)} tokens and {args.warmup + args.steps} steps do not fit "
+              f"a context of {CONTEXT}")
+        return 2
     FULL_LAYERS = SHAPE["num_hidden_layers"]
     args.layers = args.layers or FULL_LAYERS
 
