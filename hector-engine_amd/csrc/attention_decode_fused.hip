@@ -30,35 +30,52 @@
 // d + half = the same lane's element in k step ks + half/32. sn, c: the sine and cosine of
 // angle `lane` (lanes below half), fetched from the lane that holds them.
 template <int NT>
-__device__ __forceinline__ void load_q_biased(float (&x)[NT / 2][8], const uint16_t* qrow,
-                                              const void* bias, int bias_dtype, int bias_off,
-                                              bool valid, int lg) {
+struct QLoads {
+  uint4 raw[NT / 2], bias[NT / 2];
+  bool vec_bias;
+};
+
+// Issues the loads of q and, where the bias is bf16 and aligned, of its bias (eight values of
+// a k step in one load). No load sits behind a per-lane condition (the caller's head index is
+// clamped, so every lane has an address it may read; a column without a head is zeroed
+// afterwards): loads behind branches are waited for one by one, these go out together and are
+// waited for where q_biased() turns them into values, after everything else has been asked for.
+template <int NT>
+__device__ __forceinline__ void q_issue(QLoads<NT>& q, const uint16_t* qrow, const void* bias,
+                                        int bias_dtype, int bias_off, int lg) {
+  constexpr int KS = NT / 2;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) q.raw[ks] = *reinterpret_cast<const uint4*>(qrow + 32 * ks + 8 * lg);
+  q.vec_bias = bias != nullptr && bias_dtype == HE_BF16 && (((uintptr_t)bias) & 15) == 0;
+  // without such a bias the same loads read q again and their values are dropped: a branch around
+  // them would end in register copies that wait for the loads
+  const uint16_t* b = q.vec_bias ? (const uint16_t*)bias + bias_off : qrow;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) q.bias[ks] = *reinterpret_cast<const uint4*>(b + 32 * ks + 8 * lg);
+}
+
+template <int NT>
+__device__ __forceinline__ void q_biased(float (&x)[NT / 2][8], const QLoads<NT>& q, const void* bias,
+                                         int bias_dtype, int bias_off, bool valid, int lg) {
   constexpr int KS = NT / 2;
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
-    const int d0 = 32 * ks + 8 * lg;
-    uint4 raw = make_uint4(0, 0, 0, 0);
-    if (valid) raw = *reinterpret_cast<const uint4*>(qrow + d0);
-    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+    const uint32_t w[4] = {q.raw[ks].x, q.raw[ks].y, q.raw[ks].z, q.raw[ks].w};
+    const uint32_t keep = q.vec_bias ? 0xffffffffu : 0u;
+    const uint32_t bw[4] = {q.bias[ks].x & keep, q.bias[ks].y & keep, q.bias[ks].z & keep, q.bias[ks].w & keep};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      x[ks][2 * j] = __uint_as_float(w[j] << 16);
-      x[ks][2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+      const float lo = __uint_as_float(w[j] << 16) + __uint_as_float(bw[j] << 16);
+      const float hi = __uint_as_float(w[j] & 0xffff0000u) + __uint_as_float(bw[j] & 0xffff0000u);
+      x[ks][2 * j] = valid ? lo : 0.f;
+      x[ks][2 * j + 1] = valid ? hi : 0.f;
     }
-    if (valid && bias != nullptr) {
-      if (bias_dtype == HE_BF16 && (((uintptr_t)bias) & 15) == 0) {   // the eight values in one load
-        const uint4 b4 = *reinterpret_cast<const uint4*>((const uint16_t*)bias + bias_off + d0);
-        const uint32_t bw[4] = {b4.x, b4.y, b4.z, b4.w};
+  }
+  if (bias != nullptr && !q.vec_bias && valid) {   // a bias in 32-bit, or not aligned: value by value
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          x[ks][2 * j] += __uint_as_float(bw[j] << 16);
-          x[ks][2 * j + 1] += __uint_as_float(bw[j] & 0xffff0000u);
-        }
-      } else {
+    for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) x[ks][j] += load_param(bias, bias_off + d0 + j, bias_dtype);
-      }
-    }
+      for (int j = 0; j < 8; ++j) x[ks][j] += load_param(bias, bias_off + 32 * ks + 8 * lg + j, bias_dtype);
   }
 }
 
@@ -106,8 +123,8 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
   const int h = kvh * G + 16 * ht + min(lr, GT - 1);
   // loads that need nothing but the row: issued first, used last
   const uint16_t* qkv_row = qkv + (int64_t)row * qkv_stride;
-  float qx[NT / 2][8];
-  load_q_biased<NT>(qx, qkv_row + (int64_t)h * HD, bias, bias_dtype, h * HD, h_ok, lg);
+  QLoads<NT> ql;
+  q_issue<NT>(ql, qkv_row + (int64_t)h * HD, bias, bias_dtype, h * HD, lg);
   const float freq = lane < HD / 2 ? inv_freq[lane] : 0.f;
   const int seq = row_seq[row];
   const int Z = gridDim.z, z = blockIdx.z;
@@ -138,10 +155,18 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
   // unless this wavefront writes the new key into that very step
   const bool writes = write_kv && p >= kb_begin && p < kb_end;
   const bool early = has_keys && !(writes && p < kb_begin + 32);
+  // The page-table entries are asked for; what was asked for at the top is turned into values
+  // while they come, so that nothing older than the keys has to be waited for once those are on
+  // their way (behind their conditional loads the compiler waits for everything in flight).
   AttendCursor<NT> cursor;
-  if (early) attend_start<NT>(cursor, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, kb_begin, lr, lg);
+  if (early) attend_pages<NT>(cursor, pt, max_blocks, kb_begin);
+  float qx[NT / 2][8];
+  q_biased<NT>(qx, ql, bias, bias_dtype, h * HD, h_ok, lg);
+  const float angle = (float)p * freq;
+  __builtin_amdgcn_sched_barrier(0);
+  if (early) attend_first<NT>(cursor, kpool, vpool, num_pages, KVH, kvh, kb_begin, lr, lg);
   float sn = 0.f, c = 1.f;                   // lane j < HD / 2: angle j of position p
-  if (has_keys && lane < HD / 2) sincos_angle((float)p * freq, &sn, &c);
+  if (has_keys && lane < HD / 2) sincos_angle(angle, &sn, &c);
 
   // ---- the new key and value go into the cache, written by the wavefront that reads them
   if (writes) {

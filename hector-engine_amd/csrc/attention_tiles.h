@@ -142,24 +142,38 @@ struct AttendCursor {
   KVFrag<NT> cur;
 };
 
-// Starts the walk at key kb_begin (a multiple of 32): reads the page-table entries and issues
-// the loads of the first step. A caller with other work to do (a query to load and rotate)
-// does it between this and attend_walk, while the fragments are on their way.
+// Starts the walk at key kb_begin (a multiple of 32) in two parts, so that a caller can put
+// work between them: attend_pages asks for the page-table entries, attend_first issues the loads
+// of the first step. A caller with other work to do (a query to rotate) does it between
+// attend_first and attend_walk, while the fragments are on their way.
+template <int NT>
+__device__ __forceinline__ void attend_pages(AttendCursor<NT>& c, const int32_t* __restrict__ pt,
+                                             int max_blocks, int kb_begin) {
+  c.block = kb_begin >> HE_PAGE_SHIFT;
+  c.page = pt[c.block];
+  c.page_ahead = pt[min(c.block + 1, max_blocks - 1)];
+}
+
+template <int NT>
+__device__ __forceinline__ void attend_first(AttendCursor<NT>& c, const uint16_t* __restrict__ kpool,
+                                             const uint16_t* __restrict__ vpool, int num_pages, int KVH,
+                                             int kvh, int kb_begin, int lr, int lg) {
+  constexpr int HD = 16 * NT;
+  c.k_stride = (int64_t)KVH * he_k_page_elems(HD);
+  c.v_stride = (int64_t)KVH * he_v_page_elems(HD);
+  c.kp = kpool + (int64_t)kvh * he_k_page_elems(HD);
+  c.vp = vpool + (int64_t)kvh * he_v_page_elems(HD);
+  load_frag<NT>(c.cur, c.kp, c.vp, c.page, num_pages, c.k_stride, c.v_stride, kb_begin & 32, lr, lg);
+}
+
 template <int NT>
 __device__ __forceinline__ void attend_start(AttendCursor<NT>& c, const uint16_t* __restrict__ kpool,
                                              const uint16_t* __restrict__ vpool,
                                              const int32_t* __restrict__ pt, int max_blocks,
                                              int num_pages, int KVH, int kvh, int kb_begin, int lr,
                                              int lg) {
-  constexpr int HD = 16 * NT;
-  c.k_stride = (int64_t)KVH * he_k_page_elems(HD);
-  c.v_stride = (int64_t)KVH * he_v_page_elems(HD);
-  c.kp = kpool + (int64_t)kvh * he_k_page_elems(HD);
-  c.vp = vpool + (int64_t)kvh * he_v_page_elems(HD);
-  c.block = kb_begin >> HE_PAGE_SHIFT;
-  c.page = pt[c.block];
-  c.page_ahead = pt[min(c.block + 1, max_blocks - 1)];
-  load_frag<NT>(c.cur, c.kp, c.vp, c.page, num_pages, c.k_stride, c.v_stride, kb_begin & 32, lr, lg);
+  attend_pages<NT>(c, pt, max_blocks, kb_begin);
+  attend_first<NT>(c, kpool, vpool, num_pages, KVH, kvh, kb_begin, lr, lg);
 }
 
 // Runs the keys [kb_begin, kb_end) (multiples of 32) of one (sequence, kv head) against the
