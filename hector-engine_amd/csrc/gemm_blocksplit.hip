@@ -259,23 +259,29 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
 
   // Loads the epilogue needs are issued here, ahead of the weight stream, so that their
   // latency is not added at the end: the partial sums of squares of the input rows
-  // (wavefront w takes the rows w and w + nw; lanes hold strided partials) and, for the
+  // (wavefront w takes the rows w, w + nw, ... up to four; lanes hold strided partials) and, for the
   // residual epilogue (a little further down, behind the first weight loads), the residual
   // values and gains of this thread's first outputs.
   constexpr int OUT_TILES = R * MT;
   const int out_align = ((N | n0) & 3) == 0 ? 4 : (((N | n0) & 1) == 0 ? 2 : 1);
   const bool scaled = fu.scale_partials != nullptr;
   const bool to_resid = !GATED && fu.resid != nullptr;
-  const bool scale_early = scaled && fu.scale_count <= 256 && M <= 2 * nw;
-  float pv[2][4];
+  constexpr int SCALE_ROWS = 4;           // rows a wavefront takes: 16 rows with 4 wavefronts
+  const bool scale_early = scaled && fu.scale_count <= 256 && M <= SCALE_ROWS * nw;
+  float pv[SCALE_ROWS][4];
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);   // in a scalar register: rows beyond M cost a scalar branch
   if (scale_early) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int m = wave + j * nw;
+    for (int j = 0; j < SCALE_ROWS; ++j) {
+      const int m = wave_s + j * nw;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int i = lane + 64 * q;
-        pv[j][q] = (m < M && i < fu.scale_count) ? fu.scale_partials[(int64_t)m * fu.scale_count + i] : 0.f;
+      for (int q = 0; q < 4; ++q) pv[j][q] = 0.f;
+      if (m < M) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int i = lane + 64 * q;
+          if (i < fu.scale_count) pv[j][q] = fu.scale_partials[(int64_t)m * fu.scale_count + i];
+        }
       }
     }
   }
@@ -325,8 +331,8 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
   if (scaled) {
     if (scale_early) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int m = wave + j * nw;
+      for (int j = 0; j < SCALE_ROWS; ++j) {
+        const int m = wave_s + j * nw;
         if (m < M) {
           const float total = wave_sum(((pv[j][0] + pv[j][1]) + pv[j][2]) + pv[j][3]);
           if (lane == 0) row_scale[m] = 1.0f / sqrtf(total / (float)fu.scale_dim + fu.scale_eps);
