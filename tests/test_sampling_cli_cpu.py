@@ -59,3 +59,38 @@ def test_cli_argument_rules():
     assert (model, ns.ctx, temp) == ("m", 512, 0.7)
     assert parse_prompts("5,17,3;9 2") == [[5, 17, 3], [9, 2]]
     assert parse_prompts("raw:1,2") == [[1, 2]]
+
+
+def test_bench_refuses_more_than_one_gpu_and_what_does_not_fit():
+    """bench.py keeps its contract at one GPU: any other count is one line and exit status 2
+    (before anything touches a GPU), and so is a prompt that does not fit the context."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for args, needle in ((["--gpus", "2"], "one GPU"), (["--prompt", "9000"], "do not fit")):
+        r = subprocess.run([sys.executable, os.path.join(root, "bench.py")] + args, capture_output=True, text=True,
+                           timeout=120)
+        assert r.returncode == 2, r.stderr
+        assert needle in r.stdout and len(r.stdout.strip().splitlines()) == 1
+
+
+def test_bench_byte_and_flop_counts():
+    """The roofline's figures for the benchmark shape: 7.6 billion parameters' worth of bytes a step
+    and the prompt's flops (products and causal attention), as counted by hand."""
+    import importlib.util
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("bench_module", os.path.join(root, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    shape = bench.SHAPES["7b"][-1]
+    D, I, V, L = 3584, 18944, 152064, 28
+    per_layer = D * 4608 + 4608 + 3584 * D + 3 * D * I + 2 * D
+    assert bench.weight_bytes(shape, L) == 2 * (L * per_layer + D + V * D)
+    assert 14.1e9 < bench.weight_bytes(shape, L) < 14.3e9
+    assert bench.kv_bytes_per_token(shape, L) == 57344
+    T = 2048
+    flops = bench.prefill_flops(shape, L, T)
+    assert flops == L * (2 * T * (D * 4608 + 3584 * D + 3 * D * I) + 4 * 28 * 128 * T * (T + 1) // 2) + 2 * D * V
+    assert 27.4e12 < flops < 27.7e12
