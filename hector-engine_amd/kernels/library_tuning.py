@@ -7,7 +7,8 @@ Qwen2.5-7B shapes its tuner finds kernels 17-27 % faster for the 2048-row down a
 gate||up products and 20 % faster for gate||up at 64 rows. Tuning runs the first time a
 shape (rows, N, K) is seen and takes a second or so per shape, so it is meant for
 workloads whose shapes repeat (decode buckets, fixed prompt chunks); it is off unless
-asked for. Results are kept in a file and read again by the next process.
+asked for. Results are kept in a file and read again by the next process. Row counts that
+are unlikely to come again (a prompt of 1,937 tokens) are not tuned: worth_tuning().
 """
 from __future__ import annotations
 
@@ -41,6 +42,13 @@ def enabled() -> bool:
     return _enabled
 
 
+def worth_tuning(rows: int) -> bool:
+    """Whether a product of this many rows is tuned when first seen: the row counts of one-token
+    steps (up to 64) and multiples of 256 (fixed prompt chunks). Any other count runs with the
+    library's default kernel, or with a tuned one if that exact shape was tuned before."""
+    return rows <= 64 or rows % 256 == 0
+
+
 @contextlib.contextmanager
 def no_new_tuning():
     """Inside: tuned choices are used, but no shape is tuned (graph capture cannot hold the
@@ -49,8 +57,9 @@ def no_new_tuning():
         yield
         return
     t = torch.cuda.tunable
+    before = t.tuning_is_enabled()     # one such block may stand inside another
     t.tuning_enable(False)
     try:
         yield
     finally:
-        t.tuning_enable(True)
+        t.tuning_enable(before)

@@ -160,6 +160,13 @@ class Linear:
             return self._skinny(x, bias, rows, ctx, out, out_dtype, allow_split)
         if out is None:
             out = ctx.alloc((rows, N), out_dtype)
+        if library_tuning.enabled() and not library_tuning.worth_tuning(rows):
+            with library_tuning.no_new_tuning():
+                return self._library(x, bias, rows, out, out_dtype, library_f32, ctx)
+        return self._library(x, bias, rows, out, out_dtype, library_f32, ctx)
+
+    def _library(self, x, bias, rows, out, out_dtype, library_f32, ctx):
+        w = self.weight
         if library_f32:
             torch.mm(x[:rows], w.t(), out_dtype=torch.float32, out=out[:rows])
             return out
