@@ -158,6 +158,56 @@ def test_a_batch_of_a_hundred_unequal_requests(engines, plain_models, name, dtyp
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_random_traffic(engines, plain_models, dtype):
+    """Sixty batches of random sizes (1 to 24 requests), random lengths and random cuts (a prompt whole or in
+    two chunks, then token by token, shorter requests leaving early), over all configurations: every checked
+    request equals the plain implementation, and in 32-bit it equals, bit for bit, the request run alone."""
+    import random
+    rng = random.Random(11)
+    for round_ in range(60):
+        name = rng.choice(NAMES)
+        eng = engines(name, dtype, max_slots=24, max_tokens=24 * 256, max_seq_len=256)
+        cfg = plain_models[name][0]
+        longest = min(cfg.get("max_position_embeddings", 256), 250) - 1
+        reqs = [[rng.randrange(cfg["vocab_size"]) for _ in range(rng.randint(1, rng.choice([8, 40, longest])))]
+                for _ in range(rng.randint(1, 24))]
+        slots = {i: eng.acquire() for i in range(len(reqs))}
+        fed = {i: rng.randint(1, len(r)) for i, r in enumerate(reqs)}
+        got = {i: [] for i in slots}
+        first = {i: max(1, fed[i] // 2) if rng.random() < 0.3 else fed[i] for i in slots}
+        for lo, hi in ((lambda i: 0, first.get), (first.get, fed.get)):        # the prompts, some in two chunks
+            part = [i for i in slots if hi(i) > lo(i)]
+            if not part:
+                continue
+            logits = eng.step([entry(slots[i], reqs[i][lo(i):hi(i)], range(hi(i) - lo(i))) for i in part])
+            r = 0
+            for i in part:
+                got[i].append(logits[r:r + hi(i) - lo(i)].clone())
+                r += hi(i) - lo(i)
+        live = list(slots)
+        while True:
+            for i in list(live):
+                if fed[i] == len(reqs[i]):
+                    eng.release(slots.pop(i))
+                    live.remove(i)
+            if not live:
+                break
+            logits = eng.step([entry(slots[i], [reqs[i][fed[i]]], [0]) for i in live])
+            for r, i in enumerate(live):
+                got[i].append(logits[r:r + 1].clone())
+                fed[i] += 1
+        assert eng.cache.free_pages == eng.cache.num_pages
+        for i in rng.sample(range(len(reqs)), min(len(reqs), 3)):
+            whole = torch.cat(got[i])
+            close(whole, plain_logits(plain_models, name, reqs[i]), dtype)
+            if dtype == "float32":
+                s = eng.acquire()
+                alone = eng.step([entry(s, reqs[i], range(len(reqs[i])))]).clone()
+                eng.release(s)
+                assert torch.equal(alone, whole), (round_, name, i)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", NAMES)
 def test_long_decoding(engines, plain_models, name, dtype):
     """Five prompt tokens, then 250 single-token steps: page boundaries at 64, 128 and 192
