@@ -819,6 +819,104 @@ def test_attention_far_key_stands_out(ops):
         assert torch.allclose(got.reshape(H, hd)[0], v[far, 0].double(), atol=0.05), kind
 
 
+# ------------------------------------------------------------------ random sizes
+def test_gemm_blocksplit_at_random_sizes(ops):
+    """300 products of random sizes (1 to 32 rows, any N up to 6000, K in steps of 8 up to 20000), plain and gated,
+    with and without bias, bf16 and fp32 results, row-major and piece-major, against double precision."""
+    import random
+    rng = random.Random(5)
+    for case in range(300):
+        M = rng.randint(1, 32)
+        K = 8 * rng.randint(1, rng.choice([40, 300, 2500]))
+        N = rng.randint(1, rng.choice([64, 700, 6000]))
+        gated = rng.random() < 0.3 and M <= 16
+        if gated:
+            N = 2 * max(1, N // 2)
+        x = rnd(M, K, seed=case).to(torch.bfloat16)
+        w = rnd(N, K, seed=case + 1, scale=0.05).to(torch.bfloat16)
+        bias = None
+        if rng.random() < 0.5 and not gated:
+            bias = rnd(N, seed=case + 2).to(rng.choice([torch.bfloat16, torch.float32]))
+        od = torch.bfloat16 if gated else rng.choice([torch.bfloat16, torch.float32])
+        NO = N // 2 if gated else N
+        xin = rng.random() < 0.5 and M <= 16
+        op = rng.random() < 0.5 and M <= 16 and od == torch.bfloat16 and NO % 8 == 0
+        out = torch.full(ops.pieces_shape(M, NO) if op else (M, NO), 7.0, dtype=od, device="cuda")
+        xd = dev(x)
+        ops.gemm_blocksplit(out, to_pieces(xd) if xin else xd, dev(w), dev(bias) if bias is not None else None, M,
+                            gated=gated, x_pieces=xin, out_pieces=op)
+        got = (from_pieces(out) if op else out).cpu().double()
+        if gated:
+            ref = P.silu(x.double() @ w[0::2].double().T) * (x.double() @ w[1::2].double().T)
+        else:
+            ref = x.double() @ w.double().T + (bias.double() if bias is not None else 0)
+        tol = (2 ** -7 if od == torch.bfloat16 else 1e-4) * max(ref.abs().max().item(), 1e-3) * (2 if gated else 1) + 1e-6
+        err = (got - ref).abs().max().item()
+        assert err <= tol, (case, M, N, K, gated, od, xin, op, err, tol)
+
+
+def test_attention_kernels_at_random_sizes(ops):
+    """400 cases of random head counts, groups, head sizes (16 to 256 in steps of 16), windows, lengths and
+    new-token counts through the prompt kernels, the split one-token kernel and the plain kernel."""
+    import random
+    rng = random.Random(9)
+    for case in range(400):
+        hd, KVH = 16 * rng.randint(1, 16), rng.randint(1, 4)
+        H = KVH * rng.randint(1, 8)
+        window = rng.choice([0, 0, 3, 70, 300])
+        kind = rng.choice(["prefill", "prefill", "decode", "plain"])
+        lengths = [rng.randint(1, rng.choice([5, 80, 400])) for _ in range(rng.randint(1, 5))]
+        q_lens = [1 if kind == "decode" else rng.randint(1, n) for n in lengths]
+        tiles = 0 if kind != "prefill" else (rng.choice([0, 1, 2]) if hd <= 128 else rng.choice([0, 1]))
+        dtype = torch.bfloat16 if kind != "plain" else rng.choice([torch.float32, torch.bfloat16])
+        got, want = attention_case(ops, kind, dtype, H, KVH, hd, window, lengths, q_lens, case, tiles=tiles)
+        tol = 2 ** -6 if dtype == torch.bfloat16 else 1e-5
+        for g, w in zip(got, want):
+            assert torch.allclose(g, w, rtol=tol, atol=tol), (case, kind, dtype, H, KVH, hd, window, lengths, q_lens, tiles)
+
+
+def test_attention_decode_fused_at_random_sizes(ops):
+    """150 cases of the one-launch one-token attention: 1 to 40 sequences of 1 to 1500 keys, 1 to 5 kv heads with
+    groups of 1 to 9, head size 64 or 128, windows, with and without the cache write."""
+    import random
+    rng = random.Random(7)
+    theta = 10000.0
+    for case in range(150):
+        hd, KVH = rng.choice([64, 128]), rng.randint(1, 5)
+        H = KVH * rng.randint(1, 9)
+        B, window, write_kv = rng.randint(1, 40), rng.choice([0, 0, 5, 70, 300]), rng.random() < 0.7
+        lengths = [rng.randint(1, rng.choice([3, 70, 400, 1500])) for _ in range(B)]
+        slots, table, kpool, vpool = paged_setup(lengths, KVH, hd, torch.bfloat16, case)
+        old = [n if not write_kv else n - 1 for n in lengths]
+        ks = [rnd(n, KVH, hd, seed=7 * case + i).to(torch.bfloat16) for i, n in enumerate(old)]
+        vs = [rnd(n, KVH, hd, seed=7 * case + 500 + i).to(torch.bfloat16) for i, n in enumerate(old)]
+        fill_cache(table, slots, kpool, vpool, ks, vs)
+        width = (H + 2 * KVH) * hd if write_kv else H * hd
+        qkv = rnd(B, width, seed=case + 3, scale=1.5).to(torch.bfloat16)
+        bias = rnd(width, seed=case + 4).to(torch.bfloat16)
+        floats = ops.attention_decode_fused_workspace_floats(B, H, KVH, hd, 4096)
+        ws = torch.empty(floats, device="cuda") if floats else None
+        out = torch.full((B, H * hd), 7.0, dtype=torch.bfloat16, device="cuda")
+        pos = torch.tensor([n - 1 for n in lengths], dtype=torch.int32)
+        ops.attention_decode_fused(out, dev(qkv), dev(bias), dev(kpool), dev(vpool), dev(pos),
+                                   dev(torch.arange(B, dtype=torch.int32)), dev(torch.tensor(slots, dtype=torch.int32)),
+                                   dev(table), dev(P.rope_inv_freq(hd, theta)), hd, B, H, KVH, hd, window,
+                                   1.0 / math.sqrt(hd), 4096, write_kv, ws)
+        got = out.cpu().double()
+        x = qkv.double() + bias.double()
+        for s in rng.sample(range(B), min(B, 3)):
+            n = lengths[s]
+            p = torch.tensor([n - 1])
+            q = P.rope(x[s, :H * hd].reshape(1, H, hd), p, theta, hd).to(torch.bfloat16).double()
+            k_all, v_all = ks[s].double(), vs[s].double()
+            if write_kv:
+                k_new = P.rope(x[s, H * hd:(H + KVH) * hd].reshape(1, KVH, hd), p, theta, hd).to(torch.bfloat16)
+                v_new = x[s, (H + KVH) * hd:].reshape(1, KVH, hd).to(torch.bfloat16)
+                k_all, v_all = torch.cat([k_all, k_new.double()]), torch.cat([v_all, v_new.double()])
+            want = P.attention(q, k_all, v_all, p, torch.arange(n), window).reshape(-1)
+            assert torch.allclose(got[s], want, rtol=2 ** -6, atol=2 ** -6), (case, H, KVH, hd, B, window, write_kv, n)
+
+
 # ------------------------------------------------------------------ sampling
 def test_argmax_lowest_index_on_ties(ops):
     V = 1000
