@@ -179,7 +179,9 @@ __device__ __forceinline__ float key_to_float(uint32_t k) {
   const uint32_t b = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
   return __uint_as_float(b);
 }
-__device__ __forceinline__ float clean(float x) { return x != x ? -INFINITY : x; }
+// NaN counts as -inf; -0.0 becomes +0.0, which it equals: as keys the two would differ, and equal
+// values are ordered by index alone.
+__device__ __forceinline__ float clean(float x) { return x != x ? -INFINITY : (x == 0.f ? 0.f : x); }
 __device__ __forceinline__ u64 fixed_mass(float x, float m, float inv_temp) {
   const float w = expf((x - m) * inv_temp);
   return (u64)(w * SAMP_FIXED_ONE);

@@ -985,6 +985,20 @@ def test_sample_rows_equals_plain(ops, V, temperature, top_k, top_p):
         assert got == [P.argmax_lowest(r) for r in x]
 
 
+def test_sample_rows_takes_both_zeros_as_equal(ops):
+    """+0.0 and -0.0 are equal values: among them the index alone decides, as in the plain implementation
+    (as sort keys the two differ)."""
+    V = 4096
+    g = torch.Generator().manual_seed(3)
+    x = torch.where(torch.rand(2, V, generator=g) < 0.5, torch.tensor(0.0), torch.tensor(-0.0))
+    x[1, 100:200] = -1.0
+    us = [3359715596, 1234567]
+    out = torch.empty(2, dtype=torch.int32, device="cuda")
+    for temperature, top_k, top_p in ((0.8, 0, 0.1), (1.0, 50, 1.0), (0.7, 0, 1.0)):
+        ops.sample_rows(out, dev(x), 2, dev(torch.tensor(us, dtype=torch.int64).to(torch.uint32)), temperature, top_k, top_p)
+        assert out.tolist() == [P.sample(x[r], temperature, top_k, top_p, us[r]) for r in range(2)]
+
+
 @pytest.mark.parametrize("case", ["top_k beyond the list", "all equal", "ties at the threshold", "two values",
                                   "deep nucleus"])
 def test_sample_rows_list_and_whole_row_agree(ops, case):
