@@ -72,6 +72,43 @@ def test_sampled_generation_equals_plain(he, model_dirs, plain_models, name, kw)
     assert [r.tokens for r in again] == [r.tokens for r in got]
 
 
+def test_random_generations(he, model_dirs, plain_models):
+    """Sixty generations with random prompts, budgets, sampling options (greedy, temperature, top-k, top-p,
+    penalties with short and long windows), stop tokens, runs of queued steps and fewer slots than prompts:
+    the tokens of the plain implementation, request by request."""
+    import random
+    rng = random.Random(2)
+    engines = {}
+    for _ in range(60):
+        name = rng.choice(list(TINY))
+        cfg, w = plain_models[name]
+        slots = rng.choice([1, 2, 3, 8])
+        if (name, slots) not in engines:
+            engines[(name, slots)] = he.Engine(model_dirs[name], dtype="float32", max_tokens=8 * 128, max_slots=slots,
+                                               max_seq_len=128)
+        eng = engines[(name, slots)]
+        prompts = [[rng.randrange(cfg["vocab_size"]) for _ in range(rng.randint(1, 40))] for _ in range(rng.randint(1, 6))]
+        steps = rng.randint(1, 24)
+        T, top_k = rng.choice([0.0, 0.0, 0.5, 0.8, 1.0, 1.5]), rng.choice([0, 0, 1, 5, 40])
+        top_p, seed = rng.choice([1.0, 1.0, 0.9, 0.5]), rng.randint(0, 1000)
+        rep, freq, pres, win = 1.0, 0.0, 0.0, 384
+        if rng.random() < 0.3:
+            rep, freq, pres, win = rng.choice([1.0, 1.2]), rng.choice([0.0, 0.1]), rng.choice([0.0, 0.1]), rng.choice([4, 384])
+        stop = set()
+        if rng.random() < 0.4:
+            free = P.generate(cfg, w, prompts[0], steps, T, top_k, top_p, seed, 0, (), rep, freq, pres, win)
+            if free:
+                stop = {free[rng.randrange(len(free))]}
+        sampling = he.SamplingConfig(temperature=T, top_k=top_k, top_p=top_p, seed=seed, repetition_penalty=rep,
+                                     frequency_penalty=freq, presence_penalty=pres, penalty_window=win)
+        got = he.generate(eng, prompts, max_new_tokens=steps, sampling=sampling, stop_ids=sorted(stop),
+                          run_of_steps=rng.choice([1, 2, 8, 32]))
+        for i, (p, r) in enumerate(zip(prompts, got)):
+            want = P.generate(cfg, w, p, steps, T, top_k, top_p, seed, i, stop, rep, freq, pres, win)
+            assert r.tokens == want, (name, i, T, top_k, top_p, seed, (rep, freq, pres, win), stop)
+        assert eng.cache.free_pages == eng.cache.num_pages
+
+
 def test_stop_tokens_and_early_finishers(he, model_dirs, plain_models):
     cfg, w = plain_models["B"]
     prompts = prompts_for(cfg, [3, 7, 17, 30], 300)
