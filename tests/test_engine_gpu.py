@@ -157,6 +157,58 @@ def test_a_batch_of_a_hundred_unequal_requests(engines, plain_models, name, dtyp
     eng.cache.book.check_invariants()
 
 
+def test_random_configurations(tmp_path):
+    """Forty random configurations of the architecture (head sizes 16 to 256, any head and group counts, widths
+    and vocabularies of any size, 1 to 3 layers, tied or not, windows from any layer on): model folders with
+    random weights, prompts of unequal lengths in one step and then token by token, in 32-bit and in bfloat16,
+    against the plain implementation."""
+    import random
+    import hector_engine_amd as he
+    from hector_engine_amd.registry import config_from_dict
+    rng = random.Random(6)
+    for case in range(40):
+        hd, KVH = rng.choice([16, 32, 48, 64, 64, 80, 96, 128, 128, 256]), rng.randint(1, 4)
+        H, L = KVH * rng.randint(1, 7), rng.randint(1, 3)
+        cfg = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": L,
+               "hidden_size": rng.choice([8 * rng.randint(2, 40), rng.randint(16, 300)]), "num_attention_heads": H,
+               "num_key_value_heads": KVH, "head_dim": hd,
+               "intermediate_size": rng.choice([8 * rng.randint(1, 60), rng.randint(8, 400)]),
+               "vocab_size": rng.randint(20, 700), "rope_theta": rng.choice([1e4, 1e6, 5e4]),
+               "rms_norm_eps": rng.choice([1e-6, 1e-5, 3e-6]), "max_position_embeddings": 512,
+               "tie_word_embeddings": rng.random() < 0.5, "use_sliding_window": rng.random() < 0.5, "hidden_act": "silu"}
+        if cfg["use_sliding_window"]:
+            cfg.update(sliding_window=rng.choice([1, 3, 8, 70, 200]), max_window_layers=rng.randint(0, L))
+        folder = str(tmp_path / f"c{case}")
+        he.write_random_model(config_from_dict(dict(cfg)), case, folder, "bfloat16")
+        pc, w = P.read_model(folder)
+        reqs = [[rng.randrange(cfg["vocab_size"]) for _ in range(rng.randint(2, rng.choice([6, 40, 150])))]
+                for _ in range(rng.randint(1, rng.choice([3, 20])))]
+        want = [P.forward(pc, w, r) for r in reqs]
+        for dtype in DTYPES:
+            eng = he.Engine(folder, dtype=dtype, max_tokens=64 * 24 * 3, max_slots=24, max_seq_len=192)
+            slots = [eng.acquire() for _ in reqs]
+            fed = [rng.randint(1, len(r)) for r in reqs]
+            logits = eng.step([entry(s, r[:f], range(f)) for s, r, f in zip(slots, reqs, fed)])
+            got, r0 = [], 0
+            for f in fed:
+                got.append([logits[r0:r0 + f].clone()])
+                r0 += f
+            live = list(range(len(reqs)))
+            while True:
+                live = [i for i in live if fed[i] < len(reqs[i])]
+                if not live:
+                    break
+                logits = eng.step([entry(slots[i], [reqs[i][fed[i]]], [0]) for i in live])
+                for j, i in enumerate(live):
+                    got[i].append(logits[j:j + 1].clone())
+                    fed[i] += 1
+            for i in range(len(reqs)):
+                try:
+                    close(torch.cat(got[i]), want[i], dtype)
+                except AssertionError as e:
+                    raise AssertionError(f"{dtype} {cfg}: {e}") from None
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_random_traffic(engines, plain_models, dtype):
     """Sixty batches of random sizes (1 to 24 requests), random lengths and random cuts (a prompt whole or in
