@@ -25,11 +25,11 @@ def engines():
     cfg = config_from_dict(dict(SHAPE))
     made = {}
 
-    def get(dtype):
-        if dtype not in made:
-            made[dtype] = he.Engine(config=cfg, seed=3, dtype=dtype, max_tokens=4096, max_slots=8,
-                                    max_seq_len=1024)
-        return made[dtype]
+    def get(dtype, slots=8):
+        if (dtype, slots) not in made:
+            made[(dtype, slots)] = he.Engine(config=cfg, seed=3, dtype=dtype, max_tokens=max(4096, 128 * slots),
+                                             max_slots=slots, max_seq_len=1024)
+        return made[(dtype, slots)]
 
     return get
 
@@ -103,3 +103,21 @@ def test_queued_steps_at_seven_b_layer_sizes(engines):
         assert [r.tokens for r in one] == [r.tokens for r in many]
         assert all(len(r.tokens) == 27 for r in many)
     assert eng.cache.free_pages == eng.cache.num_pages
+
+
+def test_larger_batches_at_seven_b_layer_sizes(engines):
+    """Sixty-six requests of unequal lengths: as they end, the one-token steps run at 66 rows and then at every
+    row range that has kernels of its own (the library's products above 16 rows, the wavefront kernel, the
+    block-split kernel below), at the benchmark's layer sizes, against the 32-bit path."""
+    reqs = [rand_ids(152064, 4 + (i * 7) % 23, 900 + i) for i in range(66)]
+    first = [max(1, len(r) - 3 - i % 9) for i, r in enumerate(reqs)]
+    ref = run(engines("float32", 66), reqs, first)
+    got = run(engines("bfloat16", 66), reqs, first)
+    for r, g in zip(ref, got):
+        r, g = r.double(), g.double()
+        scale = r.abs().max().item()
+        assert (g - r).abs().max().item() < 0.03 * scale
+        assert ((g - r) ** 2).mean().sqrt().item() < 0.005 * scale
+        t2 = r.topk(2, -1).values
+        clear = (t2[:, 0] - t2[:, 1]) > 0.03 * scale
+        assert torch.equal(g.argmax(-1)[clear], r.argmax(-1)[clear])
