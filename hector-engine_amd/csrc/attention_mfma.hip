@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   const int hi = q_ok ? pos : -1;
   const int lo = (window > 0 && q_ok) ? max(0, pos + 1 - window) : 0;
   bf16x8 qf[KS];
-  load_q<NT>(qf, q + ((int64_t)(row0 + min(qi, q_len - 1)) * H + h) * HD, q_ok, lg);
+  load_q<NT>(qf, q + ((int64_t)(row0 + max(0, min(qi, q_len - 1))) * H + h) * HD, q_ok, lg);
 
   AttnState<NT> st;
 #pragma unroll
@@ -177,17 +177,17 @@ __device__ __forceinline__ void pf2_fetch(pf2_vec (&kreg)[Pf2<NT>::K_TURNS],
                                           const uint16_t* __restrict__ vp, int page, int num_pages,
                                           int64_t k_stride, int64_t v_stride) {
   if (page < 0 || page >= num_pages) page = 0;   // never for an admitted batch
+  // no branch around a load (a thread beyond the page's pieces reads the last one, and
+  // pf2_stage leaves it out): the loads of a page go out together
 #pragma unroll
   for (int j = 0; j < Pf2<NT>::K_TURNS; ++j) {
-    const int c = threadIdx.x + Pf2<NT>::THREADS * j;
-    if (c < Pf2<NT>::K_PIECES)
-      kreg[j] = *reinterpret_cast<const pf2_vec*>(kp + (int64_t)page * k_stride + 8 * c);
+    const int c = min((int)threadIdx.x + Pf2<NT>::THREADS * j, Pf2<NT>::K_PIECES - 1);
+    kreg[j] = *reinterpret_cast<const pf2_vec*>(kp + (int64_t)page * k_stride + 8 * c);
   }
 #pragma unroll
   for (int j = 0; j < Pf2<NT>::V_TURNS; ++j) {
-    const int c = threadIdx.x + Pf2<NT>::THREADS * j;
-    if (c < Pf2<NT>::V_PIECES)
-      vreg[j] = *reinterpret_cast<const pf2_vec*>(vp + (int64_t)page * v_stride + 8 * c);
+    const int c = min((int)threadIdx.x + Pf2<NT>::THREADS * j, Pf2<NT>::V_PIECES - 1);
+    vreg[j] = *reinterpret_cast<const pf2_vec*>(vp + (int64_t)page * v_stride + 8 * c);
   }
 }
 
@@ -233,7 +233,7 @@ struct PairTile {
     const int pos = start + qi;
     hi = ok ? pos : -1;
     lo = (window > 0 && ok) ? max(0, pos + 1 - window) : 0;
-    load_q<NT>(qf, q + ((int64_t)(row0 + min(qi, q_len - 1)) * H + h) * HD, ok, lg);
+    load_q<NT>(qf, q + ((int64_t)(row0 + max(0, min(qi, q_len - 1))) * H + h) * HD, ok, lg);
 #pragma unroll
     for (int dt = 0; dt < NT; ++dt) st.o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
     st.m = -INFINITY;

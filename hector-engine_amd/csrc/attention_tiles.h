@@ -224,6 +224,13 @@ __device__ __forceinline__ void load_q(bf16x8* qf, const uint16_t* qrow, bool va
   constexpr int HD = 16 * NT;
   constexpr int KS = (HD + 31) / 32;
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) qf[ks] = ld8(qrow + 32 * ks + 8 * lg, valid && 32 * ks + 8 * lg < HD);
+  for (int ks = 0; ks < KS; ++ks) {
+    // no branch around the load (qrow is a row that may be read, whether or not the lane's query
+    // or head counts; a piece beyond the head reads the head's start): the loads of a tile go
+    // out together, and what does not count becomes zero
+    const int d = 32 * ks + 8 * lg;
+    const uint4 v = *reinterpret_cast<const uint4*>(qrow + (d < HD ? d : 0));
+    qf[ks] = __builtin_bit_cast(bf16x8, (valid && d < HD) ? v : make_uint4(0, 0, 0, 0));
+  }
 }
 
