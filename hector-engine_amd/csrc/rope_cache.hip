@@ -228,11 +228,19 @@ __global__ __launch_bounds__(1024) void qkv_rope_cache_vec_kernel(
     return im;
   };
   const uint4 zero = make_uint4(0, 0, 0, 0);
+  // four loads with no branch around them, so that they go out together: an item without a
+  // partner, or a row without a bias, reads its own eight elements again and drops them
   auto load = [&](const Item& im, uint4 (&raw)[4]) {
-    raw[0] = *reinterpret_cast<const uint4*>(im.in + im.j);
-    raw[1] = im.rotated ? *reinterpret_cast<const uint4*>(im.in + im.j + half) : zero;
-    raw[2] = im.bias ? *reinterpret_cast<const uint4*>(im.bias + im.j) : zero;
-    raw[3] = im.bias && im.rotated ? *reinterpret_cast<const uint4*>(im.bias + im.j + half) : zero;
+    const int partner = im.rotated ? im.j + half : im.j;
+    const uint16_t* b = im.bias ? im.bias : im.in;
+    const uint4 x0 = *reinterpret_cast<const uint4*>(im.in + im.j);
+    const uint4 x1 = *reinterpret_cast<const uint4*>(im.in + partner);
+    const uint4 b0 = *reinterpret_cast<const uint4*>(b + im.j);
+    const uint4 b1 = *reinterpret_cast<const uint4*>(b + partner);
+    raw[0] = x0;
+    raw[1] = im.rotated ? x1 : zero;
+    raw[2] = im.bias ? b0 : zero;
+    raw[3] = im.bias && im.rotated ? b1 : zero;
   };
   // the loads of a thread's first item are on their way while the angles are computed
   Item first;
