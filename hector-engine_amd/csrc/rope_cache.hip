@@ -142,7 +142,7 @@ __device__ __forceinline__ uint4 pack8(const float* f) {
   return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
-// grid: one workgroup per row for q and k (blockIdx.x < rows), then one per 8 rows for v.
+// grid: one workgroup per 8 rows for v, then one per row for q and k.
 // V lies transposed in a page (8 keys of one dim are 16 contiguous bytes), so the v values of
 // a run of tokens that share such a group are gathered dim by dim and stored together: 16
 // bytes a store when the run is a whole group (a prompt), 2 bytes a token otherwise.
@@ -156,9 +156,10 @@ __global__ __launch_bounds__(1024) void qkv_rope_cache_vec_kernel(
     int num_pages, const float* __restrict__ inv_freq, int rotary_dim, int rows, int H, int KVH,
     int hd) {
   __shared__ float cs[2][ROPE_MAX_HALF];
-  if ((int)blockIdx.x >= rows) {
+  const int v_blocks = (int)gridDim.x - rows;   // they come first: theirs is the longest chain of dependent loads
+  if ((int)blockIdx.x < v_blocks) {
     // ---- v: the runs of tokens that begin in rows [r0, r0 + 8)
-    const int r0 = 8 * ((int)blockIdx.x - rows);
+    const int r0 = 8 * (int)blockIdx.x;
     const int NT = he_v_tiles(hd);
     for (int r = r0; r < min(r0 + 8, rows); ++r) {
       const int seq = row_seq[r];
@@ -175,13 +176,14 @@ __global__ __launch_bounds__(1024) void qkv_rope_cache_vec_kernel(
         const int h = e / hd, d = e - h * hd;
         const float b = v_bias ? bf16_bits_to_float(v_bias[e]) : 0.f;
         uint16_t vals[8];
+        // eight loads with no branch around them (a token beyond the run reads the run's last
+        // row and is dropped): they go out together
+#pragma unroll
+        for (int i = 0; i < 8; ++i) vals[i] = v_in[(int64_t)(r + min(i, n - 1)) * in_stride + e];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          vals[i] = 0;
-          if (i < n) {
-            const uint16_t x = v_in[(int64_t)(r + i) * in_stride + e];
-            vals[i] = v_bias ? float_to_bf16_bits(bf16_bits_to_float(x) + b) : x;
-          }
+          if (v_bias) vals[i] = float_to_bf16_bits(bf16_bits_to_float(vals[i]) + b);
+          if (i >= n) vals[i] = 0;
         }
         uint16_t* out = vpool + ((int64_t)page * KVH + h) * he_v_page_elems(hd) + he_v_index(off, d, NT);
         if (n == 8) {
@@ -198,7 +200,7 @@ __global__ __launch_bounds__(1024) void qkv_rope_cache_vec_kernel(
     return;
   }
   // ---- q and k of one row
-  const int64_t row = blockIdx.x;
+  const int64_t row = (int)blockIdx.x - v_blocks;
   const int seq = row_seq[row];
   if (seq < 0) return;  // padding row
   const int half = rotary_dim >> 1;
