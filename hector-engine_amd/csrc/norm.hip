@@ -127,22 +127,27 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const TD* __re
   const int64_t row = blockIdx.x;
   float* r = resid + row * (int64_t)D;
   const TD* d = delta ? delta + row * (int64_t)D : nullptr;
-  float v[NORM_VEC][4], g[NORM_VEC][4];
+  float v[NORM_VEC][4], g[NORM_VEC][4], a[NORM_VEC][4];
   float ss = 0.f;
+  // the loads stand in no per-thread branch (a group beyond the row reads the row's last four
+  // elements and counts as zeros), so they all go out before the first is waited for
+#pragma unroll
+  for (int e = 0; e < NORM_VEC; ++e) load4(r + min(4 * (int)(threadIdx.x + e * blockDim.x), D - 4), v[e]);
+  if (d) {
+#pragma unroll
+    for (int e = 0; e < NORM_VEC; ++e) load4(d + min(4 * (int)(threadIdx.x + e * blockDim.x), D - 4), a[e]);
+  }
+  if (out) {
+#pragma unroll
+    for (int e = 0; e < NORM_VEC; ++e) load4(w + min(4 * (int)(threadIdx.x + e * blockDim.x), D - 4), g[e]);
+  }
 #pragma unroll
   for (int e = 0; e < NORM_VEC; ++e) {
-    const int i = 4 * (threadIdx.x + e * blockDim.x);
+    const bool in = 4 * (int)(threadIdx.x + e * blockDim.x) < D;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) v[e][j] = g[e][j] = 0.f;
-    if (i < D) {
-      load4(r + i, v[e]);
-      if (d) {
-        float a[4];
-        load4(d + i, a);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) v[e][j] += a[j];
-      }
-      if (out) load4(w + i, g[e]);
+    for (int j = 0; j < 4; ++j) {
+      v[e][j] = in ? v[e][j] + (d ? a[e][j] : 0.f) : 0.f;
+      g[e][j] = (in && out) ? g[e][j] : 0.f;
     }
   }
 #pragma unroll
