@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 14
+#define HE_ABI_VERSION 15
 
 #ifdef __cplusplus
 extern "C" {
@@ -122,6 +122,19 @@ int he_attention_prefill_bf16(void* out, const void* q, const void* kpool, const
 int64_t he_argmax_workspace_bytes(int rows, int V);
 int he_argmax_rows(void* out_i32, const void* logits_f32, int rows, int V, int64_t row_stride,
                    void* workspace, int64_t workspace_bytes, void* stream);
+// Not in the reference: an argmax for callers that cannot allocate device memory (code under
+// HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). The same kernels as
+// he_argmax_rows, with the parts of the rows in a static device array of
+// HE_ARGMAX_STATIC_SCRATCH_BYTES per GPU in place of a workspace; it calls no hipMalloc / hipFree
+// and no allocating library routine. Inputs needing more scratch (rows * ceil(V / 8192) * 8
+// bytes) are refused with an error. All calls on one GPU share that GPU's array: calls that
+// overlap on one GPU (two streams, two threads) race; calls on one stream do not.
+// he_argmax_rows_static_setup looks up the current device's copy of the array (once per device;
+// the first call of he_argmax_rows_static on a device does the same), e.g. before a capture.
+#define HE_ARGMAX_STATIC_SCRATCH_BYTES 65536
+int he_argmax_rows_static_setup(void);
+int he_argmax_rows_static(void* out_i32, const void* logits_f32, int rows, int V,
+                          int64_t row_stride, void* stream);
 int he_apply_penalties(void* logits_f32, int rows, int V, int64_t row_stride, const void* ids,
                        const void* counts, const void* offsets, float rep, float freq, float pres,
                        void* stream);

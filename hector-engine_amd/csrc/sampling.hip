@@ -12,6 +12,8 @@
 // sums are exact and independent of the order of addition, and each "first
 // prefix whose cumulative count / mass reaches t" is found by a four-pass radix
 // descent over the order-preserving integer image of the floats.
+#include <mutex>
+
 #include "common.h"
 #include "hector_kernels.h"
 
@@ -132,6 +134,70 @@ extern "C" int he_argmax_rows(void* out_i32, const void* logits_f32, int rows, i
   if (rc || parts == 1) return rc;
   argmax_join_kernel<<<rows, HE_WAVE, 0, s>>>((int32_t*)out_i32, part_val, part_idx, parts);
   return he_check_launch("he_argmax_rows join");
+}
+
+// The same argmax for callers that cannot allocate: the parts of the rows go into a static
+// device array instead of a workspace the caller brings. Host code never uses the array's
+// name as an address: each device's copy is looked up once (he_argmax_rows_static_setup, or the
+// first call on that device) and the kernels get that pointer.
+static __device__ __align__(256) unsigned char he_static_scratch[HE_ARGMAX_STATIC_SCRATCH_BYTES];
+
+#define HE_MAX_DEVICES 64
+static std::mutex g_static_mutex;
+static void* g_static_ptr[HE_MAX_DEVICES];   // per device: the address of its copy of he_static_scratch
+
+// The current device's copy of the array, or null after recording an error.
+static void* static_scratch_of_current_device() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= HE_MAX_DEVICES) {
+    he_set_error("he_argmax_rows_static: no current device below %d (%s)", HE_MAX_DEVICES,
+                 hipGetErrorString(e));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> guard(g_static_mutex);
+  if (g_static_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(he_static_scratch));
+    if (e != hipSuccess || p == nullptr) {
+      he_set_error("he_argmax_rows_static: hipGetSymbolAddress on device %d: %s", dev,
+                   hipGetErrorString(e));
+      return nullptr;
+    }
+    g_static_ptr[dev] = p;
+  }
+  return g_static_ptr[dev];
+}
+
+extern "C" int he_argmax_rows_static_setup(void) {
+  return static_scratch_of_current_device() != nullptr ? 0 : -1;
+}
+
+extern "C" int he_argmax_rows_static(void* out_i32, const void* logits_f32, int rows, int V,
+                                     int64_t row_stride, void* stream) {
+  HE_REQUIRE(rows >= 0 && V > 0 && row_stride >= V, "he_argmax_rows_static: bad sizes rows=%d V=%d",
+             rows, V);
+  HE_REQUIRE(rows <= 65535, "he_argmax_rows_static: %d rows above 65535", rows);
+  if (rows == 0) return 0;
+  const int parts = (V + ARGMAX_PART - 1) / ARGMAX_PART;
+  const int64_t need = he_argmax_workspace_bytes(rows, V);
+  HE_REQUIRE(need <= HE_ARGMAX_STATIC_SCRATCH_BYTES,
+             "he_argmax_rows_static: %d rows of %d logits need %lld bytes of scratch, the static "
+             "array holds %d (use he_argmax_rows with a workspace)",
+             rows, V, (long long)need, HE_ARGMAX_STATIC_SCRATCH_BYTES);
+  void* scratch = static_scratch_of_current_device();
+  if (scratch == nullptr) return -1;
+  // every part of every row is written by the first launch before the second reads it:
+  // nothing of an earlier call's contents is read, so nothing has to be cleared
+  float* part_val = (float*)scratch;
+  int32_t* part_idx = (int32_t*)scratch + (int64_t)rows * parts;
+  hipStream_t s = (hipStream_t)stream;
+  argmax_parts_kernel<<<dim3(parts, rows), ARGMAX_THREADS, 0, s>>>(
+      (int32_t*)out_i32, part_val, part_idx, (const float*)logits_f32, V, row_stride);
+  int rc = he_check_launch("he_argmax_rows_static");
+  if (rc || parts == 1) return rc;
+  argmax_join_kernel<<<rows, HE_WAVE, 0, s>>>((int32_t*)out_i32, part_val, part_idx, parts);
+  return he_check_launch("he_argmax_rows_static join");
 }
 
 // ---------------------------------------------------------------- penalties

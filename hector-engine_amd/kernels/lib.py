@@ -16,7 +16,7 @@ _lib = None
 
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 
-EXPECTED_ABI = 14
+EXPECTED_ABI = 15
 
 c_int, c_i64, c_f32, c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
@@ -61,6 +61,8 @@ _SIGNATURES = {
                                   c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_int, c_ptr],
     "he_argmax_workspace_bytes": [c_int, c_int],
     "he_argmax_rows": [c_ptr, c_ptr, c_int, c_int, c_i64, c_ptr, c_i64, c_ptr],
+    "he_argmax_rows_static_setup": [],
+    "he_argmax_rows_static": [c_ptr, c_ptr, c_int, c_int, c_i64, c_ptr],
     "he_apply_penalties": [c_ptr, c_int, c_int, c_i64, c_ptr, c_ptr, c_ptr, c_f32, c_f32, c_f32,
                            c_ptr],
     "he_sample_rows": [c_ptr, c_ptr, c_int, c_int, c_i64, c_ptr, c_f32, c_int, c_f32, c_ptr],
