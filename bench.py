@@ -13,6 +13,13 @@ A step is one decode step of the whole batch: the engine's step function (HIP
 graph replay) plus greedy sampling. As in the library's generation loop, 8 steps are
 queued at a time: the chosen ids go into the next step on the device, and the host
 reads them once per run of 8.
+
+Procedure (the reference quotes medians with their range over repeated runs:
+tools/HQS_DECODE_OPTIMIZATION_PLAN.md:54-65): after the warm-up steps, `--repeats` (5) runs of
+exactly `--steps` steps each are timed, each bracketed by a device synchronisation; `value` and
+`ms_per_step` are the median run's, `repeats` holds all of them. The same holds for the points at
+batch 1 and at the large batch. The prefill figure is the median of three whole-prompt steps of
+one 2,048-token prompt; `prefill_packed` is one step of `--batch` such prompts packed together.
 """
 from __future__ import annotations
 
@@ -66,6 +73,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--repeats", type=int, default=5, help="timed runs of --steps steps each; the median counts")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0 = all)")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="7b")
@@ -83,9 +91,12 @@ def main() -> int:
     CONTEXT = args.context or CONTEXT
     if args.prompt:
         PROMPT_LO = PROMPT_HI = args.prompt
-    if max(PROMPT, PROMPT_HI) + args.warmup + args.steps > CONTEXT:
-        print(f"bench.py: prompts of {max(PROMPT, PROMPT_HI)} tokens and {args.warmup + args.steps} steps do not fit "
-              f"a context of {CONTEXT}")
+    if args.repeats < 1 or args.steps < 1:
+        print("bench.py: --steps and --repeats must be at least 1")
+        return 2
+    if max(PROMPT, PROMPT_HI) + args.warmup + args.repeats * args.steps > CONTEXT:
+        print(f"bench.py: prompts of {max(PROMPT, PROMPT_HI)} tokens and {args.warmup + args.repeats * args.steps} "
+              f"steps do not fit a context of {CONTEXT}")
         return 2
     FULL_LAYERS = SHAPE["num_hidden_layers"]
     args.layers = args.layers or FULL_LAYERS
@@ -128,10 +139,23 @@ def main() -> int:
                 toks += sampler.sample(logits, list(range(len(entries))), [0] * len(entries))
         return toks
 
-    def decode_run(batch, steps, warmup):
+    wbytes = weight_bytes(SHAPE, args.layers)
+    packed = {}
+
+    def decode_run(batch, steps, warmup, repeats):
+        """Prompts, warm-up steps, then `repeats` timed runs of `steps` steps. Returns per run
+        (seconds a step, bytes a step has to read)."""
         slots = [engine.acquire() for _ in range(batch)]
         ps = prompts(batch, PROMPT_LO, PROMPT_HI)
-        toks = prefill(ps, slots)
+        if batch == args.batch and batch <= 8:      # the packed prompt step of the headline batch, timed
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            toks = prefill(ps, slots)
+            torch.cuda.synchronize()
+            packed.update(tokens=sum(len(p) for p in ps), seconds=time.perf_counter() - t0,
+                          flops=sum(prefill_flops(SHAPE, args.layers, len(p)) for p in ps))
+        else:
+            toks = prefill(ps, slots)
         seqs = list(range(batch))
 
         def run(toks, count):
@@ -151,15 +175,23 @@ def main() -> int:
             return toks
 
         toks = many(toks, warmup)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        toks = many(toks, steps)
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-        avg_len = sum(len(p) for p in ps) / batch + warmup + steps / 2
+        runs = []
+        done = warmup
+        for _ in range(repeats):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            toks = many(toks, steps)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            avg_len = sum(len(p) for p in ps) / batch + done + steps / 2
+            done += steps
+            runs.append((dt / steps, wbytes + batch * avg_len * kv_bytes_per_token(SHAPE, args.layers)))
         for s in slots:
             engine.release(s)
-        return dt / steps, avg_len
+        return runs
+
+    def median_run(runs):
+        return sorted(runs)[len(runs) // 2]
 
     # ---- prefill of one 2,048-token prompt: a first run warms the library GEMMs, then the median of three
     progress(f"weights ready; prefill of {PROMPT} tokens")
@@ -179,17 +211,18 @@ def main() -> int:
 
     # ---- decode at the headline batch
     progress(f"decode at batch {args.batch}")
-    step_s, avg_len = decode_run(args.batch, args.steps, args.warmup)
-    wbytes = weight_bytes(SHAPE, args.layers)
-    step_bytes = wbytes + args.batch * avg_len * kv_bytes_per_token(SHAPE, args.layers)
+    runs = decode_run(args.batch, args.steps, args.warmup, args.repeats)
+    step_s, step_bytes = median_run(runs)
     achieved = step_bytes / step_s / 1e9
 
-    points = {}
+    points, points_frac, points_ms = {}, {}, {}
     if not args.no_points:
         for b in (1, BIG_BATCH):
             progress(f"decode at batch {b}")
-            s, _ = decode_run(b, max(8, args.steps // 2), max(3, args.warmup // 2))
+            s, nbytes = median_run(decode_run(b, args.steps, max(3, args.warmup // 2), args.repeats))
             points[f"decode_b{b}"] = round(b / s, 1)
+            points_ms[f"decode_b{b}"] = round(s * 1e3, 4)
+            points_frac[f"decode_b{b}"] = round(nbytes / s / 1e9 / HBM_PEAK_GBS, 4)
 
     PROMPTS = PROMPT_LO if PROMPT_LO == PROMPT_HI else f"{PROMPT_LO}-{PROMPT_HI}"
     line = {
@@ -221,7 +254,18 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)},
         "points": points,
+        "points_ms_per_step": points_ms,
+        "points_roofline_frac": points_frac,
+        "repeats": {"n": args.repeats, "steps_each": args.steps,
+                    "ms_per_step": [round(t * 1e3, 4) for t, _ in runs],
+                    "min": round(min(t for t, _ in runs) * 1e3, 4),
+                    "median": round(step_s * 1e3, 4),
+                    "max": round(max(t for t, _ in runs) * 1e3, 4)},
     }
+    if packed:
+        line["prefill_packed"] = {"value": round(packed["tokens"] / packed["seconds"], 1), "tokens": packed["tokens"],
+                                  "ms": round(packed["seconds"] * 1e3, 3),
+                                  "frac": round(packed["flops"] / packed["seconds"] / BF16_PEAK_FLOPS, 4)}
     print(json.dumps(line))
     return 0
 

@@ -55,6 +55,8 @@ def qwen2_spec(cfg: Qwen2Config) -> ModelSpec:
         head=PartSpec("linear_head", head_params),
         head_prefix="lm_head.",
         max_positions=cfg.max_position_embeddings,
+        # a folder of a tied model may still hold the output matrix (it is not read)
+        unused_tensors=frozenset({"lm_head.weight"}) if cfg.tie_word_embeddings else frozenset(),
     )
 
 

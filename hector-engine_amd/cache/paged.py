@@ -1,9 +1,10 @@
 """The cache on the device.
 
 Keys and values live in pages of 64 tokens. Layers are partitioned into groups
-by what they keep (kv heads, head size, all keys or a window of them); each
-group has pools of its own, [runs][pages][kv_heads][64][head_dim] for K and for
-V (V transposed inside a page: [head_dim][64]), and one page table [slots][blocks]
+by what they keep (kv heads, key and value widths, all keys or a window of them); each
+group has pools of its own, [runs][pages][kv_heads][elements of a page] for K and for
+V, the elements of a page in the order the attention kernels read their operands
+(cache/layout.py), and one page table [slots][blocks]
 shared by its runs. A sequence holds a
 slot: its row of every page table, its length, and its row of the fixed-size
 state area. Slots and pages go back to the free lists when a sequence ends and
@@ -43,7 +44,7 @@ class _Group:
         # a page of a kv head is kept in the order the attention kernels read it (cache/layout.py)
         self.kpool = torch.zeros((len(runs), num_pages, need.kv_heads, layout.k_page_elems(need.head_dim)),
                                  dtype=dtype, device=device)
-        self.vpool = torch.zeros((len(runs), num_pages, need.kv_heads, layout.v_page_elems(need.head_dim)),
+        self.vpool = torch.zeros((len(runs), num_pages, need.kv_heads, layout.v_page_elems(need.v_dim)),
                                  dtype=dtype, device=device)
         self.page_table = torch.full((max_slots, max_blocks), -1, dtype=torch.int32, device=device)
 
@@ -117,6 +118,10 @@ class PagedCache:
     def reserve(self, growth: list[tuple[int, int]]) -> None:
         """growth: (slot, new length) for every sequence of a step. Either all get
         their pages or none does."""
+        for s, n in growth:            # every check before any page is taken
+            if blocks_for(n) > self.max_blocks:
+                raise CacheFull(f"slot {s}: {n} tokens exceed the longest sequence the cache was "
+                                f"built for ({self.max_seq_len})")
         need = sum(self.book.pages_needed(s, n) for s, n in growth)
         for g in self.book.groups:
             if need > g.pool.available:
@@ -168,5 +173,5 @@ class PagedCache:
     def bytes_per_token(self) -> int:
         es = torch.empty((), dtype=self.dtype).element_size()
         return sum(len(g.runs) * g.need.kv_heads * es
-                   * (layout.k_page_elems(g.need.head_dim) + layout.v_page_elems(g.need.head_dim)) // PAGE_TOKENS
+                   * (layout.k_page_elems(g.need.head_dim) + layout.v_page_elems(g.need.v_dim)) // PAGE_TOKENS
                    for g in self.groups)

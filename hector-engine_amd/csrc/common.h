@@ -7,10 +7,11 @@
 // dtype codes used across the C ABI
 #define HE_F32 0
 #define HE_BF16 1
+#define HE_F16 2   // as the stored dtype of an uploaded tensor only
 
-// Tokens per page of the key/value cache. The K pool is laid out
-// [page][kv_head][PAGE_TOKENS][head_dim], the V pool transposed inside a page:
-// [page][kv_head][head_dim][PAGE_TOKENS].
+// Tokens per page of the key/value cache. Both pools are [page][kv_head][elements of a page];
+// inside a page the elements lie in the order the MFMA attention kernels read their operands
+// (cache_layout.h: K as [half][key tile][k step][lane][8], V as [half][dim tile][lane][8]).
 #define HE_PAGE_TOKENS 64
 #define HE_PAGE_SHIFT 6
 

@@ -2,11 +2,11 @@
 // stream and returns 0, or non-zero after recording a message for
 // he_last_error(). Pointers are device pointers unless named host_*. Shapes
 // are validated on the host before any launch. dtype codes: 0 = float32,
-// 1 = bfloat16.
+// 1 = bfloat16 (2 = float16, as the input of he_cast only).
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 15
+#define HE_ABI_VERSION 16
 
 #ifdef __cplusplus
 extern "C" {
@@ -14,6 +14,16 @@ extern "C" {
 
 const char* he_last_error(void);
 int he_abi_version(void);
+
+// ---- weight preparation ----------------------------------------------------
+// out[i] = bf16(quantiles[16 bits of the counter-based word of (key, i)] * std + mean), stored as
+// `dtype`; quantiles_f32: 65536 quantiles of the standard normal distribution (device pointer).
+int he_fill_random(void* out, int64_t n, int dtype, uint64_t key, const void* quantiles_f32,
+                   float mean, float std, void* stream);
+// out[i] = uniform integer in [0, high) from the counter-based word of (key, i).
+int he_fill_random_integers(void* out_i32, int64_t n, uint64_t key, int64_t high, void* stream);
+// out = in converted (in: float32, bfloat16 or float16; out: float32 or bfloat16, nearest even).
+int he_cast(void* out, const void* in, int64_t n, int in_dtype, int out_dtype, void* stream);
 
 // ---- row-wise ------------------------------------------------------------
 int he_embedding(void* out_f32, const void* table, const void* ids, int rows, int D, int V,

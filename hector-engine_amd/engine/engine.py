@@ -13,7 +13,7 @@ src/engine.cpp:151-269).
 from __future__ import annotations
 
 import dataclasses
-import time
+import warnings
 
 import numpy as np
 import torch
@@ -22,7 +22,7 @@ from ..cache.paged import PagedCache
 from ..cache.pages import CacheError, CacheFull  # noqa: F401
 from ..config.base import ModelConfig
 from ..kernels import lib as kernel_lib
-from ..kernels import library_tuning
+from ..kernels import library_tuning, profiler
 from ..parts.base import BuildEnv, StepContext
 from ..registry import build_model, load_config
 from ..weights.loader import load_tensors
@@ -81,9 +81,13 @@ class Engine:
                  seed: int | None = None, dtype: str = "bfloat16", max_tokens: int = 8192,
                  max_slots: int | None = None, max_seq_len: int | None = None,
                  device: str = "cuda:0", fast_kernels: bool = True, use_graphs: bool = True,
-                 tune_library: bool = False):
-        """tune_library: let the library's autotuner choose the kernel of each tall bfloat16
-        matrix product the first time its shape is seen (kernels/library_tuning.py)."""
+                 tune_library: bool = False, beyond_max_positions: bool = False, profile: bool = False):
+        """max_seq_len: the longest sequence (default: the positions the model's configuration
+        allows; more than that is refused unless beyond_max_positions says it is meant).
+        tune_library: let the library's autotuner choose the kernel of each tall bfloat16
+        matrix product the first time its shape is seen (kernels/library_tuning.py).
+        profile: time every kernel with a pair of events (kernels/profiler.py; steps then run
+        without HIP graphs); profile_summary() gives the table."""
         if dtype not in _DTYPES:
             raise ValueError(f"dtype must be one of {sorted(_DTYPES)}, got {dtype!r}")
         if not torch.cuda.is_available():
@@ -108,8 +112,7 @@ class Engine:
         self.model = build_model(self.config, self.env)
         specs = self.model.tensor_specs()
         if model_dir is not None:
-            extra = {"lm_head.weight"} if getattr(self.config, "tie_word_embeddings", False) else set()
-            tensors = load_tensors(model_dir, specs, self.dtype, self.device, extra)
+            tensors = load_tensors(model_dir, specs, self.dtype, self.device, self.model.spec.unused_tensors)
         else:
             if seed is None:
                 raise ValueError("random weights need a seed")
@@ -117,13 +120,21 @@ class Engine:
         self.model.bind(tensors)
         del tensors
         self.vocab_size = self.model.spec.vocab_size
-        max_seq_len = max_seq_len or self.model.spec.max_positions
+        allowed = self.model.spec.max_positions
+        if max_seq_len is not None and max_seq_len > allowed and not beyond_max_positions:
+            raise ValueError(f"max_seq_len {max_seq_len} exceeds the {allowed} positions the model's "
+                             "configuration allows (pass beyond_max_positions=True if that is meant)")
+        max_seq_len = max_seq_len or allowed
         self.cache = PagedCache(self.model.run_plans(), max_tokens=max_tokens,
                                 max_slots=max_slots or 256, max_seq_len=min(max_seq_len, max_tokens),
                                 dtype=self.dtype, device=self.device)
+        # the cache counts in whole pages; the engine holds sequences to the length asked for
+        self._max_seq_len = min(max_seq_len, self.cache.max_seq_len)
         self.caches = [self.cache.layer_cache(r) for r in range(len(self.model.schedule))]
         self.scratch = ScratchPool(self.device)
-        self.use_graphs = use_graphs and self.model.graph_safe()
+        self.profiler = profiler.OpProfiler() if profile else None
+        self.use_graphs = use_graphs and self.model.graph_safe() and not profile
+        self._capture_failed = False
         self._buckets: dict[int, _GraphBucket] = {}
         self._pinned = [torch.empty(1 << 16, dtype=torch.int32).pin_memory() for _ in range(4)]
         self._pinned_events: list[torch.cuda.Event | None] = [None] * 4
@@ -143,7 +154,7 @@ class Engine:
 
     @property
     def max_seq_len(self) -> int:
-        return self.cache.max_seq_len
+        return self._max_seq_len
 
     # -- the step function -------------------------------------------------------
     def step(self, entries: list[StepEntry], device_tokens: torch.Tensor | None = None) -> torch.Tensor | None:
@@ -171,9 +182,9 @@ class Engine:
             if n == 0:
                 raise StepError(f"slot {e.slot}: an entry needs at least one token")
             start = self.cache.length(e.slot)
-            if start + n > self.cache.max_seq_len:
+            if start + n > self._max_seq_len:
                 raise StepError(f"slot {e.slot}: {start} cached + {n} new tokens exceed the "
-                                f"longest sequence {self.cache.max_seq_len}")
+                                f"longest sequence {self._max_seq_len}")
             if n == 1 and type(e.tokens[0]) is int:     # the common one-token step, without numpy
                 in_range = 0 <= e.tokens[0] < self.vocab_size
             else:
@@ -189,12 +200,21 @@ class Engine:
         all_single = all(len(e.tokens) == 1 for e in entries)
         every_wanted = all(list(e.want) == [0] for e in entries)
         self.stats["steps"] += 1
-        if self.use_graphs and all_single and every_wanted and len(entries) <= GRAPH_MAX_BUCKET:
-            logits = self._graph_step(entries, device_tokens)
-        else:
-            logits = self._eager_step(entries, all_single, device_tokens)
+        with profiler.active(self.profiler):
+            if self.use_graphs and all_single and every_wanted and len(entries) <= GRAPH_MAX_BUCKET:
+                logits = self._graph_step(entries, device_tokens)
+            else:
+                logits = self._eager_step(entries, all_single, device_tokens)
         self.cache.commit(growth)
         return logits
+
+    def profile_summary(self) -> str:
+        """The table of the kernels' times since the engine was made (or since the profiler
+        was cleared): calls, total, average, share, as the reference prints its own
+        (src/engine.cpp:372-435)."""
+        if self.profiler is None:
+            return "No profiling data"
+        return self.profiler.format()
 
     # -- packing ---------------------------------------------------------------
     def _pack(self, entries, meta: _Meta, rows_padded: int, seqs_padded: int):
@@ -309,24 +329,39 @@ class Engine:
             ctx.want_all = True
             if bucket.uses == 1:
                 # first use: run eagerly; it also sizes the bucket's scratch pool
-                bucket.pool.reset()
-                self.stats["eager_steps"] += 1
-                logits = self.model.forward(bucket.views["tokens"], ctx, self.caches,
-                                            bucket.views["want_rows"], size)
-                return logits[:n]
+                return self._bucket_eager(bucket, ctx, n)
+            if self._capture_failed:
+                return self._bucket_eager(bucket, ctx, n)
             bucket.pool.reset()          # sized by the eager run; from here on it must not move
             bucket.pool.frozen = True
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
-            with library_tuning.no_new_tuning(), torch.cuda.graph(graph):
-                bucket.pool.reset()
-                bucket.logits = self.model.forward(bucket.views["tokens"], ctx, self.caches,
-                                                   bucket.views["want_rows"], size)
+            try:
+                with library_tuning.no_new_tuning(), torch.cuda.graph(graph):
+                    bucket.pool.reset()
+                    bucket.logits = self.model.forward(bucket.views["tokens"], ctx, self.caches,
+                                                       bucket.views["want_rows"], size)
+            except Exception as exc:     # the reference falls back the same way: src/engine.cpp:233-261
+                self._capture_failed = True
+                bucket.pool.frozen = False
+                del graph
+                torch.cuda.synchronize()
+                warnings.warn(f"capturing the one-token step as a HIP graph failed ({exc!r}); "
+                              "one-token steps run without graphs from here on", stacklevel=3)
+                return self._bucket_eager(bucket, ctx, n)
             bucket.graph = graph
             self.stats["graph_captures"] += 1
         bucket.graph.replay()
         self.stats["graph_replays"] += 1
         return bucket.logits[:n]
+
+    def _bucket_eager(self, bucket, ctx, n: int):
+        """The bucket's step without a graph, on its own buffers."""
+        bucket.pool.reset()
+        self.stats["eager_steps"] += 1
+        logits = self.model.forward(bucket.views["tokens"], ctx, self.caches,
+                                    bucket.views["want_rows"], bucket.size)
+        return logits[:n]
 
     # -- convenience -----------------------------------------------------------
     def synchronize(self) -> None:

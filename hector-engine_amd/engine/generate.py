@@ -18,7 +18,7 @@ from typing import Callable
 
 import torch
 
-from ..cache.pages import PAGE_TOKENS, blocks_for
+from ..cache.pages import blocks_for
 from .engine import StepEntry
 
 
@@ -73,21 +73,33 @@ RUN_OF_STEPS = 8
 
 def generate(engine, prompts: list[list[int]], *, max_new_tokens: int = 100, sampling=None,
              stop_ids=(), include_stop: bool = False, batch_size: int | None = None,
-             cancel: Callable[[], bool] | None = None, sample_fn=None,
+             cancel: Callable[[], bool] | None = None, sample_fn=None, sampler=None,
              run_of_steps: int = RUN_OF_STEPS) -> list[GenerationResult]:
     """Generates for every prompt; returns results in the order of `prompts`.
 
-    run_of_steps: with the library's own sampler and no penalties, up to so many one-token
-    steps are queued at a time: each step's ids go into the next on the device and the host
-    reads them once per run. The tokens are the same as step by step; a sequence that ends
-    inside a run keeps its slot until the run ends, and `cancel` is asked between runs."""
+    sampler: an object with the library Sampler's interface (config, sample, sample_device,
+    uniforms_device, read_later) in place of one made from `sampling`; sample_fn: a plain
+    function (logits, requests, steps, contexts) -> ids, which runs step by step.
+
+    run_of_steps: with a sampler and no penalties, up to so many one-token steps are queued at
+    a time, each step's ids going into the next on the device. The tokens are the same as step
+    by step. When nothing can end a sequence inside a run but its token budget or its cache
+    room (no stop ids, no `cancel`), the run never reaches past those and the host reads all
+    its ids at the end. Otherwise the host reads the ids of a step while the next one runs,
+    and queues nothing more once it has seen a stop token or `cancel` says so: a sequence that
+    has sampled its stop token is stepped once more at most (the step that was already
+    queued), then gives its slot back and leaves the batch."""
     from ..sampling import Sampler, SamplingConfig
-    sampler = None
+    from ..sampling.sampler import READS_IN_FLIGHT
     if sample_fn is None:
-        sampler = Sampler(sampling or SamplingConfig.deterministic(), engine.device)
+        if sampler is None:
+            sampler = Sampler(sampling or SamplingConfig.deterministic(), engine.device)
         sample_fn = sampler.sample
         if sampler.config.has_penalties or run_of_steps <= 1:
             sampler = None          # penalties need each token on the host before the next
+    else:
+        sampler = None
+    run_of_steps = min(run_of_steps, READS_IN_FLIGHT)
     stop_ids = frozenset(int(s) for s in stop_ids)
     results: list[GenerationResult | None] = [None] * len(prompts)
     pending = [(i, len(p)) for i, p in enumerate(prompts)]
@@ -121,17 +133,26 @@ def steps_in_run(generated: list[int], lengths: list[int], max_new_tokens: int, 
 
 
 def _run_of_steps(engine, sampler, slots: list[int], tokens: list[int], seqs: list[int],
-                  steps: list[int], count: int) -> list[list[int]]:
-    """Feeds `tokens` and queues `count` steps; returns the sampled ids of each, [count][rows]."""
+                  steps: list[int], count: int, stop_ids=frozenset(), cancel=None) -> list[list[int]]:
+    """Feeds `tokens` and queues up to `count` one-token steps; returns the sampled ids of the
+    steps that ran, [steps][rows]. With stop ids or `cancel`, the ids of step j are read while
+    step j + 1 runs, and the run ends with the step that was queued when a stop token (or the
+    cancellation) was seen."""
     uniforms = None if sampler.config.is_greedy else sampler.uniforms_device(seqs, steps, count)
-    ids, device_ids = [], None
+    watch = bool(stop_ids) or cancel is not None
+    reads, ids, device_ids = [], [], None
     for j in range(count):
         entries = [StepEntry(s, [t], [0]) for s, t in zip(slots, tokens)]
         logits = engine.step(entries, device_tokens=device_ids)
         device_ids = sampler.sample_device(logits, seqs, [t + j for t in steps],
                                            uniforms=None if uniforms is None else uniforms[j])
-        ids.append(device_ids)
-    return torch.stack(ids).tolist()          # the one wait of the run
+        reads.append(sampler.read_later(device_ids))
+        if watch and j >= 1:
+            ids.append(reads[j - 1].wait())
+            if not stop_ids.isdisjoint(ids[-1]) or (cancel is not None and cancel()):
+                break
+    ids += [r.wait() for r in reads[len(ids):]]
+    return ids
 
 
 def _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, include_stop, cancel,
@@ -178,7 +199,8 @@ def _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, inc
                 tokens = sample_fn(logits, active, [len(out[i]) for i in active], [out[i] for i in active])
                 continue
             run = _run_of_steps(engine, sampler, [slots[i] for i in active], [tok for _, tok in feed],
-                                active, [len(out[i]) for i in active], count)
+                                active, [len(out[i]) for i in active], count, stop_ids, cancel)
+            count = len(run)            # fewer when a stop token was seen on the way
             # all but the last step of the run are decided here, each with the cache length of its
             # moment; a sequence that ends inside the run drops the rest of its ids
             going = dict.fromkeys(active, True)

@@ -80,7 +80,7 @@ class DecoderModel:
             # the norm that reads the stream after this block: the next block's first, or the
             # final norm when every row's logits are wanted (no gather in between)
             if e < last:
-                ctx.next_norm = getattr(self.blocks[self.schedule[e + 1].layer], "mixer_norm", None)
+                ctx.next_norm = self.blocks[self.schedule[e + 1].layer].first_norm()
             else:
                 ctx.next_norm = self.final_norm if (ctx.want_all and n_want == rows) else None
             ctx.scratch.begin_layer()

@@ -16,13 +16,16 @@ _lib = None
 
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 
-EXPECTED_ABI = 15
+EXPECTED_ABI = 16
 
 c_int, c_i64, c_f32, c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
 # name -> argument types (all return int unless listed in _RESTYPES)
 _SIGNATURES = {
     "he_abi_version": [],
+    "he_fill_random": [c_ptr, c_i64, c_int, ctypes.c_uint64, c_ptr, c_f32, c_f32, c_ptr],
+    "he_fill_random_integers": [c_ptr, c_i64, ctypes.c_uint64, c_i64, c_ptr],
+    "he_cast": [c_ptr, c_ptr, c_i64, c_int, c_int, c_ptr],
     "he_embedding": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_ptr],
     "he_gather_rows_f32": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_ptr],
     "he_residual_add": [c_ptr, c_ptr, c_i64, c_int, c_ptr],

@@ -7,8 +7,9 @@ import torch
 
 from ..cache import layout
 from . import lib as _lib
+from .profiler import op as _op
 
-F32, BF16 = 0, 1
+F32, BF16, F16 = 0, 1, 2
 PAGE_TOKENS = 64
 SKINNY_MAX_M = 64
 
@@ -42,6 +43,38 @@ def _ptr(t: torch.Tensor | None) -> int | None:
     return None if t is None else t.data_ptr()
 
 
+@_op("fill_random")
+def fill_random(out, key: int, quantiles, mean: float, std: float) -> None:
+    """out (float32 or bfloat16, any shape, contiguous) = seeded normal values, element by
+    element what weights.random_init.normal_values gives on the host for the same key."""
+    _need(out, "out")
+    _need(quantiles, "quantiles", torch.float32, (65536,))
+    L = _lib.load()
+    _lib.check(L.he_fill_random(out.data_ptr(), out.numel(), dtype_code(out.dtype), key & ((1 << 64) - 1),
+                                quantiles.data_ptr(), float(mean), float(std), _stream()))
+
+
+@_op("fill_random")
+def fill_random_integers(out_i32, key: int, high: int) -> None:
+    _need(out_i32, "out", torch.int32)
+    L = _lib.load()
+    _lib.check(L.he_fill_random_integers(out_i32.data_ptr(), out_i32.numel(), key & ((1 << 64) - 1), int(high),
+                                         _stream()))
+
+
+@_op("cast")
+def cast(out, src) -> None:
+    """out (float32 or bfloat16) = src (float32, bfloat16 or float16) converted, same element count."""
+    _need(out, "out")
+    _need(src, "src")
+    if out.numel() != src.numel():
+        raise ValueError("cast: out and src differ in size")
+    code = F16 if src.dtype == torch.float16 else dtype_code(src.dtype)
+    L = _lib.load()
+    _lib.check(L.he_cast(out.data_ptr(), src.data_ptr(), src.numel(), code, dtype_code(out.dtype), _stream()))
+
+
+@_op("embedding")
 def embedding(out_f32, table, ids, rows: int) -> None:
     V, D = table.shape
     _need(table, "table")
@@ -54,6 +87,7 @@ def embedding(out_f32, table, ids, rows: int) -> None:
                               dtype_code(table.dtype), _stream()))
 
 
+@_op("gather_rows")
 def gather_rows_f32(out, src, rows_idx, n_out: int, n_src: int) -> None:
     D = src.shape[-1]
     _need(src, "src", torch.float32)
@@ -66,6 +100,7 @@ def gather_rows_f32(out, src, rows_idx, n_out: int, n_src: int) -> None:
                                     n_src, _stream()))
 
 
+@_op("residual_add")
 def residual_add(resid_f32, delta, rows: int) -> None:
     D = resid_f32.shape[-1]
     _need(resid_f32, "resid", torch.float32)
@@ -77,6 +112,7 @@ def residual_add(resid_f32, delta, rows: int) -> None:
                                  dtype_code(delta.dtype), _stream()))
 
 
+@_op("silu_mul")
 def silu_mul(out, gate_up, rows: int, interleaved: bool = False, splits: int = 0) -> None:
     """out[rows, I] = silu(gate) * up. gate_up: [rows, 2I] in out's dtype, or with
     splits > 0 the fp32 K slices [splits, rows, 2I] of the product. Its columns are all
@@ -94,6 +130,7 @@ def silu_mul(out, gate_up, rows: int, interleaved: bool = False, splits: int = 0
                              dtype_code(out.dtype), _stream()))
 
 
+@_op("add_rmsnorm")
 def add_rmsnorm(resid_f32, delta, weight, out, rows: int, eps: float, delta_splits: int = 0,
                 delta_bias=None) -> None:
     """resid += delta (if given); out = rmsnorm(resid) * weight (if out given).
@@ -130,6 +167,7 @@ def add_rmsnorm(resid_f32, delta, weight, out, rows: int, eps: float, delta_spli
                                 dtype_code(act or torch.float32), dtype_code(weight.dtype), _stream()))
 
 
+@_op("rmsnorm_rows")
 def rmsnorm_rows(out, x, weight, rows: int, D: int, x_stride: int, out_stride: int,
                  eps: float) -> None:
     if out.dtype != x.dtype:
@@ -144,6 +182,7 @@ def rmsnorm_rows(out, x, weight, rows: int, D: int, x_stride: int, out_stride: i
                                  dtype_code(weight.dtype) if weight is not None else F32, _stream()))
 
 
+@_op("gemm_plain")
 def gemm_plain(out, a, w, bias, M: int) -> None:
     """out[M,N] = a[M,K] . w[N,K]^T (+ bias), fixed summation order."""
     N, K = w.shape
@@ -165,6 +204,7 @@ def gemm_skinny_splits(M: int, N: int, K: int) -> int:
     return int(_lib.load().he_gemm_skinny_splits(M, N, K))
 
 
+@_op("gemm_skinny")
 def gemm_skinny(out, partial, a, w, bias, M: int, plan=(0, 0, 0), out_dtype=None) -> int:
     """bf16 MFMA product for M <= 64. plan = (R, U, splits), zeros for the heuristic.
     With one K slice `out` (bf16 or fp32) is written, with bias. With more slices
@@ -225,6 +265,7 @@ def gemm_blocksplit_blocks(M: int, N: int, K: int) -> int:
     return int(_lib.load().he_gemm_blocksplit_blocks(M, N, K))
 
 
+@_op("gemm_blocksplit")
 def gemm_blocksplit(out, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0), *,
                     row_scale=None, residual=None, x_pieces: bool = False, out_pieces: bool = False) -> None:
     """bf16 MFMA product for M <= 32 with K cut inside the workgroup; one launch, complete
@@ -290,6 +331,7 @@ def gemm_blocksplit(out, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0)
         int(x_pieces), int(out_pieces), _stream()))
 
 
+@_op("scale_rows")
 def scale_rows(out, x, partials, eps: float, rows: int, x_pieces: bool = False) -> None:
     """out = x / sqrt(sum(partials of the row) / D + eps) for rows x = r * gain (bf16). out is
     row-major; x_pieces: x is piece-major, shaped pieces_shape(rows, D)."""
@@ -307,6 +349,7 @@ def scale_rows(out, x, partials, eps: float, rows: int, x_pieces: bool = False) 
                                               _stream()))
 
 
+@_op("splitk_reduce")
 def splitk_reduce(out, partial, bias, M: int, splits: int) -> None:
     """out[M, N] = sum of partial[s] over the slices in index order (+ bias)."""
     N = out.shape[-1]
@@ -322,6 +365,7 @@ def splitk_reduce(out, partial, bias, M: int, splits: int) -> None:
                                   dtype_code(bias.dtype) if bias is not None else F32, _stream()))
 
 
+@_op("qkv_rope_cache")
 def qkv_rope_cache(q_out, kpool, vpool, qkv, q_cols: int, kv_cols: int, bias, positions, row_seq,
                    seq_slot, page_table, inv_freq, rotary_dim: int, rows: int, H: int, KVH: int,
                    hd: int, write_kv: bool, splits: int = 0) -> None:
@@ -393,6 +437,7 @@ def _check_attention(out, q, kpool, vpool, page_table, rows, H, KVH, hd):
         raise ValueError("attention: q/out smaller than the row count")
 
 
+@_op("attention_plain")
 def attention_plain(out, q, kpool, vpool, positions, row_seq, seq_slot, page_table, rows: int,
                     H: int, KVH: int, hd: int, window: int, scale: float) -> None:
     _check_attention(out, q, kpool, vpool, page_table, rows, H, KVH, hd)
@@ -411,6 +456,7 @@ def attention_decode_workspace_floats(rows: int, H: int, KVH: int, hd: int, max_
     return int(_lib.load().he_attention_decode_workspace_floats(rows, H, KVH, hd, max_keys))
 
 
+@_op("attention_decode")
 def attention_decode(out, q, kpool, vpool, positions, row_seq, seq_slot, page_table, rows: int,
                      H: int, KVH: int, hd: int, window: int, scale: float, max_keys: int,
                      workspace) -> None:
@@ -437,6 +483,7 @@ def attention_decode_fused_workspace_floats(rows: int, H: int, KVH: int, hd: int
     return int(_lib.load().he_attention_decode_fused_workspace_floats(rows, H, KVH, hd, max_keys))
 
 
+@_op("attention_decode_fused")
 def attention_decode_fused(out, qkv, bias, kpool, vpool, positions, row_seq, seq_slot, page_table,
                            inv_freq, rotary_dim: int, rows: int, H: int, KVH: int, hd: int,
                            window: int, scale: float, max_keys: int, write_kv: bool,
@@ -474,6 +521,7 @@ def attention_decode_fused(out, qkv, bias, kpool, vpool, positions, row_seq, seq
         workspace.numel() if workspace is not None else 0, _stream()))
 
 
+@_op("attention_prefill")
 def attention_prefill(out, q, kpool, vpool, cu_seqlens, seq_slot, seq_start, page_table,
                       num_seqs: int, max_q_len: int, total_rows: int, H: int, KVH: int, hd: int,
                       window: int, scale: float, tiles_per_wave: int = 0) -> None:
@@ -493,6 +541,7 @@ def attention_prefill(out, q, kpool, vpool, cu_seqlens, seq_slot, seq_start, pag
         kpool.shape[0], num_seqs, max_q_len, H, KVH, hd, window, float(scale), int(tiles_per_wave), _stream()))
 
 
+@_op("argmax_rows")
 def argmax_rows(out_i32, logits, rows: int) -> None:
     _need(logits, "logits", torch.float32)
     _need(out_i32, "out", torch.int32)
@@ -505,6 +554,7 @@ def argmax_rows(out_i32, logits, rows: int) -> None:
     _lib.check(L.he_argmax_rows(out_i32.data_ptr(), logits.data_ptr(), rows, V, V, _ptr(ws), need, _stream()))
 
 
+@_op("apply_penalties")
 def apply_penalties(logits, rows: int, ids, counts, offsets, rep: float, freq: float,
                     pres: float) -> None:
     _need(logits, "logits", torch.float32)
@@ -519,6 +569,7 @@ def apply_penalties(logits, rows: int, ids, counts, offsets, rep: float, freq: f
                                     float(pres), _stream()))
 
 
+@_op("sample_rows")
 def sample_rows(out_i32, logits, rows: int, uniforms_u32, temperature: float, top_k: int,
                 top_p: float) -> None:
     _need(logits, "logits", torch.float32)

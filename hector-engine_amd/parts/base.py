@@ -69,16 +69,25 @@ class ModelSpec:
     head: PartSpec
     head_prefix: str
     max_positions: int
+    # full names of tensors a model folder may hold although the model does not use them
+    # (an output matrix stored beside the embedding it is tied to)
+    unused_tensors: frozenset = frozenset()
 
 
 @dataclasses.dataclass(frozen=True)
 class KVNeed:
-    """What a mixer keeps per token in the cache: keys and values of this shape,
-    all of them (window 0) or only the last `window`."""
+    """What a mixer keeps per token in the cache: per kv head a key of `head_dim` and a value
+    of `value_dim` elements (0: as wide as the key), all of them (window 0) or only the last
+    `window`. Mixers with equal needs share a group of the cache."""
 
     kv_heads: int
     head_dim: int
     window: int = 0
+    value_dim: int = 0
+
+    @property
+    def v_dim(self) -> int:
+        return self.value_dim or self.head_dim
 
 
 @dataclasses.dataclass
@@ -227,6 +236,12 @@ class Block(Part):
     """Arrangement of a layer's parts around the residual stream."""
 
     mixer: Mixer
+
+    def first_norm(self) -> "Norm | None":
+        """The norm through which this block first reads the residual stream, when that is all
+        it reads the stream through before adding to it; None otherwise. The block that runs
+        before may then leave the stream as rows prepared for that norm (ResidualSink)."""
+        return None
 
     def forward(self, stream: "ResidualStream", ctx: StepContext, cache: LayerCache) -> None:
         raise NotImplementedError

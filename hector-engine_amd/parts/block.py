@@ -27,6 +27,9 @@ class PreNormBlock(Block):
     def children(self):
         return [self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward]
 
+    def first_norm(self):
+        return self.mixer_norm
+
     def tensor_specs(self):
         specs = {}
         for c in self.children():

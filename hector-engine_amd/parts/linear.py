@@ -36,7 +36,7 @@ from __future__ import annotations
 
 import torch
 
-from ..kernels import library_tuning, ops
+from ..kernels import library_tuning, ops, profiler
 from .base import NormedRows, PieceRows, ResidualSink, StepContext
 
 
@@ -168,7 +168,8 @@ class Linear:
     def _library(self, x, bias, rows, out, out_dtype, library_f32, ctx):
         w = self.weight
         if library_f32:
-            torch.mm(x[:rows], w.t(), out_dtype=torch.float32, out=out[:rows])
+            with profiler.span("library_gemm"):
+                torch.mm(x[:rows], w.t(), out_dtype=torch.float32, out=out[:rows])
             return out
         if out_dtype == torch.float32:
             # fp32 results of a tall product: 64 rows at a time through the MFMA kernel
@@ -176,10 +177,11 @@ class Linear:
                 r1 = min(rows, r0 + ops.SKINNY_MAX_M)
                 self._skinny(x[r0:r1], bias, r1 - r0, ctx, out[r0:r1], out_dtype, False)
             return out
-        if bias is not None:
-            torch.addmm(bias, x[:rows], w.t(), out=out[:rows])
-        else:
-            torch.mm(x[:rows], w.t(), out=out[:rows])
+        with profiler.span("library_gemm"):
+            if bias is not None:
+                torch.addmm(bias, x[:rows], w.t(), out=out[:rows])
+            else:
+                torch.mm(x[:rows], w.t(), out=out[:rows])
         return out
 
     def _into_residual(self, x, bias, rows, ctx, sink: ResidualSink):

@@ -81,11 +81,43 @@ def window_counts(context: list[int], window: int, vocab: int) -> tuple[list[int
     return list(counts.keys()), list(counts.values())
 
 
+class PendingIds:
+    """Ids on their way to the host: wait() gives them once their copy has arrived."""
+
+    def __init__(self, host: torch.Tensor, event):
+        self._host = host
+        self._event = event
+
+    def wait(self) -> list[int]:
+        if self._event is not None:
+            self._event.synchronize()
+        return self._host.tolist()
+
+
+READS_IN_FLIGHT = 64
+
+
 class Sampler:
     def __init__(self, config: SamplingConfig, device):
         config.validate()
         self.config = config
         self.device = device
+        self._ring: list[torch.Tensor | None] = [None] * READS_IN_FLIGHT   # pinned rows for read_later
+        self._ring_next = 0
+
+    def read_later(self, ids: torch.Tensor) -> PendingIds:
+        """Starts the copy of device ids (int32 [rows]) to pinned host memory without waiting
+        for it; at most READS_IN_FLIGHT such reads may be outstanding."""
+        i = self._ring_next
+        self._ring_next = (i + 1) % READS_IN_FLIGHT
+        n = ids.numel()
+        if self._ring[i] is None or self._ring[i].numel() < n:
+            self._ring[i] = torch.empty(max(256, n), dtype=torch.int32).pin_memory()
+        host = self._ring[i][:n]
+        host.copy_(ids, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        return PendingIds(host, event)
 
     def sample(self, logits: torch.Tensor, sequences: list[int], steps: list[int],
                contexts: list[list[int]] | None = None) -> list[int]:

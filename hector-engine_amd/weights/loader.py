@@ -9,6 +9,8 @@ everything becomes float32; integer tables are kept as int32.
 """
 from __future__ import annotations
 
+import warnings
+
 import torch
 
 from ..parts.base import TensorSpec
@@ -53,6 +55,10 @@ def load_tensors(model_dir: str, expected: dict[str, TensorSpec], run: torch.dty
                 raise WeightsError(f"tensor '{name}' is stored twice: {where[name].path} and {f.path}")
             where[name] = f
     check_against(expected, {n: f.shape(n) for n, f in where.items()}, allowed_extra)
+    ignored = sorted(n for n in where if n not in expected)
+    if ignored:     # allowed and unused (the reference decides by presence: src/graph_builder.cpp:250-253)
+        warnings.warn(f"{model_dir}: stored but not used by this configuration: {', '.join(ignored)}",
+                      stacklevel=2)
     out: dict[str, torch.Tensor] = {}
     for name, spec in expected.items():
         f = where[name]
@@ -61,5 +67,18 @@ def load_tensors(model_dir: str, expected: dict[str, TensorSpec], run: torch.dty
             kind = "an integer table" if spec.integer else "a floating-point tensor"
             raise WeightsError(f"tensor '{name}' is stored as {stored}, expected {kind}")
         target = run_dtype_of(stored, run, spec.integer)
-        out[name] = f.tensor(name).to(device=device, dtype=target).contiguous()
+        out[name] = _upload(f.tensor(name), target, torch.device(device))
+    return out
+
+
+def _upload(stored: torch.Tensor, target: torch.dtype, device: torch.device) -> torch.Tensor:
+    """The tensor on the device in the dtype it runs in. On the GPU the bytes go up as they are
+    stored and the conversion is the library's own kernel (bf16 -> f32 is the 16-bit shift of
+    tools/quant_bench/ref_qwen3.py:60; f32 -> bf16 rounds to nearest even)."""
+    if device.type != "cuda" or not stored.is_floating_point() or stored.dtype == target:
+        return stored.to(device=device, dtype=target).contiguous()
+    from ..kernels import ops
+    raw = stored.contiguous().to(device)
+    out = torch.empty(raw.shape, dtype=target, device=device)
+    ops.cast(out, raw)
     return out

@@ -55,7 +55,12 @@ class SafetensorsFile:
         for name, e in header.items():
             if e.get("dtype") not in _DTYPES:
                 raise WeightsError(f"{path}: tensor '{name}' has unsupported dtype {e.get('dtype')!r}")
-            a, b = e["data_offsets"]
+            try:
+                a, b = (int(x) for x in e["data_offsets"])
+            except (KeyError, TypeError, ValueError):
+                raise WeightsError(f"{path}: tensor '{name}' has no valid data_offsets") from None
+            if a < 0 or a > b:
+                raise WeightsError(f"{path}: tensor '{name}' has data_offsets [{a}, {b}]")
             count = int(np.prod(e["shape"], dtype=np.int64)) if e["shape"] else 1
             want = count * np.dtype(_DTYPES[e["dtype"]][0]).itemsize
             if b - a != want:

@@ -10,14 +10,14 @@ def rand_ids(vocab: int, n: int, seed: int) -> list[int]:
 
 def close(got: torch.Tensor, want: torch.Tensor, dtype: str) -> None:
     """float32: the engine's fp32 path against the float64 oracle, a few ulp of the
-    logits' size. bfloat16: 8 bits of mantissa at every rounding point; the bound
-    is 2 % of the largest logit, about four times what is observed."""
+    logits' size. bfloat16: 8 bits of mantissa at every rounding point; the bound is
+    1 % of the largest logit, twice the largest error seen over all tests that use it."""
     got = got.detach().cpu().double()
     want = want.double()
     assert got.shape == want.shape, (got.shape, want.shape)
     scale = want.abs().max().item()
     err = (got - want).abs().max().item()
-    tol = 2e-5 * max(scale, 1.0) if dtype == "float32" else 0.02 * scale
+    tol = 2e-5 * max(scale, 1.0) if dtype == "float32" else 0.01 * scale
     assert err <= tol, f"max error {err:.3g} above {tol:.3g} (logit scale {scale:.3g})"
 
 

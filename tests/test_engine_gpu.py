@@ -24,7 +24,7 @@ def engines(model_dirs):
     def get(name, dtype, **kw):
         key = (name, dtype, tuple(sorted(kw.items())))
         if key not in cache:
-            opts = dict(max_tokens=4096, max_slots=8, max_seq_len=1024)
+            opts = dict(max_tokens=4096, max_slots=8, max_seq_len=1024, beyond_max_positions=True)
             opts.update(kw)
             cache[key] = he.Engine(model_dirs[name], dtype=dtype, **opts)
         return cache[key]
@@ -358,7 +358,7 @@ def test_graph_replay_and_padding_change_no_result(model_dirs, plain_models, nam
     reqs = [rand_ids(vocab, n, 60 + n) for n in (40, 75, 12)]
     outs = []
     for graphs in (True, False):
-        eng = he.Engine(model_dirs[name], dtype=dtype, max_tokens=2048, max_slots=4, max_seq_len=512,
+        eng = he.Engine(model_dirs[name], dtype=dtype, max_tokens=2048, max_slots=4, max_seq_len=512, beyond_max_positions=True,
                         use_graphs=graphs)
         slots = [eng.acquire() for _ in reqs]
         eng.step([entry(s, r[:6], []) for s, r in zip(slots, reqs)])
@@ -431,7 +431,7 @@ def test_a_step_of_thousands_of_rows(model_dirs, plain_models, dtype):
     import hector_engine_amd as he
     name = "C"
     vocab = plain_models[name][0]["vocab_size"]
-    eng = he.Engine(model_dirs[name], dtype=dtype, max_tokens=24 * 448, max_slots=24, max_seq_len=448)
+    eng = he.Engine(model_dirs[name], dtype=dtype, max_tokens=24 * 448, max_slots=24, max_seq_len=448, beyond_max_positions=True)
     prompts = [rand_ids(vocab, 400 - (i % 3), 300 + i) for i in range(24)]
     slots = [eng.acquire() for _ in prompts]
     got = eng.step([entry(s, p, [0, len(p) - 1]) for s, p in zip(slots, prompts)])
@@ -446,3 +446,63 @@ def test_a_step_of_thousands_of_rows(model_dirs, plain_models, dtype):
         close(got2[i:i + 1], want[-1:], dtype)
     for s in slots:
         eng.release(s)
+
+
+def test_a_failed_capture_falls_back_to_eager_steps(model_dirs, plain_models, monkeypatch):
+    """When capturing the one-token step fails, the engine says so once and goes on without
+    graphs (the reference does the same: src/engine.cpp:233-261). The failure is made on the host:
+    torch's capture context is replaced by one that raises."""
+    import contextlib
+    import warnings
+    import hector_engine_amd as he
+    from hector_engine_amd.engine import engine as engine_module
+
+    @contextlib.contextmanager
+    def broken(graph):
+        raise RuntimeError("capture refused (made up by the test)")
+        yield
+
+    eng = he.Engine(model_dirs["D"], dtype="bfloat16", max_tokens=1024, max_slots=4)
+    monkeypatch.setattr(engine_module.torch.cuda, "graph", broken)
+    vocab = plain_models["D"][0]["vocab_size"]
+    ids = rand_ids(vocab, 30, 5)
+    want = plain_logits(plain_models, "D", ids)
+    s = eng.acquire()
+    eng.step([entry(s, ids[:10], [])])
+    rows = []
+    with warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        for t in ids[10:]:
+            rows.append(eng.step([entry(s, [t], [0])]).clone())
+    eng.release(s)
+    assert len([w for w in seen if "HIP graph failed" in str(w.message)]) == 1       # said once
+    assert eng.stats["graph_captures"] == 0 and eng.stats["graph_replays"] == 0
+    assert eng.stats["eager_steps"] == 21
+    close(torch.cat(rows), want[10:], "bfloat16")
+    # another bucket size after the failure: eager at once, no second attempt
+    a, b = eng.acquire(), eng.acquire()
+    for t in ids[:3]:
+        eng.step([entry(a, [t], [0]), entry(b, [t], [0])])
+    assert eng.stats["graph_captures"] == 0
+    eng.release(a), eng.release(b)
+
+
+def test_profile_mode_times_every_kernel(model_dirs):
+    """Engine(profile=True): every launch between two events, steps without graphs; the table names
+    the kernels with their calls, in the reference's columns."""
+    import hector_engine_amd as he
+    eng = he.Engine(model_dirs["D"], dtype="bfloat16", max_tokens=1024, max_slots=2, profile=True)
+    assert not eng.use_graphs
+    s = eng.acquire()
+    ids = rand_ids(200, 40, 9)
+    eng.step([entry(s, ids[:36], [35])])
+    for t in ids[36:]:
+        eng.step([entry(s, [t], [0])])
+    eng.release(s)
+    rows = {name: (calls, ms) for name, calls, ms, _, _ in eng.profiler.rows()}
+    assert rows["embedding"][0] == 5 and rows["attention_prefill"][0] == 2        # two layers, one prompt step
+    assert rows["attention_decode_fused"][0] == 8 and rows["gemm_blocksplit"][0] >= 4 * 2 * 4
+    assert all(ms > 0 for _, ms in rows.values())
+    text = eng.profile_summary()
+    assert text.startswith("=== Engine Profile ===") and "TOTAL" in text and "Avg(ms)" in text
+    assert eng.stats["graph_replays"] == 0

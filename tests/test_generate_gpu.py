@@ -30,7 +30,7 @@ def test_greedy_generation_equals_plain(he, model_dirs, plain_models, name, leng
     cfg, w = plain_models[name]
     prompts = prompts_for(cfg, lengths, 100)
     want = [P.generate(cfg, w, p, steps) for p in prompts]
-    eng = he.Engine(model_dirs[name], dtype="float32", max_tokens=2048, max_seq_len=512)
+    eng = he.Engine(model_dirs[name], dtype="float32", max_tokens=2048, max_seq_len=512, beyond_max_positions=True)
     got = he.generate(eng, prompts, max_new_tokens=steps)
     assert [r.tokens for r in got] == want
     assert all(r.finish_reason == "max_tokens" and r.prompt_tokens == len(p) for r, p in zip(got, prompts))
@@ -38,11 +38,11 @@ def test_greedy_generation_equals_plain(he, model_dirs, plain_models, name, leng
     for p, t in zip(prompts, want):
         assert he.generate(eng, [p], max_new_tokens=steps)[0].tokens == t
     assert [r.tokens for r in he.generate(eng, prompts[::-1], max_new_tokens=steps)] == want[::-1]
-    small = he.Engine(model_dirs[name], dtype="float32", max_tokens=2048, max_slots=2, max_seq_len=512)
+    small = he.Engine(model_dirs[name], dtype="float32", max_tokens=2048, max_slots=2, max_seq_len=512, beyond_max_positions=True)
     assert [r.tokens for r in he.generate(small, prompts, max_new_tokens=steps)] == want
     assert small.cache.free_pages == small.cache.num_pages
     # bfloat16: the same tokens wherever the oracle's choice is clear
-    eng16 = he.Engine(model_dirs[name], dtype="bfloat16", max_tokens=2048, max_seq_len=512)
+    eng16 = he.Engine(model_dirs[name], dtype="bfloat16", max_tokens=2048, max_seq_len=512, beyond_max_positions=True)
     got16 = he.generate(eng16, prompts, max_new_tokens=steps)
     for p, r, t in zip(prompts, got16, want):
         seq = list(p)
@@ -60,14 +60,14 @@ def test_greedy_generation_equals_plain(he, model_dirs, plain_models, name, leng
 def test_sampled_generation_equals_plain(he, model_dirs, plain_models, name, kw):
     cfg, w = plain_models[name]
     prompts = prompts_for(cfg, [3, 7, 17, 30], 200)
-    eng = he.Engine(model_dirs[name], dtype="float32", max_tokens=2048, max_seq_len=512)
+    eng = he.Engine(model_dirs[name], dtype="float32", max_tokens=2048, max_seq_len=512, beyond_max_positions=True)
     got = he.generate(eng, prompts, max_new_tokens=12, sampling=he.SamplingConfig(**kw))
     for i, (p, r) in enumerate(zip(prompts, got)):
         want = P.generate(cfg, w, p, 12, temperature=kw["temperature"], top_k=kw.get("top_k", 0),
                           top_p=kw.get("top_p", 1.0), seed=kw["seed"], sequence=i)
         assert r.tokens == want
     # the draw is keyed by the request's index, not by the batch: one slot at a time, same tokens
-    one = he.Engine(model_dirs[name], dtype="float32", max_tokens=2048, max_slots=1, max_seq_len=512)
+    one = he.Engine(model_dirs[name], dtype="float32", max_tokens=2048, max_slots=1, max_seq_len=512, beyond_max_positions=True)
     again = he.generate(one, prompts, max_new_tokens=12, sampling=he.SamplingConfig(**kw))
     assert [r.tokens for r in again] == [r.tokens for r in got]
 
@@ -115,7 +115,7 @@ def test_stop_tokens_and_early_finishers(he, model_dirs, plain_models):
     free = [P.generate(cfg, w, p, 12) for p in prompts]
     stop = {free[1][4], free[3][0]}                    # request 1 stops at its fifth token, request 3 at once
     want = [P.generate(cfg, w, p, 12, stop_ids=stop) for p in prompts]
-    eng = he.Engine(model_dirs["B"], dtype="float32", max_tokens=2048, max_seq_len=512)
+    eng = he.Engine(model_dirs["B"], dtype="float32", max_tokens=2048, max_seq_len=512, beyond_max_positions=True)
     got = he.generate(eng, prompts, max_new_tokens=12, stop_ids=stop)
     assert [r.tokens for r in got] == want
     assert got[3].finish_reason == "eos" and got[3].tokens == []
@@ -164,7 +164,7 @@ def test_a_step_takes_its_tokens_from_the_device(he, model_dirs):
 def test_penalties(he, model_dirs, plain_models):
     cfg, w = plain_models["A"]
     p = prompts_for(cfg, [9], 400)[0]
-    eng = he.Engine(model_dirs["A"], dtype="float32", max_tokens=1024, max_seq_len=512)
+    eng = he.Engine(model_dirs["A"], dtype="float32", max_tokens=1024, max_seq_len=512, beyond_max_positions=True)
     plainly = he.generate(eng, [p], max_new_tokens=16)[0].tokens
     cfg_s = he.SamplingConfig(temperature=0.0, repetition_penalty=1.3, frequency_penalty=0.2,
                               presence_penalty=0.1, penalty_window=6)
@@ -196,6 +196,42 @@ def test_command_line(model_dirs, plain_models):
     assert out.returncode == 0, out.stderr
     t = P.generate(cfg, w, [5, 17, 3], 6, temperature=0.8, seed=7)
     assert ",".join(map(str, t)) in out.stdout
+
+
+def test_command_line_flags(model_dirs, plain_models, tmp_path):
+    """--random CONFIG.json --seed (the model write_random_model writes from the same configuration
+    and seed), prompts from --tokens and --tokens-file, fewer slots than prompts, sampling flags in
+    place of the variables, the kernel table of --profile, and the context bound."""
+    import json
+    import hector_engine_amd as he
+    from hector_engine_amd.registry import config_from_dict
+    from tests.conftest import TINY_B
+    exe = os.path.join(ROOT, "bin", "hector_generate")
+    cfg_file = tmp_path / "config.json"
+    cfg_file.write_text(json.dumps(TINY_B))
+    folder = str(tmp_path / "model")
+    he.write_random_model(config_from_dict(dict(TINY_B)), 21, folder, "bfloat16")
+    cfg, w = P.read_model(folder)
+    prompts = [[5, 17, 3], [9, 2, 77, 13], [100, 200, 300, 1, 2]]
+    tokens_file = tmp_path / "prompts.txt"
+    tokens_file.write_text("9,2,77,13\n100 200 300 1 2\n")
+    out = subprocess.run([sys.executable, exe, "--random", str(cfg_file), "--seed", "21", "--tokens", "5,17,3",
+                          "--tokens-file", str(tokens_file), "--max-new-tokens", "7", "--temperature", "0.8",
+                          "--top-k", "0", "--top-p", "1.0", "--sampler-seed", "7", "--slots", "2", "--dtype", "float32",
+                          "--profile"], capture_output=True, text=True, timeout=180)
+    assert out.returncode == 0, out.stderr
+    for i, p in enumerate(prompts):
+        t = P.generate(cfg, w, p, 7, temperature=0.8, seed=7, sequence=i)
+        assert f"[{i}] prompt {len(p)} tokens -> 7 tokens (max_tokens): " + ",".join(map(str, t)) in out.stdout
+    assert "=== Engine Profile ===" in out.stdout and "attention_plain" in out.stdout and "TOTAL" in out.stdout
+    assert "random weights for" in out.stdout and "seed 21" in out.stdout
+    # more context than the configuration's positions is refused by name; within them --max-seq holds
+    out = subprocess.run([sys.executable, exe, folder, "5,17,3", "2", "--max-seq", "1000"], capture_output=True,
+                         text=True, timeout=120)
+    assert out.returncode != 0 and "256 positions" in out.stderr
+    out = subprocess.run([sys.executable, exe, folder, "5,17,3", "40", "--max-seq", "16", "--dtype", "float32"],
+                         capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0 and "-> 14 tokens (stop)" in out.stdout, out.stdout + out.stderr
 
 
 def test_command_line_with_the_library_tuner(model_dirs, tmp_path):

@@ -44,14 +44,16 @@ class FakeEngine:
     def length(self, s):
         return self.cache.book.length[s]
 
-    def step(self, entries):
+    def step(self, entries, device_tokens=None):
+        """device_tokens: as the engine takes them, the tokens of a one-token step in place of
+        the entries' own (here a plain list: the fake has no device)."""
         self.log.append([(e.slot, len(e.tokens)) for e in entries])
         rows = []
-        for e in entries:
+        for k, e in enumerate(entries):
             new = self.length(e.slot) + len(e.tokens)
             self.cache.book.reserve(e.slot, new)
             self.cache.book.commit(e.slot, new)
-            self.history[e.slot] += list(e.tokens)
+            self.history[e.slot] += list(e.tokens) if device_tokens is None else [device_tokens[k]]
             assert list(e.want) == [len(e.tokens) - 1]
             h = self.history[e.slot]
             rows.append((sum(h) + len(h)) % V)
@@ -61,6 +63,31 @@ class FakeEngine:
 
 def pick(rows, sequences, steps, contexts):
     return list(rows)
+
+
+class FakeSampler:
+    """The library sampler's interface without a device: ids are plain lists, and a read of
+    them is ready at once. `reads` counts how often the loop looked at a step's ids."""
+
+    def __init__(self):
+        from hector_engine_amd.sampling import SamplingConfig
+        self.config = SamplingConfig.deterministic()
+        self.waits = 0
+
+    def sample(self, rows, sequences, steps, contexts=None):
+        return list(rows)
+
+    def sample_device(self, rows, sequences, steps, contexts=None, uniforms=None):
+        return list(rows)
+
+    def read_later(self, ids):
+        outer = self
+
+        class Ready:
+            def wait(self):
+                outer.waits += 1
+                return list(ids)
+        return Ready()
 
 
 def expected(prompt, n, stop=()):
@@ -168,3 +195,55 @@ def test_steps_in_run():
     assert steps_in_run([99], [10], 100, 256, 8) == 1
     assert steps_in_run([3], [256], 100, 256, 8) == 1                 # the loop ends such a sequence before
     assert steps_in_run([1], [10], 100, 256, 1) == 1
+
+
+def test_a_stop_token_inside_a_run_of_queued_steps():
+    """Three requests through two slots, eight steps queued at a time. Request 0 samples its stop
+    token as its second token, early in a run: it is stepped once more at most (the step that was
+    queued when the host read the token), then its slot and pages are back and the batch goes on
+    without it; the waiting request starts when that batch has ended, in the slots it gave back;
+    every result equals one step at a time."""
+    prompts = [[1, 2, 3], [4] * 9, [7, 7, 7, 7, 7]]
+    stop = {expected(prompts[0], 2)[0][1]}            # the second token of request 0
+    assert all(t not in stop for p in prompts[1:] for t in expected(p, 12)[0])
+    one = generate(FakeEngine(slots=2), prompts, max_new_tokens=12, stop_ids=stop, sampler=FakeSampler(),
+                   run_of_steps=1)
+    eng = FakeEngine(slots=2)
+    many = generate(eng, prompts, max_new_tokens=12, stop_ids=stop, sampler=FakeSampler(), run_of_steps=8)
+    assert [(r.tokens, r.finish_reason) for r in many] == [(r.tokens, r.finish_reason) for r in one]
+    assert many[0].finish_reason == "eos" and len(many[0].tokens) == 1
+    assert [(r.tokens, r.finish_reason) for r in many[1:]] == [expected(p, 12) for p in prompts[1:]]
+    # step 0: both prompts. Request 0's first token is fed in step 1, which samples the stop token;
+    # step 2 was queued before the host read it; from step 3 on request 1 runs alone.
+    first_batch = [step for step in eng.log[:1 + 11]]
+    assert [n for _, n in first_batch[0]] == [3, 9]
+    assert [len(step) for step in first_batch[1:]] == [2, 2] + [1] * 9
+    # the third request starts right after, alone, in the lowest slot
+    assert eng.log[12] == [(0, 5)] and all(len(step) == 1 for step in eng.log[12:])
+    assert len(eng.log) == 12 + 12
+    assert eng.cache.book.slots.available == 2 and eng.cache.free_pages == 16 and not eng.history
+
+
+def test_runs_without_stop_ids_read_their_ids_once():
+    """Nothing can end a sequence inside a run but its budget: the run is never cut and reaches
+    exactly to the budget."""
+    eng, sampler = FakeEngine(), FakeSampler()
+    prompts = [[1, 2, 3], [5, 5]]
+    res = generate(eng, prompts, max_new_tokens=11, sampler=sampler, run_of_steps=8)
+    assert [(r.tokens, r.finish_reason) for r in res] == [expected(p, 11) for p in prompts]
+    assert len(eng.log) == 1 + 10            # the prompt step and ten one-token steps, none wasted
+    assert eng.cache.book.slots.available == 3
+
+
+def test_cancel_is_seen_inside_a_run():
+    eng = FakeEngine()
+    calls = {"n": 0}
+
+    def cancel():
+        calls["n"] += 1
+        return calls["n"] > 3
+
+    r = generate(eng, [[1, 2]], max_new_tokens=50, cancel=cancel, sampler=FakeSampler(), run_of_steps=8)[0]
+    assert r.finish_reason == "cancelled" and 1 <= len(r.tokens) <= 5
+    assert r.tokens == expected([1, 2], len(r.tokens))[0]
+    assert eng.cache.book.slots.available == 3 and eng.cache.free_pages == 16

@@ -285,6 +285,96 @@ def toys(fw):
                 r += n
             return out
 
+    @parts.register_part("mixer", "toy_running_mean_on_device")
+    class RunningMeanOnDevice(parts.Mixer):
+        """The same mixer, planned on the device: its state rows are found through ctx.seq_slot
+        and updated by index there, so that one-token steps can be captured into HIP graphs.
+        Padding rows (row_seq -1) add zeros to a row of the state."""
+
+        def __init__(self, params, prefix, env):
+            super().__init__(prefix, env)
+            self.D = parts.param(params, "hidden_size", int)
+
+        def state_bytes(self):
+            return 4 * (self.D + 1)
+
+        def tensor_specs(self):
+            return {self.prefix + "out.weight": parts.TensorSpec((self.D, self.D))}
+
+        def bind(self, tensors):
+            self.w = tensors[self.prefix + "out.weight"].float()
+
+        def forward(self, x, ctx, cache):
+            D, rows = self.D, ctx.rows
+            st = cache.state.view(torch.float32)                       # [slots, D + 1]
+            seq = ctx.row_seq[:rows].long()
+            valid = seq >= 0
+            seq = seq.clamp(min=0)
+            slot = ctx.seq_slot.long()[seq].clamp(min=0)
+            xf = x[:rows].float() * valid[:, None]
+            ones = valid.float()
+            if ctx.all_single:
+                within, place = xf, ones
+            else:     # sums over the rows of each sequence up to each row, without a trip to the host
+                c = xf.double().cumsum(0)
+                start = ctx.cu_seqlens.long()[seq]
+                before = torch.where((start > 0)[:, None], c[(start - 1).clamp(min=0)], torch.zeros_like(c))
+                within = (c - before).float()
+                place = (torch.arange(rows, device=x.device) - start + 1).float() * ones
+            sums = st[slot, :D] + within
+            counts = (st[slot, D] + place).clamp(min=1)
+            out = ctx.alloc((rows, D))
+            out.copy_(((sums / counts[:, None]) @ self.w.T).to(out.dtype))
+            st.index_add_(0, slot, torch.cat([xf, ones[:, None]], 1))
+            return out
+
+    @parts.register_part("mixer", "toy_wide_values")
+    class WideValues(parts.Mixer):
+        """One head whose keys are 16 wide and whose values are 32 wide, kept in cache pages of
+        its own group: it writes and reads them by index, in the layout the cache documents."""
+        graph_safe = False
+
+        def __init__(self, params, prefix, env):
+            super().__init__(prefix, env)
+            self.D = parts.param(params, "hidden_size", int)
+
+        def kv_need(self):
+            return parts.KVNeed(1, 16, 0, value_dim=32)
+
+        def tensor_specs(self):
+            p = self.prefix
+            return {p + "q.weight": parts.TensorSpec((16, self.D)), p + "k.weight": parts.TensorSpec((16, self.D)),
+                    p + "v.weight": parts.TensorSpec((32, self.D)), p + "o.weight": parts.TensorSpec((self.D, 32))}
+
+        def bind(self, tensors):
+            self.t = {n: tensors[self.prefix + n + ".weight"].float() for n in "qkvo"}
+
+        def forward(self, x, ctx, cache):
+            from tests.test_kernels_gpu import page_maps
+            km, vm = page_maps(16)[0].cuda(), page_maps(32)[1].cuda()
+            assert cache.kpool.shape[-1] == 64 * 32 and cache.vpool.shape[-1] == 64 * 32   # 16 -> one k step; 2 dim tiles
+            xf = x[:ctx.rows].float()
+            q, k, v = xf @ self.t["q"].T, xf @ self.t["k"].T, xf @ self.t["v"].T
+            out = ctx.alloc((ctx.rows, self.D))
+            r = 0
+            for n, start, slot in zip(ctx.host["q_lens"], ctx.host["starts"], ctx.host["slots"]):
+                table = cache.page_table[slot]
+                for j in range(n):
+                    p = start + j
+                    cache.kpool[table[p // 64], 0, km[p % 64]] = k[r + j].to(cache.kpool.dtype)
+                    cache.vpool[table[p // 64], 0, vm[p % 64]] = v[r + j].to(cache.vpool.dtype)
+                total = start + n
+                pos = torch.arange(total, device=x.device)
+                pages = table[pos // 64].long()
+                keys = cache.kpool[pages, 0][torch.arange(total, device=x.device)[:, None], km[pos % 64]].float()
+                vals = cache.vpool[pages, 0][torch.arange(total, device=x.device)[:, None], vm[pos % 64]].float()
+                scores = q[r:r + n] @ keys.T / 4.0
+                seen = pos[None, :] <= (start + torch.arange(n, device=x.device))[:, None]
+                w = torch.softmax(scores.masked_fill(~seen, float("-inf")), -1)
+                out[r:r + n] = ((w @ vals) @ self.t["o"].T).to(out.dtype)
+                r += n
+            return out
+
     @parts.register_part("position", "toy_scale_by_position")
     class ScaleByPosition(parts.PositionEncoding):
         """q, k <- q, k * (1 + pos / 100): not a rotation, so it runs through apply()."""
@@ -378,6 +468,9 @@ def toys(fw):
         def children(self):
             return [self.norm, self.mixer, self.feed_forward]
 
+        def first_norm(self):
+            return self.norm           # all it reads the stream through
+
         def tensor_specs(self):
             specs = {}
             for c in self.children():
@@ -424,8 +517,10 @@ def toys(fw):
 
         rotary = parts.PartSpec("rotary", {"head_dim": 16, "theta": 1e4})
         routed = parts.PartSpec("toy_top1_experts", {"hidden_size": D, "intermediate_size": D + 16, "experts": 3})
-        if cfg.kind == "state":
-            mixers = [attn(rotary), parts.PartSpec("toy_running_mean", {"hidden_size": D}), attn(rotary)]
+        if cfg.kind in ("state", "device_state", "wide_values"):
+            middle = {"state": "toy_running_mean", "device_state": "toy_running_mean_on_device",
+                      "wide_values": "toy_wide_values"}[cfg.kind]
+            mixers = [attn(rotary), parts.PartSpec(middle, {"hidden_size": D}), attn(rotary)]
             schedule = [parts.ScheduleEntry(0), parts.ScheduleEntry(1), parts.ScheduleEntry(2)]
         elif cfg.kind == "position":
             mixers = [attn(parts.PartSpec("toy_scale_by_position")), attn(parts.PartSpec("none"))]
@@ -441,8 +536,8 @@ def toys(fw):
             schedule = [parts.ScheduleEntry(0), parts.ScheduleEntry(1), parts.ScheduleEntry(1, cache_from=1)]
         layers = [parts.LayerSpec(f"layers.{i}.", block(m, routed if cfg.kind == "routed" and i == 1 else ff))
                   for i, m in enumerate(mixers)]
-        if cfg.kind == "parallel":   # another norm and another arrangement: a parallel block between pre-norm blocks
-            centered = parts.PartSpec("toy_centered", {"size": D, "eps": 1e-4})
+        if cfg.kind in ("parallel", "parallel_rms"):   # another arrangement (and another norm) between pre-norm blocks
+            centered = parts.PartSpec("toy_centered", {"size": D, "eps": 1e-4}) if cfg.kind == "parallel" else norm
             layers = [parts.LayerSpec("layers.0.", block(attn(rotary))),
                       parts.LayerSpec("layers.1.", parts.PartSpec("toy_parallel", {"norm": centered, "mixer": attn(rotary),
                                                                                    "feed_forward": ff})),
@@ -498,8 +593,10 @@ def toy_plain(w, kind, ids):
     rot = lambda t: P.rope(t, pos, 1e4)
     scale = lambda t: t * (1 + pos.double() / 100)[:, None, None]
     same = lambda t: t
-    if kind == "parallel":
+    if kind in ("parallel", "parallel_rms"):
         def centered(h, g):
+            if kind == "parallel_rms":
+                return P.rmsnorm(h, g, 1e-5)
             c = h - h.mean(-1, keepdim=True)
             return c / torch.sqrt((c * c).mean(-1, keepdim=True) + 1e-4) * g
 
@@ -511,8 +608,10 @@ def toy_plain(w, kind, ids):
         x = x + attn(1, n, rot)[0] + mlp(1, n)
         x = ff(2, x + attn(2, centered(x, w["layers.2.ln1.weight"]), rot)[0])
         return P.linear(P.rmsnorm(x, w["norm.weight"], 1e-5), w["head.weight"])
-    if kind == "state":
+    if kind in ("state", "device_state"):
         runs = [(0, rot, None), (1, "mean", None), (2, rot, None)]
+    elif kind == "wide_values":
+        runs = [(0, rot, None), (1, "wide", None), (2, rot, None)]
     elif kind == "position":
         runs = [(0, scale, None), (1, same, None)]
     elif kind == "twice":
@@ -526,6 +625,11 @@ def toy_plain(w, kind, ids):
         n = P.rmsnorm(x, w[f"layers.{l}.ln1.weight"], 1e-5)
         if enc == "mean":
             a = (n.cumsum(0) / torch.arange(1, S + 1)[:, None]) @ w[f"layers.{l}.mix.out.weight"].T
+        elif enc == "wide":      # one head, keys of 16 and values of 32, scale 1/4, causal
+            m = f"layers.{l}.mix."
+            scores = (n @ w[m + "q.weight"].T) @ (n @ w[m + "k.weight"].T).T / 4.0
+            scores = scores.masked_fill(pos[None, :] > pos[:, None], float("-inf"))
+            a = (torch.softmax(scores, -1) @ (n @ w[m + "v.weight"].T)) @ w[m + "o.weight"].T
         else:
             a, kvs[e] = attn(l, n, enc, kvs[src] if src is not None else None)
         x = ff(l, x + a)
@@ -536,7 +640,7 @@ def toy_plain(w, kind, ids):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("kind", ["state", "position", "twice", "shared", "parallel"])
+@pytest.mark.parametrize("kind", ["state", "position", "twice", "shared", "parallel", "parallel_rms", "wide_values"])
 def test_toy_models_build_and_step(fw, toys, tmp_path, kind, dtype):
     import hector_engine_amd as he
     from hector_engine_amd.engine.engine import StepEntry
@@ -546,7 +650,14 @@ def test_toy_models_build_and_step(fw, toys, tmp_path, kind, dtype):
     assert he.load_config(folder) == cfg
     w = {k: v.double() for k, v in P.read_safetensors(os.path.join(folder, "model.safetensors")).items()}
     eng = he.Engine(folder, dtype=dtype, max_tokens=1024, max_slots=2, max_seq_len=256)
-    assert eng.use_graphs == (kind != "state")            # the host-planning toy switches graphs off
+    assert eng.use_graphs == (kind not in ("state", "wide_values"))     # the host-planning toys switch graphs off
+    if kind == "wide_values":      # keys of 16 and values of 32: a cache group of its own, beside the attention layers'
+        assert len(eng.cache.groups) == 2 and [len(g.runs) for g in eng.cache.groups] == [2, 1]
+        need = eng.cache.groups[1].need
+        assert (need.head_dim, need.v_dim) == (16, 32) and eng.cache.groups[0].need.v_dim == 16
+        assert eng.cache.groups[1].vpool.shape[-1] == 64 * 32 and eng.cache.groups[0].vpool.shape[-1] == 64 * 16
+    if kind.startswith("parallel"):
+        assert eng.model.blocks[1].first_norm() is eng.model.blocks[1].norm
     if kind == "state":
         assert eng.cache.state_bytes_per_slot >= 4 * 65 and eng.model.run_plans()[1].kv is None
         assert len(eng.cache.groups) == 1 and len(eng.cache.groups[0].runs) == 2
@@ -631,3 +742,44 @@ def test_bad_schedules_are_refused(fw, toys):
         DecoderModel(spec, env)
     with pytest.raises(KeyError, match="registered"):
         fw.parts.build_part("mixer", fw.parts.PartSpec("no_such_mixer"), "", env)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_state_of_fixed_size_under_graph_replay(fw, toys, tmp_path, dtype):
+    """A mixer with state of its own that finds and updates its rows on the device through
+    seq_slot: its one-token steps are captured and replayed (three sequences in a bucket of four:
+    one padding row), every replay is compared with the plain implementation, and a second batch
+    takes the slots, and the state rows, that the first gave back."""
+    import hector_engine_amd as he
+    from hector_engine_amd.engine.engine import StepEntry
+    cfg = toys(architecture="ToyForCausalLM", vocab_size=97, hidden_size=64, kind="device_state")
+    folder = str(tmp_path / "device_state")
+    he.write_random_model(cfg, 8, folder)
+    w = {k: v.double() for k, v in P.read_safetensors(os.path.join(folder, "model.safetensors")).items()}
+    eng = he.Engine(folder, dtype=dtype, max_tokens=2048, max_slots=4, max_seq_len=256)
+    assert eng.use_graphs and eng.cache.state_bytes_per_slot >= 4 * 65
+    reqs = [rand_ids(97, n, 170 + n) for n in (40, 23, 31, 37, 18, 29)]
+    want = [toy_plain(w, "device_state", r) for r in reqs]
+    for batch in ([0, 1, 2], [3, 4, 5]):
+        slots = {i: eng.acquire() for i in batch}
+        fed = {i: 5 + i for i in batch}
+        got = {i: [] for i in batch}
+        logits = eng.step([StepEntry(slots[i], reqs[i][:fed[i]], list(range(fed[i]))) for i in batch])
+        r0 = 0
+        for i in batch:
+            got[i].append(logits[r0:r0 + fed[i]].clone())
+            r0 += fed[i]
+        live = list(batch)
+        while live:
+            logits = eng.step([StepEntry(slots[i], [reqs[i][fed[i]]], [0]) for i in live])
+            for j, i in enumerate(live):
+                close(logits[j:j + 1], want[i][fed[i]:fed[i] + 1], dtype)     # each replay on its own
+                got[i].append(logits[j:j + 1].clone())
+                fed[i] += 1
+            for i in list(live):
+                if fed[i] == len(reqs[i]):
+                    eng.release(slots.pop(i))
+                    live.remove(i)
+        for i in batch:
+            close(torch.cat(got[i]), want[i], dtype)
+    assert eng.stats["graph_replays"] > 40 and eng.stats["graph_captures"] >= 2

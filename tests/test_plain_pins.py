@@ -213,6 +213,78 @@ def test_a_zeroed_layer_is_the_identity_and_window_only_acts_where_configured():
     assert P.layer_window(cfgw, 0) == 0 and P.layer_window(cfgw, 1) == 4
 
 
+def test_the_final_norm_stands_directly_before_the_head():
+    """A zero gain of model.norm gives zero logits; twice the gain, twice the logits (the head is
+    linear and nothing stands between): src/graph_builder.cpp:1014-1036."""
+    for tied in (False, True):
+        cfg, w = tiny_model(tied=tied)
+        ids = [3, 14, 15, 9, 2]
+        a = P.forward(cfg, w, ids)
+        assert a.abs().max() > 0.1
+        z = dict(w)
+        z["model.norm.weight"] = torch.zeros_like(w["model.norm.weight"])
+        assert P.forward(cfg, z, ids).abs().max() == 0
+        d = dict(w)
+        d["model.norm.weight"] = 2 * w["model.norm.weight"]
+        assert torch.allclose(P.forward(cfg, d, ids), 2 * a, atol=1e-12)
+        # it normalises: scaling the last layer's output barely moves the logits (eps aside)
+        m = dict(w)
+        m["model.layers.1.mlp.down_proj.weight"] = torch.zeros_like(w["model.layers.1.mlp.down_proj.weight"])
+        m["model.layers.1.self_attn.o_proj.weight"] = torch.zeros_like(w["model.layers.1.self_attn.o_proj.weight"])
+        head = w["model.embed_tokens.weight"] if tied else w["lm_head.weight"]
+        x = P.forward(dict(cfg, num_hidden_layers=1), m, ids)        # the same model: layer 1 is the identity
+        assert torch.allclose(P.forward(cfg, m, ids), x, atol=1e-12)
+        assert x.shape == (5, head.shape[0])
+
+
+def test_the_second_norm_stands_between_the_attention_residual_and_the_feed_forward():
+    """One layer, put together by hand from the parts: x1 = x + attention(norm1(x)),
+    x2 = x1 + mlp(norm2(x1)) (src/graph_builder.cpp:1195, :1366-1396, :1415-1443,
+    kernels/fused_add_rmsnorm.cu:47-81). A zero gain of norm 2 removes the feed-forward alone; twice
+    the gain is twice the feed-forward's input, which is not twice its output (a norm behind the
+    feed-forward, or on the residual before the attention was added, fails one of these)."""
+    cfg, w = tiny_model(tied=False, layers=1)
+    ids = [7, 1, 30, 22, 5, 48]
+    pos = torch.arange(len(ids))
+    eps = cfg["rms_norm_eps"]
+    p = "model.layers.0."
+    x = P.embedding(torch.tensor(ids), w["model.embed_tokens.weight"])
+    a, _ = P.attention_block(cfg, w, p + "self_attn.", P.rmsnorm(x, w[p + "input_layernorm.weight"], eps), pos, 0)
+    x1 = x + a
+
+    def by_hand(gain):
+        n2 = P.rmsnorm(x1, gain, eps)
+        x2 = x1 + P.swiglu(n2, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+        return P.linear(P.rmsnorm(x2, w["model.norm.weight"], eps), w["lm_head.weight"])
+
+    g = w[p + "post_attention_layernorm.weight"]
+    for gain in (g, torch.zeros_like(g), 2 * g):
+        v = dict(w)
+        v[p + "post_attention_layernorm.weight"] = gain
+        assert torch.allclose(P.forward(cfg, v, ids), by_hand(gain), atol=1e-12)
+    assert not torch.allclose(by_hand(2 * g), by_hand(g), atol=1e-3)
+    no_ff = P.linear(P.rmsnorm(x1, w["model.norm.weight"], eps), w["lm_head.weight"])
+    assert torch.allclose(by_hand(torch.zeros_like(g)), no_ff, atol=1e-12)
+    # with the attention's output zeroed, x1 is the embedding itself
+    v = dict(w)
+    v[p + "self_attn.o_proj.weight"] = torch.zeros_like(w[p + "self_attn.o_proj.weight"])
+    n2 = P.rmsnorm(x, g, eps)
+    x2 = x + P.swiglu(n2, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    want = P.linear(P.rmsnorm(x2, w["model.norm.weight"], eps), w["lm_head.weight"])
+    assert torch.allclose(P.forward(cfg, v, ids), want, atol=1e-12)
+
+
+def test_greedy_below_a_temperature_of_one_hundredth():
+    """temperature < 0.01 is greedy (src/sampler.cpp:141): at 0.009 the seed does not matter, at
+    0.01 the draw is made (and, that cold, still lands on the maximum unless two logits tie)."""
+    cfg, w = tiny_model(tied=False)
+    greedy = P.generate(cfg, w, [1, 2, 3], 6)
+    assert P.generate(cfg, w, [1, 2, 3], 6, temperature=0.009, seed=5) == greedy
+    logits = torch.tensor([1.0, 1.0, 0.0])           # a tie: greedy takes the first, a draw may take the second
+    assert P.argmax_lowest(logits) == 0
+    assert P.sample(logits, 0.01, 0, 1.0, 2 ** 32 - 1) == 1
+
+
 def test_schedule_and_shared_cache_variants():
     cfg, w = tiny_model(tied=False, layers=2)
     ids = [4, 8, 15, 16, 23, 42]

@@ -3,7 +3,8 @@ command line's argument rules, all on the CPU."""
 import pytest
 
 import hector_engine_amd  # noqa: F401
-from hector_engine_amd.cli import is_plain_number, parse_args, parse_prompts
+from hector_engine_amd.cli import (context_length, gather_prompts, is_plain_number, parse_args, parse_prompts,
+                                   sampling_options)
 from hector_engine_amd.sampling import SamplingConfig, uniform_u32, window_counts
 from tests.plain import qwen2_plain as P
 
@@ -59,6 +60,57 @@ def test_cli_argument_rules():
     assert (model, ns.ctx, temp) == ("m", 512, 0.7)
     assert parse_prompts("5,17,3;9 2") == [[5, 17, 3], [9, 2]]
     assert parse_prompts("raw:1,2") == [[1, 2]]
+
+
+def test_cli_flags(tmp_path, monkeypatch):
+    """Every flag of the command line: random weights from a configuration file and a seed,
+    prompts from --tokens (repeated) and from a file, sampling options (a flag wins over the
+    reference's HELIOS_* variable, which wins over the default), context and slots, profiling."""
+    ns, model, prompt, max_tokens, temp = parse_args(
+        ["--random", "cfg.json", "--seed", "9", "--tokens", "1,2,3", "--tokens", "4 5", "--max-new-tokens", "7",
+         "--temperature", "0.8", "--top-k", "20", "--top-p", "0.5", "--sampler-seed", "3", "--max-seq", "256",
+         "--slots", "2", "--profile", "--dtype", "float32", "--stop-ids", "5,6", "--no-graph"])
+    assert (model, ns.random, ns.seed, prompt, max_tokens, temp) == (None, "cfg.json", 9, None, 7, 0.8)
+    assert (ns.ctx, ns.slots, ns.profile, ns.dtype, ns.stop_ids, ns.no_graph) == (256, 2, True, "float32", "5,6", True)
+    f = tmp_path / "prompts.txt"
+    f.write_text("7,8,9\n\n# a comment\n10 11  # two ids\n")
+    ns.tokens_file = str(f)
+    assert gather_prompts(ns, "12;13,14") == [[1, 2, 3], [4, 5], [7, 8, 9], [10, 11], [12], [13, 14]]
+    opts = sampling_options(ns, temp)
+    assert (opts["top_k"], opts["top_p"], opts["seed"], opts["temperature"]) == (20, 0.5, 3, 0.8)
+    # variables of the reference's session stand in for absent flags; flags win
+    for k, v in (("HELIOS_TOPK", "11"), ("HELIOS_TOPP", "0.7"), ("HELIOS_SEED", "5"), ("HELIOS_REP", "1.3"),
+                 ("HELIOS_FREQ", "0.2"), ("HELIOS_WINDOW", "64"), ("HELIOS_CTX", "1000")):
+        monkeypatch.setenv(k, v)
+    assert sampling_options(ns, temp)["top_k"] == 20
+    ns2, *_ = parse_args(["m", "1,2", "5", "0.9"])
+    o2 = sampling_options(ns2, 0.9)
+    assert (o2["top_k"], o2["top_p"], o2["seed"], o2["repetition_penalty"], o2["frequency_penalty"],
+            o2["penalty_window"]) == (11, 0.7, 5, 1.3, 0.2, 64)
+    greedy = sampling_options(ns2, 0.0)
+    assert (greedy["top_k"], greedy["top_p"]) == (0, 1.0)            # no truncation without sampling
+    # the context: the flag as given; else HELIOS_CTX or 4096, never beyond what the model allows
+    assert context_length(ns, 128) == 256 and context_length(ns2, 128) == 128 and context_length(ns2, 32768) == 1000
+    monkeypatch.delenv("HELIOS_CTX")
+    assert context_length(ns2, 32768) == 4096
+    with pytest.raises(SystemExit):
+        parse_args(["--model", "m", "--random", "c.json"])
+    with pytest.raises(SystemExit):
+        parse_args([])
+
+
+def test_profile_table_has_the_references_columns():
+    """Calls, total, average and share per op, largest total first, and a total line
+    (src/engine.cpp:393-434)."""
+    from hector_engine_amd.kernels.profiler import format_table, summarize
+    rows = summarize({"gemm_blocksplit": (112, 5.6), "attention_decode_fused": (28, 0.7), "never": (0, 0.0)}, 6.3)
+    assert [r[0] for r in rows] == ["gemm_blocksplit", "attention_decode_fused"]
+    assert rows[0][1:] == (112, 5.6, pytest.approx(0.05), pytest.approx(100 * 5.6 / 6.3))
+    text = format_table(rows).splitlines()
+    assert text[0] == "=== Engine Profile ===" and text[1].split() == ["Op", "Calls", "Total(ms)", "Avg(ms)", "%"]
+    assert text[3].split() == ["gemm_blocksplit", "112", "5.60", "0.050", "88.9%"]
+    assert text[-1].split() == ["TOTAL", "6.30"]
+    assert format_table([]) == "No profiling data"
 
 
 def test_bench_refuses_more_than_one_gpu_and_what_does_not_fit():
