@@ -115,7 +115,7 @@ def main() -> int:
     progress(f"{MODEL}: random weights, {args.layers} layers")
     cfg_dict = dict(SHAPE, num_hidden_layers=args.layers, architectures=["Qwen2ForCausalLM"])
     config = Qwen2Config.from_dict(cfg_dict)
-    max_batch = args.batch if args.no_points else max(args.batch, BIG_BATCH)
+    max_batch = 2 * args.batch if args.no_points else max(2 * args.batch, BIG_BATCH)
     t_load = time.perf_counter()
     engine = he.Engine(config=config, seed=0, dtype="bfloat16", max_tokens=max_batch * CONTEXT,
                        max_slots=max_batch, max_seq_len=CONTEXT, tune_library=not args.no_tune)
@@ -148,6 +148,10 @@ def main() -> int:
         slots = [engine.acquire() for _ in range(batch)]
         ps = prompts(batch, PROMPT_LO, PROMPT_HI)
         if batch == args.batch and batch <= 8:      # the packed prompt step of the headline batch, timed
+            warm = [engine.acquire() for _ in range(batch)]     # once untimed: the library's first call of a shape
+            prefill(ps, warm)
+            for s in warm:
+                engine.release(s)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             toks = prefill(ps, slots)

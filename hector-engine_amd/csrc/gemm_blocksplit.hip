@@ -2,8 +2,8 @@
 // C[M,N] = X[M,K] * W[N,K]^T (+ bias), or the gated activation of a gate||up
 // weight. One workgroup owns up to 16*R weight rows (the rows are dealt out evenly over the
 // compute units, see blocksplit_plan); its NW wavefronts take one K slice
-// each (operands straight from global memory into the MFMA registers, as in
-// gemm_skinny.hip, whose operand layout this kernel shares), leave their fp32
+// each (operands straight from global memory into the MFMA registers, in the operand
+// layout gemm_rows.hip describes), leave their fp32
 // tiles in LDS, and the workgroup adds the slices in wavefront order and writes
 // the result. The sum is complete inside one launch: no partial sums in global
 // memory, no second kernel, no atomics, and the order of the additions is fixed.

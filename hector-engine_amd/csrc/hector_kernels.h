@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 16
+#define HE_ABI_VERSION 18
 
 #ifdef __cplusplus
 extern "C" {
@@ -37,11 +37,8 @@ int he_silu_mul(void* out, const void* gate_up, int rows, int I, int interleaved
 
 // ---- norms ---------------------------------------------------------------
 // resid (fp32, in place) += delta (may be null); out (may be null) = rmsnorm(resid) * weight.
-// delta_splits > 0: delta is fp32 [delta_splits][rows][D], the K slices of a product, added
-// in index order together with delta_bias[D] (may be null).
-int he_add_rmsnorm(void* resid_f32, const void* delta, int delta_splits, const void* delta_bias,
-                   int bias_dtype, const void* weight, void* out, int rows, int D, float eps,
-                   int act_dtype, int w_dtype, void* stream);
+int he_add_rmsnorm(void* resid_f32, const void* delta, const void* weight, void* out, int rows, int D,
+                   float eps, int act_dtype, int w_dtype, void* stream);
 int he_rmsnorm_rows(void* out, const void* x, const void* weight, int rows, int D,
                     int64_t x_stride, int64_t out_stride, float eps, int dtype, int w_dtype,
                     void* stream);
@@ -50,15 +47,6 @@ int he_rmsnorm_rows(void* out, const void* x, const void* weight, int rows, int 
 int he_gemm_plain(void* C, const void* A, const void* W, const void* bias, int M, int N, int K,
                   int64_t lda, int64_t ldw, int64_t ldc, int in_dtype, int out_dtype,
                   int bias_dtype, void* stream);
-// bf16 MFMA product for M <= HE_SKINNY_MAX_M rows: every weight element is read once.
-#define HE_SKINNY_MAX_M 64
-// R, U, splits <= 0 choose the heuristic tiling. When K is cut into more than one slice, C is
-// not written: partial_f32 receives fp32 [slices][M][N] (bias not added) and *splits_used says
-// how many; the reader adds them in index order (he_splitk_reduce, he_add_rmsnorm, he_qkv_rope_cache).
-int he_gemm_skinny_bf16(void* C, void* partial_f32, int64_t partial_floats, const void* A,
-                        const void* W, const void* bias, int M, int N, int K, int out_dtype,
-                        int bias_dtype, int R, int U, int splits, int* splits_used, void* stream);
-int he_gemm_skinny_splits(int M, int N, int K);
 // bf16 MFMA product for M <= HE_BLOCKSPLIT_MAX_M with K cut inside the workgroup (NW
 // wavefronts, one slice each, added in LDS): complete in one launch.
 #define HE_BLOCKSPLIT_MAX_M 32
@@ -82,13 +70,36 @@ int he_gemm_blocksplit_fused_bf16(void* C, const void* A, const void* W, const v
 // (row-major; x_pieces: x lies piece-major for exactly `rows` rows).
 int he_scale_rows_bf16(void* out, const void* x, const void* partials, int count, int rows, int D,
                        float eps, int x_pieces, void* stream);
+// C[M,N] = the slices of partial_f32 [splits][M][N] added in index order (+ bias).
 int he_splitk_reduce(void* C, const void* partial_f32, const void* bias, int M, int N, int splits,
                      int out_dtype, int bias_dtype, void* stream);
+// bf16 MFMA product for M <= HE_GEMM_ROWS_MAX_M rows whose activation rows are shared through LDS
+// by the wavefronts of a workgroup (made for 17 to 64 rows), with the epilogues of
+// he_gemm_blocksplit_fused_bf16 (x_pieces / out_pieces for any M here). R (1, 2), NWV (4, 8),
+// splits <= 0: the heuristic. A product the plan cuts into several K slices (he_gemm_rows_plan
+// says how many) writes fp32 [slices][M][N] into partial_f32 (each slice already scaled by the owed
+// row scale) and takes no other epilogue; he_splitk_reduce or he_splitk_reduce_residual adds them.
+// With one slice and resid != null, sq_count must be the plan's `groups`.
+#define HE_GEMM_ROWS_MAX_M 64
+int he_gemm_rows_plan(int M, int N, int K, int* groups, int* splits);
+int he_gemm_rows_bf16(void* C, void* partial_f32, int64_t partial_floats, const void* A, const void* W,
+                      const void* bias, int M, int N, int K, int out_dtype, int bias_dtype, int gated,
+                      int R, int NWV, int splits, const void* scale_partials, int scale_count,
+                      float scale_eps, void* resid, const void* gain, int gain_dtype, void* xg,
+                      void* sq_out, int sq_count, int x_pieces, int out_pieces, int* splits_used,
+                      void* stream);
+// resid[M,N] (fp32, in place) += the slices of partial_f32 [splits][M][N] in index order (+ bias);
+// xg = bf16(resid * gain) (piece-major with out_pieces); sq_out[M, sq_count] = sums of resid^2 per
+// block of 1024 columns (sq_count = he_splitk_reduce_residual_blocks(N)): the rows a residual
+// epilogue leaves for the next norm.
+int he_splitk_reduce_residual_blocks(int N);
+int he_splitk_reduce_residual(void* resid_f32, const void* partial_f32, const void* bias, int bias_dtype,
+                              const void* gain, int gain_dtype, void* xg, void* sq_out, int sq_count,
+                              int M, int N, int splits, int out_pieces, void* stream);
 
 // ---- position encoding + cache write -------------------------------------
 int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const void* q_in, const void* k_in,
-                      const void* v_in, int64_t in_stride, int in_splits, const void* q_bias,
-                      const void* k_bias,
+                      const void* v_in, int64_t in_stride, const void* q_bias, const void* k_bias,
                       const void* v_bias, int bias_dtype, const void* positions,
                       const void* row_seq, const void* seq_slot, const void* page_table,
                       int max_blocks, int num_pages, const void* inv_freq, int rotary_dim, int rows,

@@ -8,12 +8,8 @@
 #include "common.h"
 #include "hector_kernels.h"
 
-// SPLIT: delta is the fp32 partial sums [splits][rows][D] of a product cut along
-// K (plus an optional bias[D]); they are added here in the order of the slice index.
-template <typename TD, typename TO, bool SPLIT>
+template <typename TD, typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
-                                   int splits, int64_t split_stride,
-                                   const void* __restrict__ delta_bias, int bias_dtype,
                                    const void* __restrict__ w, int w_dtype, TO* __restrict__ out,
                                    int D, float eps) {
   __shared__ float scratch[16];
@@ -23,15 +19,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
   if (delta != nullptr) {
     const TD* d = delta + row * (int64_t)D;
     for (int i = threadIdx.x; i < D; i += blockDim.x) {
-      float add;
-      if (SPLIT) {
-        add = 0.f;
-        for (int s = 0; s < splits; ++s) add += to_float(d[s * split_stride + i]);
-        if (delta_bias != nullptr) add += load_param(delta_bias, i, bias_dtype);
-      } else {
-        add = to_float(d[i]);
-      }
-      const float v = r[i] + add;
+      const float v = r[i] + to_float(d[i]);
       r[i] = v;
       ss += v * v;
     }
@@ -193,30 +181,16 @@ static void launch_add_rmsnorm_vec(float* resid, const void* delta, const void* 
 
 static int norm_threads(int D) { return D >= 2048 ? 512 : (D >= 512 ? 256 : (D >= 128 ? 128 : 64)); }
 
-extern "C" int he_add_rmsnorm(void* resid_f32, const void* delta, int delta_splits,
-                              const void* delta_bias, int bias_dtype, const void* weight,
-                              void* out, int rows, int D, float eps, int act_dtype, int w_dtype,
-                              void* stream) {
+extern "C" int he_add_rmsnorm(void* resid_f32, const void* delta, const void* weight, void* out,
+                              int rows, int D, float eps, int act_dtype, int w_dtype, void* stream) {
   HE_REQUIRE(rows >= 0 && D > 0, "he_add_rmsnorm: bad sizes rows=%d D=%d", rows, D);
   HE_REQUIRE(w_dtype == HE_F32 || w_dtype == HE_BF16, "he_add_rmsnorm: bad weight dtype");
-  HE_REQUIRE(delta_splits >= 0 && (delta_splits == 0 || delta != nullptr),
-             "he_add_rmsnorm: split sums without data");
   HE_REQUIRE(act_dtype == HE_F32 || act_dtype == HE_BF16, "he_add_rmsnorm: unknown dtype %d",
              act_dtype);
   if (rows == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const int threads = norm_threads(D);
-  const int64_t stride = (int64_t)rows * D;
-  if (delta_splits > 0) {
-    if (act_dtype == HE_BF16)
-      add_rmsnorm_kernel<float, bf16_t, true><<<rows, threads, 0, s>>>(
-          (float*)resid_f32, (const float*)delta, delta_splits, stride, delta_bias, bias_dtype,
-          weight, w_dtype, (bf16_t*)out, D, eps);
-    else
-      add_rmsnorm_kernel<float, float, true><<<rows, threads, 0, s>>>(
-          (float*)resid_f32, (const float*)delta, delta_splits, stride, delta_bias, bias_dtype,
-          weight, w_dtype, (float*)out, D, eps);
-  } else if ((D & 3) == 0 && D <= 4 * NORM_VEC * 512 &&
+  if ((D & 3) == 0 && D <= 4 * NORM_VEC * 512 &&
              ((((uintptr_t)resid_f32) | ((uintptr_t)delta) | ((uintptr_t)weight) | ((uintptr_t)out)) & 15) == 0) {
     if (act_dtype == HE_BF16)
       launch_add_rmsnorm_vec<bf16_t, bf16_t>((float*)resid_f32, delta, weight, w_dtype, out, rows, D, eps, s);
@@ -230,13 +204,11 @@ extern "C" int he_add_rmsnorm(void* resid_f32, const void* delta, int delta_spli
       add_rmsnorm_reg_kernel<float, float><<<rows, threads, 0, s>>>(
           (float*)resid_f32, (const float*)delta, weight, w_dtype, (float*)out, D, eps);
   } else if (act_dtype == HE_BF16) {
-    add_rmsnorm_kernel<bf16_t, bf16_t, false><<<rows, threads, 0, s>>>(
-        (float*)resid_f32, (const bf16_t*)delta, 0, 0, nullptr, 0, weight, w_dtype, (bf16_t*)out, D,
-        eps);
+    add_rmsnorm_kernel<bf16_t, bf16_t><<<rows, threads, 0, s>>>(
+        (float*)resid_f32, (const bf16_t*)delta, weight, w_dtype, (bf16_t*)out, D, eps);
   } else {
-    add_rmsnorm_kernel<float, float, false><<<rows, threads, 0, s>>>(
-        (float*)resid_f32, (const float*)delta, 0, 0, nullptr, 0, weight, w_dtype, (float*)out, D,
-        eps);
+    add_rmsnorm_kernel<float, float><<<rows, threads, 0, s>>>(
+        (float*)resid_f32, (const float*)delta, weight, w_dtype, (float*)out, D, eps);
   }
   return he_check_launch("he_add_rmsnorm");
 }

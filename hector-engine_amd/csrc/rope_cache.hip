@@ -8,27 +8,16 @@
 //   y[i]       = x[i] * cos a - x[i + r/2] * sin a
 //   y[i + r/2] = x[i] * sin a + x[i + r/2] * cos a
 // and dims >= r pass through. All of it in fp32.
-//
-// The projected rows may arrive as the fp32 partial sums [splits][rows][width]
-// of a product cut along K; they are added here in the order of the slice index.
 #include "cache_layout.h"
 #include "hector_kernels.h"
 
 #define ROPE_MAX_HALF 256
 
-template <typename TI>
-__device__ __forceinline__ float load_in(const TI* p, int splits, int64_t split_stride) {
-  if (splits <= 1) return to_float(p[0]);
-  float s = 0.f;
-  for (int i = 0; i < splits; ++i) s += to_float(p[i * split_stride]);
-  return s;
-}
-
 template <typename T, typename TI>
 __global__ void qkv_rope_cache_kernel(
     T* __restrict__ q_out, T* __restrict__ kpool, T* __restrict__ vpool,
     const TI* __restrict__ q_in, const TI* __restrict__ k_in, const TI* __restrict__ v_in,
-    int64_t in_stride, int splits, int64_t split_stride, const void* __restrict__ q_bias, const void* __restrict__ k_bias,
+    int64_t in_stride, const void* __restrict__ q_bias, const void* __restrict__ k_bias,
     const void* __restrict__ v_bias, int bias_dtype, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ row_seq, const int32_t* __restrict__ seq_slot,
     const int32_t* __restrict__ page_table, int max_blocks, int num_pages,
@@ -58,8 +47,8 @@ __global__ void qkv_rope_cache_kernel(
       const int j = it - h * per_head;
       const int base = h * hd;
       if (j < half) {
-        float x0 = load_in(in + base + j, splits, split_stride);
-        float x1 = load_in(in + base + j + half, splits, split_stride);
+        float x0 = to_float((in + base + j)[0]);
+        float x1 = to_float((in + base + j + half)[0]);
         if (q_bias) {
           x0 += load_param(q_bias, base + j, bias_dtype);
           x1 += load_param(q_bias, base + j + half, bias_dtype);
@@ -69,7 +58,7 @@ __global__ void qkv_rope_cache_kernel(
         out[base + j + half] = from_float<T>(x0 * sn + x1 * c);
       } else {
         const int d = rotary_dim + (j - half);
-        float x = load_in(in + base + d, splits, split_stride);
+        float x = to_float((in + base + d)[0]);
         if (q_bias) x += load_param(q_bias, base + d, bias_dtype);
         out[base + d] = from_float<T>(x);
       }
@@ -92,8 +81,8 @@ __global__ void qkv_rope_cache_kernel(
       T* out = kpool + ((int64_t)page * KVH + h) * he_k_page_elems(hd);   // the page, in operand order
       const int KS = he_k_steps(hd);
       if (j < half) {
-        float x0 = load_in(in + base + j, splits, split_stride);
-        float x1 = load_in(in + base + j + half, splits, split_stride);
+        float x0 = to_float((in + base + j)[0]);
+        float x1 = to_float((in + base + j + half)[0]);
         if (k_bias) {
           x0 += load_param(k_bias, base + j, bias_dtype);
           x1 += load_param(k_bias, base + j + half, bias_dtype);
@@ -103,7 +92,7 @@ __global__ void qkv_rope_cache_kernel(
         out[he_k_index(off, j + half, KS)] = from_float<T>(x0 * sn + x1 * c);
       } else {
         const int d = rotary_dim + (j - half);
-        float x = load_in(in + base + d, splits, split_stride);
+        float x = to_float((in + base + d)[0]);
         if (k_bias) x += load_param(k_bias, base + d, bias_dtype);
         out[he_k_index(off, d, KS)] = from_float<T>(x);
       }
@@ -115,7 +104,7 @@ __global__ void qkv_rope_cache_kernel(
     for (int it = threadIdx.x; it < KVH * hd; it += blockDim.x) {
       const int h = it / hd;
       const int d = it - h * hd;
-      float x = load_in(in + it, splits, split_stride);
+      float x = to_float((in + it)[0]);
       if (v_bias) x += load_param(v_bias, it, bias_dtype);
       vpool[((int64_t)page * KVH + h) * he_v_page_elems(hd) + he_v_index(off, d, he_v_tiles(hd))] =
           from_float<T>(x);
@@ -312,7 +301,7 @@ __global__ __launch_bounds__(1024) void qkv_rope_cache_vec_kernel(
 
 extern "C" int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const void* q_in,
                                  const void* k_in, const void* v_in, int64_t in_stride,
-                                 int in_splits, const void* q_bias, const void* k_bias, const void* v_bias,
+                                 const void* q_bias, const void* k_bias, const void* v_bias,
                                  int bias_dtype, const void* positions, const void* row_seq,
                                  const void* seq_slot, const void* page_table, int max_blocks,
                                  int num_pages, const void* inv_freq, int rotary_dim, int rows,
@@ -327,20 +316,18 @@ extern "C" int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const vo
   HE_REQUIRE((k_in == nullptr) == (v_in == nullptr), "he_qkv_rope_cache: k and v go together");
   HE_REQUIRE(k_in == nullptr || (kpool && vpool && page_table && max_blocks > 0 && KVH > 0),
              "he_qkv_rope_cache: cache arguments missing");
-  HE_REQUIRE(in_splits >= 0 && in_splits <= 64, "he_qkv_rope_cache: bad slice count %d", in_splits);
   HE_REQUIRE(dtype == HE_BF16 || dtype == HE_F32, "he_qkv_rope_cache: unknown dtype %d", dtype);
   if (rows == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const int threads = 256;
-  const int64_t split_stride = (int64_t)rows * in_stride;
 #define ROPE_LAUNCH(T, TI)                                                                      \
   qkv_rope_cache_kernel<T, TI><<<rows, threads, 0, s>>>(                                        \
       (T*)q_out, (T*)kpool, (T*)vpool, (const TI*)q_in, (const TI*)k_in, (const TI*)v_in,       \
-      in_stride, in_splits, split_stride, q_bias, k_bias, v_bias, bias_dtype,                   \
+      in_stride, q_bias, k_bias, v_bias, bias_dtype,                                            \
       (const int32_t*)positions, (const int32_t*)row_seq, (const int32_t*)seq_slot,             \
       (const int32_t*)page_table, max_blocks, num_pages, (const float*)inv_freq, rotary_dim, H, \
       KVH, hd)
-  const bool vec_ok = in_splits == 0 && dtype == HE_BF16 &&
+  const bool vec_ok = dtype == HE_BF16 &&
                       (q_bias == nullptr || bias_dtype == HE_BF16) &&
                       ((rotary_dim >> 1) & 7) == 0 && ((hd - rotary_dim) & 7) == 0 &&
                       (in_stride & 7) == 0 && (hd & 7) == 0 &&
@@ -357,11 +344,6 @@ extern "C" int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const vo
         (const uint16_t*)k_bias, (const uint16_t*)v_bias, (const int32_t*)positions,
         (const int32_t*)row_seq, (const int32_t*)seq_slot, (const int32_t*)page_table, max_blocks,
         num_pages, (const float*)inv_freq, rotary_dim, rows, H, KVH, hd);
-  } else if (in_splits > 0) {  // the input rows are fp32 partial sums
-    if (dtype == HE_BF16)
-      ROPE_LAUNCH(bf16_t, float);
-    else
-      ROPE_LAUNCH(float, float);
   } else if (dtype == HE_BF16) {
     ROPE_LAUNCH(bf16_t, bf16_t);
   } else {

@@ -16,7 +16,7 @@ _lib = None
 
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 
-EXPECTED_ABI = 16
+EXPECTED_ABI = 18
 
 c_int, c_i64, c_f32, c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
@@ -30,14 +30,10 @@ _SIGNATURES = {
     "he_gather_rows_f32": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_ptr],
     "he_residual_add": [c_ptr, c_ptr, c_i64, c_int, c_ptr],
     "he_silu_mul": [c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_ptr],
-    "he_add_rmsnorm": [c_ptr, c_ptr, c_int, c_ptr, c_int, c_ptr, c_ptr, c_int, c_int, c_f32, c_int,
-                       c_int, c_ptr],
+    "he_add_rmsnorm": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_f32, c_int, c_int, c_ptr],
     "he_rmsnorm_rows": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_i64, c_i64, c_f32, c_int, c_int, c_ptr],
     "he_gemm_plain": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_i64, c_i64, c_i64,
                       c_int, c_int, c_int, c_ptr],
-    "he_gemm_skinny_bf16": [c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int,
-                            c_int, c_int, c_int, c_int, ctypes.POINTER(c_int), c_ptr],
-    "he_gemm_skinny_splits": [c_int, c_int, c_int],
     "he_gemm_blocksplit_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_int,
                                 c_int, c_int, c_int, c_ptr],
     "he_gemm_blocksplit_blocks": [c_int, c_int, c_int],
@@ -46,7 +42,14 @@ _SIGNATURES = {
                                       c_ptr, c_ptr, c_int, c_int, c_int, c_ptr],
     "he_scale_rows_bf16": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_f32, c_int, c_ptr],
     "he_splitk_reduce": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_ptr],
-    "he_qkv_rope_cache": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_int, c_ptr, c_ptr, c_ptr,
+    "he_gemm_rows_plan": [c_int, c_int, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int)],
+    "he_gemm_rows_bf16": [c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_int,
+                          c_int, c_int, c_int, c_ptr, c_int, c_f32, c_ptr, c_ptr, c_int, c_ptr, c_ptr, c_int,
+                          c_int, c_int, ctypes.POINTER(c_int), c_ptr],
+    "he_splitk_reduce_residual_blocks": [c_int],
+    "he_splitk_reduce_residual": [c_ptr, c_ptr, c_ptr, c_int, c_ptr, c_int, c_ptr, c_ptr, c_int, c_int, c_int,
+                                  c_int, c_int, c_ptr],
+    "he_qkv_rope_cache": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_ptr,
                           c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_ptr, c_int, c_int,
                           c_int, c_int, c_int, c_int, c_ptr],
     "he_attention_plain": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int,

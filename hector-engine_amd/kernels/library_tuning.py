@@ -1,13 +1,12 @@
 """The library matrix product's own autotuner (torch's TunableOp over hipBLASLt / rocBLAS).
 
-Tall products (more rows than the hand-written kernels take) go to the library, as the
-reference sends every product to its BLAS library (kernels/matmul_cublas.cu:240-277).
+Tall products (more than 64 rows: more than the hand-written kernels take) go to the library,
+as the reference sends every product to its BLAS library (kernels/matmul_cublas.cu:240-277).
 The library's default choice of kernel is not always its best on MI355X: at the
 Qwen2.5-7B shapes its tuner finds kernels 17-27 % faster for the 2048-row down and
-gate||up products and 20 % faster for gate||up at 64 rows. Tuning runs the first time a
-shape (rows, N, K) is seen and takes a second or so per shape, so it is meant for
-workloads whose shapes repeat (decode buckets, fixed prompt chunks); it is off unless
-asked for. Results are kept in a file and read again by the next process. Row counts that
+gate||up products. Tuning runs the first time a shape (rows, N, K) is seen and takes a second
+or so per shape, so it is meant for workloads whose shapes repeat (fixed prompt chunks); it is
+off unless asked for. Results are kept in a file and read again by the next process. Row counts that
 are unlikely to come again (a prompt of 1,937 tokens) are not tuned: worth_tuning().
 """
 from __future__ import annotations
@@ -43,10 +42,10 @@ def enabled() -> bool:
 
 
 def worth_tuning(rows: int) -> bool:
-    """Whether a product of this many rows is tuned when first seen: the row counts of one-token
-    steps (up to 64) and multiples of 256 (fixed prompt chunks). Any other count runs with the
-    library's default kernel, or with a tuned one if that exact shape was tuned before."""
-    return rows <= 64 or rows % 256 == 0
+    """Whether a product of this many rows is tuned when first seen: multiples of 256 (fixed
+    prompt chunks). Any other count runs with the library's default kernel, or with a tuned one
+    if that exact shape was tuned before."""
+    return rows > 0 and rows % 256 == 0
 
 
 @contextlib.contextmanager

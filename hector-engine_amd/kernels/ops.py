@@ -11,7 +11,6 @@ from .profiler import op as _op
 
 F32, BF16, F16 = 0, 1, 2
 PAGE_TOKENS = 64
-SKINNY_MAX_M = 64
 
 _CODES = {torch.float32: F32, torch.bfloat16: BF16}
 
@@ -131,11 +130,8 @@ def silu_mul(out, gate_up, rows: int, interleaved: bool = False, splits: int = 0
 
 
 @_op("add_rmsnorm")
-def add_rmsnorm(resid_f32, delta, weight, out, rows: int, eps: float, delta_splits: int = 0,
-                delta_bias=None) -> None:
-    """resid += delta (if given); out = rmsnorm(resid) * weight (if out given).
-    delta_splits > 0: delta is fp32 [delta_splits, rows, D], the K slices of a product,
-    added in index order with delta_bias."""
+def add_rmsnorm(resid_f32, delta, weight, out, rows: int, eps: float) -> None:
+    """resid += delta (if given); out = rmsnorm(resid) * weight (if out given)."""
     D = resid_f32.shape[-1]
     _need(resid_f32, "resid", torch.float32)
     _need(weight, "weight", shape=(D,))
@@ -149,22 +145,15 @@ def add_rmsnorm(resid_f32, delta, weight, out, rows: int, eps: float, delta_spli
         act = out.dtype
     if delta is not None:
         _need(delta, "delta")
-        if delta_splits > 0:
-            if delta.dtype != torch.float32 or tuple(delta.shape) != (delta_splits, rows, D):
-                raise ValueError(f"add_rmsnorm: split sums must be fp32 [{delta_splits}, {rows}, {D}]")
-            if delta_bias is not None:
-                _need(delta_bias, "delta_bias", shape=(D,))
-        else:
-            if delta.shape[-1] != D or delta.numel() < rows * D:
-                raise ValueError(f"add_rmsnorm: delta does not match [rows, {D}]")
-            if act is not None and delta.dtype != act:
-                raise TypeError("add_rmsnorm: delta and out must share a dtype")
-            act = delta.dtype
+        if delta.shape[-1] != D or delta.numel() < rows * D:
+            raise ValueError(f"add_rmsnorm: delta does not match [rows, {D}]")
+        if act is not None and delta.dtype != act:
+            raise TypeError("add_rmsnorm: delta and out must share a dtype")
+        act = delta.dtype
     L = _lib.load()
-    _lib.check(L.he_add_rmsnorm(resid_f32.data_ptr(), _ptr(delta), delta_splits if delta is not None else 0,
-                                _ptr(delta_bias), dtype_code(delta_bias.dtype) if delta_bias is not None else F32,
-                                weight.data_ptr(), _ptr(out), rows, D, float(eps),
-                                dtype_code(act or torch.float32), dtype_code(weight.dtype), _stream()))
+    _lib.check(L.he_add_rmsnorm(resid_f32.data_ptr(), _ptr(delta), weight.data_ptr(), _ptr(out), rows, D,
+                                float(eps), dtype_code(act or torch.float32), dtype_code(weight.dtype),
+                                _stream()))
 
 
 @_op("rmsnorm_rows")
@@ -199,55 +188,12 @@ def gemm_plain(out, a, w, bias, M: int) -> None:
                                dtype_code(bias.dtype) if bias is not None else F32, _stream()))
 
 
-def gemm_skinny_splits(M: int, N: int, K: int) -> int:
-    """K slices the heuristic cuts this product into (1 = none)."""
-    return int(_lib.load().he_gemm_skinny_splits(M, N, K))
-
-
-@_op("gemm_skinny")
-def gemm_skinny(out, partial, a, w, bias, M: int, plan=(0, 0, 0), out_dtype=None) -> int:
-    """bf16 MFMA product for M <= 64. plan = (R, U, splits), zeros for the heuristic.
-    With one K slice `out` (bf16 or fp32) is written, with bias. With more slices
-    `partial` (fp32, room for [slices, M, N]) is written instead, without bias. Returns
-    the number of slices."""
-    import ctypes
-    N, K = w.shape
-    NO = N
-    _need(a, "a", torch.bfloat16)
-    _need(w, "w", torch.bfloat16)
-    if M > SKINNY_MAX_M:
-        raise ValueError(f"gemm_skinny: M={M} above {SKINNY_MAX_M}")
-    if a.shape[-1] != K or a.numel() < M * K:
-        raise ValueError(f"gemm_skinny: shapes a{tuple(a.shape)} w{tuple(w.shape)} M={M}")
-    if out is not None:
-        _need(out, "out")
-        if out.shape[-1] != NO or out.numel() < M * NO:
-            raise ValueError(f"gemm_skinny: out{tuple(out.shape)} does not hold [{M}, {NO}]")
-        out_dtype = out.dtype
-    if bias is not None:
-        _need(bias, "bias", shape=(N,))
-    pfloats = 0
-    if partial is not None:
-        _need(partial, "partial", torch.float32)
-        pfloats = partial.numel()
-    L = _lib.load()
-    used = ctypes.c_int(0)
-    if out is None and pfloats == 0:
-        raise ValueError("gemm_skinny: neither an output nor room for partial sums")
-    _lib.check(L.he_gemm_skinny_bf16(_ptr(out), _ptr(partial), pfloats, a.data_ptr(), w.data_ptr(),
-                                     _ptr(bias), M, N, K, dtype_code(out_dtype or torch.bfloat16),
-                                     dtype_code(bias.dtype) if bias is not None else F32,
-                                     int(plan[0]), int(plan[1]), int(plan[2]), ctypes.byref(used),
-                                     _stream()))
-    if used.value == 1 and out is None:
-        raise ValueError("gemm_skinny: one K slice was chosen but no output tensor was given")
-    return used.value
-
-
 BLOCKSPLIT_MAX_M = 32
 
 
-PIECES_MAX_M = 16
+PIECES_MAX_M = 64
+BLOCKSPLIT_PIECES_MAX_M = 16   # the block-split product reads and writes pieces up to 16 rows
+ROWS_MAX_M = 64
 
 
 def pieces_shape(M: int, D: int) -> tuple[int, int, int]:
@@ -286,6 +232,8 @@ def gemm_blocksplit(out, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0)
     _need(w, "w", torch.bfloat16)
     if M > BLOCKSPLIT_MAX_M:
         raise ValueError(f"gemm_blocksplit: M={M} above {BLOCKSPLIT_MAX_M}")
+    if (x_pieces or out_pieces) and M > BLOCKSPLIT_PIECES_MAX_M:
+        raise ValueError(f"gemm_blocksplit: piece-major rows are for up to {BLOCKSPLIT_PIECES_MAX_M} rows, not {M}")
     if x_pieces:
         _need(a, "a", shape=pieces_shape(M, K))
     elif a.shape[-1] != K or a.numel() < M * K:
@@ -331,6 +279,109 @@ def gemm_blocksplit(out, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0)
         int(x_pieces), int(out_pieces), _stream()))
 
 
+def gemm_rows_plan(M: int, N: int, K: int) -> tuple[int, int]:
+    """(workgroups along N, K slices) of gemm_rows for this product: the count of partial sums of
+    squares its residual epilogue gives, and whether it leaves plain sums or partial sums."""
+    import ctypes
+    g, s = ctypes.c_int(0), ctypes.c_int(0)
+    _lib.check(_lib.load().he_gemm_rows_plan(M, N, K, ctypes.byref(g), ctypes.byref(s)))
+    return g.value, s.value
+
+
+@_op("gemm_rows")
+def gemm_rows(out, partial, a, w, bias, M: int, gated: bool = False, plan=(0, 0, 0), *, row_scale=None,
+              residual=None, x_pieces: bool = False, out_pieces: bool = False) -> int:
+    """bf16 MFMA product for M <= 64 whose activation rows go through LDS once per workgroup; the
+    epilogues of gemm_blocksplit (see there: bias, gated, row_scale, residual, x_pieces, out_pieces).
+    plan = (R, NWV, splits), zeros = heuristic. A product cut into several K slices writes its fp32
+    sums into `partial` ([slices, M, N], each already scaled by row_scale) and takes no other
+    epilogue. Returns the number of slices."""
+    import ctypes
+    N, K = w.shape
+    NO = N // 2 if gated else N
+    _need(a, "a", torch.bfloat16)
+    _need(w, "w", torch.bfloat16)
+    if not 0 < M <= ROWS_MAX_M:
+        raise ValueError(f"gemm_rows: M={M} outside [1, {ROWS_MAX_M}]")
+    if x_pieces:
+        _need(a, "a", shape=pieces_shape(M, K))
+    elif a.shape[-1] != K or a.numel() < M * K:
+        raise ValueError(f"gemm_rows: shapes a{tuple(a.shape)} w{tuple(w.shape)} M={M}")
+    if out is not None:
+        _need(out, "out")
+        if out_pieces:
+            _need(out, "out", torch.bfloat16, pieces_shape(M, NO))
+        elif out.shape[-1] != NO or out.numel() < M * NO:
+            raise ValueError(f"gemm_rows: out{tuple(out.shape)} for M={M} N={NO}")
+    pf = 0
+    if partial is not None:
+        _need(partial, "partial", torch.float32)
+        pf = partial.numel()
+    if bias is not None:
+        _need(bias, "bias", shape=(N,))
+    sp, sc, se = None, 0, 0.0
+    if row_scale is not None:
+        partials, se = row_scale
+        _need(partials, "row_scale partials", torch.float32)
+        if partials.dim() != 2 or partials.shape[0] < M:
+            raise ValueError("gemm_rows: row_scale partials must be [M, count]")
+        sp, sc = partials.data_ptr(), partials.shape[1]
+    rp = gp = xp = qp = None
+    gdt, qc = F32, 0
+    if residual is not None:
+        resid, gain, xg, sq = residual
+        _need(resid, "resid", torch.float32)
+        _need(gain, "gain", shape=(N,))
+        _need(xg, "xg", torch.bfloat16)
+        _need(sq, "sq", torch.float32)
+        if out_pieces:
+            _need(xg, "xg", shape=pieces_shape(M, N))
+        if resid.shape[-1] != N or resid.numel() < M * N or xg.numel() < M * N \
+                or (not out_pieces and xg.shape[-1] != N) or sq.dim() != 2 or sq.shape[0] < M:
+            raise ValueError("gemm_rows: residual buffers do not match [M, N]")
+        rp, gp, xp, qp = resid.data_ptr(), gain.data_ptr(), xg.data_ptr(), sq.data_ptr()
+        gdt, qc = dtype_code(gain.dtype), sq.shape[1]
+    used = ctypes.c_int(0)
+    L = _lib.load()
+    _lib.check(L.he_gemm_rows_bf16(
+        _ptr(out), _ptr(partial), pf, a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K,
+        dtype_code(out.dtype) if out is not None else BF16,
+        dtype_code(bias.dtype) if bias is not None else F32, int(gated),
+        int(plan[0]), int(plan[1]), int(plan[2]), sp, sc, float(se), rp, gp, gdt, xp, qp, qc,
+        int(x_pieces), int(out_pieces), ctypes.byref(used), _stream()))
+    return used.value
+
+
+def splitk_reduce_residual_blocks(N: int) -> int:
+    return int(_lib.load().he_splitk_reduce_residual_blocks(N))
+
+
+@_op("splitk_reduce_residual")
+def splitk_reduce_residual(resid, partial, bias, gain, xg, sq, M: int, splits: int,
+                           out_pieces: bool = False) -> None:
+    """resid [M, N] (fp32, in place) += the K slices partial [splits, M, N] in index order (+ bias);
+    xg = bf16(resid * gain), piece-major with out_pieces; sq [M, blocks] = sums of resid^2 per block
+    of columns (blocks = splitk_reduce_residual_blocks(N))."""
+    N = resid.shape[-1]
+    _need(resid, "resid", torch.float32)
+    _need(partial, "partial", torch.float32)
+    _need(gain, "gain", shape=(N,))
+    _need(xg, "xg", torch.bfloat16)
+    _need(sq, "sq", torch.float32)
+    if out_pieces:
+        _need(xg, "xg", shape=pieces_shape(M, N))
+    if resid.numel() < M * N or partial.numel() < splits * M * N or xg.numel() < M * N \
+            or sq.dim() != 2 or sq.shape[0] < M or (not out_pieces and xg.shape[-1] != N):
+        raise ValueError("splitk_reduce_residual: buffers do not match [splits, M, N]")
+    if bias is not None:
+        _need(bias, "bias", shape=(N,))
+    L = _lib.load()
+    _lib.check(L.he_splitk_reduce_residual(
+        resid.data_ptr(), partial.data_ptr(), _ptr(bias), dtype_code(bias.dtype) if bias is not None else F32,
+        gain.data_ptr(), dtype_code(gain.dtype), xg.data_ptr(), sq.data_ptr(), sq.shape[1], M, N, splits,
+        int(out_pieces), _stream()))
+
+
 @_op("scale_rows")
 def scale_rows(out, x, partials, eps: float, rows: int, x_pieces: bool = False) -> None:
     """out = x / sqrt(sum(partials of the row) / D + eps) for rows x = r * gain (bf16). out is
@@ -368,24 +419,20 @@ def splitk_reduce(out, partial, bias, M: int, splits: int) -> None:
 @_op("qkv_rope_cache")
 def qkv_rope_cache(q_out, kpool, vpool, qkv, q_cols: int, kv_cols: int, bias, positions, row_seq,
                    seq_slot, page_table, inv_freq, rotary_dim: int, rows: int, H: int, KVH: int,
-                   hd: int, write_kv: bool, splits: int = 0) -> None:
-    """qkv: [rows, q_cols (+ 2 kv_cols)] projected rows without bias, or with splits > 0 the
-    fp32 K slices [splits, rows, width] of that product; bias (optional) has the same
+                   hd: int, write_kv: bool) -> None:
+    """qkv: [rows, q_cols (+ 2 kv_cols)] projected rows without bias; bias (optional) has the same
     column layout. Rotated q goes to q_out [rows, H*hd]; k, v go into the pools at
     (slot, position) when write_kv."""
     _need(qkv, "qkv")
     _need(q_out, "q_out")
-    if splits > 0:
-        if qkv.dtype != torch.float32 or qkv.dim() != 3 or qkv.shape[0] != splits or qkv.shape[1] != rows:
-            raise ValueError("qkv_rope_cache: split sums must be fp32 [splits, rows, width]")
-    elif qkv.dtype != q_out.dtype:
+    if qkv.dtype != q_out.dtype:
         raise TypeError("qkv_rope_cache: qkv and q_out must share a dtype")
     width = qkv.shape[-1]
     if q_cols != H * hd or (write_kv and (kv_cols != KVH * hd or width != q_cols + 2 * kv_cols)):
         raise ValueError("qkv_rope_cache: column layout does not match the head sizes")
     if not write_kv and width < q_cols:
         raise ValueError("qkv_rope_cache: qkv narrower than the query columns")
-    if qkv.numel() < max(splits, 1) * rows * width or q_out.numel() < rows * q_cols:
+    if qkv.numel() < rows * width or q_out.numel() < rows * q_cols:
         raise ValueError("qkv_rope_cache: buffers smaller than the row count")
     _need(positions, "positions", torch.int32)
     _need(row_seq, "row_seq", torch.int32)
@@ -419,7 +466,7 @@ def qkv_rope_cache(q_out, kpool, vpool, qkv, q_cols: int, kv_cols: int, bias, po
     L = _lib.load()
     _lib.check(L.he_qkv_rope_cache(
         q_out.data_ptr(), _ptr(kpool) if write_kv else None, _ptr(vpool) if write_kv else None,
-        base, k_in, v_in, width, splits, qb, kb, vb, bias_code, positions.data_ptr(), row_seq.data_ptr(),
+        base, k_in, v_in, width, qb, kb, vb, bias_code, positions.data_ptr(), row_seq.data_ptr(),
         seq_slot.data_ptr(), _ptr(page_table) if write_kv else None, max_blocks, num_pages,
         _ptr(inv_freq) if rotary_dim else None, rotary_dim, rows, H, KVH if write_kv else 0, hd,
         dtype_code(q_out.dtype), _stream()))

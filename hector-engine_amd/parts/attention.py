@@ -18,7 +18,7 @@ import torch
 from ..kernels import ops
 from .base import (BuildEnv, KVNeed, LayerCache, Mixer, PartSpec, PieceRows, StepContext, TensorSpec,
                    build_part, param, register_part)
-from .linear import Linear, SplitSum
+from .linear import Linear
 
 
 @register_part("mixer", "attention")
@@ -109,14 +109,10 @@ class Attention(Mixer):
                                        ctx.row_seq, ctx.seq_slot, cache.page_table, rot[0], rot[1],
                                        rows, H, KVH, hd, self.window, self.scale, ctx.max_keys,
                                        writes, ws, out_pieces=pieces)
-            return self.o_proj(PieceRows(out) if pieces else out, rows, ctx, allow_split=True,
-                               sink=ctx.take_sink())
+            return self.o_proj(PieceRows(out) if pieces else out, rows, ctx, sink=ctx.take_sink())
         # With a rotation (or no encoding) the bias is added inside the fused kernel;
         # any other encoding sees q and k with their bias already added.
-        qkv = proj(x, rows, ctx, use_bias=not fused_bias, allow_split=fused_bias)
-        splits = 0
-        if isinstance(qkv, SplitSum):        # K slices: the q/k/v kernel adds them while it reads
-            splits, qkv = qkv.splits, qkv.partial
+        qkv = proj(x, rows, ctx, use_bias=not fused_bias)
         if not fused_bias:
             q_cols, kv_cols = H * hd, KVH * hd
             qv = qkv[:, :q_cols].unflatten(1, (H, hd))
@@ -126,8 +122,7 @@ class Attention(Mixer):
         inv_freq, r = rot if rot is not None else (None, 0)
         ops.qkv_rope_cache(q, cache.kpool, cache.vpool, qkv, H * hd, KVH * hd,
                            proj.bias if fused_bias else None, ctx.positions, ctx.row_seq,
-                           ctx.seq_slot, cache.page_table, inv_freq, r, rows, H, KVH, hd, writes,
-                           splits)
+                           ctx.seq_slot, cache.page_table, inv_freq, r, rows, H, KVH, hd, writes)
         out = ctx.alloc((rows, H * hd))
         if not self.fast:
             ops.attention_plain(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
@@ -143,4 +138,4 @@ class Attention(Mixer):
             ops.attention_prefill(out, q, cache.kpool, cache.vpool, ctx.cu_seqlens, ctx.seq_slot,
                                   ctx.seq_start, cache.page_table, ctx.num_seqs, ctx.max_q_len,
                                   rows, H, KVH, hd, self.window, self.scale)
-        return self.o_proj(out, rows, ctx, allow_split=True, sink=ctx.take_sink())
+        return self.o_proj(out, rows, ctx, sink=ctx.take_sink())

@@ -183,10 +183,8 @@ class Norm(Part):
 
     def add_norm(self, resid: torch.Tensor, delta, rows: int, ctx: StepContext,
                  want_out: bool = True) -> torch.Tensor | None:
-        """resid (fp32 [rows, D], in place) += delta; returns norm(resid) in the
-        activation dtype (or None when want_out is False). delta is a tensor, None, or
-        the split sums of a product (parts.linear.SplitSum); a norm that does not add
-        slices itself turns them into a tensor with parts.linear.as_tensor."""
+        """resid (fp32 [rows, D], in place) += delta (a tensor in the activation dtype, or
+        None); returns norm(resid) in the activation dtype (or None when want_out is False)."""
         raise NotImplementedError
 
 
@@ -219,8 +217,8 @@ class Mixer(Part):
         return 0
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache):
-        """x: [rows, D] normed activations. Returns [rows, D], as a tensor or as the
-        split sums of its last product."""
+        """x: [rows, D] normed activations. Returns [rows, D], or None when its last product
+        has added the result to the residual stream through the sink it was offered."""
         raise NotImplementedError
 
 
@@ -228,7 +226,8 @@ class FeedForward(Part):
     accepts_normed_rows = False
 
     def forward(self, x: torch.Tensor, ctx: StepContext):
-        """Returns [rows, D], as a tensor or as the split sums of its last product."""
+        """Returns [rows, D], or None when its last product has added the result to the residual
+        stream through the sink it was offered."""
         raise NotImplementedError
 
 
@@ -303,8 +302,8 @@ class ResidualStream:
         self.prepared: tuple[Norm, NormedRows] | None = None   # rows already made for that norm
 
     def add(self, delta, ctx: StepContext) -> None:
-        """delta: a tensor [rows, D], the split sums of a product, or None when the
-        producer has added its result through a ResidualSink."""
+        """delta: a tensor [rows, D], or None when the producer has added its result through a
+        ResidualSink."""
         if delta is None:
             return
         self.prepared = None
@@ -334,8 +333,7 @@ class ResidualStream:
     def materialize(self, ctx: StepContext) -> torch.Tensor:
         if self.pending is not None:
             from ..kernels import ops
-            from .linear import as_tensor
-            ops.residual_add(self.resid, as_tensor(self.pending, ctx), self.rows)
+            ops.residual_add(self.resid, self.pending, self.rows)
             self.pending = None
         return self.resid
 

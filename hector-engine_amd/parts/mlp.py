@@ -9,7 +9,7 @@ import torch
 
 from ..kernels import ops
 from .base import BuildEnv, FeedForward, NormedRows, PieceRows, StepContext, TensorSpec, param, register_part
-from .linear import Linear, SplitSum
+from .linear import Linear
 
 # rows of the intermediate activations held at once in a long prompt step
 _ROW_CHUNK = 8192
@@ -55,20 +55,16 @@ class GatedMLP(FeedForward):
         if rows <= _ROW_CHUNK:
             act = x.scaled.dtype if isinstance(x, NormedRows) else x.dtype
             if self.gate_up.gated_silu_rows(rows, ctx, act):
-                # few rows: the activation is the product's epilogue, and its result goes to the
+                # up to 64 rows: the activation is the product's epilogue, and its result goes to the
                 # down projection piece-major where that reads it so
-                pieces = self.inter % 8 == 0 and self.down.reads_pieces(rows, ctx)
+                pieces = self.inter % 8 == 0 and self.down.reads_pieces(rows, ctx) and self.gate_up.gated_pieces(rows)
                 h = ctx.alloc(ops.pieces_shape(rows, self.inter) if pieces else (rows, self.inter))
                 self.gate_up.gated_silu(x, rows, ctx, h, out_pieces=pieces)
-                return self.down(PieceRows(h) if pieces else h, rows, ctx, allow_split=True,
-                                 sink=ctx.take_sink())
+                return self.down(PieceRows(h) if pieces else h, rows, ctx, sink=ctx.take_sink())
             h = ctx.alloc((rows, self.inter))
-            gu = self.gate_up(x, rows, ctx, allow_split=True)
-            if isinstance(gu, SplitSum):     # K slices: the activation kernel adds them while it reads
-                ops.silu_mul(h, gu.partial, rows, True, gu.splits)
-            else:
-                ops.silu_mul(h, gu, rows, True)
-            return self.down(h, rows, ctx, allow_split=True, sink=ctx.take_sink())
+            gu = self.gate_up(x, rows, ctx)
+            ops.silu_mul(h, gu, rows, True)
+            return self.down(h, rows, ctx, sink=ctx.take_sink())
         if not isinstance(x, torch.Tensor):
             x = x.tensor(ctx)
         out = ctx.alloc((rows, self.hidden))

@@ -8,7 +8,6 @@ import torch
 
 from ..kernels import ops
 from .base import BuildEnv, Norm, StepContext, TensorSpec, param, register_part
-from .linear import SplitSum
 
 
 @register_part("norm", "rmsnorm")
@@ -30,9 +29,5 @@ class RMSNorm(Norm):
 
     def add_norm(self, resid, delta, rows, ctx: StepContext, want_out: bool = True):
         out = ctx.alloc((rows, self.size)) if want_out else None
-        if isinstance(delta, SplitSum):      # the K slices of a product: added while read
-            ops.add_rmsnorm(resid, delta.partial, self.weight, out, rows, self.eps,
-                            delta_splits=delta.splits, delta_bias=delta.bias)
-        else:
-            ops.add_rmsnorm(resid, delta, self.weight, out, rows, self.eps)
+        ops.add_rmsnorm(resid, delta, self.weight, out, rows, self.eps)
         return out

@@ -238,33 +238,33 @@ def test_command_line_with_the_library_tuner(model_dirs, tmp_path):
     """--tune-gemm: tall bfloat16 products go through the library's tuner (its own process, since the
     tuner is process-wide); the same tokens as without it where the decision is clear."""
     exe = os.path.join(ROOT, "bin", "hector_generate")
-    prompt = ",".join(str(7 + (i * 37) % 200) for i in range(48))          # 48 rows: a library product
+    prompt = ",".join(str(7 + (i * 37) % 290) for i in range(256))         # 256 rows: a library product
     env = dict(os.environ, TMPDIR=str(tmp_path))
     runs = []
     for extra in ([], ["--tune-gemm"]):
-        out = subprocess.run([sys.executable, exe, model_dirs["A"], prompt, "4", "--dtype", "bfloat16"] + extra,
+        out = subprocess.run([sys.executable, exe, model_dirs["C"], prompt, "4", "--dtype", "bfloat16"] + extra,
                              capture_output=True, text=True, timeout=300, env=env)
         assert out.returncode == 0, out.stderr
         runs.append([l for l in out.stdout.splitlines() if l.startswith("[0]")])
     assert runs[0] and runs[1]
     first = lambda lines: lines[0].rsplit(": ", 1)[-1].split(",")[0]       # "...(max_tokens): 12,7,..."
     assert first(runs[0]).isdigit() and first(runs[0]) == first(runs[1])
-    # a row count that will hardly come again (77: above the one-token steps, no multiple of 256) runs
-    # without the tuner's trials; the file of results holds the 48-row products only
-    odd = ",".join(str(3 + (i * 29) % 200) for i in range(77))
-    out = subprocess.run([sys.executable, exe, model_dirs["A"], odd, "2", "--dtype", "bfloat16", "--tune-gemm"],
+    # a row count that will hardly come again (77: above the hand-written kernels' 64, no multiple of 256)
+    # runs without the tuner's trials; the file of results holds the 256-row products only
+    odd = ",".join(str(3 + (i * 29) % 290) for i in range(77))
+    out = subprocess.run([sys.executable, exe, model_dirs["C"], odd, "2", "--dtype", "bfloat16", "--tune-gemm"],
                          capture_output=True, text=True, timeout=300, env=env)
     assert out.returncode == 0, out.stderr
     results = [os.path.join(d, f) for d, _, fs in os.walk(str(tmp_path)) for f in fs if f.endswith(".csv")]
     assert results
     text = "".join(open(f).read() for f in results)
-    assert "_48_" in text and "_77_" not in text
+    assert "_256_" in text and "_77_" not in text
 
 
 def test_tuning_policy_and_nested_blocks():
     from hector_engine_amd.kernels import library_tuning
-    assert all(library_tuning.worth_tuning(r) for r in (1, 17, 64, 256, 2048, 16384))
-    assert not any(library_tuning.worth_tuning(r) for r in (65, 77, 1937, 2049))
+    assert all(library_tuning.worth_tuning(r) for r in (256, 2048, 16384))
+    assert not any(library_tuning.worth_tuning(r) for r in (1, 17, 64, 65, 77, 1937, 2049))
 
 
 def test_smoke_entry():

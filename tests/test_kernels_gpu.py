@@ -123,106 +123,21 @@ def test_gemm_plain_rows_do_not_depend_on_the_batch(ops):
         assert torch.equal(one.cpu()[0], full.cpu()[r])      # bit-equal
 
 
-@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 64])
-@pytest.mark.parametrize("N,K", [(301, 136), (1000, 520), (37, 4104), (4608, 3584)])
-@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
-def test_gemm_skinny(ops, M, N, K, out_dtype):
-    if (N, K) == (4608, 3584) and M not in (1, 8, 64):
-        pytest.skip("large shape at three row counts only")
-    a = rnd(M, K, seed=14).to(torch.bfloat16)
-    w = rnd(N, K, seed=15, scale=0.05).to(torch.bfloat16)
-    b = rnd(N, seed=16).to(torch.bfloat16)
-    out = torch.empty(M, N, dtype=out_dtype, device="cuda")
-    splits = ops.gemm_skinny_splits(M, N, K)
-    if splits == 1:
-        assert ops.gemm_skinny(out, None, dev(a), dev(w), dev(b), M) == 1
-    else:
-        partial = torch.empty(splits, M, N, device="cuda")
-        assert ops.gemm_skinny(None, partial, dev(a), dev(w), None, M) == splits
-        ops.splitk_reduce(out, partial, dev(b), M, splits)
-    ref = a.double() @ w.double().T + b.double()
-    scale = ref.abs().max().item()
-    err = (out.cpu().double() - ref).abs().max().item()
-    tol = 2e-5 * scale * math.sqrt(K / 64) if out_dtype == torch.float32 else 2 ** -8 * scale + 1e-6
-    assert err <= tol, (err, tol)
-    # the plain kernel agrees too (same inputs, fp32 accumulation)
-    plain = torch.empty(M, N, dtype=out_dtype, device="cuda")
-    ops.gemm_plain(plain, dev(a), dev(w), dev(b), M)
-    assert (plain.cpu().double() - ref).abs().max().item() <= tol
-
-
-PLANS = [(1, 1, 1), (1, 2, 3), (1, 4, 8), (2, 1, 1), (2, 2, 5), (2, 4, 2), (4, 1, 1), (4, 2, 4)]
-
-
-@pytest.mark.parametrize("M", [1, 16, 20, 64])
-@pytest.mark.parametrize("R,U,splits", PLANS)
-def test_gemm_skinny_every_plan(ops, M, R, U, splits):
-    """Every tiling the kernel can be launched with gives the same product; K slices are
-    added in index order by the reader, so two runs agree bit for bit."""
-    MT = (M + 15) // 16
-    if (MT == 1 and (R, U) in ((4, 4),)) or (MT == 2 and (R == 1 or U == 4)) or \
-            (MT >= 3 and ((R, U) not in ((4, 1), (2, 1), (2, 2)))):
-        pytest.skip("not instantiated")
-    N, K = 1000, 1544
-    a = rnd(M, K, seed=70).to(torch.bfloat16)
-    w = rnd(N, K, seed=71, scale=0.05).to(torch.bfloat16)
-    b = rnd(N, seed=72).to(torch.bfloat16)
-    ref = a.double() @ w.double().T + b.double()
-    outs = []
-    for _ in range(2):
-        out = torch.empty(M, N, dtype=torch.float32, device="cuda")
-        partial = torch.empty(64, M, N, device="cuda")
-        used = ops.gemm_skinny(out, partial, dev(a), dev(w), dev(b), M, plan=(R, U, splits))
-        assert 1 <= used <= splits and (used > 1) == (splits > 1)
-        if used > 1:
-            ops.splitk_reduce(out, partial, dev(b), M, used)
-        outs.append(out.cpu())
-    assert torch.equal(outs[0], outs[1])
-    assert (outs[0].double() - ref).abs().max().item() <= 1e-4 * ref.abs().max().item()
-
-
-def test_split_sums_are_added_by_the_norm_and_the_qkv_kernel(ops):
-    """The fused norm and the q/k/v kernel read the K slices of a product directly and give
-    what they give for the reduced tensor."""
+def test_splitk_reduce_and_the_gated_activation_add_slices_in_order(ops):
+    """K slices of a product are added in index order (+ bias) by splitk_reduce, and by the gated
+    activation while it reads them."""
     rows, D, S = 5, 96, 3
     parts = rnd(S, rows, D, seed=76)
     bias = rnd(D, seed=77)
-    resid = rnd(rows, D, seed=78)
-    w = 1 + 0.1 * rnd(D, seed=79)
-    a, b_ = dev(resid.clone()), dev(resid.clone())
-    out_a = torch.empty(rows, D, dtype=torch.bfloat16, device="cuda")
-    out_b = torch.empty_like(out_a)
-    ops.add_rmsnorm(a, dev(parts), dev(w), out_a, rows, 1e-6, delta_splits=S, delta_bias=dev(bias))
     summed = torch.empty(rows, D, device="cuda")
     ops.splitk_reduce(summed, dev(parts), dev(bias), rows, S)
-    want = resid.double() + parts.double().sum(0) + bias.double()
-    assert torch.allclose(a.cpu().double(), want, atol=1e-5)
-    ops.add_rmsnorm(b_, summed.to(torch.bfloat16), dev(w), out_b, rows, 1e-6)
-    assert torch.allclose(out_a.float(), out_b.float(), atol=2 ** -6, rtol=2 ** -6)
-    # q/k/v kernel: H=2, KVH=1, hd=32 -> width 128
-    H, KVH, hd = 2, 1, 32
-    width = (H + 2 * KVH) * hd
-    parts = rnd(S, rows, width, seed=80)
-    qb = rnd(width, seed=81).to(torch.bfloat16)
-    slots, table, kpool, vpool = paged_setup([rows], KVH, hd, torch.bfloat16, 82)
-    pos = torch.arange(rows, dtype=torch.int32)
-    meta = (dev(pos), dev(torch.zeros(rows, dtype=torch.int32)), dev(torch.tensor(slots, dtype=torch.int32)), dev(table))
-    inv = dev(P.rope_inv_freq(hd, 1e4))
-    res = []
-    for split in (True, False):
-        q_out = torch.zeros(rows, H * hd, dtype=torch.bfloat16, device="cuda")
-        kp, vp = dev(kpool), dev(vpool)
-        if split:
-            ops.qkv_rope_cache(q_out, kp, vp, dev(parts), H * hd, KVH * hd, dev(qb), *meta, inv, hd, rows,
-                               H, KVH, hd, True, splits=S)
-        else:
-            x = parts.sum(0)
-            q_ref = P.rope((x + qb.float())[:, :H * hd].reshape(rows, H, hd).double(), pos, 1e4)
-            res.append(q_ref.reshape(rows, H * hd))
-            continue
-        res.append(q_out.cpu().double())
-        assert (kp != 0).sum().item() > 0 and (vp != 0).sum().item() > 0
-    assert torch.allclose(res[0], res[1], atol=2 ** -6, rtol=2 ** -6)
+    want = ((parts[0] + parts[1]) + parts[2]) + bias
+    assert torch.equal(summed.cpu(), want)
+    h = torch.empty(rows, D // 2, dtype=torch.bfloat16, device="cuda")
+    ops.silu_mul(h, dev(parts), rows, True, S)
+    x = parts.double().sum(0)
+    ref = P.silu(x[:, 0::2]) * x[:, 1::2]
+    assert torch.allclose(h.cpu().double(), ref, rtol=2 ** -7, atol=2 ** -7)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -412,9 +327,13 @@ def test_gemm_blocksplit_piece_major(ops, M, N, K):
 def test_piece_major_rows_are_refused_beyond_their_sizes(ops):
     from hector_engine_amd.kernels.lib import KernelLibraryError
     with pytest.raises(ValueError, match="piece-major"):
-        ops.pieces_shape(17, 64)
+        ops.pieces_shape(65, 64)
     with pytest.raises(ValueError, match="piece-major"):
         ops.pieces_shape(4, 60)
+    with pytest.raises(ValueError, match="up to 16 rows"):      # the block-split product's own limit
+        ops.gemm_blocksplit(torch.empty(ops.pieces_shape(17, 64), dtype=torch.bfloat16, device="cuda"),
+                            torch.zeros(17, 64, dtype=torch.bfloat16, device="cuda"),
+                            torch.zeros(64, 64, dtype=torch.bfloat16, device="cuda"), None, 17, out_pieces=True)
     M, N, K = 4, 64, 64
     x = torch.zeros(ops.pieces_shape(M, K), dtype=torch.bfloat16, device="cuda")
     w = torch.zeros(N, K, dtype=torch.bfloat16, device="cuda")
@@ -442,15 +361,6 @@ def test_gemm_blocksplit_residual_epilogue_checks_its_buffers(ops):
         ops.gemm_blocksplit(None, x, w, None, M, residual=(resid, gain, xg, torch.zeros(M, 1, device="cuda")))
     with pytest.raises(ValueError):
         ops.gemm_blocksplit(None, x, w, None, M, gated=True, residual=(resid, gain, xg, torch.zeros(M, 4, device="cuda")))
-
-
-def test_gemm_skinny_refuses_bad_sizes(ops):
-    from hector_engine_amd.kernels.lib import KernelLibraryError
-    a = torch.zeros(2, 20, dtype=torch.bfloat16, device="cuda")
-    w = torch.zeros(16, 20, dtype=torch.bfloat16, device="cuda")
-    out = torch.empty(2, 16, dtype=torch.bfloat16, device="cuda")
-    with pytest.raises(KernelLibraryError, match="multiple of 8"):
-        ops.gemm_skinny(out, None, a, w, None, 2)
 
 
 # ------------------------------------------------------------------ rope + cache + attention

@@ -49,11 +49,6 @@ def make_ctx(fw, env, q_lens, starts, slots):
         host={"q_lens": q_lens, "starts": starts, "slots": slots})
 
 
-def as_tensor(x, ctx):
-    from hector_engine_amd.parts.linear import as_tensor as f
-    return f(x, ctx)
-
-
 def rnd(*shape, seed=0, scale=1.0):
     g = torch.Generator().manual_seed(seed)
     return torch.randn(*shape, generator=g) * scale
@@ -115,7 +110,7 @@ def test_gated_mlp_part(fw, dtype, rows, inter):
     mlp.bind({k: v.cuda() for k, v in w.items()})
     ctx = make_ctx(fw, env, [rows], [0], [0])
     x = rnd(rows, 80, seed=9).to(dtype)
-    out = as_tensor(mlp.forward(x.cuda(), ctx), ctx)
+    out = mlp.forward(x.cuda(), ctx)
     want = P.swiglu(x.double(), w["m.gate_proj.weight"].double(), w["m.up_proj.weight"].double(),
                     w["m.down_proj.weight"].double())
     assert torch.allclose(out.cpu().double(), want, **tol(dtype))
@@ -152,7 +147,7 @@ def test_attention_part_prompt_then_tokens(fw, dtype, fast, window):
     # the prompts in one step
     cache.reserve(list(zip(slots, lens)))
     ctx = make_ctx(fw, env, lens, [0, 0], slots)
-    out = as_tensor(att.forward(torch.cat([x[:n] for x, n in zip(xs, lens)]).cuda(), ctx, lc), ctx).cpu().double()
+    out = att.forward(torch.cat([x[:n] for x, n in zip(xs, lens)]).cuda(), ctx, lc).cpu().double()
     cache.commit(list(zip(slots, lens)))
     near(out[:70], want[0][:70], dtype)
     near(out[70:], want[1][:3], dtype)
@@ -162,7 +157,7 @@ def test_attention_part_prompt_then_tokens(fw, dtype, fast, window):
         cache.reserve(list(zip(slots, new)))
         ctx = make_ctx(fw, env, [1, 1], [n + t for n in lens], slots)
         x = torch.stack([xs[0][70 + t], xs[1][3 + t]])
-        out = as_tensor(att.forward(x.cuda(), ctx, lc), ctx).cpu().double()
+        out = att.forward(x.cuda(), ctx, lc).cpu().double()
         cache.commit(list(zip(slots, new)))
         near(out[0], want[0][70 + t], dtype)
         near(out[1], want[1][3 + t], dtype)
@@ -443,10 +438,9 @@ def toys(fw):
             self.w = tensors[self.prefix + "weight"].float()
 
         def add_norm(self, resid, delta, rows, ctx, want_out=True):
-            from hector_engine_amd.parts.linear import as_tensor
             r = resid[:rows]
             if delta is not None:
-                r += as_tensor(delta, ctx)[:rows].float()
+                r += delta[:rows].float()
             if not want_out:
                 return None
             c = r - r.mean(-1, keepdim=True)
