@@ -323,13 +323,13 @@ attention_prefill_pair_kernel(
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int lr = lane & 15, lg = lane >> 4;
-  // Workgroups go to the eight XCDs in turn, and each XCD has an L2 of its own. The work is
+  // Workgroups go to the HE_XCDS XCDs in turn, and each XCD has an L2 of its own. The work is
   // numbered so that an XCD gets a contiguous range of (head, sequence, query tiles): its
   // workgroups then read the pages of one or two kv heads, not of all, and its L2 holds them.
   const int total = gridDim.x * gridDim.y * gridDim.z;
   const int launched = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-  const int xcd = launched & 7, share = total >> 3, extra = total & 7;
-  const int work = xcd * share + min(xcd, extra) + (launched >> 3);
+  const int xcd = launched % HE_XCDS, share = total / HE_XCDS, extra = total % HE_XCDS;
+  const int work = xcd * share + min(xcd, extra) + launched / HE_XCDS;
   const int tile_x = work % gridDim.x;
   const int seq = (work / gridDim.x) % gridDim.z, h = work / (gridDim.x * gridDim.z);
   const int slot = seq_slot[seq];

@@ -52,6 +52,20 @@ def source_hash() -> str:
     return h.hexdigest()
 
 
+def private_folder() -> str:
+    """The per-user folder under the temporary directory (fallback build, tuning file).
+    Created with mode 0700; a folder of that name that belongs to someone else, or that
+    others may write, is refused: a library found there would be loaded as code."""
+    folder = os.path.join(tempfile.gettempdir(), f"hector-engine_amd-{os.getuid()}")
+    os.makedirs(folder, mode=0o700, exist_ok=True)
+    st = os.lstat(folder)
+    import stat
+    if not stat.S_ISDIR(st.st_mode) or st.st_uid != os.getuid() or st.st_mode & 0o022:
+        raise RuntimeError(f"{folder} is not a private folder of this user (owner {st.st_uid}, "
+                           f"mode {stat.S_IMODE(st.st_mode):o}): remove it or set TMPDIR")
+    return folder
+
+
 def _writable(folder: str) -> bool:
     try:
         os.makedirs(folder, exist_ok=True)
@@ -65,8 +79,11 @@ def _writable(folder: str) -> bool:
 
 
 def _candidate_dirs() -> list[str]:
-    fallback = os.path.join(tempfile.gettempdir(), f"hector-engine_amd-{os.getuid()}")
-    return [CSRC, fallback]
+    """The source folder, then the private fallback (left out when it cannot be trusted)."""
+    try:
+        return [CSRC, private_folder()]
+    except (OSError, RuntimeError):
+        return [CSRC]
 
 
 def _stamp_path(folder: str) -> str:
@@ -106,7 +123,8 @@ def build(force: bool = True, jobs: int | None = None) -> str:
     folder = next((d for d in _candidate_dirs() if _writable(d)), None)
     if folder is None:
         raise RuntimeError("no writable folder for the kernel library build")
-    obj_dir = os.path.join(folder, "_build")
+    # objects of this process only: two processes that build at once do not share files
+    obj_dir = os.path.join(folder, "_build", f"obj{os.getpid()}")
     os.makedirs(obj_dir, exist_ok=True)
     srcs = sources()
     jobs = jobs or max(1, min(len(srcs), int(os.environ.get("MAX_JOBS", "0")) or os.cpu_count() or 4, 16))
@@ -131,8 +149,11 @@ def build(force: bool = True, jobs: int | None = None) -> str:
     if proc.returncode != 0:
         raise RuntimeError(f"link failed:\n{proc.stderr[-6000:]}")
     os.replace(tmp, lib)
-    with open(_stamp_path(folder), "w") as f:
+    stamp_tmp = _stamp_path(folder) + f".tmp{os.getpid()}"
+    with open(stamp_tmp, "w") as f:
         f.write(digest)
+    os.replace(stamp_tmp, _stamp_path(folder))
+    shutil.rmtree(obj_dir, ignore_errors=True)
     _log(f"built {lib} in {time.time() - t0:.0f} s")
     return lib
 

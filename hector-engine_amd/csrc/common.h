@@ -16,6 +16,8 @@
 #define HE_PAGE_SHIFT 6
 
 #define HE_WAVE 64
+// L2 domains (XCDs) of the part; consecutive workgroups of a launch go to them in turn
+#define HE_XCDS 8
 
 struct bf16_t {
   uint16_t v;

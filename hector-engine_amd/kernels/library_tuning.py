@@ -6,30 +6,36 @@ The library's default choice of kernel is not always its best on MI355X: at the
 Qwen2.5-7B shapes its tuner finds kernels 17-27 % faster for the 2048-row down and
 gate||up products. Tuning runs the first time a shape (rows, N, K) is seen and takes a second
 or so per shape, so it is meant for workloads whose shapes repeat (fixed prompt chunks); it is
-off unless asked for. Results are kept in a file and read again by the next process. Row counts that
+off unless asked for. Results are kept in a file and read again by the next process (so the
+kernels chosen, and with them the last bits of bfloat16 results, follow that file: name one with
+HECTOR_TUNING_FILE or enable(path=...) where runs must repeat exactly). Row counts that
 are unlikely to come again (a prompt of 1,937 tokens) are not tuned: worth_tuning().
 """
 from __future__ import annotations
 
 import contextlib
 import os
-import tempfile
 
 import torch
+
+from . import lib as _lib
 
 _enabled = False
 
 
-def results_path() -> str:
-    folder = os.path.join(tempfile.gettempdir(), f"hector-engine_amd-{os.getuid()}")
-    os.makedirs(folder, exist_ok=True)
-    return os.path.join(folder, "library_gemm_tuning.csv")
+def results_path(path: str | None = None) -> str:
+    """The tuning file: the given path, else HECTOR_TUNING_FILE, else a file in this user's
+    private folder under the temporary directory."""
+    path = path or os.environ.get("HECTOR_TUNING_FILE")
+    if path:
+        return os.path.abspath(path)
+    return os.path.join(_lib._build_module().private_folder(), "library_gemm_tuning.csv")
 
 
-def enable(max_seconds_per_shape: int = 30, max_iterations: int = 10) -> None:
+def enable(max_seconds_per_shape: int = 30, max_iterations: int = 10, path: str | None = None) -> None:
     global _enabled
     t = torch.cuda.tunable
-    t.set_filename(results_path())
+    t.set_filename(results_path(path))
     t.enable(True)
     t.tuning_enable(True)
     t.set_max_tuning_duration(max_seconds_per_shape)
