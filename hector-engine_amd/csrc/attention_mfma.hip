@@ -88,306 +88,6 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   }
 }
 
-// ------------------------------------------------------------------ prefill, K/V through LDS
-// grid (ceil(max_q_len / 128), H, num_seqs), 256 threads. The workgroup takes 128
-// consecutive queries of one sequence and head, wavefront w the 32 queries 32w..32w+31 as
-// two tiles. The keys are walked a page (64 keys) at a time: the page's K and V^T are copied
-// once into LDS as the cache holds them, in the order the MFMA operands are read (one
-// operand of all 64 lanes is one contiguous KiB, so the reads have no bank conflicts, and
-// neither have the staging stores), and every operand a
-// wavefront reads from LDS feeds two MFMAs, one per tile - with one tile a wavefront the LDS
-// reads (32 KiB a page and wavefront), not the matrix cores, set the pace. The page in LDS
-// is double-buffered: the next page is written into the other buffer while this one is
-// used, one barrier a page; the page after that is on its way into registers meanwhile.
-// Head sizes up to 128. The staging arrays are native vectors: arrays of the uint4 struct
-// are not kept in registers by the compiler (it moves them to LDS or scratch).
-#define PF2_WAVES 4
-#define PF2_QUERIES (32 * PF2_WAVES)
-
-// Online softmax of one tile's scores of a step of 32 keys (see attend_frag); returns P^T
-// as the B operand of the value product.
-template <int NT, bool MASK>
-__device__ __forceinline__ bf16x8 softmax_step(AttnState<NT>& st, const floatx4* s, int key_base,
-                                               int lo, int hi, float scale_log2, int lg) {
-  // raw scores (masked ones at -inf), their maximum, then p = 2^(raw * scale - m) with the
-  // scale folded into the subtraction (scale > 0, so the maximum commutes with it)
-  float p[2][4];
-  float mx = -INFINITY;
-#pragma unroll
-  for (int t = 0; t < 2; ++t)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      float v = s[t][r];
-      if (MASK) {
-        const int key = key_base + 8 * lg + 4 * t + r;
-        v = (key >= lo && key <= hi) ? v : -INFINITY;
-      }
-      p[t][r] = v;
-      mx = fmaxf(mx, v);
-    }
-  mx = xor32_max(xor16_max(mx)) * scale_log2;
-  // the reference point follows the maximum only when that has grown by more than
-  // 2^HE_SOFTMAX_SLACK: p stays below that factor, and the accumulators are rarely rescaled
-  const float m_new = mx > st.m + HE_SOFTMAX_SLACK ? mx : st.m;
-  const bool moved = __builtin_amdgcn_ballot_w64(m_new != st.m) != 0;   // wave-uniform
-  const float m_use = m_new == -INFINITY ? 0.f : m_new;
-  float sum = 0.f;
-  uint32_t packed[4];
-#pragma unroll
-  for (int t = 0; t < 2; ++t)
-#pragma unroll
-    for (int r = 0; r < 4; r += 2) {
-      const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(p[t][r], scale_log2, -m_use));
-      const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(p[t][r + 1], scale_log2, -m_use));
-      sum += e0 + e1;
-      packed[2 * t + (r >> 1)] = pack2_bf16(e0, e1);
-    }
-  if (moved) {
-    const float alpha = __builtin_amdgcn_exp2f(st.m - m_use);
-    st.l = st.l * alpha + sum;
-    st.m = m_new;
-#pragma unroll
-    for (int dt = 0; dt < NT; ++dt) st.o[dt] *= alpha;
-  } else {
-    st.l += sum;
-  }
-  return __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
-}
-
-typedef uint32_t pf2_vec __attribute__((ext_vector_type(4)));   // 16 bytes, a native vector
-
-// A page of K and of V^T of one kv head, global memory -> registers -> LDS, 16-byte pieces,
-// one per thread and turn. The cache keeps its pages in operand order (cache_layout.h), so
-// the copy is straight: piece c goes to slot c, neighbouring threads write neighbouring
-// slots, and an operand read (64 lanes x 16 bytes, contiguous) has no bank conflicts.
-template <int NT>
-struct Pf2 {
-  static constexpr int HD = 16 * NT;
-  static constexpr int KS = (HD + 31) / 32;
-  static constexpr int THREADS = 64 * PF2_WAVES;
-  static constexpr int K_PIECES = 2 * 2 * KS * 64, V_PIECES = 2 * NT * 64;
-  static constexpr int K_TURNS = (K_PIECES + THREADS - 1) / THREADS;
-  static constexpr int V_TURNS = (V_PIECES + THREADS - 1) / THREADS;
-};
-
-template <int NT>
-__device__ __forceinline__ void pf2_fetch(pf2_vec (&kreg)[Pf2<NT>::K_TURNS],
-                                          pf2_vec (&vreg)[Pf2<NT>::V_TURNS],
-                                          const uint16_t* __restrict__ kp,
-                                          const uint16_t* __restrict__ vp, int page, int num_pages,
-                                          int64_t k_stride, int64_t v_stride) {
-  if (page < 0 || page >= num_pages) page = 0;   // never for an admitted batch
-  // no branch around a load (a thread beyond the page's pieces reads the last one, and
-  // pf2_stage leaves it out): the loads of a page go out together
-#pragma unroll
-  for (int j = 0; j < Pf2<NT>::K_TURNS; ++j) {
-    const int c = min((int)threadIdx.x + Pf2<NT>::THREADS * j, Pf2<NT>::K_PIECES - 1);
-    kreg[j] = *reinterpret_cast<const pf2_vec*>(kp + (int64_t)page * k_stride + 8 * c);
-  }
-#pragma unroll
-  for (int j = 0; j < Pf2<NT>::V_TURNS; ++j) {
-    const int c = min((int)threadIdx.x + Pf2<NT>::THREADS * j, Pf2<NT>::V_PIECES - 1);
-    vreg[j] = *reinterpret_cast<const pf2_vec*>(vp + (int64_t)page * v_stride + 8 * c);
-  }
-}
-
-template <int NT>
-__device__ __forceinline__ void pf2_stage(const pf2_vec (&kreg)[Pf2<NT>::K_TURNS],
-                                          const pf2_vec (&vreg)[Pf2<NT>::V_TURNS], pf2_vec* k_lds,
-                                          pf2_vec* v_lds) {
-#pragma unroll
-  for (int j = 0; j < Pf2<NT>::K_TURNS; ++j) {
-    const int c = threadIdx.x + Pf2<NT>::THREADS * j;
-    if (c < Pf2<NT>::K_PIECES) k_lds[c] = kreg[j];
-  }
-#pragma unroll
-  for (int j = 0; j < Pf2<NT>::V_TURNS; ++j) {
-    const int c = threadIdx.x + Pf2<NT>::THREADS * j;
-    if (c < Pf2<NT>::V_PIECES) v_lds[c] = vreg[j];
-  }
-}
-
-// One tile of 16 queries (a query per column) of such a wavefront.
-template <int NT>
-struct PairTile {
-  static constexpr int HD = 16 * NT;
-  static constexpr int KS = (HD + 31) / 32;
-  bf16x8 qf[KS];
-  AttnState<NT> st;
-  int qi, hi, lo, clear_lo, clear_hi;
-  int first, last;   // positions any query of the tile sees; first > last: no tile here
-  bool ok;
-
-  // whether the 32 keys from key_base on hold a key some query of the tile sees
-  __device__ __forceinline__ bool active(int key_base) const {
-    return key_base <= last && key_base + 31 >= first;
-  }
-
-  __device__ __forceinline__ void init(const uint16_t* __restrict__ q, int row0, int q_len,
-                                       int start, int qt, bool valid, int H, int h, int window,
-                                       int lr, int lg) {
-    qi = qt + lr;
-    ok = valid && qi < q_len;
-    last = valid ? start + min(qt + 15, q_len - 1) : -1;
-    first = !valid ? 0x7fffffff : (window > 0 ? max(0, start + qt + 1 - window) : 0);
-    const int pos = start + qi;
-    hi = ok ? pos : -1;
-    lo = (window > 0 && ok) ? max(0, pos + 1 - window) : 0;
-    load_q<NT>(qf, q + ((int64_t)(row0 + max(0, min(qi, q_len - 1))) * H + h) * HD, ok, lg);
-#pragma unroll
-    for (int dt = 0; dt < NT; ++dt) st.o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
-    st.m = -INFINITY;
-    st.l = 0.f;
-    // keys every query of a full tile sees: from its last query's window start to its first
-    // query's position
-    const int tlast = start + min(qt + 15, q_len - 1);
-    clear_lo = window > 0 ? max(0, tlast + 1 - window) : 0;
-    clear_hi = qt + 15 < q_len ? start + qt : -1;
-  }
-
-  __device__ __forceinline__ bf16x8 softmax(const floatx4* s, int key_base, float scale_log2,
-                                            int lg) {
-    if (key_base >= clear_lo && key_base + 31 <= clear_hi)
-      return softmax_step<NT, false>(st, s, key_base, lo, hi, scale_log2, lg);
-    return softmax_step<NT, true>(st, s, key_base, lo, hi, scale_log2, lg);
-  }
-
-  __device__ __forceinline__ void store(uint16_t* __restrict__ out, int row0, int H, int h, int lr,
-                                        int lg) {
-    float l = st.l;
-    l = xor32_sum(xor16_sum(l));
-    if (!ok) return;
-    const float inv = l > 0.f ? 1.f / l : 0.f;
-    uint16_t* orow = out + ((int64_t)(row0 + qi) * H + h) * HD;
-#pragma unroll
-    for (int dt = 0; dt < NT; ++dt) {
-      uint2 w;
-      w.x = pack2_bf16(st.o[dt][0] * inv, st.o[dt][1] * inv);
-      w.y = pack2_bf16(st.o[dt][2] * inv, st.o[dt][3] * inv);
-      *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * lg) = w;
-    }
-  }
-};
-
-// One step of 32 keys (half hb of the page in LDS) for the tiles that see keys in it. With
-// both, every operand read from LDS feeds two MFMAs.
-template <int NT, bool D0, bool D1>
-__device__ __forceinline__ void pf2_step(PairTile<NT>& t0, PairTile<NT>& t1, const pf2_vec* k_lds,
-                                         const pf2_vec* v_lds, int hb, int key_base,
-                                         float scale_log2, int lr, int lg) {
-  constexpr int HD = 16 * NT;
-  constexpr int KS = (HD + 31) / 32;
-  floatx4 s0[2], s1[2];
-#pragma unroll
-  for (int t = 0; t < 2; ++t) s0[t] = s1[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int t = 0; t < 2; ++t)
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      pf2_vec v = {0u, 0u, 0u, 0u};
-      if (32 * ks + 8 * lg < HD) v = k_lds[((hb * 2 + t) * KS + ks) * 64 + 16 * lg + lr];
-      const bf16x8 kf = __builtin_bit_cast(bf16x8, v);
-      if (D0) s0[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, t0.qf[ks], s0[t], 0, 0, 0);
-      if (D1) s1[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, t1.qf[ks], s1[t], 0, 0, 0);
-    }
-  bf16x8 p0, p1;
-  if (D0) p0 = t0.softmax(s0, key_base, scale_log2, lg);
-  if (D1) p1 = t1.softmax(s1, key_base, scale_log2, lg);
-#pragma unroll
-  for (int dt = 0; dt < NT; ++dt) {
-    const bf16x8 vf = __builtin_bit_cast(bf16x8, v_lds[(hb * NT + dt) * 64 + 16 * lg + lr]);
-    if (D0) t0.st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p0, t0.st.o[dt], 0, 0, 0);
-    if (D1) t1.st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p1, t1.st.o[dt], 0, 0, 0);
-  }
-}
-
-// The query tiles (16 queries) of a sequence are paired from both ends: tile a with tile
-// T - 1 - a. Under the causal mask an early tile sees few keys and a late one many; a pair
-// sees the same number of keys whatever a is, so every wavefront (one pair) and every
-// workgroup (four pairs) does the same work and none waits for a longest one. Where both
-// tiles of a pair see keys of a step the LDS operands are shared; the late tile walks the
-// rest alone.
-template <int NT>
-__global__ __launch_bounds__(64 * PF2_WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void
-attention_prefill_pair_kernel(
-    uint16_t* __restrict__ out, const uint16_t* __restrict__ q,
-    const uint16_t* __restrict__ kpool, const uint16_t* __restrict__ vpool,
-    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_slot,
-    const int32_t* __restrict__ seq_start, const int32_t* __restrict__ page_table, int max_blocks,
-    int num_pages, int H, int KVH, int window, float scale) {
-  constexpr int HD = 16 * NT;
-  constexpr int KS = (HD + 31) / 32;
-  // a page as the cache holds it: k[((hb*2 + t)*KS + ks)*64 + lane], v[(hb*NT + dt)*64 + lane]
-  __shared__ pf2_vec k_lds[2][Pf2<NT>::K_PIECES];
-  __shared__ pf2_vec v_lds[2][Pf2<NT>::V_PIECES];
-
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int lr = lane & 15, lg = lane >> 4;
-  // Workgroups go to the HE_XCDS XCDs in turn, and each XCD has an L2 of its own. The work is
-  // numbered so that an XCD gets a contiguous range of (head, sequence, query tiles): its
-  // workgroups then read the pages of one or two kv heads, not of all, and its L2 holds them.
-  const int total = gridDim.x * gridDim.y * gridDim.z;
-  const int launched = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-  const int xcd = launched % HE_XCDS, share = total / HE_XCDS, extra = total % HE_XCDS;
-  const int work = xcd * share + min(xcd, extra) + launched / HE_XCDS;
-  const int tile_x = work % gridDim.x;
-  const int seq = (work / gridDim.x) % gridDim.z, h = work / (gridDim.x * gridDim.z);
-  const int slot = seq_slot[seq];
-  if (slot < 0) return;
-  const int row0 = cu_seqlens[seq];
-  const int q_len = cu_seqlens[seq + 1] - row0;
-  const int tiles = (q_len + 15) >> 4;
-  const int pairs = (tiles + 1) >> 1;
-  const int pair0 = PF2_WAVES * tile_x;          // the workgroup's first pair: its earliest and latest tile
-  if (pair0 >= pairs) return;
-  const int start = seq_start[seq];
-  const int kvh = h / (H / KVH);
-  const int32_t* pt = page_table + (int64_t)slot * max_blocks;
-  const int64_t k_stride = (int64_t)KVH * he_k_page_elems(HD), v_stride = (int64_t)KVH * he_v_page_elems(HD);
-  const uint16_t* kp = kpool + (int64_t)kvh * he_k_page_elems(HD);
-  const uint16_t* vp = vpool + (int64_t)kvh * he_v_page_elems(HD);
-
-  const int pair = pair0 + wave;
-  const int ta = pair, tb = tiles - 1 - pair;    // ta <= tb while pair < pairs
-  PairTile<NT> t0, t1;
-  t0.init(q, row0, q_len, start, 16 * ta, pair < pairs, H, h, window, lr, lg);
-  t1.init(q, row0, q_len, start, 16 * tb, pair < pairs && tb > ta, H, h, window, lr, lg);
-  const float scale_log2 = scale * 1.4426950408889634f;
-
-  // pages from the first key the earliest tile sees to the last key of the latest tile
-  const int blk_last = start + min(16 * (tiles - 1 - pair0) + 15, q_len - 1);
-  const int blk_first = window > 0 ? max(0, start + 16 * pair0 + 1 - window) : 0;
-  const int pb0 = blk_first >> HE_PAGE_SHIFT, pb1 = blk_last >> HE_PAGE_SHIFT;
-
-  pf2_vec kreg[Pf2<NT>::K_TURNS], vreg[Pf2<NT>::V_TURNS];
-  pf2_fetch<NT>(kreg, vreg, kp, vp, pt[pb0], num_pages, k_stride, v_stride);
-  pf2_stage<NT>(kreg, vreg, k_lds[0], v_lds[0]);
-  if (pb0 < pb1) pf2_fetch<NT>(kreg, vreg, kp, vp, pt[pb0 + 1], num_pages, k_stride, v_stride);
-  __syncthreads();
-  for (int pb = pb0; pb <= pb1; ++pb) {
-    const int buf = (pb - pb0) & 1;
-    if (pb < pb1) {
-      // everyone left the other buffer before the last barrier
-      pf2_stage<NT>(kreg, vreg, k_lds[buf ^ 1], v_lds[buf ^ 1]);
-      if (pb + 1 < pb1) pf2_fetch<NT>(kreg, vreg, kp, vp, pt[pb + 2], num_pages, k_stride, v_stride);
-    }
-#pragma unroll
-    for (int hb = 0; hb < 2; ++hb) {
-      const int key_base = (pb << HE_PAGE_SHIFT) + 32 * hb;
-      const bool a0 = t0.active(key_base), a1 = t1.active(key_base);   // the same in all lanes
-      if (a0 && a1)
-        pf2_step<NT, true, true>(t0, t1, k_lds[buf], v_lds[buf], hb, key_base, scale_log2, lr, lg);
-      else if (a1)
-        pf2_step<NT, false, true>(t0, t1, k_lds[buf], v_lds[buf], hb, key_base, scale_log2, lr, lg);
-      else if (a0)
-        pf2_step<NT, true, false>(t0, t1, k_lds[buf], v_lds[buf], hb, key_base, scale_log2, lr, lg);
-    }
-    __syncthreads();
-  }
-  t0.store(out, row0, H, h, lr, lg);
-  t1.store(out, row0, H, h, lr, lg);
-}
-
 // ------------------------------------------------------------------ decode
 // grid (nsplit, KVH * head_tiles, rows), 64 threads. Columns are the query heads
 // of one kv group (16 per head tile). The keys of a sequence are cut into slices
@@ -629,15 +329,15 @@ extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* k
                                          const void* seq_slot, const void* seq_start,
                                          const void* page_table, int max_blocks, int num_pages,
                                          int num_seqs, int max_q_len, int H, int KVH, int hd,
-                                         int window, float scale, int tiles_per_wave,
+                                         int window, float scale, int kernel,
                                          void* stream) {
   HE_REQUIRE(num_seqs >= 0 && max_q_len >= 0 && H > 0 && KVH > 0 && hd > 0,
              "he_attention_prefill_bf16: bad sizes");
-  HE_REQUIRE(tiles_per_wave >= 0 && tiles_per_wave <= 2,
-             "he_attention_prefill_bf16: %d query tiles a wavefront (0 = the library's choice, 1, 2)",
-             tiles_per_wave);
-  HE_REQUIRE(tiles_per_wave < 2 || hd <= 128,
-             "he_attention_prefill_bf16: %d tiles a wavefront need head_dim %d <= 128", tiles_per_wave, hd);
+  HE_REQUIRE(kernel >= 0 && kernel <= 2,
+             "he_attention_prefill_bf16: kernel %d (0 = the library's choice; 1: 16 queries a wavefront, "
+             "operands from global memory; 2: 32 queries a wavefront, pages shared through LDS)", kernel);
+  HE_REQUIRE(kernel < 2 || hd <= 128,
+             "he_attention_prefill_bf16: kernel %d needs head_dim %d <= 128", kernel, hd);
   HE_REQUIRE(scale > 0.f, "he_attention_prefill_bf16: the score scale must be positive");
   HE_REQUIRE(H % KVH == 0, "he_attention_prefill_bf16: heads %d not a multiple of kv heads %d", H,
              KVH);
@@ -649,23 +349,11 @@ extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* k
              "he_attention_prefill_bf16: buffers must be 16-byte aligned");
   if (num_seqs == 0 || max_q_len == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  if (tiles_per_wave == 0) tiles_per_wave = (hd > 128 || max_q_len <= 16) ? 1 : 2;
-  if (tiles_per_wave == 2) {   // K/V pages shared through LDS by 128 queries
-    dim3 grid128((max_q_len + 127) / 128, H, num_seqs);
-#define PREFILL_LDS(NTV)                                                                        \
-  case NTV:                                                                                     \
-    attention_prefill_pair_kernel<NTV><<<grid128, 64 * PF2_WAVES, 0, s>>>(                      \
-        (uint16_t*)out, (const uint16_t*)q, (const uint16_t*)kpool, (const uint16_t*)vpool,     \
-        (const int32_t*)cu_seqlens, (const int32_t*)seq_slot, (const int32_t*)seq_start,        \
-        (const int32_t*)page_table, max_blocks, num_pages, H, KVH, window, scale);              \
-    break;
-    switch (hd / 16) {
-      PREFILL_LDS(1) PREFILL_LDS(2) PREFILL_LDS(3) PREFILL_LDS(4)
-      PREFILL_LDS(5) PREFILL_LDS(6) PREFILL_LDS(7) PREFILL_LDS(8)
-    }
-#undef PREFILL_LDS
-    return he_check_launch("he_attention_prefill_bf16");
-  }
+  if (kernel == 0) kernel = (hd > 128 || max_q_len <= 16) ? 1 : 2;
+  if (kernel == 2)
+    return he_attention_prefill_wide(out, q, kpool, vpool, cu_seqlens, seq_slot, seq_start, page_table,
+                                     max_blocks, num_pages, num_seqs, max_q_len, H, KVH, hd, window, scale,
+                                     stream);
   dim3 grid((max_q_len + 63) / 64, H, num_seqs);
   ATTN_SWITCH(hd / 16, (attention_prefill_kernel<NT><<<grid, 256, 0, s>>>(
                            (uint16_t*)out, (const uint16_t*)q, (const uint16_t*)kpool,

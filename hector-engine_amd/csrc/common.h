@@ -148,6 +148,12 @@ int he_check_launch(const char* what);
 int he_attention_merge_parts(void* out, const float* ws_o, const float* ws_ml, const void* row_seq,
                              int rows, int H, int hd, int parts, int out_pieces, void* stream);
 
+// attention_prefill_wide.hip: prompt attention, 32 queries a wavefront (head sizes up to 128; arguments checked by the caller)
+int he_attention_prefill_wide(void* out, const void* q, const void* kpool, const void* vpool,
+                              const void* cu_seqlens, const void* seq_slot, const void* seq_start,
+                              const void* page_table, int max_blocks, int num_pages, int num_seqs,
+                              int max_q_len, int H, int KVH, int hd, int window, float scale, void* stream);
+
 #define HE_REQUIRE(cond, ...)      \
   do {                             \
     if (!(cond)) {                 \

@@ -132,12 +132,15 @@ int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_t qkv_strid
                                    int hd, int window, float scale, int max_keys, int write_kv,
                                    int out_pieces, void* workspace_f32, int64_t workspace_floats,
                                    void* stream);
-// bf16, prompt steps: tiles of queries of one sequence against its cache rows.
+// bf16, prompt steps: tiles of queries of one sequence against its cache rows. kernel: 0 leaves
+// the choice to the library; 1: 16 queries a wavefront, operands straight from global memory
+// (any head size up to 256); 2: 32 queries a wavefront, pages shared through LDS, the softmax
+// beside the matrix products (head sizes up to 128).
 int he_attention_prefill_bf16(void* out, const void* q, const void* kpool, const void* vpool,
                               const void* cu_seqlens, const void* seq_slot, const void* seq_start,
                               const void* page_table, int max_blocks, int num_pages, int num_seqs,
                               int max_q_len, int H, int KVH, int hd, int window, float scale,
-                              int tiles_per_wave, void* stream);
+                              int kernel, void* stream);
 
 // ---- sampling ------------------------------------------------------------
 int64_t he_argmax_workspace_bytes(int rows, int V);

@@ -571,10 +571,10 @@ def attention_decode_fused(out, qkv, bias, kpool, vpool, positions, row_seq, seq
 @_op("attention_prefill")
 def attention_prefill(out, q, kpool, vpool, cu_seqlens, seq_slot, seq_start, page_table,
                       num_seqs: int, max_q_len: int, total_rows: int, H: int, KVH: int, hd: int,
-                      window: int, scale: float, tiles_per_wave: int = 0) -> None:
-    """tiles_per_wave: 0 leaves the kernel to the library (by head size and prompt length);
-    1 or 2 name it: one query tile a wavefront without LDS, or two with the pages shared
-    through LDS (head sizes up to 128)."""
+                      window: int, scale: float, kernel: int = 0) -> None:
+    """kernel: 0 leaves the choice to the library (by head size and prompt length); 1 or 2
+    name it: 16 queries a wavefront with operands from global memory, or 32 queries a
+    wavefront with the pages shared through LDS (head sizes up to 128)."""
     _check_attention(out, q, kpool, vpool, page_table, total_rows, H, KVH, hd)
     _need(q, "q", torch.bfloat16)
     for name, t in (("cu_seqlens", cu_seqlens), ("seq_slot", seq_slot), ("seq_start", seq_start)):
@@ -585,7 +585,7 @@ def attention_prefill(out, q, kpool, vpool, cu_seqlens, seq_slot, seq_start, pag
     _lib.check(L.he_attention_prefill_bf16(
         out.data_ptr(), q.data_ptr(), kpool.data_ptr(), vpool.data_ptr(), cu_seqlens.data_ptr(),
         seq_slot.data_ptr(), seq_start.data_ptr(), page_table.data_ptr(), page_table.shape[1],
-        kpool.shape[0], num_seqs, max_q_len, H, KVH, hd, window, float(scale), int(tiles_per_wave), _stream()))
+        kpool.shape[0], num_seqs, max_q_len, H, KVH, hd, window, float(scale), int(kernel), _stream()))
 
 
 @_op("argmax_rows")

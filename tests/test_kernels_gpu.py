@@ -476,12 +476,15 @@ def test_qkv_rope_cache(ops, dtype, H, KVH, hd, rot):
     assert (kp != 0).sum().item() <= rows * KVH * hd
 
 
-def attention_case(ops, kind, dtype, H, KVH, hd, window, lengths, q_lens, seed, pad=0, tiles=0):
-    """Runs one attention kernel over a crafted cache; returns (got, want) lists per sequence."""
+def attention_case(ops, kind, dtype, H, KVH, hd, window, lengths, q_lens, seed, pad=0, tiles=0, plant=None):
+    """Runs one attention kernel over a crafted cache; returns (got, want) lists per sequence.
+    plant(ks, vs) may change keys and values before they go into the cache."""
     B = len(lengths)
     slots, table, kpool, vpool = paged_setup(lengths, KVH, hd, dtype, seed)
     ks = [rnd(n, KVH, hd, seed=seed + 10 + i).to(dtype) for i, n in enumerate(lengths)]
     vs = [rnd(n, KVH, hd, seed=seed + 20 + i).to(dtype) for i, n in enumerate(lengths)]
+    if plant is not None:
+        plant(ks, vs)
     fill_cache(table, slots, kpool, vpool, ks, vs)
     qs = [rnd(m, H, hd, seed=seed + 30 + i, scale=2.0).to(dtype) for i, m in enumerate(q_lens)]
     rows = sum(q_lens)
@@ -506,7 +509,7 @@ def attention_case(ops, kind, dtype, H, KVH, hd, window, lengths, q_lens, seed, 
                              dev(table), rows + pad, H, KVH, hd, window, scale, max_keys, ws)
     else:
         ops.attention_prefill(out, dev(q), *args, dev(cu), dev(seq_slot), dev(seq_start), dev(table),
-                              B, max(q_lens), rows, H, KVH, hd, window, scale, tiles_per_wave=tiles)
+                              B, max(q_lens), rows, H, KVH, hd, window, scale, kernel=tiles)
     got, want = [], []
     r = 0
     for i, (n, m) in enumerate(zip(lengths, q_lens)):
@@ -545,8 +548,9 @@ def test_attention_decode(ops, H, KVH, hd, window):
 @pytest.mark.parametrize("window", [0, 70])
 @pytest.mark.parametrize("tiles", [0, 1, 2])
 def test_attention_prefill(ops, H, KVH, hd, window, tiles):
-    """Each of the prompt kernels (1 or 2 query tiles a wavefront; 0 = the library's choice):
-    whole prompts, a continuation (200 cached + 37 new) and a single token."""
+    """Each of the prompt kernels (1: 16 queries a wavefront without LDS, 2: 32 queries a wavefront
+    with the pages shared through LDS; 0 = the library's choice): whole prompts, a continuation
+    (200 cached + 37 new) and a single token."""
     if tiles >= 2 and hd > 128:
         from hector_engine_amd.kernels.lib import KernelLibraryError
         with pytest.raises(KernelLibraryError, match="head_dim"):
@@ -564,12 +568,39 @@ def test_attention_prefill(ops, H, KVH, hd, window, tiles):
 def test_attention_prefill_of_many_tiles(ops, H, KVH, hd, window, tiles):
     """Prompts of several workgroups' worth of query tiles: an even and an odd number of tiles, a
     last tile that is not full, a continuation whose first position is no multiple of 32 (its tiles'
-    diagonals then fall into different steps of 32 keys), and a prompt short enough that the pairs
-    from both ends meet inside one workgroup."""
+    diagonals then fall into different steps of 32 keys), and short prompts."""
     got, want = attention_case(ops, "prefill", torch.bfloat16, H, KVH, hd, window,
                                [1024, 713, 530, 48, 272], [1024, 713, 330, 48, 17], 43, tiles=tiles)
     for g, w in zip(got, want):
         assert torch.allclose(g, w, rtol=2 ** -6, atol=2 ** -6)
+
+
+@pytest.mark.parametrize("H,KVH,hd,window", [(7, 1, 128, 0), (4, 2, 64, 0), (3, 1, 80, 0), (4, 1, 128, 200)])
+def test_attention_prefill_shared_pages_edges(ops, H, KVH, hd, window):
+    """The kernel that shares pages through LDS, where its loops change over. Continuations whose
+    first new position is 31 or 63 past a multiple of 64 (the first query of a tile is then the last
+    key of a step, and of a page), a last tile of one query, one new token behind 700 cached ones, a
+    prompt of exactly one page, and 129 queries (a second workgroup for one query)."""
+    lengths = [64 * 5 + 31 + 97, 64 * 3 + 63 + 160, 64 * 4 + 33, 701, 64, 129]
+    q_lens = [97, 160, 33, 1, 64, 129]
+    got, want = attention_case(ops, "prefill", torch.bfloat16, H, KVH, hd, window, lengths, q_lens, 47, tiles=2)
+    for g, w in zip(got, want):
+        assert torch.allclose(g, w, rtol=2 ** -6, atol=2 ** -6)
+
+
+@pytest.mark.parametrize("tiles", [1, 2])
+def test_attention_prefill_reference_point_moves(ops, tiles):
+    """Random scores never make the softmax's reference point move after the first step, so the
+    branch that rescales the accumulators would go untested: two keys far before the diagonal are
+    made large (scores of several hundred for about half of the queries, first at key 300, larger
+    still at key 700), and one inside the last page."""
+    def plant(ks, vs):
+        ks[0][300] *= 40
+        ks[0][700] *= 160
+        ks[0][1000] *= 300
+    got, want = attention_case(ops, "prefill", torch.bfloat16, 7, 1, 128, 0, [1024], [1024], 48, tiles=tiles,
+                               plant=plant)
+    assert torch.allclose(got[0], want[0], rtol=2 ** -6, atol=2 ** -6)
 
 
 @pytest.mark.parametrize("H,KVH,hd", [(4, 1, 64), (28, 4, 128), (6, 3, 64), (40, 2, 128)])
