@@ -19,6 +19,9 @@
 // the P^T V product wants from it. A query is a column (l%16), so its softmax
 // statistics are reduced over registers and two lane swaps (xor 16, 32) only.
 // Softmax, its running maximum and sum, and both accumulators are fp32.
+// The prompt kernel here reads its operands from global memory; head sizes up to 128 and
+// prompts of more than 16 tokens go to the kernel in attention_prefill_wide.hip, which shares
+// pages through LDS (he_attention_prefill_bf16 chooses).
 #include "common.h"
 #include "hector_kernels.h"
 
