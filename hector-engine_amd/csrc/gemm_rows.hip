@@ -174,7 +174,7 @@ __global__ __launch_bounds__(64 * NWV) void gemm_rows_kernel(
   constexpr int BL = (MT * 256 + NT - 1) / NT;
   __shared__ __align__(16) unsigned char xs[2][MT * 4096];
   __shared__ float row_sq[NWV][16 * MT];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lr = lane & 15, lg = lane >> 4;
   // the workgroup's weight rows [n0, n_end): at most 16 R NWV, fewer when the rows are dealt out
   // evenly over the compute units (the last wavefronts then have a partly empty tile, or none)
@@ -222,17 +222,6 @@ __global__ __launch_bounds__(64 * NWV) void gemm_rows_kernel(
     const int cc = c + rot;
     return k_begin + (cc >= nchunks ? cc - nchunks : cc) * ROWS_KC;
   };
-  if (nchunks > 0) {
-    rows_load_b<MT, NT, XP, TAIL>(bst0, X, M, K, kof(0), k_end);
-    if (nchunks > 1) rows_load_b<MT, NT, XP, TAIL>(bst1, X, M, K, kof(1), k_end);
-    if (n_wave < n_end) {
-      rows_load_a<R, TAIL>(a0, wp, W, kof(0), lg, k_end);
-      if (nchunks > 1) rows_load_a<R, TAIL>(a1, wp, W, kof(1), lg, k_end);
-    }
-    rows_store_b<MT, NT>(bst0, xs[0]);
-    if (nchunks > 2) rows_load_b<MT, NT, XP, TAIL>(bst0, X, M, K, kof(2), k_end);
-  }
-  __syncthreads();
   // one chunk (A_: its weights, B_: its LDS buffer, N_: the register set of the next chunk's
   // rows). GUARD: near the end of the slice some of it is left out. WORK: false in a wavefront
   // without weight rows (rows dealt out evenly leave some): it only helps to copy the rows.
@@ -246,8 +235,27 @@ __global__ __launch_bounds__(64 * NWV) void gemm_rows_kernel(
     __syncthreads();                                                                               \
   }
   int j = 0;
-  if (n_wave < n_end) {
-    for (; j + 4 < nchunks; j += 2) {   // steady state without conditions: the compiler counts the loads in flight
+  if (n_wave < n_end && nchunks > 4) {
+    // The usual case, with nothing conditional ahead of its loop. The compiler places its waits
+    // for loads by what may be in flight on any path into a loop; with the loads below behind
+    // conditions (as in the general case further down) it had to assume, inside the loop and in
+    // every turn, that the rows' loads were the newest, and drained the weights of the next chunk
+    // with them: one chunk of weights in flight instead of two. The loads are issued in the
+    // order of the loop (rows, then weights) so that both ways into it look alike.
+    // (the scheduler would move the loads among each other; each sched_barrier keeps one group in its place)
+    rows_load_b<MT, NT, XP, TAIL>(bst0, X, M, K, kof(0), k_end);
+    __builtin_amdgcn_sched_barrier(0);
+    rows_load_b<MT, NT, XP, TAIL>(bst1, X, M, K, kof(1), k_end);
+    __builtin_amdgcn_sched_barrier(0);
+    rows_load_a<R, TAIL>(a0, wp, W, kof(0), lg, k_end);
+    __builtin_amdgcn_sched_barrier(0);
+    rows_store_b<MT, NT>(bst0, xs[0]);
+    rows_load_b<MT, NT, XP, TAIL>(bst0, X, M, K, kof(2), k_end);
+    __builtin_amdgcn_sched_barrier(0);
+    rows_load_a<R, TAIL>(a1, wp, W, kof(1), lg, k_end);
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    for (; j + 4 < nchunks; j += 2) {
       ROWS_STEP(a0, 0, bst1, j, false, true)
       ROWS_STEP(a1, 1, bst0, j + 1, false, true)
     }
@@ -257,10 +265,27 @@ __global__ __launch_bounds__(64 * NWV) void gemm_rows_kernel(
       ROWS_STEP(a1, 1, bst0, j + 1, true, true)
     }
   } else {
-    for (; j < nchunks; j += 2) {
-      ROWS_STEP(a0, 0, bst1, j, true, false)
-      if (j + 1 >= nchunks) break;
-      ROWS_STEP(a1, 1, bst0, j + 1, true, false)
+    if (nchunks > 0) {
+      rows_load_b<MT, NT, XP, TAIL>(bst0, X, M, K, kof(0), k_end);
+      if (nchunks > 1) rows_load_b<MT, NT, XP, TAIL>(bst1, X, M, K, kof(1), k_end);
+      if (n_wave < n_end) rows_load_a<R, TAIL>(a0, wp, W, kof(0), lg, k_end);
+      rows_store_b<MT, NT>(bst0, xs[0]);
+      if (nchunks > 2) rows_load_b<MT, NT, XP, TAIL>(bst0, X, M, K, kof(2), k_end);
+      if (n_wave < n_end && nchunks > 1) rows_load_a<R, TAIL>(a1, wp, W, kof(1), lg, k_end);
+    }
+    __syncthreads();
+    if (n_wave < n_end) {
+      for (; j < nchunks; j += 2) {
+        ROWS_STEP(a0, 0, bst1, j, true, true)
+        if (j + 1 >= nchunks) break;
+        ROWS_STEP(a1, 1, bst0, j + 1, true, true)
+      }
+    } else {
+      for (; j < nchunks; j += 2) {
+        ROWS_STEP(a0, 0, bst1, j, true, false)
+        if (j + 1 >= nchunks) break;
+        ROWS_STEP(a1, 1, bst0, j + 1, true, false)
+      }
     }
   }
 #undef ROWS_STEP
@@ -382,13 +407,16 @@ struct RowsPlan {
 // slice, their weight rows dealt out evenly over the workgroups the chip holds at once (two
 // a compute unit: 37888 rows as 499 workgroups of 76, the last three of whose eight wavefronts
 // only help to copy the activation rows; not 296 of 128, of which 40 would run after the
-// others); narrow ones are cut along K until the grid holds about a workgroup a compute unit.
+// others; above 32 rows one workgroup of sixteen wavefronts a compute unit); narrow ones are cut along K until the grid holds about a workgroup a compute unit.
 static RowsPlan rows_plan(int M, int N, int K, int R, int NWV, int splits) {
   RowsPlan p;
   p.MT = M <= 32 ? 2 : 4;
   if (R <= 0 || NWV <= 0) {
     if (N >= 65536) R = 2, NWV = 8;                        // the output head
-    else if (N >= 16384) R = 1, NWV = 8;                   // gate||up
+    else if (N >= 16384) R = 1, NWV = p.MT == 4 ? 16 : 8;  // gate||up: at 33 to 64 rows one workgroup a compute
+                                                           // unit, so that the unit fetches the activation rows
+                                                           // once, not twice (gate||up at 64 rows 61.1 -> 57.2 us;
+                                                           // without that copying it takes 53.6)
     else R = 1, NWV = (K >= 8192 || N >= 4096) ? 8 : 4;
   }
   p.R = R;
@@ -396,9 +424,9 @@ static RowsPlan rows_plan(int M, int N, int K, int R, int NWV, int splits) {
   const int cap = 16 * R * NWV;
   int rows = cap;
   if (N >= 16384 && splits <= 1) {
-    // dealt out evenly over the workgroups the chip holds at once: one of eight wavefronts with two
-    // tiles each a compute unit (the head), two otherwise
-    const int slots = 256 * (R == 2 && NWV == 8 ? 1 : 2);
+    // dealt out evenly over the workgroups the chip holds at once: one a compute unit where a workgroup
+    // has 256 rows (the head; sixteen wavefronts), two otherwise
+    const int slots = 256 * ((R == 2 && NWV == 8) || NWV == 16 ? 1 : 2);
     const int rounds = (N + slots * cap - 1) / (slots * cap);
     rows = ((N + slots * rounds - 1) / (slots * rounds) + 3) & ~3;
     if (rows > cap) rows = cap;
@@ -452,7 +480,7 @@ static int dispatch_rows(const RowsPlan& p, void* C, float* partial, const void*
     launch_rows<MT_, R_, NWV_, GATED, TC>(p, C, partial, X, W, bias, bias_dtype, M, N, K, fu, x_pieces, s); \
     return 0;                                                                                  \
   }
-  RW(2, 1, 4) RW(4, 1, 4) RW(4, 2, 4) RW(2, 1, 8) RW(4, 1, 8) RW(2, 2, 8) RW(4, 2, 8)
+  RW(2, 1, 4) RW(4, 1, 4) RW(4, 2, 4) RW(2, 1, 8) RW(4, 1, 8) RW(2, 2, 8) RW(4, 2, 8) RW(2, 1, 16) RW(4, 1, 16)
 #undef RW
   he_set_error("he_gemm_rows_bf16: no kernel for MT=%d R=%d NWV=%d", p.MT, p.R, p.NWV);
   return -1;
@@ -477,7 +505,7 @@ extern "C" int he_gemm_rows_bf16(void* C, void* partial_f32, int64_t partial_flo
   HE_REQUIRE(!out_pieces || ((resid != nullptr || out_dtype == HE_BF16) && ((gated ? N / 2 : N) & 7) == 0),
              "he_gemm_rows_bf16: a piece-major output is bf16 and a multiple of 8 wide");
   HE_REQUIRE(R <= 0 || R == 1 || R == 2, "he_gemm_rows_bf16: R=%d is not 1 or 2", R);
-  HE_REQUIRE(NWV <= 0 || NWV == 4 || NWV == 8, "he_gemm_rows_bf16: %d wavefronts, not 4 or 8", NWV);
+  HE_REQUIRE(NWV <= 0 || NWV == 4 || NWV == 8 || NWV == 16, "he_gemm_rows_bf16: %d wavefronts, not 4, 8 or 16", NWV);
   HE_REQUIRE((R <= 0) == (NWV <= 0), "he_gemm_rows_bf16: give both R and NWV, or neither");
   HE_REQUIRE(!(R == 2 && NWV == 4) || M > 32,
              "he_gemm_rows_bf16: two tiles a wavefront in four wavefronts are for more than 32 rows");

@@ -9,7 +9,7 @@ from tests.test_kernels_gpu import alternate_rows, dev, from_pieces, rnd, to_pie
 
 pytestmark = pytest.mark.gpu
 
-PLANS = [(0, 0, 0), (1, 8, 1), (2, 8, 1), (1, 4, 1), (1, 4, 3), (1, 8, 4), (2, 8, 16), (2, 4, 1)]
+PLANS = [(0, 0, 0), (1, 8, 1), (2, 8, 1), (1, 4, 1), (1, 4, 3), (1, 8, 4), (2, 8, 16), (2, 4, 1), (1, 16, 1), (1, 16, 2)]
 SHAPES = [(301, 136), (1000, 1544), (37, 4104), (4608, 3584), (2051, 264), (512, 128), (20002, 136)]
 
 
@@ -65,7 +65,7 @@ def test_gemm_rows(ops, M, N, K, plan):
 
 @pytest.mark.parametrize("M", [1, 17, 32, 50, 64])
 @pytest.mark.parametrize("I,K", [(160, 64), (1008, 520), (37, 136), (1515, 264), (4000, 1024), (9475, 264)])
-@pytest.mark.parametrize("plan", [(0, 0, 1), (1, 4, 1), (2, 4, 1), (1, 8, 1), (2, 8, 1)])
+@pytest.mark.parametrize("plan", [(0, 0, 1), (1, 4, 1), (2, 4, 1), (1, 8, 1), (2, 8, 1), (1, 16, 1)])
 def test_gemm_rows_gated_epilogue(ops, M, I, K, plan):
     if plan == (2, 4, 1) and M <= 32:
         pytest.skip("two tiles a wavefront in four wavefronts: above 32 rows")
@@ -163,7 +163,9 @@ def test_gemm_rows_refuses_what_it_cannot_do(ops):
                       dev(rnd(20, 100, seed=3).to(torch.bfloat16)), dev(rnd(64, 100, seed=4).to(torch.bfloat16)), None, 20)
     groups, splits = ops.gemm_rows_plan(64, 3584, 18944)
     assert groups * splits >= 192 and splits > 1                      # few rows, long K: cut across workgroups
-    # wide products: one slice, the rows dealt out evenly (76 a workgroup, not 64 or 80; 200, not 256)
-    assert ops.gemm_rows_plan(64, 37888, 3584) == (499, 1) and ops.gemm_rows_plan(64, 152064, 3584) == (761, 1)
+    # wide products: one slice, the rows dealt out evenly (76 a workgroup, not 64 or 80; 200, not 256;
+    # above 32 rows one workgroup of 148 rows a compute unit)
+    assert ops.gemm_rows_plan(32, 37888, 3584) == (499, 1) and ops.gemm_rows_plan(64, 152064, 3584) == (761, 1)
+    assert ops.gemm_rows_plan(64, 37888, 3584) == (256, 1)
     with pytest.raises(KernelLibraryError, match="more than 32 rows"):
         ops.gemm_rows(out, None, a, w, None, 20, plan=(2, 4, 1))
