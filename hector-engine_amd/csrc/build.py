@@ -126,7 +126,8 @@ def build(force: bool = True, jobs: int | None = None) -> str:
     # objects of this process only: two processes that build at once do not share files
     obj_dir = os.path.join(folder, "_build", f"obj{os.getpid()}")
     os.makedirs(obj_dir, exist_ok=True)
-    srcs = sources()
+    # the product kernels have the most instantiations and take longest: they start first
+    srcs = sorted(sources(), key=lambda s: (not os.path.basename(s).startswith("gemm_"), s))
     jobs = jobs or max(1, min(len(srcs), int(os.environ.get("MAX_JOBS", "0")) or os.cpu_count() or 4, 16))
     _log(f"compiling {len(srcs)} sources for {ARCH} with {jobs} jobs into {folder}")
     t0 = time.time()

@@ -39,7 +39,7 @@ def product(ops, a, w, bias, M, plan, out_dtype=torch.float32, **kw):
     return out.cpu(), used
 
 
-@pytest.mark.parametrize("M", [1, 16, 17, 20, 32, 33, 47, 64])
+@pytest.mark.parametrize("M", [1, 16, 17, 20, 32, 33, 47, 48, 49, 64])
 @pytest.mark.parametrize("N,K", SHAPES)
 @pytest.mark.parametrize("plan", PLANS)
 def test_gemm_rows(ops, M, N, K, plan):
@@ -63,7 +63,7 @@ def test_gemm_rows(ops, M, N, K, plan):
         assert torch.equal(outp, outs[0])
 
 
-@pytest.mark.parametrize("M", [1, 17, 32, 50, 64])
+@pytest.mark.parametrize("M", [1, 17, 32, 40, 50, 64])
 @pytest.mark.parametrize("I,K", [(160, 64), (1008, 520), (37, 136), (1515, 264), (4000, 1024), (9475, 264)])
 @pytest.mark.parametrize("plan", [(0, 0, 1), (1, 4, 1), (2, 4, 1), (1, 8, 1), (2, 8, 1), (1, 16, 1)])
 def test_gemm_rows_gated_epilogue(ops, M, I, K, plan):
