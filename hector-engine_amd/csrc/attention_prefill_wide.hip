@@ -34,10 +34,11 @@
 // running maximum only when that has grown by more than 2^PW_SLACK, and the accumulators are
 // rescaled only then. Epochs that hold a masked step (the diagonal, a window's start, the
 // first and the last of a tile) run through a plain variant of the same contract.
-// Workgroups with many keys are launched first, over all heads and sequences; an XCD sees
-// neighbouring heads. Head sizes up to 128.
+// Workgroups with many keys are launched first, over all heads and sequences (a launch that
+// fits on the chip at once puts its lightest beside its heaviest); an XCD sees neighbouring
+// heads. Head sizes up to 128.
 //
-// Measured at 28 heads of 128, 4 kv heads (causal flops): 0.57 PFLOP/s at 2048 tokens,
+// Measured at 28 heads of 128, 4 kv heads (causal flops): 0.61 PFLOP/s at 2048 tokens,
 // 0.94 at 8192, 1.1 at 16384, 0.85 for eight prompts of 2048. In the long runs the shader
 // clock sits near 1.4 GHz (s_memtime against the 100 MHz counter), so 1.1 PFLOP/s is four
 // fifths of what the matrix cores give at that clock; at 2048 tokens the launch is as long
@@ -353,9 +354,19 @@ attention_prefill_wide_kernel(
   const int launched = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
   int gcd = HE_XCDS;
   while (rows % gcd) gcd >>= 1;               // HE_XCDS is a power of two
-  const int rho = launched % rows;
+  // When the whole launch is on the chip at once (two workgroups a compute unit), a unit's second
+  // workgroup is the one launched HE_CUS after its first (the 33rd of its XCD): the heaviest gets
+  // the lightest beside it, and so on, and every unit has about the same to do (2048 tokens,
+  // 28 heads: 52.1 -> 49.6 us).
+  int rank = launched;
+  if ((int)(gridDim.x * rows) <= 2 * HE_CUS) {
+    const int x = launched % HE_XCDS, j = launched / HE_XCDS;
+    const int of_xcd = ((int)(gridDim.x * rows) - x + HE_XCDS - 1) / HE_XCDS;
+    rank = x + HE_XCDS * (j < HE_CUS / HE_XCDS ? j : of_xcd - 1 - (j - HE_CUS / HE_XCDS));
+  }
+  const int rho = rank % rows;
   const int row = (rho % gcd) * (rows / gcd) + rho / gcd;
-  const int bx = gridDim.x - 1 - launched / rows;
+  const int bx = gridDim.x - 1 - rank / rows;
   const int seq = row % gridDim.z, h = row / gridDim.z;
   const int slot = seq_slot[seq];
   if (slot < 0) return;

@@ -18,6 +18,8 @@
 #define HE_WAVE 64
 // L2 domains (XCDs) of the part; consecutive workgroups of a launch go to them in turn
 #define HE_XCDS 8
+// compute units of the part (the grids of the products count in them as well)
+#define HE_CUS 256
 
 struct bf16_t {
   uint16_t v;
