@@ -273,9 +273,9 @@ static void fused_shape(int rows, int H, int KVH, int hd, int max_keys, int* nw,
   const int gt = G < 16 ? G : 16;
   const int groups = rows * KVH * ((G + 15) / 16);
   int w = (int64_t)8 * gt * (hd + 2) * 4 <= 65536 ? 8 : 4, zz = 1;
-  if (groups < 256) {
+  if (groups < HE_CUS) {
     w = 4;
-    zz = (256 + groups - 1) / groups;
+    zz = (HE_CUS + groups - 1) / groups;
     const int cap = max_keys > 16384 ? 32 : 16;
     if (zz > cap) zz = cap;
     const int most = (max_keys + 4 * FUSED_MIN_CHUNK - 1) / (4 * FUSED_MIN_CHUNK);

@@ -48,14 +48,14 @@ static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int
     else if (p.MT == 1) r = 4, u = 2, nw = 4;
     else r = 2, u = 2, nw = 4;
   } else if (K >= 8192) {           // long K
-    const int groups = (N + 31) / 32, last_round = groups % 256;   // with two tiles a workgroup
+    const int groups = (N + 31) / 32, last_round = groups % HE_CUS;   // with two tiles a workgroup
     if (N < 4096) {                 // few weight rows: one tile a workgroup, or the chip is not filled
       r = 1, u = 1, nw = p.MT == 1 ? 8 : 4;
     } else if (p.MT == 2) {
       r = 2, u = 2, nw = 4;
     } else if (M > 8 && N >= 10240) {
       r = 4, u = 2, nw = 4;         // the activation rows are read half as often
-    } else if (groups < 256) {
+    } else if (groups < HE_CUS) {
       r = 2, u = 1, nw = 8;         // under one workgroup a compute unit: more wavefronts each
     } else if (groups < 1024 && last_round > 0 && last_round <= 128) {
       r = 1, u = 1, nw = 8;         // the last round of whole tiles would fill under half of the chip:
@@ -82,8 +82,8 @@ static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int
   // stored in pairs.
   int rows = 0;
   if (R <= 0 && r <= 2 && N >= 2048 && N < 65536) {
-    const int rounds = (N + 256 * 32 - 1) / (256 * 32);
-    rows = ((N + 256 * rounds - 1) / (256 * rounds) + 1) & ~1;
+    const int rounds = (N + HE_CUS * 32 - 1) / (HE_CUS * 32);
+    rows = ((N + HE_CUS * rounds - 1) / (HE_CUS * rounds) + 1) & ~1;
     r = rows > 16 ? 2 : 1;
   }
   p.R = R > 0 ? R : r;

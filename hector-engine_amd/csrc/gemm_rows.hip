@@ -49,7 +49,7 @@ static RowsPlan rows_plan(int M, int N, int K, int R, int NWV, int splits) {
   if (N >= 16384 && splits <= 1) {
     // dealt out evenly over the workgroups the chip holds at once: one a compute unit where a workgroup
     // has 256 rows (the head; sixteen wavefronts), two otherwise
-    const int slots = 256 * ((R == 2 && NWV == 8) || NWV == 16 ? 1 : 2);
+    const int slots = HE_CUS * ((R == 2 && NWV == 8) || NWV == 16 ? 1 : 2);
     const int rounds = (N + slots * cap - 1) / (slots * cap);
     rows = ((N + slots * rounds - 1) / (slots * rounds) + 3) & ~3;
     if (rows > cap) rows = cap;
