@@ -181,6 +181,11 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
 // Joins the slices of one (row, head): grid (H, rows), four wavefronts; wavefront w adds
 // the slices s = w, w + 4, ... and the four sums are added in wavefront order. The number
 // of slices that hold keys is recomputed exactly as the decode kernel computes it.
+// The launch is a chain of trips to memory and little else, so the loads that need no
+// loaded value to know their address go out together at the start: the row's sequence, the
+// slices' statistics and the first 32 slices' outputs (when every part was stored, that is
+// all of them), and a row without a sequence is dealt with at the store.
+#define MERGE_PER 8   // slices a wavefront holds at once
 __global__ __launch_bounds__(256) void attention_merge_kernel(
     uint16_t* __restrict__ out, const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq, int H, int HD,
@@ -195,43 +200,60 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(
     const int64_t c = (int64_t)h * HD + d;
     return out_pieces ? out + ((c >> 3) * gridDim.y + row) * 8 + (c & 7) : out + row * H * (int64_t)HD + c;
   };
-  if (row_seq[row] < 0) {
-    for (int d = threadIdx.x; d < HD; d += 256) *at(d) = 0;
-    return;
-  }
+  const bool live = row_seq[row] >= 0;
   int active = nsplit;                     // all_parts: every part was stored, empty ones as (-inf, 0, 0)
   if (!all_parts) {
-    const int n_keys = positions[row] + 1;
-    const int first = window > 0 ? max(0, n_keys - window) : 0;
-    const int span_lo = first & ~31;
-    int chunk = (n_keys - span_lo + nsplit - 1) / nsplit;
-    chunk = max(DECODE_MIN_CHUNK, (chunk + 31) & ~31);
-    active = (n_keys - span_lo + chunk - 1) / chunk;
+    active = 0;
+    if (live) {
+      const int n_keys = positions[row] + 1;
+      const int first = window > 0 ? max(0, n_keys - window) : 0;
+      const int span_lo = first & ~31;
+      int chunk = (n_keys - span_lo + nsplit - 1) / nsplit;
+      chunk = max(DECODE_MIN_CHUNK, (chunk + 31) & ~31);
+      active = (n_keys - span_lo + chunk - 1) / chunk;
+    }
   }
   const int64_t base = (row * H + h) * nsplit;
+  // outputs of the slices s0 + wave + 4 i at the dims d0 + lane + 64 j; what does not exist reads as 0
+  auto load_slices = [&](float (&ov)[MERGE_PER][4], int d0, int s0) {
+#pragma unroll
+    for (int i = 0; i < MERGE_PER; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int s = s0 + wave + 4 * i, d = d0 + lane + 64 * j;
+        ov[i][j] = s < active && d < HD ? ws_o[(base + s) * HD + d] : 0.f;
+      }
+  };
   const float m = lane < active ? ws_ml[2 * (base + lane)] : -INFINITY;
   const float l = lane < active ? ws_ml[2 * (base + lane) + 1] : 0.f;
+  float ov[MERGE_PER][4];
+  load_slices(ov, 0, 0);
   const float M = wave_max(m);
   const float w = m > -INFINITY ? __builtin_amdgcn_exp2f(m - M) : 0.f;   // m is in the base-2 domain
   const float L = wave_sum(l * w);          // every wavefront computes the same weights
-  if (wave == 0) wgt[lane] = w;
+  if (wave == 0) wgt[lane] = w;             // 0 from `active` on
   __syncthreads();
   const float inv = L > 0.f ? 1.f / L : 0.f;
   for (int d0 = 0; d0 < HD; d0 += 256) {
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < active; s0 += 4 * MERGE_PER) {
+      if (d0 + s0 > 0) load_slices(ov, d0, s0);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int d = d0 + lane + 64 * j;
-      float acc = 0.f;
-      if (d < HD)
-        for (int s = wave; s < active; s += 4) acc += ws_o[(base + s) * HD + d] * wgt[s];
-      part[wave][lane + 64 * j] = acc;
+      for (int i = 0; i < MERGE_PER; ++i) {
+        const int s = s0 + wave + 4 * i;
+        const float ws = s < active ? wgt[s] : 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] += ov[i][j] * ws;
+      }
     }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) part[wave][lane + 64 * j] = acc[j];
     __syncthreads();
     const int d = d0 + threadIdx.x;
     if (d < HD) {
-      const float acc = ((part[0][threadIdx.x] + part[1][threadIdx.x]) + part[2][threadIdx.x]) +
+      const float sum = ((part[0][threadIdx.x] + part[1][threadIdx.x]) + part[2][threadIdx.x]) +
                         part[3][threadIdx.x];
-      *at(d) = float_to_bf16_bits(acc * inv);
+      *at(d) = live ? float_to_bf16_bits(sum * inv) : (uint16_t)0;
     }
     __syncthreads();
   }
