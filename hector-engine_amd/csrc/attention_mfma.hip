@@ -200,7 +200,7 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(
     const int64_t c = (int64_t)h * HD + d;
     return out_pieces ? out + ((c >> 3) * gridDim.y + row) * 8 + (c & 7) : out + row * H * (int64_t)HD + c;
   };
-  const bool live = row_seq[row] >= 0;
+  const bool live = row_seq == nullptr || row_seq[row] >= 0;
   int active = nsplit;                     // all_parts: every part was stored, empty ones as (-inf, 0, 0)
   if (!all_parts) {
     active = 0;
@@ -340,6 +340,58 @@ extern "C" int he_attention_decode_bf16(void* out, const void* q, const void* kp
   return he_check_launch("he_attention_decode_bf16 merge");
 }
 
+// The same join for many rows (the parts of a prompt step): one wavefront per (row, head), four
+// of them a workgroup, no LDS and no barrier; a lane has the dims 2 lane, 2 lane + 1 (+ 128, ...).
+// Parts are added in their order. Every part was stored; out is row-major.
+__global__ __launch_bounds__(256) void attention_merge_rows_kernel(
+    uint16_t* __restrict__ out, const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+    int64_t pairs, int HD, int nsplit) {
+  const int lane = threadIdx.x & 63;
+  const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);   // row * H + h
+  if (pair >= pairs) return;
+  const int64_t base = pair * nsplit;
+  const float2 ml = lane < nsplit ? *reinterpret_cast<const float2*>(ws_ml + 2 * (base + lane))
+                                  : make_float2(-INFINITY, 0.f);
+  auto load_parts = [&](float2 (&ov)[MERGE_PER], int d0, int s0) {
+#pragma unroll
+    for (int i = 0; i < MERGE_PER; ++i)
+      ov[i] = s0 + i < nsplit && d0 < HD ? *reinterpret_cast<const float2*>(ws_o + (base + s0 + i) * HD + d0)
+                                         : make_float2(0.f, 0.f);
+  };
+  float2 ov[MERGE_PER];
+  load_parts(ov, 2 * lane, 0);   // on their way while the weights are made
+  // lane s has the weight of part s (0 from nsplit on); all lanes take part in the sums
+  const float M = wave_max(ml.x);
+  const float w = ml.x > -INFINITY ? __builtin_amdgcn_exp2f(ml.x - M) : 0.f;   // base-2 domain
+  const float L = wave_sum(ml.y * w);
+  const float inv = L > 0.f ? 1.f / L : 0.f;
+  for (int d0 = 2 * lane; d0 < HD; d0 += 128) {
+    float2 acc = make_float2(0.f, 0.f);
+    for (int s0 = 0; s0 < nsplit; s0 += MERGE_PER) {
+      if (d0 >= 128 || s0 > 0) load_parts(ov, d0, s0);
+#pragma unroll
+      for (int i = 0; i < MERGE_PER; ++i) {
+        // v_readlane: the lane is the same for all, and it need not be active
+        const float w_s = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), (s0 + i) & 63));
+        acc.x += ov[i].x * w_s;
+        acc.y += ov[i].y * w_s;
+      }
+    }
+    *reinterpret_cast<uint32_t*>(out + pair * HD + d0) = pack2_bf16(acc.x * inv, acc.y * inv);
+  }
+}
+
+int he_attention_merge_rows(void* out, const float* ws_o, const float* ws_ml, int rows, int H, int hd,
+                            int parts, void* stream) {
+  HE_REQUIRE(parts >= 1 && parts <= 64 && hd % 2 == 0, "he_attention_merge_rows: %d parts (at most 64), head_dim %d", parts, hd);
+  const int64_t pairs = (int64_t)rows * H;
+  HE_REQUIRE((pairs + 3) / 4 < (1ll << 31), "he_attention_merge_rows: too many rows for one launch");
+  if (pairs == 0) return 0;
+  attention_merge_rows_kernel<<<(unsigned)((pairs + 3) / 4), 256, 0, (hipStream_t)stream>>>(
+      (uint16_t*)out, ws_o, ws_ml, pairs, hd, parts);
+  return he_check_launch("he_attention_merge_rows");
+}
+
 // Joins parts [rows][H][parts] of (O fp32 [hd], then (m, l) pairs) that were all stored.
 int he_attention_merge_parts(void* out, const float* ws_o, const float* ws_ml, const void* row_seq,
                              int rows, int H, int hd, int parts, int out_pieces, void* stream) {
@@ -349,14 +401,37 @@ int he_attention_merge_parts(void* out, const float* ws_o, const float* ws_ml, c
   return he_check_launch("he_attention_merge_parts");
 }
 
+// Parts the keys of a prompt step are cut into (he_attention_prefill_bf16's `parts`): a step with few
+// blocks of 128 queries and many keys (a short continuation of a long sequence) would leave most of the
+// chip idle, each of its workgroups walking all the pages alone. As many parts as bring the launch to two
+// workgroups a compute unit, each of at least 16 pages, at most 16. most_keys: the most keys a sequence
+// of the step has (or a bound). Measured at 28 heads of 128, 4 kv heads (us without parts -> with, join
+// included): 64 tokens after 8000 114 -> 27, 200 after 8000 129 -> 45, 512 after 7680 130 -> 76, 4 x 128
+// after 4000 74 -> 51, 512 after 30000 457 -> 233; 1024 after 7168 144 -> 134 (two parts); a whole prompt
+// of 2048 tokens has workgroups enough and stays whole (47 us; 71 in two parts).
+extern "C" int he_attention_prefill_parts(int num_seqs, int max_q_len, int H, int hd, int most_keys) {
+  if (num_seqs <= 0 || H <= 0 || hd <= 0 || hd > 128 || hd % 16 || max_q_len <= 16) return 1;
+  const int64_t blocks = (int64_t)((max_q_len + 127) / 128) * H * num_seqs;
+  int64_t parts = 2 * HE_CUS / blocks;
+  const int pages = (most_keys + HE_PAGE_TOKENS - 1) / HE_PAGE_TOKENS;
+  if (parts > pages / 16) parts = pages / 16;
+  if (parts > 16) parts = 16;
+  return parts < 1 ? 1 : (int)parts;
+}
+
+extern "C" int64_t he_attention_prefill_workspace_floats(int total_rows, int H, int hd, int parts) {
+  return parts > 1 ? (int64_t)total_rows * H * parts * (hd + 2) : 0;
+}
+
 extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* kpool,
                                          const void* vpool, const void* cu_seqlens,
                                          const void* seq_slot, const void* seq_start,
                                          const void* page_table, int max_blocks, int num_pages,
                                          int num_seqs, int max_q_len, int H, int KVH, int hd,
-                                         int window, float scale, int kernel,
+                                         int window, float scale, int kernel, int total_rows,
+                                         int parts, void* workspace_f32, int64_t workspace_floats,
                                          void* stream) {
-  HE_REQUIRE(num_seqs >= 0 && max_q_len >= 0 && H > 0 && KVH > 0 && hd > 0,
+  HE_REQUIRE(num_seqs >= 0 && max_q_len >= 0 && H > 0 && KVH > 0 && hd > 0 && total_rows >= 0,
              "he_attention_prefill_bf16: bad sizes");
   HE_REQUIRE(kernel >= 0 && kernel <= 2,
              "he_attention_prefill_bf16: kernel %d (0 = the library's choice; 1: 16 queries a wavefront, "
@@ -375,10 +450,24 @@ extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* k
   if (num_seqs == 0 || max_q_len == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   if (kernel == 0) kernel = (hd > 128 || max_q_len <= 16) ? 1 : 2;
-  if (kernel == 2)
-    return he_attention_prefill_wide(out, q, kpool, vpool, cu_seqlens, seq_slot, seq_start, page_table,
-                                     max_blocks, num_pages, num_seqs, max_q_len, H, KVH, hd, window, scale,
-                                     stream);
+  if (parts < 1) parts = 1;
+  HE_REQUIRE(parts == 1 || kernel == 2,
+             "he_attention_prefill_bf16: keys in %d parts are for kernel 2 (head sizes up to 128, more than 16 queries)", parts);
+  if (kernel == 2) {
+    float* ws_o = (float*)workspace_f32;
+    float* ws_ml = ws_o + (int64_t)total_rows * H * parts * hd;
+    if (parts > 1) {
+      const int64_t need = he_attention_prefill_workspace_floats(total_rows, H, hd, parts);
+      HE_REQUIRE(parts <= 64 && ws_o != nullptr && workspace_floats >= need && (((uintptr_t)ws_o) & 15) == 0,
+                 "he_attention_prefill_bf16: %d parts (at most 64) need %lld floats of workspace (16-byte aligned), %lld given",
+                 parts, (long long)need, (long long)workspace_floats);
+    }
+    int rc = he_attention_prefill_wide(out, q, kpool, vpool, cu_seqlens, seq_slot, seq_start, page_table,
+                                       max_blocks, num_pages, num_seqs, max_q_len, H, KVH, hd, window, scale,
+                                       parts, ws_o, ws_ml, stream);
+    if (rc || parts == 1) return rc;
+    return he_attention_merge_rows(out, ws_o, ws_ml, total_rows, H, hd, parts, stream);
+  }
   dim3 grid((max_q_len + 63) / 64, H, num_seqs);
   ATTN_SWITCH(hd / 16, (attention_prefill_kernel<NT><<<grid, 256, 0, s>>>(
                            (uint16_t*)out, (const uint16_t*)q, (const uint16_t*)kpool,

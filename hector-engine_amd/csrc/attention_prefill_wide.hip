@@ -38,6 +38,12 @@
 // fits on the chip at once puts its lightest beside its heaviest); an XCD sees neighbouring
 // heads. Head sizes up to 128.
 //
+// parts > 1: grid.x counts (block of queries, part). The pages of a block are dealt out evenly to its
+// parts; a part runs the same loops over its own pages and leaves unnormalised sums, reference
+// point and sum of weights per query and head (ws_o, ws_ml) for attention_merge_rows_kernel
+// (attention_mfma.hip). For steps of few queries against many keys, which would otherwise keep
+// a fraction of the chip busy.
+//
 // Measured at 28 heads of 128, 4 kv heads (causal flops): 0.61 PFLOP/s at 2048 tokens,
 // 0.94 at 8192, 1.1 at 16384, 0.85 for eight prompts of 2048. In the long runs the shader
 // clock sits near 1.4 GHz (s_memtime against the 100 MHz counter), so 1.1 PFLOP/s is four
@@ -336,7 +342,8 @@ attention_prefill_wide_kernel(
     const uint16_t* __restrict__ kpool, const uint16_t* __restrict__ vpool,
     const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_slot,
     const int32_t* __restrict__ seq_start, const int32_t* __restrict__ page_table, int max_blocks,
-    int num_pages, int H, int KVH, int window, float scale) {
+    int num_pages, int H, int KVH, int window, float scale, int parts, float* __restrict__ ws_o,
+    float* __restrict__ ws_ml) {
   constexpr int HD = Pw<NT>::HD, KS = Pw<NT>::KS, DT = Pw<NT>::DT;
   constexpr int KP = Pw<NT>::K_PIECES, VP = Pw<NT>::V_PIECES;
   __shared__ uint4 k_lds[2 * KP];
@@ -366,7 +373,8 @@ attention_prefill_wide_kernel(
   }
   const int rho = rank % rows;
   const int row = (rho % gcd) * (rows / gcd) + rho / gcd;
-  const int bx = gridDim.x - 1 - rank / rows;
+  const int gx = gridDim.x - 1 - rank / rows;   // gridDim.x = query blocks x parts
+  const int bx = gx / parts, part = gx - bx * parts;
   const int seq = row % gridDim.z, h = row / gridDim.z;
   const int slot = seq_slot[seq];
   if (slot < 0) return;
@@ -385,12 +393,27 @@ attention_prefill_wide_kernel(
   // the workgroup's pages: from the first key its first query sees to its last query
   const int blk_last = start + min(q0 + PW_QUERIES, q_len) - 1;
   const int blk_first = window > 0 ? max(0, start + q0 + 1 - window) : 0;
-  const int pbA = blk_first >> HE_PAGE_SHIFT, pbB = blk_last >> HE_PAGE_SHIFT;
+  int pbA = blk_first >> HE_PAGE_SHIFT, pbB = blk_last >> HE_PAGE_SHIFT;
+  if (parts > 1) {
+    // this workgroup's share of the block's pages; one without pages leaves empty parts
+    const int per = (pbB - pbA + parts) / parts;
+    pbA += part * per;
+    pbB = min(pbB, pbA + per - 1);
+  }
 
   // the wavefront's tile; a query beyond the sequence doubles the last one and is not stored
   const int qt = q0 + 32 * wave;
   const bool tile = qt < q_len;
   const int qi = min(qt + col, q_len - 1);
+  if (pbA > pbB) {
+    // a part without pages (more parts than the block has pages): empty parts for its queries
+    if (tile && qt + col < q_len) {
+      const int64_t idx = ((int64_t)(row0 + qi) * H + h) * parts + part;
+      if (g == 0) *reinterpret_cast<float2*>(ws_ml + 2 * idx) = make_float2(-INFINITY, 0.f);
+      for (int d = 4 * g; d < HD; d += 8) *reinterpret_cast<float4*>(ws_o + idx * HD + d) = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    return;
+  }
   WideTile<NT> t;
   t.hi = start + qi;
   t.lo = window > 0 ? max(0, t.hi + 1 - window) : 0;
@@ -409,10 +432,11 @@ attention_prefill_wide_kernel(
   const int first_pos = start + qt, last_pos = start + min(qt + 31, q_len - 1);
   const int lo_min = window > 0 ? max(0, first_pos + 1 - window) : 0;
   const int lo_max = window > 0 ? max(0, last_pos + 1 - window) : 0;
-  const int hsA = tile ? lo_min >> 5 : 1, hsB = tile ? last_pos >> 5 : 0;
+  // (a part has the steps of its own pages only)
+  const int hsA = tile ? max(lo_min >> 5, 2 * pbA) : 1, hsB = tile ? min(last_pos >> 5, 2 * pbB + 1) : 0;
   const int hsI0 = (lo_max + 31) >> 5, hsI1 = (first_pos + 1) >> 5;
   // epochs of the loop without masks: steps 2j-2 .. 2j+1 are the tile's, 2j-1 and 2j unmasked
-  int jF0 = max(max((hsA + 3) >> 1, (hsI0 + 2) >> 1), pbA + 1), jF1 = (hsI1 - 1) >> 1;
+  int jF0 = max(max((hsA + 3) >> 1, (hsI0 + 2) >> 1), pbA + 1), jF1 = min((hsI1 - 1) >> 1, pbB);
   if (!tile || hsI1 < 1 || jF0 > jF1) { jF0 = pbB + 2; jF1 = pbB + 1; }
 
   const int kl = ((lane >> 4) & 1) * KS * 64 + 16 * g + (lane & 15);
@@ -475,6 +499,22 @@ attention_prefill_wide_kernel(
 
   const float l = xor32_sum(t.l);
   if (!tile || qt + col >= q_len) return;
+  if (parts > 1) {
+    // one of several parts of the keys: the sums as they stand, with their reference point, for
+    // attention_merge_kernel (O fp32 [hd], then (m, l) with m in the base-2 domain)
+    const int64_t idx = ((int64_t)(row0 + qi) * H + h) * parts + part;
+    if (g == 0) *reinterpret_cast<float2*>(ws_ml + 2 * idx) = make_float2(t.m, l);
+    float* orow = ws_o + idx * HD + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        if (32 * dt + 8 * a >= HD) continue;
+        *reinterpret_cast<float4*>(orow + 32 * dt + 8 * a) =
+            make_float4(t.o[dt][4 * a], t.o[dt][4 * a + 1], t.o[dt][4 * a + 2], t.o[dt][4 * a + 3]);
+      }
+    return;
+  }
   const float inv = l > 0.f ? 1.f / l : 0.f;
   uint16_t* orow = out + ((int64_t)(row0 + qi) * H + h) * HD + 4 * g;
 #pragma unroll
@@ -492,17 +532,23 @@ attention_prefill_wide_kernel(
 int he_attention_prefill_wide(void* out, const void* q, const void* kpool, const void* vpool,
                               const void* cu_seqlens, const void* seq_slot, const void* seq_start,
                               const void* page_table, int max_blocks, int num_pages, int num_seqs,
-                              int max_q_len, int H, int KVH, int hd, int window, float scale, void* stream) {
+                              int max_q_len, int H, int KVH, int hd, int window, float scale,
+                              int parts, float* ws_o, float* ws_ml, void* stream) {
   HE_REQUIRE(hd % 16 == 0 && hd >= 16 && hd <= 128,
              "he_attention_prefill_wide: head_dim %d must be a multiple of 16 up to 128", hd);
-  dim3 grid((max_q_len + PW_QUERIES - 1) / PW_QUERIES, H, num_seqs);
+  HE_REQUIRE(parts >= 1 && parts <= 64 && (parts == 1 || (ws_o != nullptr && ws_ml != nullptr)),
+             "he_attention_prefill_wide: %d parts (1 to 64, with room for them)", parts);
+  const int64_t gx = (int64_t)((max_q_len + PW_QUERIES - 1) / PW_QUERIES) * parts;
+  HE_REQUIRE(gx * H * num_seqs < (1ll << 31), "he_attention_prefill_wide: grid too large");
+  dim3 grid((unsigned)gx, H, num_seqs);
   hipStream_t s = (hipStream_t)stream;
 #define PREFILL_WIDE(NTV)                                                                       \
   case NTV:                                                                                     \
     attention_prefill_wide_kernel<NTV><<<grid, 64 * PW_WAVES, 0, s>>>(                          \
         (uint16_t*)out, (const uint16_t*)q, (const uint16_t*)kpool, (const uint16_t*)vpool,     \
         (const int32_t*)cu_seqlens, (const int32_t*)seq_slot, (const int32_t*)seq_start,        \
-        (const int32_t*)page_table, max_blocks, num_pages, H, KVH, window, scale);              \
+        (const int32_t*)page_table, max_blocks, num_pages, H, KVH, window, scale, parts, ws_o,  \
+        ws_ml);                                                                                 \
     break;
   switch (hd / 16) {
     PREFILL_WIDE(1) PREFILL_WIDE(2) PREFILL_WIDE(3) PREFILL_WIDE(4)

@@ -146,15 +146,19 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 // ---- error channel -------------------------------------------------------
 void he_set_error(const char* fmt, ...);
 int he_check_launch(const char* what);
-// attention_mfma.hip: joins attention parts that were all stored (used by the fused one-token kernel)
+// attention_mfma.hip: joins attention parts that were all stored (the fused one-token kernel's, the
+// prompt kernel's); row_seq may be null: every row has a sequence
 int he_attention_merge_parts(void* out, const float* ws_o, const float* ws_ml, const void* row_seq,
                              int rows, int H, int hd, int parts, int out_pieces, void* stream);
 
-// attention_prefill_wide.hip: prompt attention, 32 queries a wavefront (head sizes up to 128; arguments checked by the caller)
+// attention_prefill_wide.hip: prompt attention, 32 queries a wavefront (head sizes up to 128; arguments
+// checked by the caller). parts > 1: the keys of a block of queries are cut into that many parts, each
+// a workgroup of its own that leaves its sums in ws_o / ws_ml for he_attention_merge_parts.
 int he_attention_prefill_wide(void* out, const void* q, const void* kpool, const void* vpool,
                               const void* cu_seqlens, const void* seq_slot, const void* seq_start,
                               const void* page_table, int max_blocks, int num_pages, int num_seqs,
-                              int max_q_len, int H, int KVH, int hd, int window, float scale, void* stream);
+                              int max_q_len, int H, int KVH, int hd, int window, float scale,
+                              int parts, float* ws_o, float* ws_ml, void* stream);
 
 #define HE_REQUIRE(cond, ...)      \
   do {                             \

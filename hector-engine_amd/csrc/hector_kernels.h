@@ -135,12 +135,18 @@ int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_t qkv_strid
 // bf16, prompt steps: tiles of queries of one sequence against its cache rows. kernel: 0 leaves
 // the choice to the library; 1: 16 queries a wavefront, operands straight from global memory
 // (any head size up to 256); 2: 32 queries a wavefront, pages shared through LDS, the softmax
-// beside the matrix products (head sizes up to 128).
+// beside the matrix products (head sizes up to 128). parts > 1 (kernel 2 only): the keys of a
+// block of queries are cut into that many parts that run side by side and are joined by a
+// second launch; the workspace holds he_attention_prefill_workspace_floats() floats.
+// he_attention_prefill_parts() is the number the library would take for a step.
+int he_attention_prefill_parts(int num_seqs, int max_q_len, int H, int hd, int most_keys);
+int64_t he_attention_prefill_workspace_floats(int total_rows, int H, int hd, int parts);
 int he_attention_prefill_bf16(void* out, const void* q, const void* kpool, const void* vpool,
                               const void* cu_seqlens, const void* seq_slot, const void* seq_start,
                               const void* page_table, int max_blocks, int num_pages, int num_seqs,
                               int max_q_len, int H, int KVH, int hd, int window, float scale,
-                              int kernel, void* stream);
+                              int kernel, int total_rows, int parts, void* workspace_f32,
+                              int64_t workspace_floats, void* stream);
 
 // ---- sampling ------------------------------------------------------------
 int64_t he_argmax_workspace_bytes(int rows, int V);

@@ -64,7 +64,10 @@ _SIGNATURES = {
                                        c_ptr, c_ptr, c_int, c_int, c_ptr, c_int, c_int, c_int, c_int,
                                        c_int, c_int, c_f32, c_int, c_int, c_int, c_ptr, c_i64, c_ptr],
     "he_attention_prefill_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int,
-                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_int, c_ptr],
+                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_int,
+                                  c_int, c_int, c_ptr, c_i64, c_ptr],
+    "he_attention_prefill_parts": [c_int, c_int, c_int, c_int, c_int],
+    "he_attention_prefill_workspace_floats": [c_int, c_int, c_int, c_int],
     "he_argmax_workspace_bytes": [c_int, c_int],
     "he_argmax_rows": [c_ptr, c_ptr, c_int, c_int, c_i64, c_ptr, c_i64, c_ptr],
     "he_argmax_rows_static_setup": [],
@@ -76,6 +79,7 @@ _SIGNATURES = {
 _RESTYPES = {
     "he_attention_decode_workspace_floats": c_i64,
     "he_attention_decode_fused_workspace_floats": c_i64,
+    "he_attention_prefill_workspace_floats": c_i64,
     "he_argmax_workspace_bytes": c_i64,
 }
 

@@ -568,24 +568,40 @@ def attention_decode_fused(out, qkv, bias, kpool, vpool, positions, row_seq, seq
         workspace.numel() if workspace is not None else 0, _stream()))
 
 
+def attention_prefill_parts(num_seqs: int, max_q_len: int, H: int, hd: int, most_keys: int) -> int:
+    """Parts the library would cut the keys of this prompt step into (1: none): more than one
+    for a step of few queries against many keys, which would otherwise leave most of the chip idle."""
+    return int(_lib.load().he_attention_prefill_parts(num_seqs, max_q_len, H, hd, most_keys))
+
+
+def attention_prefill_workspace_floats(total_rows: int, H: int, hd: int, parts: int) -> int:
+    return int(_lib.load().he_attention_prefill_workspace_floats(total_rows, H, hd, parts))
+
+
 @_op("attention_prefill")
 def attention_prefill(out, q, kpool, vpool, cu_seqlens, seq_slot, seq_start, page_table,
                       num_seqs: int, max_q_len: int, total_rows: int, H: int, KVH: int, hd: int,
-                      window: int, scale: float, kernel: int = 0) -> None:
+                      window: int, scale: float, kernel: int = 0, parts: int = 1, workspace=None) -> None:
     """kernel: 0 leaves the choice to the library (by head size and prompt length); 1 or 2
     name it: 16 queries a wavefront with operands from global memory, or 32 queries a
-    wavefront with the pages shared through LDS (head sizes up to 128)."""
+    wavefront with the pages shared through LDS (head sizes up to 128). parts > 1 (kernel 2):
+    the keys in that many parts side by side, joined by a second launch; the workspace holds
+    attention_prefill_workspace_floats() floats."""
     _check_attention(out, q, kpool, vpool, page_table, total_rows, H, KVH, hd)
     _need(q, "q", torch.bfloat16)
     for name, t in (("cu_seqlens", cu_seqlens), ("seq_slot", seq_slot), ("seq_start", seq_start)):
         _need(t, name, torch.int32)
     if cu_seqlens.numel() < num_seqs + 1 or seq_slot.numel() < num_seqs or seq_start.numel() < num_seqs:
         raise ValueError("attention_prefill: metadata shorter than the sequence count")
+    if workspace is not None:
+        _need(workspace, "workspace", torch.float32)
     L = _lib.load()
     _lib.check(L.he_attention_prefill_bf16(
         out.data_ptr(), q.data_ptr(), kpool.data_ptr(), vpool.data_ptr(), cu_seqlens.data_ptr(),
         seq_slot.data_ptr(), seq_start.data_ptr(), page_table.data_ptr(), page_table.shape[1],
-        kpool.shape[0], num_seqs, max_q_len, H, KVH, hd, window, float(scale), int(kernel), _stream()))
+        kpool.shape[0], num_seqs, max_q_len, H, KVH, hd, window, float(scale), int(kernel),
+        total_rows, int(parts), _ptr(workspace), workspace.numel() if workspace is not None else 0,
+        _stream()))
 
 
 @_op("argmax_rows")

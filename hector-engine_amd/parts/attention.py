@@ -135,7 +135,14 @@ class Attention(Mixer):
                                  ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,
                                  self.scale, ctx.max_keys, ws)
         else:
+            # few queries against many keys (a continuation of a long sequence): the keys in parts
+            most = max(s + n for s, n in zip(ctx.host["starts"], ctx.host["q_lens"])) if ctx.host else ctx.max_keys
+            if self.window > 0:
+                most = min(most, self.window + ctx.max_q_len)
+            parts = ops.attention_prefill_parts(ctx.num_seqs, ctx.max_q_len, H, hd, most)
+            ws = ctx.alloc((ops.attention_prefill_workspace_floats(rows, H, hd, parts),), torch.float32) \
+                if parts > 1 else None
             ops.attention_prefill(out, q, cache.kpool, cache.vpool, ctx.cu_seqlens, ctx.seq_slot,
                                   ctx.seq_start, cache.page_table, ctx.num_seqs, ctx.max_q_len,
-                                  rows, H, KVH, hd, self.window, self.scale)
+                                  rows, H, KVH, hd, self.window, self.scale, parts=parts, workspace=ws)
         return self.o_proj(out, rows, ctx, sink=ctx.take_sink())

@@ -476,7 +476,7 @@ def test_qkv_rope_cache(ops, dtype, H, KVH, hd, rot):
     assert (kp != 0).sum().item() <= rows * KVH * hd
 
 
-def attention_case(ops, kind, dtype, H, KVH, hd, window, lengths, q_lens, seed, pad=0, tiles=0, plant=None):
+def attention_case(ops, kind, dtype, H, KVH, hd, window, lengths, q_lens, seed, pad=0, tiles=0, plant=None, parts=1):
     """Runs one attention kernel over a crafted cache; returns (got, want) lists per sequence.
     plant(ks, vs) may change keys and values before they go into the cache."""
     B = len(lengths)
@@ -508,8 +508,9 @@ def attention_case(ops, kind, dtype, H, KVH, hd, window, lengths, q_lens, seed, 
         ops.attention_decode(out, dev(q), *args, dev(positions), dev(row_seq), dev(seq_slot),
                              dev(table), rows + pad, H, KVH, hd, window, scale, max_keys, ws)
     else:
+        ws = torch.empty(ops.attention_prefill_workspace_floats(rows, H, hd, parts), device="cuda") if parts > 1 else None
         ops.attention_prefill(out, dev(q), *args, dev(cu), dev(seq_slot), dev(seq_start), dev(table),
-                              B, max(q_lens), rows, H, KVH, hd, window, scale, kernel=tiles)
+                              B, max(q_lens), rows, H, KVH, hd, window, scale, kernel=tiles, parts=parts, workspace=ws)
     got, want = [], []
     r = 0
     for i, (n, m) in enumerate(zip(lengths, q_lens)):
@@ -586,6 +587,55 @@ def test_attention_prefill_shared_pages_edges(ops, H, KVH, hd, window):
     got, want = attention_case(ops, "prefill", torch.bfloat16, H, KVH, hd, window, lengths, q_lens, 47, tiles=2)
     for g, w in zip(got, want):
         assert torch.allclose(g, w, rtol=2 ** -6, atol=2 ** -6)
+
+
+@pytest.mark.parametrize("H,KVH,hd,window", [(7, 1, 128, 0), (4, 2, 64, 0), (3, 1, 80, 70), (4, 1, 128, 300), (2, 1, 16, 0)])
+@pytest.mark.parametrize("parts", [2, 3, 5, 16])
+def test_attention_prefill_keys_in_parts(ops, H, KVH, hd, window, parts):
+    """The keys of a block of queries cut into parts that run side by side and are joined: short
+    continuations of long sequences (what the parts are for), whole prompts whose first blocks have
+    fewer pages than there are parts (parts without pages), a window (parts before its start hold
+    nothing), one new token, a block of one query, starts that are no multiple of 32."""
+    lengths = [1500 + 40, 64 * 9 + 31 + 97, 700, 701, 129, 64 * 4 + 33]
+    q_lens = [40, 97, 700, 1, 129, 33]
+    got, want = attention_case(ops, "prefill", torch.bfloat16, H, KVH, hd, window, lengths, q_lens, 51, tiles=2,
+                               parts=parts)
+    for g, w in zip(got, want):
+        assert torch.allclose(g, w, rtol=2 ** -6, atol=2 ** -6)
+
+
+def test_attention_prefill_keys_in_parts_reference_points(ops):
+    """Parts whose reference points lie far apart: one key in the first part and one in the last
+    are made large, so the join weighs parts by 2^(hundreds) against each other."""
+    def plant(ks, vs):
+        ks[0][100] *= 60
+        ks[0][1900] *= 200
+    got, want = attention_case(ops, "prefill", torch.bfloat16, 7, 1, 128, 0, [2000], [90], 52, tiles=2,
+                               plant=plant, parts=4)
+    assert torch.allclose(got[0], want[0], rtol=2 ** -6, atol=2 ** -6)
+
+
+def test_attention_prefill_parts_rule_and_errors(ops):
+    """The library's own choice: none for a whole prompt that fills the chip or for a short context, several
+    for a short continuation of a long sequence; parts are refused for the kernel that cannot run them and
+    without room for them."""
+    from hector_engine_amd.kernels.lib import KernelLibraryError
+    assert ops.attention_prefill_parts(1, 2048, 28, 128, 2048) == 1
+    assert ops.attention_prefill_parts(1, 300, 28, 128, 300) == 1
+    assert ops.attention_prefill_parts(1, 200, 28, 128, 8200) == 8
+    assert ops.attention_prefill_parts(1, 64, 28, 128, 8064) == 7
+    assert ops.attention_prefill_parts(1, 64, 28, 128, 40000) == 16
+    assert ops.attention_prefill_parts(1, 200, 28, 256, 8200) == 1      # head size of the other kernel
+    assert ops.attention_prefill_parts(8, 16, 28, 128, 8200) == 1       # so few queries run the other kernel
+    with pytest.raises(KernelLibraryError, match="kernel 2"):
+        attention_case(ops, "prefill", torch.bfloat16, 4, 1, 64, 0, [300], [100], 53, tiles=1, parts=2)
+    q = torch.zeros(100, 4 * 64, dtype=torch.bfloat16, device="cuda")
+    pool = torch.zeros(8, 1, 64 * 64, dtype=torch.bfloat16, device="cuda")
+    i32 = lambda *v: torch.tensor(v, dtype=torch.int32, device="cuda")
+    with pytest.raises(KernelLibraryError, match="workspace"):
+        ops.attention_prefill(torch.empty_like(q), q, pool, pool, i32(0, 100), i32(0), i32(200),
+                              torch.arange(8, dtype=torch.int32, device="cuda").reshape(1, 8), 1, 100, 100, 4, 1, 64,
+                              0, 0.125, kernel=2, parts=2, workspace=torch.empty(10, device="cuda"))
 
 
 @pytest.mark.parametrize("tiles", [1, 2])

@@ -315,3 +315,35 @@ def test_engine_through_a_window_of_4096_at_10000_tokens(tmp_path):
         eng.release(s)
         assert eng.cache.free_pages == eng.cache.num_pages
         del eng
+
+
+def test_engine_short_continuations_of_long_sequences(tmp_path):
+    """A few new tokens behind thousands of cached ones, the step whose prompt attention cuts the keys
+    into parts: 70 tokens after 3,000 and, in the same step, 130 after 2,100 and a whole prompt of 40;
+    every position against the plain implementation."""
+    import hector_engine_amd as he
+    from hector_engine_amd.engine.engine import StepEntry
+    from hector_engine_amd.kernels import ops
+    from hector_engine_amd.registry import config_from_dict
+    from tests.helpers import close, rand_ids
+    cfg = {"architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 96,
+           "num_attention_heads": 3, "num_key_value_heads": 1, "head_dim": 32, "intermediate_size": 80,
+           "vocab_size": 157, "rope_theta": 10000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 4096,
+           "tie_word_embeddings": False}
+    assert ops.attention_prefill_parts(3, 130, 3, 32, 3070) > 1
+    folder = str(tmp_path)
+    he.write_random_model(config_from_dict(dict(cfg)), 29, folder, "bfloat16")
+    reqs = [rand_ids(157, 3070, 81), rand_ids(157, 2230, 82), rand_ids(157, 40, 83)]
+    fed = [3000, 2100, 0]
+    pcfg, w = P.read_model(folder)
+    want = [P.forward(pcfg, w, r)[f:] for r, f in zip(reqs, fed)]
+    for dtype in ("float32", "bfloat16"):
+        eng = he.Engine(folder, dtype=dtype, max_tokens=8192, max_slots=3)
+        slots = [eng.acquire() for _ in reqs]
+        assert eng.step([StepEntry(s, r[:f], []) for s, r, f in zip(slots[:2], reqs, fed)]) is None
+        out = eng.step([StepEntry(s, r[f:], list(range(len(r) - f))) for s, r, f in zip(slots, reqs, fed)])
+        r0 = 0
+        for r, f, wnt in zip(reqs, fed, want):
+            close(out[r0:r0 + len(r) - f], wnt, dtype)
+            r0 += len(r) - f
+        del eng
