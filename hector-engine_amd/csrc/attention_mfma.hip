@@ -404,17 +404,19 @@ int he_attention_merge_parts(void* out, const float* ws_o, const float* ws_ml, c
 // Parts the keys of a prompt step are cut into (he_attention_prefill_bf16's `parts`): a step with few
 // blocks of 128 queries and many keys (a short continuation of a long sequence) would leave most of the
 // chip idle, each of its workgroups walking all the pages alone. As many parts as bring the launch to two
-// workgroups a compute unit, each of at least 16 pages, at most 16. most_keys: the most keys a sequence
-// of the step has (or a bound). Measured at 28 heads of 128, 4 kv heads (us without parts -> with, join
-// included): 64 tokens after 8000 114 -> 27, 200 after 8000 129 -> 45, 512 after 7680 130 -> 76, 4 x 128
-// after 4000 74 -> 51, 512 after 30000 457 -> 233; 1024 after 7168 144 -> 134 (two parts); a whole prompt
-// of 2048 tokens has workgroups enough and stays whole (47 us; 71 in two parts).
+// workgroups a compute unit, each of at least 4 pages, at most 16; none for a step whose sequences have
+// fewer than four keys a query (a whole prompt has workgroups enough, and the join would cost more than the
+// parts save: 2048 tokens 47 us whole, 71 in two parts). most_keys: the most keys a sequence of the step
+// has (or a bound). Measured at 28 heads of 128, 4 kv heads (us without parts -> with, join included):
+// 8 tokens after 8000 108 -> 18, 64 after 8000 114 -> 27, 200 after 8000 129 -> 45, 512 after 7680 130 -> 76,
+// 4 x 128 after 4000 74 -> 51, 512 after 30000 457 -> 233, 1024 after 7168 144 -> 134.
 extern "C" int he_attention_prefill_parts(int num_seqs, int max_q_len, int H, int hd, int most_keys) {
-  if (num_seqs <= 0 || H <= 0 || hd <= 0 || hd > 128 || hd % 16 || max_q_len <= 16) return 1;
+  if (num_seqs <= 0 || H <= 0 || hd <= 0 || hd > 128 || hd % 16 || max_q_len <= 0) return 1;
+  if ((int64_t)most_keys < 4 * (int64_t)max_q_len) return 1;
   const int64_t blocks = (int64_t)((max_q_len + 127) / 128) * H * num_seqs;
   int64_t parts = 2 * HE_CUS / blocks;
   const int pages = (most_keys + HE_PAGE_TOKENS - 1) / HE_PAGE_TOKENS;
-  if (parts > pages / 16) parts = pages / 16;
+  if (parts > pages / 4) parts = pages / 4;
   if (parts > 16) parts = 16;
   return parts < 1 ? 1 : (int)parts;
 }
@@ -449,10 +451,10 @@ extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* k
              "he_attention_prefill_bf16: buffers must be 16-byte aligned");
   if (num_seqs == 0 || max_q_len == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  if (kernel == 0) kernel = (hd > 128 || max_q_len <= 16) ? 1 : 2;
+  if (kernel == 0) kernel = hd > 128 ? 1 : 2;
   if (parts < 1) parts = 1;
   HE_REQUIRE(parts == 1 || kernel == 2,
-             "he_attention_prefill_bf16: keys in %d parts are for kernel 2 (head sizes up to 128, more than 16 queries)", parts);
+             "he_attention_prefill_bf16: keys in %d parts are for kernel 2 (head sizes up to 128)", parts);
   if (kernel == 2) {
     float* ws_o = (float*)workspace_f32;
     float* ws_ml = ws_o + (int64_t)total_rows * H * parts * hd;

@@ -622,11 +622,13 @@ def test_attention_prefill_parts_rule_and_errors(ops):
     from hector_engine_amd.kernels.lib import KernelLibraryError
     assert ops.attention_prefill_parts(1, 2048, 28, 128, 2048) == 1
     assert ops.attention_prefill_parts(1, 300, 28, 128, 300) == 1
-    assert ops.attention_prefill_parts(1, 200, 28, 128, 8200) == 8
-    assert ops.attention_prefill_parts(1, 64, 28, 128, 8064) == 7
-    assert ops.attention_prefill_parts(1, 64, 28, 128, 40000) == 16
+    assert ops.attention_prefill_parts(1, 1024, 28, 128, 2048) == 1     # fewer than four keys a query
+    assert ops.attention_prefill_parts(1, 200, 28, 128, 8200) == 9
+    assert ops.attention_prefill_parts(1, 64, 28, 128, 8064) == 16
+    assert ops.attention_prefill_parts(1, 8, 28, 128, 508) == 2
+    assert ops.attention_prefill_parts(1, 16, 28, 128, 2016) == 8
+    assert ops.attention_prefill_parts(4, 8, 28, 128, 3008) == 4
     assert ops.attention_prefill_parts(1, 200, 28, 256, 8200) == 1      # head size of the other kernel
-    assert ops.attention_prefill_parts(8, 16, 28, 128, 8200) == 1       # so few queries run the other kernel
     with pytest.raises(KernelLibraryError, match="kernel 2"):
         attention_case(ops, "prefill", torch.bfloat16, 4, 1, 64, 0, [300], [100], 53, tiles=1, parts=2)
     q = torch.zeros(100, 4 * 64, dtype=torch.bfloat16, device="cuda")
