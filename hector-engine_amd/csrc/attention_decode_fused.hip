@@ -268,7 +268,12 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
 // 4 wavefronts and as many workgroups per pair as bring the grid to about 256 (one per
 // compute unit; at 32 sequences that is 41 us against 52 us for one workgroup per pair), at
 // most 16 (32 for contexts beyond 16384), while a slice keeps 64 keys at max_keys.
-static void fused_shape(int rows, int H, int KVH, int hd, int max_keys, int* nw, int* Z) {
+// spread: the caller knows that one sequence has several times the keys of the others; the
+// grid above would leave that sequence to a few workgroups (64 sequences, two of them with
+// 30000 keys and the others with 500: 279 us, with 8 workgroups per pair 102; 32 sequences
+// 186 -> 87; 8 sequences, one long, 56 -> 47 with 16): twice as many workgroups per pair,
+// 8 to 16. A short sequence's spare workgroups find no keys and leave empty parts.
+static void fused_shape(int rows, int H, int KVH, int hd, int max_keys, int spread, int* nw, int* Z) {
   const int G = H / KVH;
   const int gt = G < 16 ? G : 16;
   const int groups = rows * KVH * ((G + 15) / 16);
@@ -281,6 +286,12 @@ static void fused_shape(int rows, int H, int KVH, int hd, int max_keys, int* nw,
     const int most = (max_keys + 4 * FUSED_MIN_CHUNK - 1) / (4 * FUSED_MIN_CHUNK);
     if (zz > most) zz = most;
     if (zz < 1) zz = 1;
+  }
+  if (spread) {
+    const int most = (max_keys + 4 * FUSED_MIN_CHUNK - 1) / (4 * FUSED_MIN_CHUNK);
+    int sz = 2 * zz < 8 ? 8 : 2 * zz > 16 ? (zz > 16 ? zz : 16) : 2 * zz;
+    if (sz > most) sz = most;
+    if (sz > zz) zz = sz, w = 4;
   }
   *nw = w;
   *Z = zz;
@@ -295,10 +306,10 @@ extern "C" int he_attention_decode_fused_ok(int H, int KVH, int hd, int rotary_d
 }
 
 extern "C" int64_t he_attention_decode_fused_workspace_floats(int rows, int H, int KVH, int hd,
-                                                              int max_keys) {
+                                                              int max_keys, int spread) {
   if (rows <= 0 || !he_attention_decode_fused_ok(H, KVH, hd, hd) || max_keys <= 0) return 0;
   int nw, Z;
-  fused_shape(rows, H, KVH, hd, max_keys, &nw, &Z);
+  fused_shape(rows, H, KVH, hd, max_keys, spread, &nw, &Z);
   return Z == 1 ? 0 : (int64_t)rows * H * Z * (hd + 2);
 }
 
@@ -309,7 +320,7 @@ extern "C" int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_
                                               const void* page_table, int max_blocks,
                                               int num_pages, const void* inv_freq, int rotary_dim,
                                               int rows, int H, int KVH, int hd, int window,
-                                              float scale, int max_keys, int write_kv,
+                                              float scale, int max_keys, int spread, int write_kv,
                                               int out_pieces, void* workspace_f32,
                                               int64_t workspace_floats, void* stream) {
   HE_REQUIRE(rows >= 0 && H > 0 && KVH > 0 && hd > 0 && max_keys > 0,
@@ -329,7 +340,7 @@ extern "C" int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_
   const int head_tiles = (G + 15) / 16;
   const int gt = G < 16 ? G : 16;
   int nw, Z;
-  fused_shape(rows, H, KVH, hd, max_keys, &nw, &Z);
+  fused_shape(rows, H, KVH, hd, max_keys, spread, &nw, &Z);
   const int64_t need = Z == 1 ? 0 : (int64_t)rows * H * Z * (hd + 2);
   HE_REQUIRE(Z == 1 || (workspace_f32 != nullptr && workspace_floats >= need &&
                         (((uintptr_t)workspace_f32) & 15) == 0),

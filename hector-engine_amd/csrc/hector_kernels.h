@@ -121,16 +121,19 @@ int64_t he_attention_decode_workspace_floats(int rows, int H, int KVH, int hd, i
 // merge (a second launch joins the parts where few sequences are cut across workgroups).
 // qkv: the un-biased projection rows [rows, (H + 2 KVH) hd]. he_attention_decode_fused_ok: 1
 // when the sizes are taken (head_dim 64 or 128, rotated whole). out_pieces: out lies piece-major
-// (as he_gemm_blocksplit_fused_bf16 reads it with x_pieces).
+// (as he_gemm_blocksplit_fused_bf16 reads it with x_pieces). spread: one sequence of the step has
+// several times the keys of the others; every sequence's keys are then cut across more workgroups.
 int he_attention_decode_fused_ok(int H, int KVH, int hd, int rotary_dim);
-int64_t he_attention_decode_fused_workspace_floats(int rows, int H, int KVH, int hd, int max_keys);
+int64_t he_attention_decode_fused_workspace_floats(int rows, int H, int KVH, int hd, int max_keys,
+                                                   int spread);
 int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_t qkv_stride, const void* bias,
                                    int bias_dtype, void* kpool, void* vpool, const void* positions,
                                    const void* row_seq, const void* seq_slot,
                                    const void* page_table, int max_blocks, int num_pages,
                                    const void* inv_freq, int rotary_dim, int rows, int H, int KVH,
-                                   int hd, int window, float scale, int max_keys, int write_kv,
-                                   int out_pieces, void* workspace_f32, int64_t workspace_floats,
+                                   int hd, int window, float scale, int max_keys, int spread,
+                                   int write_kv, int out_pieces, void* workspace_f32,
+                                   int64_t workspace_floats,
                                    void* stream);
 // bf16, prompt steps: tiles of queries of one sequence against its cache rows. kernel: 0 leaves
 // the choice to the library; 1: 16 queries a wavefront, operands straight from global memory

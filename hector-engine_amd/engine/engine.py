@@ -135,7 +135,7 @@ class Engine:
         self.profiler = profiler.OpProfiler() if profile else None
         self.use_graphs = use_graphs and self.model.graph_safe() and not profile
         self._capture_failed = False
-        self._buckets: dict[int, _GraphBucket] = {}
+        self._buckets: dict[tuple[int, bool], _GraphBucket] = {}
         self._pinned = [torch.empty(1 << 16, dtype=torch.int32).pin_memory() for _ in range(4)]
         self._pinned_events: list[torch.cuda.Event | None] = [None] * 4
         self._pinned_next = 0
@@ -289,6 +289,15 @@ class Engine:
                            max_q_len=max_q_len, max_keys=self.cache.max_seq_len,
                            all_single=all_single, env=self.env, scratch=pool)
 
+    def _uneven_keys(self, entries) -> bool:
+        """Whether one sequence of a one-token step has several times the keys of the others (and
+        thousands of them): the attention kernels then cut every sequence's keys across more
+        workgroups, or the long sequence would be left to a few of them. A step with the flag has a
+        graph of its own."""
+        lens = [self.cache.length(e.slot) for e in entries]
+        longest = max(lens)
+        return longest >= 4096 and longest * len(lens) >= 4 * sum(lens)
+
     def _eager_step(self, entries, all_single: bool, device_tokens=None):
         rows = sum(len(e.tokens) for e in entries)
         wants = sum(len(e.want) for e in entries)
@@ -302,6 +311,7 @@ class Engine:
             views["tokens"][:len(entries)].copy_(device_tokens)
         ctx = self._context(views, rows, len(entries), max(len(e.tokens) for e in entries),
                             all_single, self.scratch)
+        ctx.uneven_keys = all_single and self._uneven_keys(entries)
         ctx.host = {"q_lens": [len(e.tokens) for e in entries],
                     "starts": [self.cache.length(e.slot) for e in entries],
                     "slots": [e.slot for e in entries]}
@@ -313,9 +323,10 @@ class Engine:
     def _graph_step(self, entries, device_tokens=None):
         n = len(entries)
         size = 1 << (n - 1).bit_length()
-        bucket = self._buckets.get(size)
+        uneven = self._uneven_keys(entries)
+        bucket = self._buckets.get((size, uneven))
         if bucket is None:
-            bucket = self._buckets[size] = _GraphBucket(size, self.device)
+            bucket = self._buckets[(size, uneven)] = _GraphBucket(size, self.device)
         # every row of the bucket gets logits; padding rows are inert (row_seq -1)
         padded = [StepEntry(e.slot, e.tokens, [0]) for e in entries]
         host, idx, _ = self._pack(padded, bucket.meta, size, size)
@@ -327,6 +338,7 @@ class Engine:
         if bucket.graph is None:
             ctx = self._context(bucket.views, size, size, 1, True, bucket.pool)
             ctx.want_all = True
+            ctx.uneven_keys = uneven
             if bucket.uses == 1:
                 # first use: run eagerly; it also sizes the bucket's scratch pool
                 return self._bucket_eager(bucket, ctx, n)

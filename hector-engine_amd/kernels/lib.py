@@ -59,10 +59,10 @@ _SIGNATURES = {
                                  c_i64, c_ptr],
     "he_attention_decode_workspace_floats": [c_int, c_int, c_int, c_int, c_int],
     "he_attention_decode_fused_ok": [c_int, c_int, c_int, c_int],
-    "he_attention_decode_fused_workspace_floats": [c_int, c_int, c_int, c_int, c_int],
+    "he_attention_decode_fused_workspace_floats": [c_int, c_int, c_int, c_int, c_int, c_int],
     "he_attention_decode_fused_bf16": [c_ptr, c_ptr, c_i64, c_ptr, c_int, c_ptr, c_ptr, c_ptr, c_ptr,
                                        c_ptr, c_ptr, c_int, c_int, c_ptr, c_int, c_int, c_int, c_int,
-                                       c_int, c_int, c_f32, c_int, c_int, c_int, c_ptr, c_i64, c_ptr],
+                                       c_int, c_int, c_f32, c_int, c_int, c_int, c_int, c_ptr, c_i64, c_ptr],
     "he_attention_prefill_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int,
                                   c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_int,
                                   c_int, c_int, c_ptr, c_i64, c_ptr],

@@ -526,17 +526,20 @@ def attention_decode_fused_ok(H: int, KVH: int, hd: int, rotary_dim: int) -> boo
     return int(_lib.load().he_attention_decode_fused_ok(H, KVH, hd, rotary_dim)) > 0
 
 
-def attention_decode_fused_workspace_floats(rows: int, H: int, KVH: int, hd: int, max_keys: int) -> int:
-    return int(_lib.load().he_attention_decode_fused_workspace_floats(rows, H, KVH, hd, max_keys))
+def attention_decode_fused_workspace_floats(rows: int, H: int, KVH: int, hd: int, max_keys: int,
+                                           spread: bool = False) -> int:
+    return int(_lib.load().he_attention_decode_fused_workspace_floats(rows, H, KVH, hd, max_keys, int(spread)))
 
 
 @_op("attention_decode_fused")
 def attention_decode_fused(out, qkv, bias, kpool, vpool, positions, row_seq, seq_slot, page_table,
                            inv_freq, rotary_dim: int, rows: int, H: int, KVH: int, hd: int,
                            window: int, scale: float, max_keys: int, write_kv: bool,
-                           workspace, out_pieces: bool = False) -> None:
+                           workspace, out_pieces: bool = False, spread: bool = False) -> None:
     """One-token steps in one launch: bias, rotation of q and of the new key, cache write,
-    attention over the cache, merge. qkv: bf16 [rows, (H + 2 KVH) hd] without bias; q columns
+    attention over the cache, merge. spread: one sequence has several times the keys of the
+    others (every sequence's keys are then cut across more workgroups; the workspace is asked for
+    with the same flag). qkv: bf16 [rows, (H + 2 KVH) hd] without bias; q columns
     alone where the run reads another run's cache (write_kv False). out_pieces: out is written
     piece-major for exactly `rows` rows (see :func:`to_pieces`)."""
     width = (H + 2 * KVH) * hd if write_kv else H * hd
@@ -564,7 +567,7 @@ def attention_decode_fused(out, qkv, bias, kpool, vpool, positions, row_seq, seq
         dtype_code(bias.dtype) if bias is not None else F32, kpool.data_ptr(), vpool.data_ptr(),
         positions.data_ptr(), row_seq.data_ptr(), seq_slot.data_ptr(), page_table.data_ptr(),
         page_table.shape[1], kpool.shape[0], inv_freq.data_ptr(), rotary_dim, rows, H, KVH, hd,
-        window, float(scale), max_keys, int(write_kv), int(out_pieces), _ptr(workspace),
+        window, float(scale), max_keys, int(spread), int(write_kv), int(out_pieces), _ptr(workspace),
         workspace.numel() if workspace is not None else 0, _stream()))
 
 

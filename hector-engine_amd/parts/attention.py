@@ -103,12 +103,12 @@ class Attention(Mixer):
             qkv = proj(x, rows, ctx, use_bias=False)
             pieces = self.o_proj.reads_pieces(rows, ctx)       # the layout the output product reads best
             out = ctx.alloc(ops.pieces_shape(rows, H * hd) if pieces else (rows, H * hd))
-            floats = ops.attention_decode_fused_workspace_floats(rows, H, KVH, hd, ctx.max_keys)
+            floats = ops.attention_decode_fused_workspace_floats(rows, H, KVH, hd, ctx.max_keys, ctx.uneven_keys)
             ws = ctx.alloc((floats,), torch.float32) if floats else None
             ops.attention_decode_fused(out, qkv, proj.bias, cache.kpool, cache.vpool, ctx.positions,
                                        ctx.row_seq, ctx.seq_slot, cache.page_table, rot[0], rot[1],
                                        rows, H, KVH, hd, self.window, self.scale, ctx.max_keys,
-                                       writes, ws, out_pieces=pieces)
+                                       writes, ws, out_pieces=pieces, spread=ctx.uneven_keys)
             return self.o_proj(PieceRows(out) if pieces else out, rows, ctx, sink=ctx.take_sink())
         # With a rotation (or no encoding) the bias is added inside the fused kernel;
         # any other encoding sees q and k with their bias already added.

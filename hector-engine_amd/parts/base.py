@@ -124,6 +124,7 @@ class StepContext:
         self.env = env
         self.scratch = scratch            # ScratchPool: alloc(shape, dtype)
         self.host = host                  # {"q_lens", "starts", "slots"}: lists per sequence, eager steps only
+        self.uneven_keys = False          # one sequence has several times the keys of the others (a hint for the grids)
         self.want_all = False             # the wanted rows are all rows, in order
         self.next_norm = None             # the norm that reads the stream after the running block (set by the model)
         self.sink = None                  # ResidualSink offered to the running mixer / feed-forward

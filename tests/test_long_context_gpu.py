@@ -107,12 +107,14 @@ def case_id(c):
 
 
 @pytest.mark.parametrize("case", CASES, ids=case_id)
-@pytest.mark.parametrize("kind", ["split", "fused"])
+@pytest.mark.parametrize("kind", ["split", "fused", "fused_spread"])
 def test_one_token_attention_at_long_contexts(ops, kind, case):
     """The split one-token kernel (rotated q given) and the one-launch kernel (bias, rotation,
     cache write, attention) at 1, 8 and 64 rows, up to 20,000 keys, with max_keys below and above
     16,384 (the most slices a sequence is cut into differs), and through a window of 4,096 whose
-    dead pages have been given back."""
+    dead pages have been given back; the one-launch kernel also with the grid for a step whose
+    sequences have very unequal lengths (more workgroups a sequence, most of them without keys
+    for the short ones)."""
     rows, max_keys, long_lengths, window = case
     lengths = decode_batch(rows, long_lengths)
     B = len(lengths)
@@ -127,7 +129,7 @@ def test_one_token_attention_at_long_contexts(ops, kind, case):
     qkv = rnd(B, width, seed=301, scale=1.0).to(torch.bfloat16)
     qkv[:, :H * HD] *= 4                                  # long queries: few keys carry a head's result
     bias = rnd(width, seed=302, scale=0.25).to(torch.bfloat16)
-    fused = kind == "fused"
+    fused, spread = kind.startswith("fused"), kind == "fused_spread"
     x = qkv.double() + (bias.double() if fused else 0)
     pos = torch.tensor([n - 1 for n in lengths])
     q = x[:, :H * HD].reshape(B, H, HD)
@@ -154,11 +156,12 @@ def test_one_token_attention_at_long_contexts(ops, kind, case):
     seq_slot = dev(torch.tensor(cache.slots, dtype=torch.int32))
     out = torch.full((B, H * HD), 7.0, dtype=torch.bfloat16, device="cuda")
     if fused:
-        floats = ops.attention_decode_fused_workspace_floats(B, H, KVH, HD, max_keys)
+        floats = ops.attention_decode_fused_workspace_floats(B, H, KVH, HD, max_keys, spread)
+        assert not spread or floats >= B * H * 8 * (HD + 2)       # at least 8 workgroups a sequence and kv head
         ws = torch.empty(floats, device="cuda") if floats else None
         ops.attention_decode_fused(out, dev(qkv), dev(bias), cache.kpool, cache.vpool, positions, row_seq,
                                    seq_slot, dev(cache.table), dev(P.rope_inv_freq(HD, theta)), HD, B, H, KVH,
-                                   HD, window, scale, max_keys, True, ws)
+                                   HD, window, scale, max_keys, True, ws, spread=spread)
     else:
         ws = torch.empty(max(1, ops.attention_decode_workspace_floats(B, H, KVH, HD, max_keys)), device="cuda")
         ops.attention_decode(out, dev(q.to(torch.bfloat16).reshape(B, H * HD)), cache.kpool, cache.vpool,
@@ -346,4 +349,50 @@ def test_engine_short_continuations_of_long_sequences(tmp_path):
         for r, f, wnt in zip(reqs, fed, want):
             close(out[r0:r0 + len(r) - f], wnt, dtype)
             r0 += len(r) - f
+        del eng
+
+
+def test_engine_one_long_sequence_among_short_ones(tmp_path):
+    """One-token steps of a batch in which one sequence has thousands of keys and the others a few dozen:
+    the step is flagged (the attention grid spreads every sequence over more workgroups), has a graph of
+    its own, and gives the plain implementation's logits; when the long sequence has ended the others go on
+    in the ordinary graph."""
+    import hector_engine_amd as he
+    from hector_engine_amd.engine.engine import StepEntry
+    from hector_engine_amd.registry import config_from_dict
+    from tests.helpers import close, rand_ids
+    cfg = {"architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 128,
+           "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 64, "intermediate_size": 88,
+           "vocab_size": 173, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "max_position_embeddings": 8192,
+           "tie_word_embeddings": True}
+    folder = str(tmp_path)
+    he.write_random_model(config_from_dict(dict(cfg)), 31, folder, "bfloat16")
+    reqs = [rand_ids(173, 4310, 91)] + [rand_ids(173, 30 + 3 * i, 92 + i) for i in range(5)]
+    steps = 6
+    pcfg, w = P.read_model(folder)
+    want = [P.forward(pcfg, w, r) for r in reqs]
+    for dtype in ("float32", "bfloat16"):
+        eng = he.Engine(folder, dtype=dtype, max_tokens=8192, max_slots=8)
+        slots = [eng.acquire() for _ in reqs]
+        fed = [len(r) - steps - (3 if i else 0) for i, r in enumerate(reqs)]
+        eng.step([StepEntry(s, r[:f], []) for s, r, f in zip(slots, reqs, fed)])
+        entries = lambda live: [StepEntry(slots[i], [reqs[i][fed[i]]], [0]) for i in live]   # noqa: E731
+        for t in range(steps):
+            live = list(range(len(reqs)))
+            assert eng._uneven_keys(entries(live))
+            out = eng.step(entries(live))
+            for j, i in enumerate(live):
+                close(out[j:j + 1], want[i][fed[i]:fed[i] + 1], dtype)
+                fed[i] += 1
+        captured = eng.stats["graph_captures"]
+        eng.release(slots[0])
+        for t in range(3):
+            live = list(range(1, len(reqs)))
+            assert not eng._uneven_keys(entries(live))
+            out = eng.step(entries(live))
+            for j, i in enumerate(live):
+                close(out[j:j + 1], want[i][fed[i]:fed[i] + 1], dtype)
+                fed[i] += 1
+        if dtype == "bfloat16":
+            assert captured == 1 and eng.stats["graph_captures"] == 2
         del eng
