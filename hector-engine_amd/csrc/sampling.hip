@@ -322,13 +322,22 @@ __device__ u64 set_total(const Source& src, float m, float inv_temp, Cut cut, Sa
 // Adds every lane's pending (bin, run) to the histogram. Lanes of a wavefront that hold the
 // same bin - all of them in the passes over the upper key bytes - are summed first and one
 // lane adds the sum: a thousand 64-bit LDS atomics on one address take tens of microseconds.
+// Where the lanes' bins differ (the passes over the lower key bytes) that summing, a dozen
+// exchanges across the wavefront a bin, would be the slow part: once a bin is shared by fewer
+// than eight lanes, or three bins have been dealt with, the lanes left add their own.
 __device__ __forceinline__ void flush_runs(u64* hist, int bin, u64 run) {
   const int lane = threadIdx.x & (HE_WAVE - 1);
   unsigned long long pending = __builtin_amdgcn_ballot_w64(bin >= 0);
+  int dealt = 0;
   while (pending) {
     const int leader = __builtin_ctzll(pending);
     const int lb = __shfl(bin, leader, HE_WAVE);
     const bool same = bin == lb;
+    const unsigned long long sharing = __builtin_amdgcn_ballot_w64(same);
+    if (__builtin_popcountll(sharing) < 8 || dealt == 3) {
+      if ((pending >> lane) & 1ull) atomicAdd(&hist[bin], run);
+      return;
+    }
     u64 v = same ? run : 0ull;
 #pragma unroll
     for (int off = HE_WAVE / 2; off > 0; off >>= 1) {
@@ -337,7 +346,8 @@ __device__ __forceinline__ void flush_runs(u64* hist, int bin, u64 run) {
       v += ((u64)hi << 32) | lo;
     }
     if (lane == leader) atomicAdd(&hist[lb], v);
-    pending &= ~__builtin_amdgcn_ballot_w64(same);
+    pending &= ~sharing;
+    ++dealt;
   }
 }
 
@@ -550,10 +560,19 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_rows_kernel(
   // pass 1: row maximum
   float best = -INFINITY;
   if (((stride & 3) == 0) && ((((uintptr_t)logits) & 15) == 0)) {
+    // four loads on their way at a time: one workgroup reads the whole row, and a load takes
+    // about a microsecond
     const int V4 = V & ~3;
-    for (int i = 4 * threadIdx.x; i < V4; i += 4 * SAMP_THREADS) {
-      const float4 v = *reinterpret_cast<const float4*>(x + i);
-      best = fmaxf(fmaxf(best, clean(v.x)), fmaxf(clean(v.y), fmaxf(clean(v.z), clean(v.w))));
+    for (int i0 = 4 * threadIdx.x; i0 < V4; i0 += 16 * SAMP_THREADS) {
+      float4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = i0 + u * 4 * SAMP_THREADS;
+        v[u] = i < V4 ? *reinterpret_cast<const float4*>(x + i) : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        best = fmaxf(fmaxf(best, clean(v[u].x)), fmaxf(clean(v[u].y), fmaxf(clean(v[u].z), clean(v[u].w))));
     }
     for (int i = V4 + threadIdx.x; i < V; i += SAMP_THREADS) best = fmaxf(best, clean(x[i]));
   } else {
@@ -627,24 +646,33 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_rows_kernel(
     filled += __builtin_popcountll(appenders);
   };
   if (V > SAMP_LIST && ((stride & 3) == 0) && ((((uintptr_t)logits) & 15) == 0)) {
-    // 16 bytes a load, the next one on its way while this one is looked at; all lanes of a
-    // wavefront make the same number of turns
+    // 16 bytes a load, four loads a group, the next group on its way while this one is looked
+    // at; all lanes of a wavefront make the same number of turns
     const int V4 = V & ~3;
-    const int turns = (V4 + 4 * SAMP_THREADS - 1) / (4 * SAMP_THREADS);
+    constexpr int STEP = 4 * SAMP_THREADS;
+    const int groups = (V4 + 4 * STEP - 1) / (4 * STEP);
     int i = 4 * threadIdx.x;
-    float4 cur = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (i < V4) cur = *reinterpret_cast<const float4*>(x + i);
-    for (int t = 0; t < turns; ++t) {
-      const int nx = i + 4 * SAMP_THREADS;
-      float4 nxt = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (nx < V4) nxt = *reinterpret_cast<const float4*>(x + nx);
-      const bool in = i < V4;
-      take(cur.x, i, in);
-      take(cur.y, i + 1, in);
-      take(cur.z, i + 2, in);
-      take(cur.w, i + 3, in);
-      cur = nxt;
-      i = nx;
+    float4 cur[4], nxt[4];
+    auto load_group = [&](float4 (&g)[4], int at) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        g[u] = at + u * STEP < V4 ? *reinterpret_cast<const float4*>(x + at + u * STEP) : make_float4(0.f, 0.f, 0.f, 0.f);
+    };
+    load_group(cur, i);
+    for (int gi = 0; gi < groups; ++gi) {
+      load_group(nxt, i + 4 * STEP);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int at = i + u * STEP;
+        const bool in = at < V4;
+        take(cur[u].x, at, in);
+        take(cur[u].y, at + 1, in);
+        take(cur[u].z, at + 2, in);
+        take(cur[u].w, at + 3, in);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) cur[u] = nxt[u];
+      i += 4 * STEP;
     }
     const int j = V4 + threadIdx.x;
     take(j < V ? x[j] : 0.f, j, j < V);   // at most three elements are left
