@@ -171,6 +171,12 @@ int he_argmax_rows_static(void* out_i32, const void* logits_f32, int rows, int V
 int he_apply_penalties(void* logits_f32, int rows, int V, int64_t row_stride, const void* ids,
                        const void* counts, const void* offsets, float rep, float freq, float pres,
                        void* stream);
+// The penalties of he_apply_penalties from a ring of recent tokens on the device: window [rows][W]
+// (token number n at n % W), appended [rows] = tokens ever appended. last_ids (or null) are appended
+// first, one a row. W up to 4096.
+int he_apply_penalties_window(void* logits_f32, int rows, int V, int64_t row_stride, void* window_i32,
+                              void* appended_i32, int W, const void* last_ids_i32, float rep, float freq,
+                              float pres, void* stream);
 int he_sample_rows(void* out_i32, const void* logits_f32, int rows, int V, int64_t row_stride,
                    const void* uniforms_u32, float temperature, int top_k, float top_p,
                    void* stream);

@@ -233,6 +233,65 @@ extern "C" int he_apply_penalties(void* logits_f32, int rows, int V, int64_t row
   return he_check_launch("he_apply_penalties");
 }
 
+// The same penalties from a window of recent tokens that lives on the device, so that a run of
+// queued steps needs no token on the host in between: window [rows][W] is a ring (the token
+// appended as number n lies at n % W), appended[row] counts what was ever appended. One
+// workgroup a row first appends last_ids[row] (the token sampled by the step before; null:
+// nothing), then counts the distinct ids among the last min(appended, W) tokens and changes
+// each one's logit once, with the arithmetic of penalties_kernel.
+#define PEN_WINDOW_MAX 4096
+__global__ __launch_bounds__(256) void penalties_window_kernel(
+    float* __restrict__ logits, int V, int64_t stride, int32_t* __restrict__ window,
+    int32_t* __restrict__ appended, int W, const int32_t* __restrict__ last_ids, float rep,
+    float freq, float pres) {
+  __shared__ int32_t ids[PEN_WINDOW_MAX];
+  float* x = logits + blockIdx.x * stride;
+  int32_t* ring = window + (int64_t)blockIdx.x * W;
+  int total = appended[blockIdx.x];
+  const int fresh = last_ids != nullptr ? last_ids[blockIdx.x] : 0;
+  const int at = total % W;
+  if (last_ids != nullptr) ++total;
+  const int n = total < W ? total : W;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) ids[i] = last_ids != nullptr && i == at ? fresh : ring[i];
+  __syncthreads();          // every thread has read the count before it is written
+  if (threadIdx.x == 0 && last_ids != nullptr) {
+    ring[at] = fresh;
+    appended[blockIdx.x] = total;
+  }
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int id = ids[i];
+    if (id < 0 || id >= V) continue;
+    int count = 0;
+    bool first = true;
+    for (int j = 0; j < n; ++j) {
+      const bool same = ids[j] == id;
+      count += same;
+      first = first && !(same && j < i);
+    }
+    if (!first) continue;
+    float v = x[id];
+    if (rep != 1.0f) v = v > 0.f ? v / rep : v * rep;
+    if (freq != 0.0f) v -= freq * (float)count;
+    if (pres != 0.0f) v -= pres;
+    x[id] = v;
+  }
+}
+
+extern "C" int he_apply_penalties_window(void* logits_f32, int rows, int V, int64_t row_stride,
+                                         void* window_i32, void* appended_i32, int W,
+                                         const void* last_ids_i32, float rep, float freq, float pres,
+                                         void* stream) {
+  HE_REQUIRE(rows >= 0 && V > 0 && row_stride >= V, "he_apply_penalties_window: bad sizes");
+  HE_REQUIRE(W >= 1 && W <= PEN_WINDOW_MAX, "he_apply_penalties_window: a window of %d tokens (1 to %d)", W,
+             PEN_WINDOW_MAX);
+  HE_REQUIRE(window_i32 != nullptr && appended_i32 != nullptr, "he_apply_penalties_window: no window");
+  if (rows == 0) return 0;
+  penalties_window_kernel<<<rows, 256, 0, (hipStream_t)stream>>>(
+      (float*)logits_f32, V, row_stride, (int32_t*)window_i32, (int32_t*)appended_i32, W,
+      (const int32_t*)last_ids_i32, rep, freq, pres);
+  return he_check_launch("he_apply_penalties_window");
+}
+
 // ---------------------------------------------------------------- sampling
 typedef unsigned long long u64;
 

@@ -81,8 +81,9 @@ def generate(engine, prompts: list[list[int]], *, max_new_tokens: int = 100, sam
     uniforms_device, read_later) in place of one made from `sampling`; sample_fn: a plain
     function (logits, requests, steps, contexts) -> ids, which runs step by step.
 
-    run_of_steps: with a sampler and no penalties, up to so many one-token steps are queued at
-    a time, each step's ids going into the next on the device. The tokens are the same as step
+    run_of_steps: with a sampler, up to so many one-token steps are queued at a time, each
+    step's ids going into the next on the device (and into the penalty windows, which then live
+    there for the run). The tokens are the same as step
     by step. When nothing can end a sequence inside a run but its token budget or its cache
     room (no stop ids, no `cancel`), the run never reaches past those and the host reads all
     its ids at the end. Otherwise the host reads the ids of a step while the next one runs,
@@ -95,8 +96,9 @@ def generate(engine, prompts: list[list[int]], *, max_new_tokens: int = 100, sam
         if sampler is None:
             sampler = Sampler(sampling or SamplingConfig.deterministic(), engine.device)
         sample_fn = sampler.sample
-        if sampler.config.has_penalties or run_of_steps <= 1:
-            sampler = None          # penalties need each token on the host before the next
+        if run_of_steps <= 1 or (sampler.config.has_penalties
+                                 and not getattr(sampler, "window_on_device", False)):
+            sampler = None          # step by step: each token on the host before the next
     else:
         sampler = None
     run_of_steps = min(run_of_steps, READS_IN_FLIGHT)
@@ -133,19 +135,23 @@ def steps_in_run(generated: list[int], lengths: list[int], max_new_tokens: int, 
 
 
 def _run_of_steps(engine, sampler, slots: list[int], tokens: list[int], seqs: list[int],
-                  steps: list[int], count: int, stop_ids=frozenset(), cancel=None) -> list[list[int]]:
+                  steps: list[int], count: int, stop_ids=frozenset(), cancel=None,
+                  contexts: list[list[int]] | None = None) -> list[list[int]]:
     """Feeds `tokens` and queues up to `count` one-token steps; returns the sampled ids of the
     steps that ran, [steps][rows]. With stop ids or `cancel`, the ids of step j are read while
     step j + 1 runs, and the run ends with the step that was queued when a stop token (or the
     cancellation) was seen."""
     uniforms = None if sampler.config.is_greedy else sampler.uniforms_device(seqs, steps, count)
+    # the penalty windows (the generated tokens, the ones fed now included) go to the device once
+    window = sampler.window_device(contexts) if sampler.config.has_penalties and contexts is not None else None
     watch = bool(stop_ids) or cancel is not None
     reads, ids, device_ids = [], [], None
     for j in range(count):
         entries = [StepEntry(s, [t], [0]) for s, t in zip(slots, tokens)]
         logits = engine.step(entries, device_tokens=device_ids)
+        more = {} if window is None else {"window": window, "last_ids": device_ids}
         device_ids = sampler.sample_device(logits, seqs, [t + j for t in steps],
-                                           uniforms=None if uniforms is None else uniforms[j])
+                                           uniforms=None if uniforms is None else uniforms[j], **more)
         reads.append(sampler.read_later(device_ids))
         if watch and j >= 1:
             ids.append(reads[j - 1].wait())
@@ -199,7 +205,8 @@ def _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, inc
                 tokens = sample_fn(logits, active, [len(out[i]) for i in active], [out[i] for i in active])
                 continue
             run = _run_of_steps(engine, sampler, [slots[i] for i in active], [tok for _, tok in feed],
-                                active, [len(out[i]) for i in active], count, stop_ids, cancel)
+                                active, [len(out[i]) for i in active], count, stop_ids, cancel,
+                                [out[i] for i in active])
             count = len(run)            # fewer when a stop token was seen on the way
             # all but the last step of the run are decided here, each with the cache length of its
             # moment; a sequence that ends inside the run drops the rest of its ids

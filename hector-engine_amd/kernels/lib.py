@@ -74,6 +74,8 @@ _SIGNATURES = {
     "he_argmax_rows_static": [c_ptr, c_ptr, c_int, c_int, c_i64, c_ptr],
     "he_apply_penalties": [c_ptr, c_int, c_int, c_i64, c_ptr, c_ptr, c_ptr, c_f32, c_f32, c_f32,
                            c_ptr],
+    "he_apply_penalties_window": [c_ptr, c_int, c_int, c_i64, c_ptr, c_ptr, c_int, c_ptr, c_f32, c_f32,
+                                  c_f32, c_ptr],
     "he_sample_rows": [c_ptr, c_ptr, c_int, c_int, c_i64, c_ptr, c_f32, c_int, c_f32, c_ptr],
 }
 _RESTYPES = {

@@ -635,6 +635,31 @@ def apply_penalties(logits, rows: int, ids, counts, offsets, rep: float, freq: f
                                     float(pres), _stream()))
 
 
+PENALTY_WINDOW_MAX = 4096
+
+
+@_op("apply_penalties_window")
+def apply_penalties_window(logits, rows: int, window, appended, last_ids, rep: float, freq: float,
+                           pres: float) -> None:
+    """The penalties of apply_penalties from a ring of recent tokens on the device: window int32
+    [rows, W] (token number n at n % W), appended int32 [rows] (tokens ever appended). last_ids
+    (int32 [rows] or None) are appended first. Changes logits in place."""
+    _need(logits, "logits", torch.float32)
+    _need(window, "window", torch.int32)
+    _need(appended, "appended", torch.int32)
+    V = logits.shape[-1]
+    if window.dim() != 2 or window.shape[0] < rows or appended.numel() < rows or logits.numel() < rows * V:
+        raise ValueError("apply_penalties_window: buffers smaller than the row count")
+    if last_ids is not None:
+        _need(last_ids, "last_ids", torch.int32)
+        if last_ids.numel() < rows:
+            raise ValueError("apply_penalties_window: fewer ids than rows")
+    L = _lib.load()
+    _lib.check(L.he_apply_penalties_window(logits.data_ptr(), rows, V, V, window.data_ptr(),
+                                           appended.data_ptr(), window.shape[1], _ptr(last_ids),
+                                           float(rep), float(freq), float(pres), _stream()))
+
+
 @_op("sample_rows")
 def sample_rows(out_i32, logits, rows: int, uniforms_u32, temperature: float, top_k: int,
                 top_p: float) -> None:

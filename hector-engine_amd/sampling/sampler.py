@@ -134,14 +134,44 @@ class Sampler:
                       for j in range(count)], dtype=np.uint32)
         return torch.from_numpy(u.view(np.int32)).to(self.device)
 
+    @property
+    def window_on_device(self) -> bool:
+        """Whether the penalties of these options can run from a window kept on the device."""
+        return self.config.has_penalties and 1 <= self.config.penalty_window <= ops.PENALTY_WINDOW_MAX
+
+    def window_device(self, contexts: list[list[int]]):
+        """The penalty windows of these rows on the device, for a run of steps whose tokens stay
+        there: (ring int32 [rows, W], appended int32 [rows]), or None when the options have no
+        penalties (or a window the kernel does not take). One upload; sample_device then appends
+        each step's ids itself."""
+        cfg = self.config
+        W = cfg.penalty_window
+        if not self.window_on_device:
+            return None
+        rows = len(contexts)
+        host = np.zeros((rows, W + 1), dtype=np.int32)
+        for r, ctx in enumerate(contexts):
+            last = ctx[max(0, len(ctx) - W):]
+            host[r, :len(last)] = last          # oldest first: the next token overwrites the oldest
+            host[r, W] = len(last)
+        dev = torch.from_numpy(host).to(self.device)
+        return dev[:, :W].contiguous(), dev[:, W].contiguous()
+
     def sample_device(self, logits: torch.Tensor, sequences: list[int], steps: list[int],
                       contexts: list[list[int]] | None = None,
-                      uniforms: torch.Tensor | None = None) -> torch.Tensor:
+                      uniforms: torch.Tensor | None = None, window=None,
+                      last_ids: torch.Tensor | None = None) -> torch.Tensor:
         """The same, the ids left on the device (int32 [rows]). With `uniforms` (a row of
-        uniforms_device) and no penalties nothing is copied or waited for."""
+        uniforms_device) and no penalties nothing is copied or waited for. window: what
+        window_device gave, in place of `contexts`; last_ids: the ids the step before sampled,
+        which the window has not seen yet (they are appended first). The penalties then change
+        `logits` itself."""
         cfg = self.config
         rows, V = logits.shape
-        if cfg.has_penalties and contexts is not None and any(contexts):
+        if window is not None:
+            ops.apply_penalties_window(logits, rows, window[0], window[1], last_ids, cfg.repetition_penalty,
+                                       cfg.frequency_penalty, cfg.presence_penalty)
+        elif cfg.has_penalties and contexts is not None and any(contexts):
             ids, counts, offsets = [], [], [0]
             for ctx in contexts:
                 i, c = window_counts(ctx, cfg.penalty_window, V)

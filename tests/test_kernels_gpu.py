@@ -954,6 +954,53 @@ def test_penalties(ops):
         assert torch.allclose(d.cpu()[r], want, rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("W", [1, 5, 16, 300])
+def test_penalties_from_a_window_on_the_device(ops, W):
+    """The window as a ring on the device, fed one token a row and step: after every step the logits
+    equal the plain penalties over the last W tokens (ids repeat, some lie outside the vocabulary, the
+    ring wraps several times), and equal the kernel that takes the host's counts bit for bit."""
+    V, rows, steps = 97, 3, 40
+    g = torch.Generator().manual_seed(63)
+    start = [[5, 5, 96], [], list(range(10, 10 + 2 * W))]
+    ring = torch.zeros(rows, W, dtype=torch.int32)
+    appended = torch.zeros(rows, dtype=torch.int32)
+    for r, ctx in enumerate(start):
+        last = ctx[max(0, len(ctx) - W):]
+        ring[r, :len(last)] = torch.tensor(last, dtype=torch.int32)
+        appended[r] = len(last)
+    ring, appended = dev(ring), dev(appended)
+    ctx = [list(c) for c in start]
+    fresh = None
+    for step in range(steps):
+        x = rnd(rows, V, seed=100 + step)
+        d = dev(x.clone())
+        ops.apply_penalties_window(d, rows, ring, appended, fresh, 1.2, 0.15, 0.05)
+        ids, counts, offsets = [], [], [0]
+        for r in range(rows):
+            want = P.apply_penalties(x[r], ctx[r], W, 1.2, 0.15, 0.05)
+            assert torch.allclose(d.cpu()[r], want, rtol=1e-6, atol=1e-6), (step, r)
+            seen = {}
+            for tok in ctx[r][max(0, len(ctx[r]) - W):]:
+                if 0 <= tok < V:
+                    seen[tok] = seen.get(tok, 0) + 1
+            ids.append(list(seen))
+            counts.append(list(seen.values()))
+            offsets.append(offsets[-1] + len(seen))
+        flat = lambda v: dev(torch.tensor([a for part in v for a in part], dtype=torch.int32))   # noqa: E731
+        d2 = dev(x.clone())
+        if offsets[-1]:
+            ops.apply_penalties(d2, rows, flat(ids), flat(counts), dev(torch.tensor(offsets, dtype=torch.int32)),
+                                1.2, 0.15, 0.05)
+        assert torch.equal(d2, d)
+        new = torch.randint(-2, V + 3, (rows,), generator=g).tolist()    # some ids outside the vocabulary
+        if step % 3 == 0:
+            new[0] = 5                                                   # repeats
+        fresh = dev(torch.tensor(new, dtype=torch.int32))
+        for r in range(rows):
+            ctx[r].append(new[r])
+    assert appended.cpu().tolist() == [min(len(s), W) + steps - 1 for s in start]
+
+
 @pytest.mark.parametrize("V", [301, 5000, 152064])
 @pytest.mark.parametrize("temperature,top_k,top_p", [(0.8, 0, 1.0), (1.0, 50, 0.9), (0.7, 40, 1.0),
                                                      (1.3, 0, 0.5), (0.05, 0, 1.0), (1.0, 1, 1.0)])
