@@ -238,6 +238,28 @@ def test_a_weight_stored_in_32_bit_stays_so_under_bfloat16(fw):
     assert torch.allclose(out.cpu().double(), want, rtol=2 ** -7, atol=2 ** -7)
 
 
+@pytest.mark.parametrize("rows", [65, 200, 512, 513])
+@pytest.mark.parametrize("N,K,bias", [(72, 8192, True), (300, 9024, False), (40, 8200, True)])
+def test_a_long_k_product_in_slices_through_the_library(fw, rows, N, K, bias):
+    """More than 64 rows against a weight with a long K and few output columns (a down projection):
+    up to 512 rows the library runs it as a batched product over K slices whose fp32 results are added
+    in slice order; above, or where K does not divide, as one product. Either way the double-precision
+    result, within bfloat16's rounding of the output."""
+    from hector_engine_amd.parts.linear import Linear
+    env = env_for(fw, torch.bfloat16)
+    w = rnd(N, K, seed=11, scale=0.05).to(torch.bfloat16)
+    b = rnd(N, seed=12).to(torch.bfloat16) if bias else None
+    lin = Linear(w.cuda(), b.cuda() if bias else None)
+    slices = lin._library_slices(rows)
+    assert slices == (1 if rows > 512 else 8 if K % 64 == 0 else 1 if K % 16 else 2 if K % 32 else 4)
+    ctx = make_ctx(fw, env, [rows], [0], [0])
+    x = rnd(rows, K, seed=13).to(torch.bfloat16)
+    out = lin(x.cuda(), rows, ctx)
+    want = x.double() @ w.double().T + (b.double() if bias else 0)
+    assert out.dtype == torch.bfloat16
+    assert torch.allclose(out.cpu().double(), want, rtol=2 ** -7, atol=2 ** -6 * want.abs().max().item())
+
+
 # ---------------------------------------------------------------------------
 # toys: registered here, in the test, through the public registries only
 # ---------------------------------------------------------------------------
