@@ -81,6 +81,9 @@ def main() -> int:
     ap.add_argument("--prompt", type=int, default=0,
                     help="another prompt length of the decode batches (the prefill figure stays at 2048 tokens)")
     ap.add_argument("--no-points", action="store_true", help="skip the points at batch 1 and at the large batch")
+    ap.add_argument("--continuation", default="", metavar="AFTER:NEW",
+                    help="also time a step of NEW tokens of a sequence that holds AFTER tokens already "
+                         "(a new turn of a conversation); reported as \"continuation\"")
     ap.add_argument("--no-tune", action="store_true",
                     help="leave the library's default kernels for the tall matrix products")
     args = ap.parse_args()
@@ -98,6 +101,17 @@ def main() -> int:
         print(f"bench.py: prompts of {max(PROMPT, PROMPT_HI)} tokens and {args.warmup + args.repeats * args.steps} "
               f"steps do not fit a context of {CONTEXT}")
         return 2
+    cont = None
+    if args.continuation:
+        try:
+            cont = tuple(int(v) for v in args.continuation.split(":"))
+            assert len(cont) == 2 and cont[0] >= 0 and cont[1] >= 1
+        except (ValueError, AssertionError):
+            print("bench.py: --continuation takes AFTER:NEW, two token counts")
+            return 2
+        if sum(cont) > CONTEXT:
+            print(f"bench.py: a continuation of {cont[1]} tokens after {cont[0]} does not fit a context of {CONTEXT}")
+            return 2
     FULL_LAYERS = SHAPE["num_hidden_layers"]
     args.layers = args.layers or FULL_LAYERS
 
@@ -213,6 +227,25 @@ def main() -> int:
     prefill_s = sorted(times)[1]
     flops = prefill_flops(SHAPE, args.layers, PROMPT)
 
+    # ---- a step of a few new tokens behind a long sequence: the median of three
+    continuation = None
+    if cont is not None:
+        progress(f"{cont[1]} tokens after {cont[0]}")
+        before, fresh = prompts(1, cont[0], cont[0])[0], prompts(1, cont[1], cont[1])[0]
+        times = []
+        for run in range(4):
+            slot = engine.acquire()
+            if before:
+                engine.step([StepEntry(slot, before, [])])
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            engine.step([StepEntry(slot, fresh, [len(fresh) - 1])])
+            torch.cuda.synchronize()
+            if run > 0:
+                times.append(time.perf_counter() - t0)
+            engine.release(slot)
+        continuation = {"after": cont[0], "tokens": cont[1], "ms": round(sorted(times)[1] * 1e3, 3)}
+
     # ---- decode at the headline batch
     progress(f"decode at batch {args.batch}")
     runs = decode_run(args.batch, args.steps, args.warmup, args.repeats)
@@ -266,6 +299,8 @@ def main() -> int:
                     "median": round(step_s * 1e3, 4),
                     "max": round(max(t for t, _ in runs) * 1e3, 4)},
     }
+    if continuation:
+        line["continuation"] = continuation
     if packed:
         line["prefill_packed"] = {"value": round(packed["tokens"] / packed["seconds"], 1), "tokens": packed["tokens"],
                                   "ms": round(packed["seconds"] * 1e3, 3),
