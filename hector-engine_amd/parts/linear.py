@@ -137,13 +137,14 @@ class Linear:
         256 x 256 outputs would be a dozen or two for a chip of 256 compute units, each walking all
         of K. As a batched product over K slices with fp32 results, which he_splitk_reduce adds
         in slice order, the Qwen2.5-7B down projection takes 58 us instead of 99 at 128 rows, 50
-        instead of 122 at 200, 54 instead of 126 at 256, 81 instead of 197 at 512. Products with
+        instead of 122 at 200, 54 instead of 126 at 256, 80 instead of 197 at 512 (four slices); the
+        Qwen2.5-32B one 68 instead of 180 at 128 rows, the Qwen2-72B one (four slices) 142 instead of 226. Products with
         K below 8192 gain nothing (q||k||v, o, gate||up: measured)."""
         N, K = self.weight.shape
-        if rows > 512 or K < 8192 or K < 4 * N:
+        if rows > 512 or K < 8192 or K < 3 * N:
             return 1
         tiles = -(-rows // 256) * -(-N // 256)
-        slices = 8 if tiles <= 32 else 4 if tiles <= 64 else 1
+        slices = 8 if tiles <= 20 else 4 if tiles <= 40 else 2 if tiles <= 64 else 1
         while slices > 1 and K % (8 * slices):
             slices //= 2
         return slices

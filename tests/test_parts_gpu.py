@@ -251,7 +251,10 @@ def test_a_long_k_product_in_slices_through_the_library(fw, rows, N, K, bias):
     b = rnd(N, seed=12).to(torch.bfloat16) if bias else None
     lin = Linear(w.cuda(), b.cuda() if bias else None)
     slices = lin._library_slices(rows)
-    assert slices == (1 if rows > 512 else 8 if K % 64 == 0 else 1 if K % 16 else 2 if K % 32 else 4)
+    want = 1 if rows > 512 else 8          # a handful of the library's tiles at these sizes
+    while want > 1 and K % (8 * want):
+        want //= 2
+    assert slices == want
     ctx = make_ctx(fw, env, [rows], [0], [0])
     x = rnd(rows, K, seed=13).to(torch.bfloat16)
     out = lin(x.cuda(), rows, ctx)

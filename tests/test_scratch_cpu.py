@@ -67,3 +67,18 @@ def test_an_arena_that_was_too_small_is_made_whole_at_the_next_step_and_a_frozen
         assert "cannot grow" in str(e)
     else:
         raise AssertionError("a frozen pool grew")
+
+
+def test_which_library_products_are_cut_along_k():
+    """The rule that sends a long-K product of up to 512 rows to the library in K slices: the down projections of
+    the Qwen2 shapes in 2 to 8 slices, nothing for short K, wide outputs, more than 512 rows, or a K that does not divide."""
+    from hector_engine_amd.parts.linear import Linear
+
+    def slices(N, K, rows):
+        return Linear(torch.empty(N, K, dtype=torch.bfloat16, device="meta"))._library_slices(rows)
+    assert [slices(3584, 18944, r) for r in (65, 200, 256, 512, 513, 2048)] == [8, 8, 8, 4, 1, 1]
+    assert slices(5120, 27648, 128) == 8 and slices(5120, 27648, 300) == 4
+    assert slices(8192, 29568, 128) == 4 and slices(8192, 29568, 300) == 2
+    assert slices(4608, 3584, 200) == 1 and slices(37888, 3584, 200) == 1 and slices(3584, 3584, 128) == 1
+    assert slices(152064, 3584, 100) == 1
+    assert slices(64, 8200, 100) == 1 and slices(64, 8208, 100) == 2 and slices(64, 8224, 100) == 4
