@@ -82,3 +82,17 @@ def test_which_library_products_are_cut_along_k():
     assert slices(4608, 3584, 200) == 1 and slices(37888, 3584, 200) == 1 and slices(3584, 3584, 128) == 1
     assert slices(152064, 3584, 100) == 1
     assert slices(64, 8200, 100) == 1 and slices(64, 8208, 100) == 2 and slices(64, 8224, 100) == 4
+
+
+def test_which_one_token_steps_count_as_uneven():
+    """The engine's flag for a step in which one sequence has several times the keys of the others: the longest
+    has 4096 or more and at least four times the mean; a single sequence, equal lengths or short ones do not count."""
+    import types
+    from hector_engine_amd.engine.engine import Engine, StepEntry
+
+    def uneven(lengths):
+        fake = types.SimpleNamespace(cache=types.SimpleNamespace(length=lambda slot: lengths[slot]))
+        return Engine._uneven_keys(fake, [StepEntry(i, [1], [0]) for i in range(len(lengths))])
+    assert uneven([30000] + [200] * 7) and uneven([30000, 30000] + [500] * 62) and uneven([4096, 10, 10, 10, 10])
+    assert not uneven([30000]) and not uneven([8000] * 8) and not uneven([16000, 16000] + [1000] * 6)
+    assert not uneven([4000, 10, 10, 10, 10]) and not uneven([5000, 4000, 3000])
