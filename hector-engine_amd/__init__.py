@@ -13,7 +13,7 @@ bookkeeping import without a GPU.
 from __future__ import annotations
 
 __all__ = ["Engine", "StepEntry", "generate", "GenerationResult", "SamplingConfig", "Sampler",
-           "load_config", "register_architecture", "register_part", "write_random_model",
+           "load_config", "register_architecture", "register_part", "register_init", "write_random_model",
            "build_kernels"]
 
 _LAZY = {
@@ -26,6 +26,7 @@ _LAZY = {
     "load_config": ("registry", "load_config"),
     "register_architecture": ("registry", "register_architecture"),
     "register_part": ("parts.base", "register_part"),
+    "register_init": ("weights.random_init", "register_init"),
     "write_random_model": ("weights.random_init", "write_random_model"),
 }
 

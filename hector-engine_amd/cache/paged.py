@@ -3,8 +3,8 @@
 Keys and values live in pages of 64 tokens. Layers are partitioned into groups
 by what they keep (kv heads, key and value widths, all keys or a window of them); each
 group has pools of its own, [runs][pages][kv_heads][elements of a page] for K and for
-V, the elements of a page in the order the attention kernels read their operands
-(cache/layout.py), and one page table [slots][blocks]
+V, a page as large as the group's mixers ask for (KVNeed.k_elems, KVNeed.v_elems: the order
+inside a page is theirs), and one page table [slots][blocks]
 shared by its runs. A sequence holds a
 slot: its row of every page table, its length, and its row of the fixed-size
 state area. Slots and pages go back to the free lists when a sequence ends and
@@ -21,7 +21,6 @@ import dataclasses
 import torch
 
 from ..parts.base import KVNeed, LayerCache
-from . import layout
 from .pages import PAGE_TOKENS, CacheError, CacheFull, GroupPages, SlotBook, blocks_for  # noqa: F401
 
 
@@ -41,11 +40,9 @@ class _Group:
         self.runs = runs
         # zero-filled once (as the reference's cache is: src/kv_cache.hpp:161-203): a masked
         # key still enters the matrix products with weight 0, so it must never be NaN
-        # a page of a kv head is kept in the order the attention kernels read it (cache/layout.py)
-        self.kpool = torch.zeros((len(runs), num_pages, need.kv_heads, layout.k_page_elems(need.head_dim)),
-                                 dtype=dtype, device=device)
-        self.vpool = torch.zeros((len(runs), num_pages, need.kv_heads, layout.v_page_elems(need.v_dim)),
-                                 dtype=dtype, device=device)
+        # a page is as large as the mixers of the group say; what lies where inside it is theirs
+        self.kpool = torch.zeros((len(runs), num_pages, need.kv_heads, need.k_elems), dtype=dtype, device=device)
+        self.vpool = torch.zeros((len(runs), num_pages, need.kv_heads, need.v_elems), dtype=dtype, device=device)
         self.page_table = torch.full((max_slots, max_blocks), -1, dtype=torch.int32, device=device)
 
 
@@ -103,6 +100,14 @@ class PagedCache:
 
     def release(self, slot: int) -> None:
         self._clear(self.book.release(slot))
+
+    def truncate(self, slot: int, new_length: int) -> None:
+        """Keeps the first new_length tokens of the slot and gives back the pages beyond
+        (cache/pages.py: SlotBook.truncate). A model that keeps fixed-size state per
+        sequence cannot be rewound: the state has seen the dropped tokens."""
+        if self.state is not None and new_length < self.length(slot):
+            raise CacheError(f"slot {slot}: a model with per-sequence state cannot be truncated")
+        self._clear(self.book.truncate(slot, new_length))
 
     def length(self, slot: int) -> int:
         try:
@@ -172,6 +177,5 @@ class PagedCache:
 
     def bytes_per_token(self) -> int:
         es = torch.empty((), dtype=self.dtype).element_size()
-        return sum(len(g.runs) * g.need.kv_heads * es
-                   * (layout.k_page_elems(g.need.head_dim) + layout.v_page_elems(g.need.v_dim)) // PAGE_TOKENS
+        return sum(len(g.runs) * g.need.kv_heads * es * (g.need.k_elems + g.need.v_elems) // PAGE_TOKENS
                    for g in self.groups)

@@ -142,14 +142,50 @@ class SlotBook:
             if g.window <= 0:
                 continue
             row = g.table[slot]
-            dead = (new_length - g.window - (PAGE_TOKENS - 1)) // PAGE_TOKENS + 1 \
-                if new_length - g.window >= PAGE_TOKENS - 1 else 0
-            for b in range(min(dead, len(row))):
+            for b in range(min(self._dead_blocks(new_length, g.window), len(row))):
                 if row[b] >= 0:
                     g.pool.give_back(row[b])
                     row[b] = -1
                     cleared.append((gi, slot, b))
         return cleared
+
+    def truncate(self, slot: int, new_length: int) -> list[tuple[int, int, int]]:
+        """Shortens the slot to its first new_length tokens (the reference's rewind:
+        src/kv_cache.hpp:93-96; what lies beyond is never read again and is overwritten by
+        the next tokens). Pages that hold no position below new_length go back to their
+        pools. A windowed group must still hold every key the token at new_length will see:
+        the pages it gave back at the present length must be pages it would have given back
+        at new_length too, or nothing is changed and the call raises. Returns cleared
+        (group, slot, block)."""
+        self._check(slot)
+        if not 0 <= new_length <= self.length[slot]:
+            raise CacheError(f"slot {slot}: cannot truncate from {self.length[slot]} to {new_length}")
+        for gi, g in enumerate(self.groups):
+            if g.window <= 0:
+                continue
+            dead = self._dead_blocks(new_length, g.window)
+            if any(page < 0 for page in g.table[slot][dead:]):
+                raise CacheError(f"slot {slot}: group {gi} keeps a window of {g.window} keys and has given "
+                                 f"back pages that a sequence of {new_length} tokens still reads")
+        keep = blocks_for(new_length)
+        cleared = []
+        for gi, g in enumerate(self.groups):
+            row = g.table[slot]
+            for b in range(keep, len(row)):
+                if row[b] >= 0:
+                    g.pool.give_back(row[b])
+                    cleared.append((gi, slot, b))
+            del row[keep:]
+        self.length[slot] = new_length
+        return cleared
+
+    @staticmethod
+    def _dead_blocks(length: int, window: int) -> int:
+        """Leading blocks of a windowed group that no query at or beyond position `length`
+        reads: block b is dead once its last position 64b+63 <= length - window."""
+        if length - window < PAGE_TOKENS - 1:
+            return 0
+        return (length - window - (PAGE_TOKENS - 1)) // PAGE_TOKENS + 1
 
     def check_invariants(self) -> None:
         """Every page is free or held by exactly one (slot, block)."""

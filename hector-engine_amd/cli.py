@@ -13,7 +13,9 @@ HELIOS_TOPK, HELIOS_TOPP, HELIOS_SEED, and HELIOS_CTX (helios_chat.cpp:549); a
 flag wins over its variable. Options of this library's own: --random CONFIG.json
 --seed N (random weights instead of a folder), --tokens / --tokens-file,
 --max-new-tokens, --temperature, --top-k, --top-p, --sampler-seed, --max-seq,
---slots, --dtype, --stop-ids, --no-graph, --tune-gemm, --profile.
+--slots, --dtype, --stop-ids, --no-graph, --tune-gemm, --profile, --sync-each-launch.
+Without --stop-ids a sequence ends at the model's own end-of-sequence ids: `eos_token_id` of
+the folder's generation_config.json, else of its config.json.
 It prints the generated ids and the reference's closing report
 (test_generate_kv.cpp:294-300).
 """
@@ -80,6 +82,8 @@ def parse_args(argv: list[str]):
                          "per new shape)")
     ap.add_argument("--profile", action="store_true",
                     help="time every kernel with a pair of events (no HIP graphs) and print the table")
+    ap.add_argument("--sync-each-launch", action="store_true",
+                    help="debugging: wait for the GPU after every launch and name the op in an error")
     ap.add_argument("rest", nargs="*")
     ns = ap.parse_args(argv)
     rest = list(ns.rest)
@@ -160,16 +164,15 @@ def main(argv: list[str] | None = None) -> int:
         prompts = [[first]]
     ctx = context_length(ns, model_spec(config).max_positions)
     sampling = he.SamplingConfig(**sampling_options(ns, temperature))
-    if ns.stop_ids is not None:
-        stop_ids = [int(t) for t in ns.stop_ids.split(",") if t]
-    else:
-        stop_ids = list(getattr(config, "eos_token_id", None) or [])
+    # None: the model's own end-of-sequence ids (generation_config.json, else config.json)
+    stop_ids = [int(t) for t in ns.stop_ids.split(",") if t] if ns.stop_ids is not None else None
     slots = max(1, min(len(prompts), ns.slots or len(prompts)))
     pages = slots * ((ctx + 63) // 64)
     start = time.perf_counter()
     source = dict(config=config, seed=ns.seed) if ns.random is not None else dict(model_dir=model)
     engine = he.Engine(dtype=ns.dtype, max_tokens=pages * 64, max_slots=slots, max_seq_len=ctx,
-                       use_graphs=not ns.no_graph, tune_library=ns.tune_gemm, profile=ns.profile, **source)
+                       use_graphs=not ns.no_graph, tune_library=ns.tune_gemm, profile=ns.profile,
+                       sync_each_launch=ns.sync_each_launch, **source)
     what = f"random weights for {ns.random}, seed {ns.seed}" if ns.random is not None else model
     print(f"Model: {what}  ({config.architecture}, {ns.dtype})  loaded in "
           f"{(time.perf_counter() - start) * 1e3:.0f} ms")

@@ -78,6 +78,28 @@ def load_config_dict(model_dir: str) -> dict:
     return data
 
 
+def stop_token_ids(model_dir: str | None, config: "ModelConfig") -> list[int]:
+    """The token ids that end a sequence when the caller names none: `eos_token_id` of the
+    folder's generation_config.json when that file has the key (an instruction-tuned
+    checkpoint lists its end-of-turn id there beside the end-of-text id), else `eos_token_id`
+    of config.json, else none. The reference takes the id from the model's own files too
+    (src/inference_session.cpp:357)."""
+    if model_dir is not None:
+        path = os.path.join(model_dir, "generation_config.json")
+        if os.path.exists(path):
+            try:
+                with open(path) as f:
+                    data = json.load(f)
+            except json.JSONDecodeError as exc:
+                raise ConfigError(f"{path}: not valid JSON: {exc}") from None
+            if not isinstance(data, dict):
+                raise ConfigError(f"{path}: top level must be an object")
+            ids = read_int_list(data, "eos_token_id", None)
+            if ids is not None:
+                return ids
+    return list(getattr(config, "eos_token_id", None) or [])
+
+
 def architecture_name(data: dict) -> str:
     """architectures[0], the name the registry is keyed by."""
     archs = data.get("architectures")

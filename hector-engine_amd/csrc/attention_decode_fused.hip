@@ -278,9 +278,10 @@ static void fused_shape(int rows, int H, int KVH, int hd, int max_keys, int spre
   const int gt = G < 16 ? G : 16;
   const int groups = rows * KVH * ((G + 15) / 16);
   int w = (int64_t)8 * gt * (hd + 2) * 4 <= 65536 ? 8 : 4, zz = 1;
-  if (groups < HE_CUS) {
+  const int cus = he_cus();
+  if (groups < cus) {
     w = 4;
-    zz = (HE_CUS + groups - 1) / groups;
+    zz = (cus + groups - 1) / groups;
     const int cap = max_keys > 16384 ? 32 : 16;
     if (zz > cap) zz = cap;
     const int most = (max_keys + 4 * FUSED_MIN_CHUNK - 1) / (4 * FUSED_MIN_CHUNK);

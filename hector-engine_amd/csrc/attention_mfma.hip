@@ -414,7 +414,7 @@ extern "C" int he_attention_prefill_parts(int num_seqs, int max_q_len, int H, in
   if (num_seqs <= 0 || H <= 0 || hd <= 0 || hd > 128 || hd % 16 || max_q_len <= 0) return 1;
   if ((int64_t)most_keys < 4 * (int64_t)max_q_len) return 1;
   const int64_t blocks = (int64_t)((max_q_len + 127) / 128) * H * num_seqs;
-  int64_t parts = 2 * HE_CUS / blocks;
+  int64_t parts = 2 * he_cus() / blocks;
   const int pages = (most_keys + HE_PAGE_TOKENS - 1) / HE_PAGE_TOKENS;
   if (parts > pages / 4) parts = pages / 4;
   if (parts > 16) parts = 16;

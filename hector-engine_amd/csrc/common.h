@@ -18,7 +18,8 @@
 #define HE_WAVE 64
 // L2 domains (XCDs) of the part; consecutive workgroups of a launch go to them in turn
 #define HE_XCDS 8
-// compute units of the part (the grids of the products count in them as well)
+// compute units of the MI355X: the default of he_cus(), and what the prompt attention's order of
+// work inside the kernel is written for
 #define HE_CUS 256
 
 struct bf16_t {
@@ -146,6 +147,8 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 // ---- error channel -------------------------------------------------------
 void he_set_error(const char* fmt, ...);
 int he_check_launch(const char* what);
+// compute units of the current device (errors.hip); the host-side plans count in them
+int he_cus();
 // attention_mfma.hip: joins attention parts that were all stored (the fused one-token kernel's, the
 // prompt kernel's); row_seq may be null: every row has a sequence
 int he_attention_merge_parts(void* out, const float* ws_o, const float* ws_ml, const void* row_seq,

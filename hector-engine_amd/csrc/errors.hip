@@ -26,4 +26,24 @@ int he_check_launch(const char* what) {
 
 extern "C" const char* he_last_error(void) { return g_error; }
 
+// Compute units of the current device, asked once per device and process. The grids of the
+// products and of the attention kernels count in them; HE_CUS (the MI355X's 256, at which the
+// rules were measured) stands in where the device cannot be asked.
+int he_cus() {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    (void)hipGetLastError();
+    return HE_CUS;
+  }
+  int n = cached[dev];
+  if (n > 0) return n;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+    (void)hipGetLastError();
+    n = HE_CUS;
+  }
+  cached[dev] = n;
+  return n;
+}
+
 extern "C" int he_abi_version(void) { return HE_ABI_VERSION; }

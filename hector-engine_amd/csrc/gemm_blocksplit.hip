@@ -41,6 +41,7 @@
 // and Qwen2-72B shapes). The rule depends on the sizes only, so a product always runs the same way.
 static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int U, int NW) {
   BlockSplitPlan p;
+  const int cus = he_cus();
   p.MT = (M + 15) / 16;
   int r, u, nw;
   if (N >= 65536) {                 // output head
@@ -48,14 +49,14 @@ static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int
     else if (p.MT == 1) r = 4, u = 2, nw = 4;
     else r = 2, u = 2, nw = 4;
   } else if (K >= 8192) {           // long K
-    const int groups = (N + 31) / 32, last_round = groups % HE_CUS;   // with two tiles a workgroup
+    const int groups = (N + 31) / 32, last_round = groups % cus;   // with two tiles a workgroup
     if (N < 4096) {                 // few weight rows: one tile a workgroup, or the chip is not filled
       r = 1, u = 1, nw = p.MT == 1 ? 8 : 4;
     } else if (p.MT == 2) {
       r = 2, u = 2, nw = 4;
     } else if (M > 8 && N >= 10240) {
       r = 4, u = 2, nw = 4;         // the activation rows are read half as often
-    } else if (groups < HE_CUS) {
+    } else if (groups < cus) {
       r = 2, u = 1, nw = 8;         // under one workgroup a compute unit: more wavefronts each
     } else if (groups < 1024 && last_round > 0 && last_round <= 128) {
       r = 1, u = 1, nw = 8;         // the last round of whole tiles would fill under half of the chip:
@@ -74,7 +75,7 @@ static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int
     u = p.MT == 1 && K < 5120 ? 4 : 1;   // 5120 x 5120 at 8 rows: 12.8 us unrolled once, 13.5 us four times
     nw = 8;
   }
-  // Weight rows are dealt out evenly over the 256 compute units (or twice, three times ... 256
+  // Weight rows are dealt out evenly over the compute units (256 of them: or twice, three times ... 256
   // workgroups, at most 32 rows each) rather than in whole tiles of 16: 4608 rows as 256
   // workgroups of 18 rows instead of 144 of 32, the 37888 rows of gate||up as 1280 of 30
   // instead of 1184 of 32 (4.6 a compute unit). The last tile of such a workgroup is partly
@@ -82,8 +83,8 @@ static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int
   // stored in pairs.
   int rows = 0;
   if (R <= 0 && r <= 2 && N >= 2048 && N < 65536) {
-    const int rounds = (N + HE_CUS * 32 - 1) / (HE_CUS * 32);
-    rows = ((N + HE_CUS * rounds - 1) / (HE_CUS * rounds) + 1) & ~1;
+    const int rounds = (N + cus * 32 - 1) / (cus * 32);
+    rows = ((N + cus * rounds - 1) / (cus * rounds) + 1) & ~1;
     r = rows > 16 ? 2 : 1;
   }
   p.R = R > 0 ? R : r;

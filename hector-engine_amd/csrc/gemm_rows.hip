@@ -49,7 +49,7 @@ static RowsPlan rows_plan(int M, int N, int K, int R, int NWV, int splits) {
   if (N >= 16384 && splits <= 1) {
     // dealt out evenly over the workgroups the chip holds at once: one a compute unit where a workgroup
     // has 256 rows (the head; sixteen wavefronts), two otherwise
-    const int slots = HE_CUS * ((R == 2 && NWV == 8) || NWV == 16 ? 1 : 2);
+    const int slots = he_cus() * ((R == 2 && NWV == 8) || NWV == 16 ? 1 : 2);
     const int rounds = (N + slots * cap - 1) / (slots * cap);
     rows = ((N + slots * rounds - 1) / (slots * rounds) + 3) & ~3;
     if (rows > cap) rows = cap;
@@ -59,7 +59,7 @@ static RowsPlan rows_plan(int M, int N, int K, int R, int NWV, int splits) {
   int s = splits;
   if (s <= 0) {
     s = 1;
-    while (p.groups * s < 192 && K / (2 * s) >= 512 && s < 32) s *= 2;
+    while (p.groups * s < he_cus() * 3 / 4 && K / (2 * s) >= 512 && s < 32) s *= 2;   // 192 workgroups on 256 units
   }
   int ks = (K + s - 1) / s;
   ks = (ks + ROWS_KC - 1) / ROWS_KC * ROWS_KC;

@@ -20,7 +20,7 @@ import torch
 
 from ..cache.paged import PagedCache
 from ..cache.pages import CacheError, CacheFull  # noqa: F401
-from ..config.base import ModelConfig
+from ..config.base import ModelConfig, stop_token_ids
 from ..kernels import lib as kernel_lib
 from ..kernels import library_tuning, profiler
 from ..parts.base import BuildEnv, StepContext
@@ -74,6 +74,7 @@ class _GraphBucket:
         self.graph: torch.cuda.CUDAGraph | None = None
         self.logits: torch.Tensor | None = None
         self.uses = 0
+        self.capture_failed: str | None = None    # why this bucket runs without a graph
 
 
 class Engine:
@@ -81,13 +82,17 @@ class Engine:
                  seed: int | None = None, dtype: str = "bfloat16", max_tokens: int = 8192,
                  max_slots: int | None = None, max_seq_len: int | None = None,
                  device: str = "cuda:0", fast_kernels: bool = True, use_graphs: bool = True,
-                 tune_library: bool = False, beyond_max_positions: bool = False, profile: bool = False):
+                 tune_library: bool = False, beyond_max_positions: bool = False, profile: bool = False,
+                 sync_each_launch: bool = False):
         """max_seq_len: the longest sequence (default: the positions the model's configuration
         allows; more than that is refused unless beyond_max_positions says it is meant).
         tune_library: let the library's autotuner choose the kernel of each tall bfloat16
         matrix product the first time its shape is seen (kernels/library_tuning.py).
         profile: time every kernel with a pair of events (kernels/profiler.py; steps then run
-        without HIP graphs); profile_summary() gives the table."""
+        without HIP graphs); profile_summary() gives the table.
+        sync_each_launch: a debugging mode (the reference's sync_after_each_op, src/engine.cpp:318-334):
+        steps run without HIP graphs and the host waits for the GPU after every launch, so that
+        a fault is reported with the name of the op that raised it."""
         if dtype not in _DTYPES:
             raise ValueError(f"dtype must be one of {sorted(_DTYPES)}, got {dtype!r}")
         if not torch.cuda.is_available():
@@ -109,6 +114,8 @@ class Engine:
             self.config = config
         else:
             raise ValueError("give a model folder, or a configuration and a seed")
+        # what ends a sequence when a caller of generate() names no stop ids
+        self.stop_ids = stop_token_ids(model_dir, self.config)
         self.model = build_model(self.config, self.env)
         specs = self.model.tensor_specs()
         if model_dir is not None:
@@ -133,14 +140,17 @@ class Engine:
         self.caches = [self.cache.layer_cache(r) for r in range(len(self.model.schedule))]
         self.scratch = ScratchPool(self.device)
         self.profiler = profiler.OpProfiler() if profile else None
-        self.use_graphs = use_graphs and self.model.graph_safe() and not profile
-        self._capture_failed = False
+        self.sync_each_launch = sync_each_launch
+        self.use_graphs = use_graphs and self.model.graph_safe() and not profile and not sync_each_launch
         self._buckets: dict[tuple[int, bool], _GraphBucket] = {}
+        self._uneven_sticky: dict[int, bool] = {}     # per bucket size: the flag of the step before
         self._pinned = [torch.empty(1 << 16, dtype=torch.int32).pin_memory() for _ in range(4)]
         self._pinned_events: list[torch.cuda.Event | None] = [None] * 4
         self._pinned_next = 0
         self._iota_cache = np.arange(64, dtype=np.int32)
-        self.stats = {"steps": 0, "graph_replays": 0, "graph_captures": 0, "eager_steps": 0}
+        self.stats = {"steps": 0, "graph_replays": 0, "graph_captures": 0, "eager_steps": 0,
+                      "graph_capture_failures": 0}
+        self.capture_failures: list[str] = []         # one line per bucket whose capture failed
 
     # -- slots ----------------------------------------------------------------
     def acquire(self) -> int:
@@ -151,6 +161,13 @@ class Engine:
 
     def length(self, slot: int) -> int:
         return self.cache.length(slot)
+
+    def truncate(self, slot: int, length: int) -> None:
+        """Drops the tokens of the slot beyond its first `length` (a turn that is taken back:
+        the reference rewinds its cache so, src/kv_cache.hpp:93-96, src/inference_session.cpp:682-693)
+        and gives back the pages that held only them. The next step of the slot continues at
+        position `length`, with the logits a fresh run of the kept tokens would give."""
+        self.cache.truncate(slot, length)
 
     @property
     def max_seq_len(self) -> int:
@@ -200,7 +217,7 @@ class Engine:
         all_single = all(len(e.tokens) == 1 for e in entries)
         every_wanted = all(list(e.want) == [0] for e in entries)
         self.stats["steps"] += 1
-        with profiler.active(self.profiler):
+        with profiler.active(self.profiler), profiler.sync_each_launch(self.sync_each_launch):
             if self.use_graphs and all_single and every_wanted and len(entries) <= GRAPH_MAX_BUCKET:
                 logits = self._graph_step(entries, device_tokens)
             else:
@@ -289,14 +306,16 @@ class Engine:
                            max_q_len=max_q_len, max_keys=self.cache.max_seq_len,
                            all_single=all_single, env=self.env, scratch=pool)
 
-    def _uneven_keys(self, entries) -> bool:
+    def _uneven_keys(self, entries, was: bool = False) -> bool:
         """Whether one sequence of a one-token step has several times the keys of the others (and
         thousands of them): the attention kernels then cut every sequence's keys across more
         workgroups, or the long sequence would be left to a few of them. A step with the flag has a
-        graph of its own."""
+        graph of its own. was: the flag of the step before; it then stays up until the longest
+        sequence has fewer than three times the mean (four to raise it), so that a batch at the
+        edge does not go back and forth between two graphs."""
         lens = [self.cache.length(e.slot) for e in entries]
         longest = max(lens)
-        return longest >= 4096 and longest * len(lens) >= 4 * sum(lens)
+        return longest >= 4096 and longest * len(lens) >= (3 if was else 4) * sum(lens)
 
     def _eager_step(self, entries, all_single: bool, device_tokens=None):
         rows = sum(len(e.tokens) for e in entries)
@@ -323,7 +342,7 @@ class Engine:
     def _graph_step(self, entries, device_tokens=None):
         n = len(entries)
         size = 1 << (n - 1).bit_length()
-        uneven = self._uneven_keys(entries)
+        uneven = self._uneven_sticky[size] = self._uneven_keys(entries, self._uneven_sticky.get(size, False))
         bucket = self._buckets.get((size, uneven))
         if bucket is None:
             bucket = self._buckets[(size, uneven)] = _GraphBucket(size, self.device)
@@ -342,7 +361,7 @@ class Engine:
             if bucket.uses == 1:
                 # first use: run eagerly; it also sizes the bucket's scratch pool
                 return self._bucket_eager(bucket, ctx, n)
-            if self._capture_failed:
+            if bucket.capture_failed is not None:
                 return self._bucket_eager(bucket, ctx, n)
             bucket.pool.reset()          # sized by the eager run; from here on it must not move
             bucket.pool.frozen = True
@@ -354,13 +373,20 @@ class Engine:
                     bucket.logits = self.model.forward(bucket.views["tokens"], ctx, self.caches,
                                                        bucket.views["want_rows"], size)
             except Exception as exc:     # the reference falls back the same way: src/engine.cpp:233-261
-                self._capture_failed = True
+                # This bucket alone runs without a graph from here on. The same step is run again
+                # eagerly below: an error that is the step's own (a kernel's refusal, a part's
+                # bug) is raised again there and reaches the caller; only a failure of the
+                # capture itself ends in the fallback.
+                bucket.capture_failed = f"{size} rows{', uneven' if uneven else ''}: {exc!r}"
+                self.capture_failures.append(bucket.capture_failed)
+                self.stats["graph_capture_failures"] += 1
                 bucket.pool.frozen = False
                 del graph
                 torch.cuda.synchronize()
-                warnings.warn(f"capturing the one-token step as a HIP graph failed ({exc!r}); "
-                              "one-token steps run without graphs from here on", stacklevel=3)
-                return self._bucket_eager(bucket, ctx, n)
+                logits = self._bucket_eager(bucket, ctx, n)
+                warnings.warn(f"capturing the one-token step of {bucket.capture_failed} as a HIP graph "
+                              "failed; steps of this size run without a graph from here on", stacklevel=3)
+                return logits
             bucket.graph = graph
             self.stats["graph_captures"] += 1
         bucket.graph.replay()

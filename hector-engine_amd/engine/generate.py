@@ -72,10 +72,13 @@ RUN_OF_STEPS = 8
 
 
 def generate(engine, prompts: list[list[int]], *, max_new_tokens: int = 100, sampling=None,
-             stop_ids=(), include_stop: bool = False, batch_size: int | None = None,
+             stop_ids=None, include_stop: bool = False, batch_size: int | None = None,
              cancel: Callable[[], bool] | None = None, sample_fn=None, sampler=None,
              run_of_steps: int = RUN_OF_STEPS) -> list[GenerationResult]:
     """Generates for every prompt; returns results in the order of `prompts`.
+
+    stop_ids: the token ids that end a sequence; None: the model's own (engine.stop_ids: the
+    end-of-sequence ids of its generation_config.json or config.json), (): none.
 
     sampler: an object with the library Sampler's interface (config, sample, sample_device,
     uniforms_device, read_later) in place of one made from `sampling`; sample_fn: a plain
@@ -102,6 +105,8 @@ def generate(engine, prompts: list[list[int]], *, max_new_tokens: int = 100, sam
     else:
         sampler = None
     run_of_steps = min(run_of_steps, READS_IN_FLIGHT)
+    if stop_ids is None:
+        stop_ids = getattr(engine, "stop_ids", ())
     stop_ids = frozenset(int(s) for s in stop_ids)
     results: list[GenerationResult | None] = [None] * len(prompts)
     pending = [(i, len(p)) for i, p in enumerate(prompts)]

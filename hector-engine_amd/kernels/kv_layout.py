@@ -1,5 +1,6 @@
-"""Sizes and indices of a cache page (64 tokens of one kv head) as the attention kernels
-keep it: in the order in which the MFMA kernels read their operands, so that every operand
+"""Sizes and indices of a cache page (64 tokens of one kv head) as the attention kernels of
+this library keep it (the attention part asks the cache for pages of these sizes through its
+KVNeed; the cache itself knows no layout): in the order in which the MFMA kernels read their operands, so that every operand
 load is one contiguous KiB (csrc/cache_layout.h holds the same formulas for the device).
 
   K: [half h][key tile t][k step ks][lane = 16 lg + lr][e]   key = 32 h + 8 (lr // 4) + 4 t + lr % 4

@@ -5,7 +5,7 @@ from __future__ import annotations
 
 import torch
 
-from ..cache import layout
+from . import kv_layout as layout
 from . import lib as _lib
 from .profiler import op as _op
 

@@ -7,6 +7,11 @@ matrix product of parts.linear) is bracketed by two events on the current stream
 are read when the table is asked for, not after each launch, so the launches still follow one
 another without a wait in between. Steps run eagerly while profiling: a captured graph has no
 place for events between its nodes.
+
+The same hooks serve a debugging mode in the manner of the reference's sync_after_each_op
+(src/engine.cpp:318-334): inside sync_each_launch() the host waits for the GPU after every
+launch, so that a fault a kernel raises asynchronously is reported with the name of the op
+that caused it, not at some later call.
 """
 from __future__ import annotations
 
@@ -16,6 +21,13 @@ import functools
 import torch
 
 _active: "OpProfiler | None" = None
+_sync_each = False
+# events of launches not yet read: collect() is called on the way once so many are waiting
+MAX_PENDING = 4096
+
+
+class LaunchFault(RuntimeError):
+    """The GPU reported an error right after the named launch (sync_each_launch mode)."""
 
 
 class OpProfiler:
@@ -33,16 +45,22 @@ class OpProfiler:
         finally:
             stop.record()
             self._pending.append((name, start, stop))
+            if len(self._pending) >= MAX_PENDING:
+                # a long profiled generation would pile up events without bound; the oldest
+                # have long completed, so reading them costs no wait to speak of
+                self._collect(len(self._pending) // 2)
 
     def collect(self) -> None:
-        if self._pending:
-            self._pending[-1][2].synchronize()
-        for name, start, stop in self._pending:
+        self._collect(len(self._pending))
+
+    def _collect(self, count: int) -> None:
+        """Reads the `count` oldest pending event pairs into the totals."""
+        for name, start, stop in self._pending[:count]:
             stop.synchronize()
             entry = self._totals.setdefault(name, [0, 0.0])
             entry[0] += 1
             entry[1] += start.elapsed_time(stop)
-        self._pending.clear()
+        del self._pending[:count]
 
     def clear(self) -> None:
         self.collect()
@@ -90,8 +108,37 @@ def active(profiler: "OpProfiler | None"):
         _active = before
 
 
+@contextlib.contextmanager
+def sync_each_launch(on: bool = True):
+    """Inside (with on): the host waits for the GPU after every launch and raises LaunchFault
+    naming the op when the wait reports an error."""
+    global _sync_each
+    before, _sync_each = _sync_each, bool(on)
+    try:
+        yield
+    finally:
+        _sync_each = before
+
+
+def _wait_after(name: str) -> None:
+    try:
+        torch.cuda.synchronize()
+    except RuntimeError as exc:
+        raise LaunchFault(f"the GPU reported an error after the launch of '{name}': {exc}") from exc
+
+
+@contextlib.contextmanager
+def _synced(name: str):
+    with (_active.span(name) if _active is not None else contextlib.nullcontext()):
+        yield
+    _wait_after(name)
+
+
 def span(name: str):
-    """A context that times what runs inside under `name` when a profiler is active."""
+    """A context that times what runs inside under `name` when a profiler is active (and waits
+    for it in sync_each_launch mode)."""
+    if _sync_each:
+        return _synced(name)
     return _active.span(name) if _active is not None else contextlib.nullcontext()
 
 
@@ -100,9 +147,9 @@ def op(name: str):
     def deco(fn):
         @functools.wraps(fn)
         def timed(*args, **kwargs):
-            if _active is None:
+            if _active is None and not _sync_each:
                 return fn(*args, **kwargs)
-            with _active.span(name):
+            with span(name):
                 return fn(*args, **kwargs)
         return timed
     return deco

@@ -15,7 +15,7 @@ import math
 
 import torch
 
-from ..kernels import ops
+from ..kernels import kv_layout, ops
 from .base import (BuildEnv, KVNeed, LayerCache, Mixer, PartSpec, PieceRows, StepContext, TensorSpec,
                    build_part, param, register_part)
 from .linear import Linear
@@ -50,7 +50,9 @@ class Attention(Mixer):
         return [self.position]
 
     def kv_need(self):
-        return KVNeed(self.KVH, self.hd, self.window)
+        # pages in the order the attention kernels read their operands
+        return KVNeed(self.KVH, self.hd, self.window, k_page_elems=kv_layout.k_page_elems(self.hd),
+                      v_page_elems=kv_layout.v_page_elems(self.hd))
 
     def tensor_specs(self):
         p, hd = self.prefix, self.hd

@@ -32,7 +32,8 @@ class PartSpec:
 class TensorSpec:
     """A weight tensor a part expects: shape, and how the random mode fills it.
 
-    init: ("normal", std) | ("gain", mean, std) | ("zeros",)
+    init: ("normal", std) | ("gain", mean, std) | ("zeros",) | ("constant", value), or any kind
+    registered with weights.random_init.register_init
     integer: integer tables are kept as int32, everything else follows the run dtype rule.
     """
 
@@ -74,20 +75,40 @@ class ModelSpec:
     unused_tensors: frozenset = frozenset()
 
 
+PAGE_TOKENS = 64     # tokens of a cache page
+
+
 @dataclasses.dataclass(frozen=True)
 class KVNeed:
     """What a mixer keeps per token in the cache: per kv head a key of `head_dim` and a value
     of `value_dim` elements (0: as wide as the key), all of them (window 0) or only the last
-    `window`. Mixers with equal needs share a group of the cache."""
+    `window`. Mixers with equal needs share a group of the cache.
+
+    k_page_elems, v_page_elems: the elements of one page (64 tokens of one kv head) in the
+    group's two pools. The order inside a page is the mixer's own business: the cache hands out
+    pages of these sizes and never looks inside. 0: 64 x head_dim and 64 x value_dim, token by
+    token. A mixer with kernels that want their operands padded or tiled (the attention part:
+    kernels/kv_layout.py), or that keeps something else per token (a latent, a code), says so
+    here."""
 
     kv_heads: int
     head_dim: int
     window: int = 0
     value_dim: int = 0
+    k_page_elems: int = 0
+    v_page_elems: int = 0
 
     @property
     def v_dim(self) -> int:
         return self.value_dim or self.head_dim
+
+    @property
+    def k_elems(self) -> int:
+        return self.k_page_elems or PAGE_TOKENS * self.head_dim
+
+    @property
+    def v_elems(self) -> int:
+        return self.v_page_elems or PAGE_TOKENS * self.v_dim
 
 
 @dataclasses.dataclass
@@ -142,7 +163,7 @@ class StepContext:
 class LayerCache:
     """The cache as one run of a layer sees it."""
 
-    kpool: torch.Tensor | None        # [pages, kv_heads, elements of a page] in the kernels' operand order (cache/layout.py)
+    kpool: torch.Tensor | None        # [pages, kv_heads, elements of a page (KVNeed.k_elems)], the order inside a page the mixer's own
     vpool: torch.Tensor | None
     page_table: torch.Tensor | None   # int32 [slots, blocks] of the layer's group
     writes: bool                      # False: the keys/values are another run's

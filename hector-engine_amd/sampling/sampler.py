@@ -95,6 +95,11 @@ class PendingIds:
 
 
 READS_IN_FLIGHT = 64
+# The kernel that keeps the penalty window on the device counts the distinct ids of a window by
+# comparing its entries with one another in LDS: quadratic in the window. Up to this many
+# entries that costs less than the trip to the host it saves; longer windows (the kernel takes
+# up to ops.PENALTY_WINDOW_MAX) are counted on the host, step by step, which is linear.
+WINDOW_ON_DEVICE_MAX = 1024
 
 
 class Sampler:
@@ -137,7 +142,8 @@ class Sampler:
     @property
     def window_on_device(self) -> bool:
         """Whether the penalties of these options can run from a window kept on the device."""
-        return self.config.has_penalties and 1 <= self.config.penalty_window <= ops.PENALTY_WINDOW_MAX
+        return self.config.has_penalties \
+            and 1 <= self.config.penalty_window <= min(WINDOW_ON_DEVICE_MAX, ops.PENALTY_WINDOW_MAX)
 
     def window_device(self, contexts: list[list[int]]):
         """The penalty windows of these rows on the device, for a run of steps whose tokens stay

@@ -94,6 +94,35 @@ def integer_values(key: int, n: int, high: int) -> np.ndarray:
     return (((w >> np.uint64(32)) * np.uint64(high)) >> np.uint64(32)).astype(np.int32)
 
 
+# How a TensorSpec's `init` becomes values: kind -> rule(init) -> (mean, std) of the normal
+# values the tensor is filled with (std 0: the constant `mean`). A part with another kind of
+# initial values registers its rule; nothing else changes.
+_init_rules: dict = {}
+
+
+def register_init(kind: str, rule=None):
+    """Registers rule(init: tuple) -> (mean, std) for TensorSpec.init tuples that start with
+    `kind`; usable as a decorator."""
+    def deco(f):
+        _init_rules[kind] = f
+        return f
+    return deco(rule) if rule is not None else deco
+
+
+register_init("normal", lambda init: (0.0, float(init[1])))
+register_init("gain", lambda init: (float(init[1]), float(init[2])))
+register_init("zeros", lambda init: (0.0, 0.0))
+register_init("constant", lambda init: (float(init[1]), 0.0))
+
+
+def init_moments(name: str, init: tuple) -> tuple[float, float]:
+    try:
+        rule = _init_rules[init[0]]
+    except (KeyError, IndexError):
+        raise ValueError(f"tensor '{name}': unknown init {init}; registered kinds: {sorted(_init_rules)}") from None
+    return rule(init)
+
+
 def random_tensor(name: str, spec: TensorSpec, seed: int, dtype: torch.dtype, device) -> torch.Tensor:
     device = torch.device(device)
     key = tensor_key(seed, name)
@@ -109,15 +138,9 @@ def random_tensor(name: str, spec: TensorSpec, seed: int, dtype: torch.dtype, de
             ops.fill_random_integers(out, key, high)
             return out
         return torch.from_numpy(integer_values(key, n, high)).reshape(shape)
-    kind = spec.init[0]
-    if kind == "zeros":
-        return torch.zeros(shape, dtype=dtype, device=device)
-    if kind == "normal":
-        mean, std = 0.0, spec.init[1]
-    elif kind == "gain":
-        mean, std = spec.init[1], spec.init[2]
-    else:
-        raise ValueError(f"tensor '{name}': unknown init {spec.init}")
+    mean, std = init_moments(name, spec.init)
+    if std == 0.0:
+        return torch.full(shape, mean, dtype=dtype, device=device)
     if on_gpu:
         out = torch.empty(shape, dtype=dtype, device=device)
         ops.fill_random(out, key, _quantiles_device(device), mean, std)

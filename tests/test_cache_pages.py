@@ -118,3 +118,84 @@ def test_random_traffic_keeps_every_invariant():
     for s in list(live):
         b.release(s)
     assert all(g.pool.available == 40 for g in b.groups) and b.slots.available == 6
+
+
+def test_truncate_gives_back_whole_pages_beyond_the_new_length():
+    b = book(pages=16, windows=(0, 0))
+    s = b.acquire()
+    b.reserve(s, 300)
+    b.commit(s, 300)
+    assert b.groups[0].pool.available == 16 - 5
+    cleared = b.truncate(s, 130)                      # 130 tokens lie in 3 pages
+    assert sorted(cleared) == [(0, s, 3), (0, s, 4), (1, s, 3), (1, s, 4)]
+    assert b.length[s] == 130 and b.groups[0].pool.available == 16 - 3
+    b.check_invariants()
+    assert b.truncate(s, 129) == [] and b.length[s] == 129      # same pages, shorter
+    b.reserve(s, 200)                                 # grows again into pages handed out anew
+    b.commit(s, 200)
+    b.check_invariants()
+    b.truncate(s, 0)
+    assert b.groups[0].table[s] == [] and b.groups[0].pool.available == 16
+    with pytest.raises(CacheError, match="truncate"):
+        b.truncate(s, 1)                              # longer than the slot
+    with pytest.raises(CacheError):
+        b.truncate(3, 0)                              # never acquired
+    b.release(s)
+    b.check_invariants()
+
+
+def test_truncate_of_a_windowed_group_needs_the_window_it_gave_back():
+    b = book(pages=32, max_blocks=16, windows=(0, 70))
+    s = b.acquire()
+    b.reserve(s, 400)
+    b.commit(s, 400)               # positions <= 330 left the window: blocks 0..4 were given back
+    assert [p < 0 for p in b.groups[1].table[s]] == [True] * 5 + [False] * 2
+    b.truncate(s, 390)             # a query at 390 reads keys > 320: block 5 (320..383) is still there
+    assert b.length[s] == 390
+    before = (list(b.groups[0].table[s]), list(b.groups[1].table[s]), b.groups[1].pool.available)
+    with pytest.raises(CacheError, match="window"):
+        b.truncate(s, 380)         # a query at 380 reads keys > 310: block 4 (256..319) is gone
+    assert before == (list(b.groups[0].table[s]), list(b.groups[1].table[s]), b.groups[1].pool.available)
+    assert b.length[s] == 390      # nothing was changed
+    b.check_invariants()
+
+
+def test_random_traffic_with_truncation_keeps_every_invariant():
+    rng = random.Random(1)
+    b = book(pages=40, slots=5, max_blocks=12, windows=(0, 100))
+    live = {}
+    for _ in range(3000):
+        op = rng.random()
+        if op < 0.2 and len(live) < 5:
+            live[b.acquire()] = 0
+        elif op < 0.3 and live:
+            s = rng.choice(list(live))
+            b.release(s)
+            del live[s]
+        elif op < 0.5 and live:
+            s = rng.choice(list(live))
+            new = rng.randint(0, live[s])
+            try:
+                b.truncate(s, new)
+                live[s] = new
+            except CacheError:
+                pass                                   # the window's pages were gone: nothing changed
+        elif live:
+            s = rng.choice(list(live))
+            new = live[s] + rng.choice([1, 1, 5, 64, 100])
+            try:
+                b.reserve(s, new)
+                b.commit(s, new)
+                live[s] = new
+            except CacheFull:
+                pass
+        b.check_invariants()
+        assert all(b.length[s] == n for s, n in live.items())
+        for s, n in live.items():                      # every position a next query reads has a page
+            for g in b.groups:
+                first = max(0, n - g.window + 1) if g.window else 0
+                assert len(g.table[s]) == blocks_for(n)
+                assert all(g.table[s][blk] >= 0 for blk in range(first // 64, blocks_for(n)))
+    for s in list(live):
+        b.release(s)
+    assert all(g.pool.available == 40 for g in b.groups)

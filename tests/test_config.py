@@ -82,3 +82,28 @@ def test_round_trip_through_a_folder(tmp_path):
 def test_int_and_bool_coercion():
     c = config_from_dict(dict(TINY_A, rope_theta=10000, tie_word_embeddings=1, eos_token_id=3))
     assert c.rope_theta == 10000.0 and c.tie_word_embeddings is True and c.eos_token_id == [3]
+
+
+def test_stop_ids_come_from_generation_config_then_config(tmp_path):
+    """An instruction-tuned folder lists its end-of-turn id in generation_config.json beside the
+    end-of-text id of config.json: both end a sequence. Without that file, or without the key
+    in it, config.json's id counts; with neither, nothing ends a sequence by itself."""
+    from hector_engine_amd.config.base import ConfigError, stop_token_ids
+    cfg = config_from_dict(dict(TINY_A, eos_token_id=151643 % 256))
+    folder = tmp_path / "m"
+    folder.mkdir()
+    assert stop_token_ids(str(folder), cfg) == [151643 % 256]
+    assert stop_token_ids(None, cfg) == [151643 % 256]
+    (folder / "generation_config.json").write_text(json.dumps({"eos_token_id": [7, 9], "temperature": 0.7}))
+    assert stop_token_ids(str(folder), cfg) == [7, 9]
+    (folder / "generation_config.json").write_text(json.dumps({"eos_token_id": 11}))
+    assert stop_token_ids(str(folder), cfg) == [11]
+    (folder / "generation_config.json").write_text(json.dumps({"temperature": 0.7}))
+    assert stop_token_ids(str(folder), cfg) == [151643 % 256]
+    assert stop_token_ids(str(folder), config_from_dict(dict(TINY_A))) == []
+    (folder / "generation_config.json").write_text("{not json")
+    with pytest.raises(ConfigError, match="generation_config.json"):
+        stop_token_ids(str(folder), cfg)
+    (folder / "generation_config.json").write_text(json.dumps({"eos_token_id": "x"}))
+    with pytest.raises(ConfigError, match="eos_token_id"):
+        stop_token_ids(str(folder), cfg)

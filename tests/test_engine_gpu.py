@@ -449,9 +449,11 @@ def test_a_step_of_thousands_of_rows(model_dirs, plain_models, dtype):
 
 
 def test_a_failed_capture_falls_back_to_eager_steps(model_dirs, plain_models, monkeypatch):
-    """When capturing the one-token step fails, the engine says so once and goes on without
-    graphs (the reference does the same: src/engine.cpp:233-261). The failure is made on the host:
-    torch's capture context is replaced by one that raises."""
+    """When capturing the one-token step of a batch size fails, the engine says so once, records why,
+    and runs steps of that size without a graph (the reference falls back the same way:
+    src/engine.cpp:233-261). The failure is made on the host: torch's capture context is replaced by
+    one that raises. An error that is the step's own is not swallowed: it comes back from the eager
+    run of the same step and reaches the caller."""
     import contextlib
     import warnings
     import hector_engine_amd as he
@@ -479,12 +481,29 @@ def test_a_failed_capture_falls_back_to_eager_steps(model_dirs, plain_models, mo
     assert eng.stats["graph_captures"] == 0 and eng.stats["graph_replays"] == 0
     assert eng.stats["eager_steps"] == 21
     close(torch.cat(rows), want[10:], "bfloat16")
-    # another bucket size after the failure: eager at once, no second attempt
+    assert eng.stats["graph_capture_failures"] == 1 and "made up by the test" in eng.capture_failures[0]
+    # the fallback is the bucket's own: another batch size tries its own capture
+    monkeypatch.undo()
     a, b = eng.acquire(), eng.acquire()
-    for t in ids[:3]:
-        eng.step([entry(a, [t], [0]), entry(b, [t], [0])])
-    assert eng.stats["graph_captures"] == 0
-    eng.release(a), eng.release(b)
+    pair = [eng.step([entry(a, [t], [0]), entry(b, [t], [0])]).clone() for t in ids[:4]]
+    assert eng.stats["graph_captures"] == 1 and eng.stats["graph_replays"] >= 2
+    close(torch.cat([r[:1] for r in pair]), want[:4], "bfloat16")
+    # an error of the step itself (here: of the model's forward) during the capture is raised
+    forward, calls = eng.model.forward, []
+
+    def failing(*args, **kw):
+        calls.append(1)
+        if len(calls) > 1:
+            raise ValueError("a part's own bug (made up by the test)")
+        return forward(*args, **kw)
+    monkeypatch.setattr(eng.model, "forward", failing)
+    c = eng.acquire()
+    three = [entry(x, [ids[0]], [0]) for x in (a, b, c)]
+    eng.step(three)                                   # the bucket of four rows: first use, eager
+    with pytest.raises(ValueError, match="own bug"):
+        eng.step([entry(x, [ids[1]], [0]) for x in (a, b, c)])
+    for x in (a, b, c):
+        eng.release(x)
 
 
 def test_profile_mode_times_every_kernel(model_dirs):
@@ -506,3 +525,111 @@ def test_profile_mode_times_every_kernel(model_dirs):
     text = eng.profile_summary()
     assert text.startswith("=== Engine Profile ===") and "TOTAL" in text and "Avg(ms)" in text
     assert eng.stats["graph_replays"] == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_a_request_joins_three_that_decode(engines, plain_models, name, dtype):
+    """Three sequences decode through the replayed graph; in one step a fourth joins with a prompt
+    of 37 tokens while the three bring one token each; then all four decode. Every logit of every
+    request against the plain implementation."""
+    eng = engines(name, dtype)
+    vocab = plain_models[name][0]["vocab_size"]
+    requests = [rand_ids(vocab, n, 700 + i) for i, n in enumerate((29, 42, 79, 41))]
+    prompt = [20, 33, 70]
+    slots = [eng.acquire() for _ in range(3)]
+    out = [[] for _ in requests]
+    replays = eng.stats["graph_replays"]
+    logits = eng.step([entry(s, r[:n], range(n)) for s, r, n in zip(slots, requests, prompt)])
+    for i, part in enumerate(logits.split(prompt)):
+        out[i].append(part.clone())
+    fed = list(prompt) + [0]
+    for _ in range(4):                                   # eager, captured, replayed, replayed
+        logits = eng.step([entry(s, [requests[i][fed[i]]], [0]) for i, s in enumerate(slots)])
+        for i in range(3):
+            out[i].append(logits[i:i + 1].clone())
+            fed[i] += 1
+    assert eng.stats["graph_replays"] >= replays + 2
+    # the mixed step: one token each of the three, the fourth's whole prompt
+    slots.append(eng.acquire())
+    logits = eng.step([entry(slots[i], [requests[i][fed[i]]], [0]) for i in range(3)]
+                      + [entry(slots[3], requests[3][:37], range(37))])
+    for i in range(3):
+        out[i].append(logits[i:i + 1].clone())
+        fed[i] += 1
+    out[3].append(logits[3:].clone())
+    fed[3] = 37
+    for _ in range(4):
+        logits = eng.step([entry(s, [requests[i][fed[i]]], [0]) for i, s in enumerate(slots)])
+        for i in range(4):
+            out[i].append(logits[i:i + 1].clone())
+            fed[i] += 1
+    assert fed == [len(r) for r in requests]
+    for s in slots:
+        eng.release(s)
+    for i, ids in enumerate(requests):
+        close(torch.cat(out[i]), plain_logits(plain_models, name, ids), dtype)
+    if dtype == "float32":
+        s = eng.acquire()
+        alone = eng.step([entry(s, requests[3], range(41))]).clone()
+        eng.release(s)
+        assert torch.equal(alone, torch.cat(out[3]))    # joining a running batch changed no bit
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_truncate_then_refeed_equals_a_fresh_run(engines, plain_models, name, dtype):
+    """A turn that is taken back: 150 tokens are fed, the slot is cut back, other tokens follow.
+    The logits are those of a sequence that never held the dropped tokens (bit for bit in 32-bit),
+    the pages beyond the cut are free again, and a cut that a windowed layer can no longer serve
+    (its older pages are gone) is refused and changes nothing."""
+    from hector_engine_amd.cache import CacheError
+    eng = engines(name, dtype)
+    cfg = plain_models[name][0]
+    vocab = cfg["vocab_size"]
+    first, other = rand_ids(vocab, 150, 31), rand_ids(vocab, 40, 32)
+    free = eng.cache.free_pages
+    s = eng.acquire()
+    eng.step([entry(s, first, [])])
+    keep = 70
+    if cfg.get("use_sliding_window"):
+        # the windowed layers (8, 70 or 40 keys) have given back their first page or two: a query at
+        # position 70 would read keys that are gone, one at 141 reads only what is still held
+        with pytest.raises(CacheError, match="window"):
+            eng.truncate(s, keep)
+        assert eng.length(s) == 150 and eng.cache.free_pages == free - 3
+        keep = 141
+    eng.truncate(s, keep)
+    assert eng.length(s) == keep and eng.cache.free_pages == free - (keep + 63) // 64
+    cut = eng.step([entry(s, other, range(40))]).clone()
+    eng.release(s)
+    s = eng.acquire()
+    eng.step([entry(s, first[:keep], [])])
+    fresh = eng.step([entry(s, other, range(40))]).clone()
+    eng.release(s)
+    want = plain_logits(plain_models, name, first[:keep] + other)[keep:]
+    close(cut, want, dtype)
+    if dtype == "float32":
+        assert torch.equal(cut, fresh)
+    with pytest.raises(CacheError):
+        eng.truncate(s, 0)                                # the slot is no longer held
+    assert eng.cache.free_pages == free
+    eng.cache.book.check_invariants()
+
+
+def test_sync_each_launch_mode_gives_the_same_logits(model_dirs, plain_models):
+    """The debugging mode (a wait after every launch, no graphs) changes no bit of the 32-bit path."""
+    import hector_engine_amd as he
+    ids = rand_ids(200, 40, 77)
+    outs = []
+    for mode in (False, True):
+        eng = he.Engine(model_dirs["D"], dtype="float32", max_tokens=1024, max_slots=2, sync_each_launch=mode)
+        s = eng.acquire()
+        rows = [eng.step([entry(s, ids[:30], range(30))]).clone()]
+        rows += [eng.step([entry(s, [t], [0])]).clone() for t in ids[30:]]
+        outs.append(torch.cat(rows))
+        assert eng.use_graphs is not mode
+        if mode:
+            assert eng.stats["graph_replays"] == 0
+    assert torch.equal(outs[0], outs[1])
+    close(outs[1], plain_logits(plain_models, "D", ids), "float32")

@@ -271,3 +271,34 @@ def test_smoke_entry():
     sys.path.insert(0, ROOT)
     import __graft_entry__
     __graft_entry__.smoke()
+
+
+def test_default_stop_ids_are_the_model_folders_own(he, model_dirs, plain_models, tmp_path):
+    """Without stop ids from the caller a sequence ends at the ids the model folder names: those of
+    its generation_config.json (here: a list of two, as instruction-tuned checkpoints have), else
+    those of its config.json; stop_ids=() switches them off."""
+    import json
+    import shutil
+    cfg, w = plain_models["A"]
+    prompts = prompts_for(cfg, [5, 9], 900)
+    free = [P.generate(cfg, w, p, 10) for p in prompts]
+    stop = [free[0][3], free[1][6]]
+    want = [P.generate(cfg, w, p, 10, stop_ids=set(stop)) for p in prompts]
+    assert len(want[0]) <= 3 and len(want[1]) <= 6
+    folder = str(tmp_path / "with_generation_config")
+    shutil.copytree(model_dirs["A"], folder)
+    with open(os.path.join(folder, "generation_config.json"), "w") as f:
+        json.dump({"eos_token_id": stop, "do_sample": True}, f)
+    eng = he.Engine(folder, dtype="float32", max_tokens=1024, max_seq_len=128)
+    assert eng.stop_ids == stop
+    got = he.generate(eng, prompts, max_new_tokens=10)
+    assert [r.tokens for r in got] == want and got[0].finish_reason == "eos"
+    assert [r.tokens for r in he.generate(eng, prompts, max_new_tokens=10, stop_ids=())] == free
+    # config.json's id counts when generation_config.json is absent
+    os.remove(os.path.join(folder, "generation_config.json"))
+    data = json.load(open(os.path.join(folder, "config.json")))
+    data["eos_token_id"] = stop[0]
+    json.dump(data, open(os.path.join(folder, "config.json"), "w"))
+    eng = he.Engine(folder, dtype="float32", max_tokens=1024, max_seq_len=128)
+    assert eng.stop_ids == [stop[0]]
+    assert he.generate(eng, prompts[:1], max_new_tokens=10)[0].tokens == want[0]

@@ -238,6 +238,41 @@ def test_float32_equals_plain_at_seven_b_layer_sizes(folder):
     assert torch.equal(got16.argmax(-1)[clear], want.argmax(-1)[clear])
 
 
+@pytest.mark.skipif(TUNED, reason="the comparison with the plain implementation runs once")
+def test_unequal_batch_equals_plain_at_seven_b_layer_sizes(folder):
+    """Three requests of unequal lengths in one batch, their prompts in one step, then one token
+    each, the shortest ending first: every position of every request against the plain
+    implementation (on vocabulary columns), in true 32-bit and in bfloat16, and once more from the
+    slots the first batch gave back."""
+    import hector_engine_amd as he
+    reqs = [rand_ids(152064, n, 900 + n) for n in (41, 23, 60)]
+    first = [30, 19, 33]                    # the second request has 4 tokens left, the first 11, the third 27
+    cols = sorted(set(range(5, 152064, 97)) | set(range(152064 - 40, 152064)))
+    want = [plain_logits_on_columns(folder, ids, cols) for ids in reqs]
+    for dtype in ("float32", "bfloat16"):
+        eng = he.Engine(folder, dtype=dtype, max_tokens=1024, max_slots=3, max_seq_len=256)
+        for batch in range(2):
+            got = run(eng, reqs, first)
+            assert eng.cache.free_pages == eng.cache.num_pages
+            for g, w in zip(got, want):
+                g = g[:, cols].cpu().double()
+                scale = w.abs().max().item()
+                d = g - w
+                if dtype == "float32":
+                    assert d.abs().max().item() <= 2e-5 * (18944 / 160) ** 0.5 * scale
+                    assert torch.equal(g.argmax(-1), w.argmax(-1))
+                else:
+                    assert d.abs().max().item() < 0.03 * scale
+                    assert (d ** 2).mean().sqrt().item() < 0.005 * scale
+                    t2 = w.topk(2, -1).values
+                    clear = (t2[:, 0] - t2[:, 1]) > 0.03 * scale
+                    assert torch.equal(g.argmax(-1)[clear], w.argmax(-1)[clear])
+        if dtype == "bfloat16":
+            assert eng.stats["graph_replays"] > 0
+        del eng
+        torch.cuda.empty_cache()
+
+
 @pytest.mark.skipif(TUNED, reason="this is the run it starts")
 def test_the_same_with_the_library_tuner_on():
     """The benchmark runs with the library's tuner choosing the kernel of every product above 16

@@ -132,7 +132,10 @@ def test_attention_part_prompt_then_tokens(fw, dtype, fast, window):
     D, H, KVH, hd = 80, 6, 3, 32
     env = env_for(fw, dtype, fast)
     att = fw.parts.build_part("mixer", attention_spec(fw, D, H, KVH, hd, window), "a.", env)
-    assert att.kv_need() == fw.parts.KVNeed(KVH, hd, window) and att.state_bytes() == 0
+    need = att.kv_need()
+    assert (need.kv_heads, need.head_dim, need.window, need.v_dim) == (KVH, hd, window, hd) and att.state_bytes() == 0
+    # its pages are as large as its kernels keep them: keys in steps of 32 dims, values in tiles of 16
+    assert (need.k_elems, need.v_elems) == (64 * 32 * ((hd + 31) // 32), 64 * 16 * ((hd + 15) // 16))
     w = attention_weights(att.tensor_specs(), dtype)
     att.bind({k: v.cuda() for k, v in w.items()})
     cache = fw.PagedCache([fw.RunPlan(att.kv_need(), None)], max_tokens=1024, max_slots=4, max_seq_len=512,
@@ -272,6 +275,10 @@ def toys(fw):
     from hector_engine_amd.config.base import ModelConfig, architecture_name, read_field
     parts = fw.parts
 
+    # initial values of a kind of the toys' own: a rule registered from here gives a TensorSpec's
+    # ("toy_near", centre) its mean and spread in the random-weights mode
+    he.register_init("toy_near", lambda init: (float(init[1]), 0.05))
+
     @parts.register_part("mixer", "toy_running_mean")
     class RunningMean(parts.Mixer):
         """out_t = Wo . mean_{j<=t} x_j. Its state, the running sum and the count, lives in the
@@ -350,8 +357,10 @@ def toys(fw):
 
     @parts.register_part("mixer", "toy_wide_values")
     class WideValues(parts.Mixer):
-        """One head whose keys are 16 wide and whose values are 32 wide, kept in cache pages of
-        its own group: it writes and reads them by index, in the layout the cache documents."""
+        """One head whose keys are 16 wide (kept with 4 more elements a token: a code of its own)
+        and whose values are 32 wide, in cache pages of its own group and of its own sizes: 64 x 20
+        and 64 x 32 elements, token by token. The cache hands out pages of the sizes the mixer
+        names and never looks inside them."""
         graph_safe = False
 
         def __init__(self, params, prefix, env):
@@ -359,7 +368,7 @@ def toys(fw):
             self.D = parts.param(params, "hidden_size", int)
 
         def kv_need(self):
-            return parts.KVNeed(1, 16, 0, value_dim=32)
+            return parts.KVNeed(1, 16, 0, value_dim=32, k_page_elems=64 * 20)     # v: the default, 64 x value_dim
 
         def tensor_specs(self):
             p = self.prefix
@@ -370,9 +379,10 @@ def toys(fw):
             self.t = {n: tensors[self.prefix + n + ".weight"].float() for n in "qkvo"}
 
         def forward(self, x, ctx, cache):
-            from tests.test_kernels_gpu import page_maps
-            km, vm = page_maps(16)[0].cuda(), page_maps(32)[1].cuda()
-            assert cache.kpool.shape[-1] == 64 * 32 and cache.vpool.shape[-1] == 64 * 32   # 16 -> one k step; 2 dim tiles
+            assert cache.kpool.shape[-1] == 64 * 20 and cache.vpool.shape[-1] == 64 * 32   # the sizes it asked for
+            ar = torch.arange(64, device=x.device)[:, None]
+            km = ar * 20 + torch.arange(16, device=x.device)[None, :]       # token t: elements 20 t .. 20 t + 15, then its code
+            vm = ar * 32 + torch.arange(32, device=x.device)[None, :]
             xf = x[:ctx.rows].float()
             q, k, v = xf @ self.t["q"].T, xf @ self.t["k"].T, xf @ self.t["v"].T
             out = ctx.alloc((ctx.rows, self.D))
@@ -382,12 +392,15 @@ def toys(fw):
                 for j in range(n):
                     p = start + j
                     cache.kpool[table[p // 64], 0, km[p % 64]] = k[r + j].to(cache.kpool.dtype)
+                    cache.kpool[table[p // 64], 0, 20 * (p % 64) + 16:20 * (p % 64) + 20] = float(p % 7)   # the code
                     cache.vpool[table[p // 64], 0, vm[p % 64]] = v[r + j].to(cache.vpool.dtype)
                 total = start + n
                 pos = torch.arange(total, device=x.device)
                 pages = table[pos // 64].long()
                 keys = cache.kpool[pages, 0][torch.arange(total, device=x.device)[:, None], km[pos % 64]].float()
                 vals = cache.vpool[pages, 0][torch.arange(total, device=x.device)[:, None], vm[pos % 64]].float()
+                codes = cache.kpool[pages, 0][torch.arange(total, device=x.device), 20 * (pos % 64) + 16].float()
+                assert torch.equal(codes, (pos % 7).float())      # what it wrote beside the keys is still there
                 scores = q[r:r + n] @ keys.T / 4.0
                 seen = pos[None, :] <= (start + torch.arange(n, device=x.device))[:, None]
                 w = torch.softmax(scores.masked_fill(~seen, float("-inf")), -1)
@@ -457,10 +470,11 @@ def toys(fw):
             self.eps = parts.param(params, "eps", float)
 
         def tensor_specs(self):
-            return {self.prefix + "weight": parts.TensorSpec((self.size,), ("gain", 1.0, 0.1))}
+            return {self.prefix + "weight": parts.TensorSpec((self.size,), ("toy_near", 0.9))}
 
         def bind(self, tensors):
             self.w = tensors[self.prefix + "weight"].float()
+            assert 0.6 < self.w.mean().item() < 1.2 and self.w.std().item() > 0     # the registered rule made them
 
         def add_norm(self, resid, delta, rows, ctx, want_out=True):
             r = resid[:rows]

@@ -173,3 +173,22 @@ def test_expected_names_are_the_hf_names():
             assert f"model.layers.{l}.{n}" in names
     assert not any("o_proj.bias" in n for n in names)
     assert len(names) == 3 * 12 + 3
+
+
+def test_init_rules_are_a_registry():
+    """The random mode fills a tensor by the rule registered for the kind its TensorSpec names: the
+    built-in kinds, a rule registered from outside, and an unknown kind as an error that lists them."""
+    from hector_engine_amd.parts.base import TensorSpec
+    from hector_engine_amd.weights import register_init
+    from hector_engine_amd.weights.random_init import random_tensor
+    z = random_tensor("t", TensorSpec((3, 5), ("zeros",)), 0, torch.float32, CPU)
+    c = random_tensor("t", TensorSpec((3, 5), ("constant", 0.5)), 0, torch.bfloat16, CPU)
+    assert torch.equal(z, torch.zeros(3, 5)) and torch.equal(c, torch.full((3, 5), 0.5, dtype=torch.bfloat16))
+    with pytest.raises(ValueError, match="unknown init.*registered kinds.*normal"):
+        random_tensor("t", TensorSpec((4,), ("test_wide", 3.0)), 0, torch.float32, CPU)
+    register_init("test_wide", lambda init: (float(init[1]), 2.0))
+    w = random_tensor("t", TensorSpec((4000,), ("test_wide", 3.0)), 0, torch.float32, CPU)
+    assert abs(w.mean().item() - 3.0) < 0.15 and abs(w.std().item() - 2.0) < 0.15
+    g = random_tensor("t", TensorSpec((4000,), ("gain", 1.0, 0.1)), 0, torch.float32, CPU)
+    n = random_tensor("t", TensorSpec((4000,), ("normal", 0.1)), 0, torch.float32, CPU)
+    assert torch.allclose(g, 1.0 + n, atol=0.01)          # the same draws, another mean (bfloat16 values)
