@@ -9,6 +9,14 @@ The default is the 7B shape; --shape runs the same measurement at the layer size
 Qwen2.5-32B (context 8192, prompts of 512 to 2048 tokens, batches 1 / 8 / 64) or
 Qwen2-72B (context 4096, prompts of 2048 tokens, batches 1 / 8 / 32).
 
+Beside the points at batch 1 and at the large batch the default run adds three more (--no-extra
+leaves them out), each with its share of the HBM peak in `points_roofline_frac`:
+  decode_b64_t7800   the large batch behind prompts of 7,800 tokens (30 GB of keys and values a step:
+                     the one-token attention is then the kernel most of the time goes to)
+  decode_b8_32b      batch 8 at the Qwen2.5-32B layer sizes (all 64 layers), prompts of 512 to 2,048 tokens
+  decode_b1_fp32     batch 1 of the 7B shape in true 32-bit (28.3 GB of weights a step), and with it
+                     `prefill_fp32`, the 2,048-token prompt in 32-bit against the fp32 peak
+
 A step is one decode step of the whole batch: the engine's step function (HIP
 graph replay) plus greedy sampling. As in the library's generation loop, 8 steps are
 queued at a time: the chosen ids go into the next step on the device, and the host
@@ -47,17 +55,19 @@ PROMPT = 2048
 RUN = 8          # one-token steps queued at a time
 HBM_PEAK_GBS = 8000.0
 BF16_PEAK_FLOPS = 2.5e15
+FP32_PEAK_FLOPS = 157.3e12
+LONG_PROMPT = 7800   # the long-context point: prompts of so many tokens in the shape's context
 
 
-def weight_bytes(c, layers):
+def weight_bytes(c, layers, itemsize=2):
     D, H, KVH, hd, I, V = (c["hidden_size"], c["num_attention_heads"], c["num_key_value_heads"],
                            c["head_dim"], c["intermediate_size"], c["vocab_size"])
     per_layer = D * (H + 2 * KVH) * hd + (H + 2 * KVH) * hd + H * hd * D + 3 * D * I + 2 * D
-    return 2 * (layers * per_layer + D + V * D)      # lm_head read once; embedding rows are negligible
+    return itemsize * (layers * per_layer + D + V * D)      # lm_head read once; embedding rows are negligible
 
 
-def kv_bytes_per_token(c, layers):
-    return 2 * layers * c["num_key_value_heads"] * c["head_dim"] * 2
+def kv_bytes_per_token(c, layers, itemsize=2):
+    return 2 * layers * c["num_key_value_heads"] * c["head_dim"] * itemsize
 
 
 def prefill_flops(c, layers, T):
@@ -81,6 +91,8 @@ def main() -> int:
     ap.add_argument("--prompt", type=int, default=0,
                     help="another prompt length of the decode batches (the prefill figure stays at 2048 tokens)")
     ap.add_argument("--no-points", action="store_true", help="skip the points at batch 1 and at the large batch")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="skip the long-context point, the Qwen2.5-32B point and the 32-bit point")
     ap.add_argument("--continuation", default="", metavar="AFTER:NEW",
                     help="also time a step of NEW tokens of a sequence that holds AFTER tokens already "
                          "(a new turn of a conversation); reported as \"continuation\"")
@@ -126,112 +138,143 @@ def main() -> int:
     def progress(what):
         print(f"[bench {time.perf_counter() - t_start:6.1f}s] {what}", file=sys.stderr, flush=True)
 
-    progress(f"{MODEL}: random weights, {args.layers} layers")
-    cfg_dict = dict(SHAPE, num_hidden_layers=args.layers, architectures=["Qwen2ForCausalLM"])
-    config = Qwen2Config.from_dict(cfg_dict)
-    max_batch = 2 * args.batch if args.no_points else max(2 * args.batch, BIG_BATCH)
-    t_load = time.perf_counter()
-    engine = he.Engine(config=config, seed=0, dtype="bfloat16", max_tokens=max_batch * CONTEXT,
-                       max_slots=max_batch, max_seq_len=CONTEXT, tune_library=not args.no_tune)
-    sampler = he.Sampler(he.SamplingConfig.deterministic(), engine.device)
-    torch.cuda.synchronize()
-    load_s = time.perf_counter() - t_load
     rng = np.random.default_rng(0)
 
-    def prompts(n, lo=PROMPT, hi=PROMPT):
-        return [rng.integers(0, SHAPE["vocab_size"], int(rng.integers(lo, hi + 1))).tolist() for _ in range(n)]
+    class Model:
+        """An engine of one shape and precision with what the measurements need of it."""
 
-    def prefill(ps, slots):
-        """Prompts in groups of 8 sequences a step; returns the first sampled tokens."""
-        toks = []
-        # prompts of random lengths give row counts that never come again: not worth the tuner's trials
-        tuning = library_tuning.no_new_tuning() if PROMPT_LO != PROMPT_HI else contextlib.nullcontext()
-        with tuning:
-            for g in range(0, len(ps), 8):
-                entries = [StepEntry(s, p, [len(p) - 1]) for s, p in zip(slots[g:g + 8], ps[g:g + 8])]
-                logits = engine.step(entries)
-                toks += sampler.sample(logits, list(range(len(entries))), [0] * len(entries))
-        return toks
-
-    wbytes = weight_bytes(SHAPE, args.layers)
-    packed = {}
-
-    def decode_run(batch, steps, warmup, repeats):
-        """Prompts, warm-up steps, then `repeats` timed runs of `steps` steps. Returns per run
-        (seconds a step, bytes a step has to read)."""
-        slots = [engine.acquire() for _ in range(batch)]
-        ps = prompts(batch, PROMPT_LO, PROMPT_HI)
-        if batch == args.batch and batch <= 8:      # the packed prompt step of the headline batch, timed
-            warm = [engine.acquire() for _ in range(batch)]     # once untimed: the library's first call of a shape
-            prefill(ps, warm)
-            for s in warm:
-                engine.release(s)
-            torch.cuda.synchronize()
+        def __init__(self, shape, layers, dtype, max_batch, context, tune):
+            self.shape, self.layers, self.context = shape, layers, context
+            self.itemsize = 2 if dtype == "bfloat16" else 4
+            config = Qwen2Config.from_dict(dict(shape, num_hidden_layers=layers, architectures=["Qwen2ForCausalLM"]))
             t0 = time.perf_counter()
-            toks = prefill(ps, slots)
+            self.engine = he.Engine(config=config, seed=0, dtype=dtype, max_tokens=max_batch * context,
+                                    max_slots=max_batch, max_seq_len=context, tune_library=tune)
+            self.sampler = he.Sampler(he.SamplingConfig.deterministic(), self.engine.device)
             torch.cuda.synchronize()
-            packed.update(tokens=sum(len(p) for p in ps), seconds=time.perf_counter() - t0,
-                          flops=sum(prefill_flops(SHAPE, args.layers, len(p)) for p in ps))
-        else:
-            toks = prefill(ps, slots)
-        seqs = list(range(batch))
+            self.load_s = time.perf_counter() - t0
+            self.wbytes = weight_bytes(shape, layers, self.itemsize)
+            self.packed = {}
 
-        def run(toks, count):
-            """`count` steps queued back to back: each step's ids go into the next on the device,
-            the host reads the ids of all of them at the end (as the generation loop does)."""
-            ids, history = None, []
-            for _ in range(count):
-                logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)], device_tokens=ids)
-                ids = sampler.sample_device(logits, seqs, [0] * batch)
-                history.append(ids)
-            return torch.stack(history).tolist()[-1]
+        def prompts(self, n, lo, hi):
+            return [rng.integers(0, self.shape["vocab_size"], int(rng.integers(lo, hi + 1))).tolist() for _ in range(n)]
 
-        def many(toks, count):
-            while count > 0:
-                toks = run(toks, min(RUN, count))
-                count -= RUN
+        def prefill(self, ps, slots, fixed_length):
+            """Prompts in groups of 8 sequences a step; returns the first sampled tokens."""
+            toks = []
+            # prompts of random lengths give row counts that never come again: not worth the tuner's trials
+            tuning = contextlib.nullcontext() if fixed_length else library_tuning.no_new_tuning()
+            with tuning:
+                for g in range(0, len(ps), 8):
+                    entries = [StepEntry(s, p, [len(p) - 1]) for s, p in zip(slots[g:g + 8], ps[g:g + 8])]
+                    logits = self.engine.step(entries)
+                    toks += self.sampler.sample(logits, list(range(len(entries))), [0] * len(entries))
             return toks
 
-        toks = many(toks, warmup)
-        runs = []
-        done = warmup
-        for _ in range(repeats):
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            toks = many(toks, steps)
-            torch.cuda.synchronize()
-            dt = time.perf_counter() - t0
-            avg_len = sum(len(p) for p in ps) / batch + done + steps / 2
-            done += steps
-            runs.append((dt / steps, wbytes + batch * avg_len * kv_bytes_per_token(SHAPE, args.layers)))
-        for s in slots:
-            engine.release(s)
-        return runs
+        def prompt_step(self, tokens):
+            """Seconds of one whole-prompt step of `tokens` tokens: a first run warms the library's
+            products, then the median of three."""
+            p = self.prompts(1, tokens, tokens)[0]
+            times = []
+            for run in range(4):
+                slot = self.engine.acquire()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                self.engine.step([StepEntry(slot, p, [tokens - 1])])
+                torch.cuda.synchronize()
+                if run > 0:
+                    times.append(time.perf_counter() - t0)
+                self.engine.release(slot)
+            return sorted(times)[1]
+
+        def decode_run(self, batch, lo, hi, steps, warmup, repeats, time_prefill=False):
+            """Prompts of lo to hi tokens, warm-up steps, then `repeats` timed runs of `steps` steps.
+            Returns per run (seconds a step, bytes a step has to read)."""
+            engine, sampler = self.engine, self.sampler
+            slots = [engine.acquire() for _ in range(batch)]
+            ps = self.prompts(batch, lo, hi)
+            if time_prefill:      # the packed prompt step of the headline batch, timed
+                warm = [engine.acquire() for _ in range(batch)]     # once untimed: the library's first call of a shape
+                self.prefill(ps, warm, lo == hi)
+                for s in warm:
+                    engine.release(s)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                toks = self.prefill(ps, slots, lo == hi)
+                torch.cuda.synchronize()
+                self.packed.update(tokens=sum(len(p) for p in ps), seconds=time.perf_counter() - t0,
+                                   flops=sum(prefill_flops(self.shape, self.layers, len(p)) for p in ps))
+            else:
+                toks = self.prefill(ps, slots, lo == hi)
+            seqs = list(range(batch))
+
+            def run(toks, count):
+                """`count` steps queued back to back: each step's ids go into the next on the device,
+                the host reads the ids of all of them at the end (as the generation loop does)."""
+                ids, history = None, []
+                for _ in range(count):
+                    logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)], device_tokens=ids)
+                    ids = sampler.sample_device(logits, seqs, [0] * batch)
+                    history.append(ids)
+                return torch.stack(history).tolist()[-1]
+
+            def many(toks, count):
+                while count > 0:
+                    toks = run(toks, min(RUN, count))
+                    count -= RUN
+                return toks
+
+            toks = many(toks, warmup)
+            runs = []
+            done = warmup
+            kv = kv_bytes_per_token(self.shape, self.layers, self.itemsize)
+            for _ in range(repeats):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                toks = many(toks, steps)
+                torch.cuda.synchronize()
+                dt = time.perf_counter() - t0
+                avg_len = sum(len(p) for p in ps) / batch + done + steps / 2
+                done += steps
+                runs.append((dt / steps, self.wbytes + batch * avg_len * kv))
+            for s in slots:
+                engine.release(s)
+            if engine.capture_failures:
+                # a step that fell back from its HIP graph would pass as a (slower) number
+                raise RuntimeError(f"bench.py: one-token steps ran without their graph: {engine.capture_failures}")
+            return runs
+
+        def close(self):
+            del self.engine, self.sampler
+            torch.cuda.empty_cache()
 
     def median_run(runs):
         return sorted(runs)[len(runs) // 2]
 
-    # ---- prefill of one 2,048-token prompt: a first run warms the library GEMMs, then the median of three
+    points, points_frac, points_ms = {}, {}, {}
+
+    def point(name, model, batch, lo, hi, steps, warmup, repeats):
+        progress(name)
+        s, nbytes = median_run(model.decode_run(batch, lo, hi, steps, warmup, repeats))
+        points[name] = round(batch / s, 1)
+        points_ms[name] = round(s * 1e3, 4)
+        points_frac[name] = round(nbytes / s / 1e9 / HBM_PEAK_GBS, 4)
+
+    progress(f"{MODEL}: random weights, {args.layers} layers")
+    max_batch = 2 * args.batch if args.no_points else max(2 * args.batch, BIG_BATCH)
+    model = Model(SHAPE, args.layers, "bfloat16", max_batch, CONTEXT, not args.no_tune)
+    engine, load_s = model.engine, model.load_s
+
+    # ---- prefill of one 2,048-token prompt
     progress(f"weights ready; prefill of {PROMPT} tokens")
-    p = prompts(1)[0]
-    times = []
-    for run in range(4):
-        slot = engine.acquire()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        engine.step([StepEntry(slot, p, [PROMPT - 1])])
-        torch.cuda.synchronize()
-        if run > 0:
-            times.append(time.perf_counter() - t0)
-        engine.release(slot)
-    prefill_s = sorted(times)[1]
+    prefill_s = model.prompt_step(PROMPT)
     flops = prefill_flops(SHAPE, args.layers, PROMPT)
 
     # ---- a step of a few new tokens behind a long sequence: the median of three
     continuation = None
     if cont is not None:
         progress(f"{cont[1]} tokens after {cont[0]}")
-        before, fresh = prompts(1, cont[0], cont[0])[0], prompts(1, cont[1], cont[1])[0]
+        before, fresh = model.prompts(1, cont[0], cont[0])[0], model.prompts(1, cont[1], cont[1])[0]
         times = []
         for run in range(4):
             slot = engine.acquire()
@@ -248,18 +291,35 @@ def main() -> int:
 
     # ---- decode at the headline batch
     progress(f"decode at batch {args.batch}")
-    runs = decode_run(args.batch, args.steps, args.warmup, args.repeats)
+    runs = model.decode_run(args.batch, PROMPT_LO, PROMPT_HI, args.steps, args.warmup, args.repeats,
+                            time_prefill=args.batch <= 8)
     step_s, step_bytes = median_run(runs)
     achieved = step_bytes / step_s / 1e9
+    packed = model.packed
 
-    points, points_frac, points_ms = {}, {}, {}
     if not args.no_points:
         for b in (1, BIG_BATCH):
-            progress(f"decode at batch {b}")
-            s, nbytes = median_run(decode_run(b, args.steps, max(3, args.warmup // 2), args.repeats))
-            points[f"decode_b{b}"] = round(b / s, 1)
-            points_ms[f"decode_b{b}"] = round(s * 1e3, 4)
-            points_frac[f"decode_b{b}"] = round(nbytes / s / 1e9 / HBM_PEAK_GBS, 4)
+            point(f"decode_b{b}", model, b, PROMPT_LO, PROMPT_HI, args.steps, max(3, args.warmup // 2), args.repeats)
+    extra = not args.no_extra and not args.no_points and args.shape == "7b" and args.layers == FULL_LAYERS
+    prefill_fp32 = None
+    if extra:
+        # the large batch behind long prompts: 32 steps a run keep the sequences inside the context
+        long_prompt = min(LONG_PROMPT, CONTEXT - 8 - 3 * 32 - 8)
+        point(f"decode_b{BIG_BATCH}_t{LONG_PROMPT}", model, BIG_BATCH, long_prompt, long_prompt, 32, 8, 3)
+    model.close()
+    if extra:
+        name32, ctx32, (lo32, hi32), _, shape32 = SHAPES["32b"]
+        progress(f"{name32}: random weights, {shape32['num_hidden_layers']} layers")
+        other = Model(shape32, shape32["num_hidden_layers"], "bfloat16", 8, ctx32, not args.no_tune)
+        point("decode_b8_32b", other, 8, lo32, hi32, 32, 8, 3)
+        other.close()
+        progress(f"{MODEL} in 32-bit")
+        other = Model(SHAPE, args.layers, "float32", 1, CONTEXT, False)
+        fp32_s = other.prompt_step(PROMPT)
+        prefill_fp32 = {"value": round(PROMPT / fp32_s, 1), "tokens": PROMPT, "ms": round(fp32_s * 1e3, 3),
+                        "frac": round(flops / fp32_s / FP32_PEAK_FLOPS, 4)}
+        point("decode_b1_fp32", other, 1, PROMPT_LO, PROMPT_HI, 16, 4, 3)
+        other.close()
 
     PROMPTS = PROMPT_LO if PROMPT_LO == PROMPT_HI else f"{PROMPT_LO}-{PROMPT_HI}"
     line = {
@@ -284,6 +344,8 @@ def main() -> int:
             "global_batch": args.batch, "seq_len": CONTEXT, "prompt_len": PROMPTS,
             "parallelism": "single GPU", "sampling": "greedy, ids read every 8 steps", "load_s": round(load_s, 1),
             "library_gemm_autotuned": not args.no_tune,
+            "points_of_other_shapes": "decode_b8_32b: Qwen2.5-32B layer sizes, 64 layers, prompts 512-2048; "
+                                      "decode_b1_fp32 and prefill_fp32: this shape in true 32-bit" if extra else "none",
         },
         "prefill": {"value": round(PROMPT / prefill_s, 1), "tokens": PROMPT,
                     "ms": round(prefill_s * 1e3, 3),
@@ -299,6 +361,8 @@ def main() -> int:
                     "median": round(step_s * 1e3, 4),
                     "max": round(max(t for t, _ in runs) * 1e3, 4)},
     }
+    if prefill_fp32:
+        line["prefill_fp32"] = prefill_fp32
     if continuation:
         line["continuation"] = continuation
     if packed:
