@@ -96,6 +96,9 @@ def main() -> int:
     ap.add_argument("--continuation", default="", metavar="AFTER:NEW",
                     help="also time a step of NEW tokens of a sequence that holds AFTER tokens already "
                          "(a new turn of a conversation); reported as \"continuation\"")
+    ap.add_argument("--short-steps", action="store_true",
+                    help="also time prompt steps of 16, 64 and 256 tokens and a step of 8 one-token entries plus a "
+                         "64-token prompt, as replayed graphs and issued launch by launch; reported as \"short_steps\"")
     ap.add_argument("--no-tune", action="store_true",
                     help="leave the library's default kernels for the tall matrix products")
     args = ap.parse_args()
@@ -289,6 +292,47 @@ def main() -> int:
             engine.release(slot)
         continuation = {"after": cont[0], "tokens": cont[1], "ms": round(sorted(times)[1] * 1e3, 3)}
 
+    # ---- short prompt steps and a mixed step: the replayed graph of their bucket against launches from the host
+    short_steps = None
+    if args.short_steps:
+        progress("short steps")
+        short_steps = {}
+
+        def timed(step, reset):
+            times = []
+            for run in range(7):
+                reset()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                step()
+                torch.cuda.synchronize()
+                if run > 2:               # the bucket's first step runs eagerly, its second is captured
+                    times.append(time.perf_counter() - t0)
+            return round(sorted(times)[len(times) // 2] * 1e3, 3)
+
+        for label, n_decoding, n_prompt in (("prompt16", 0, 16), ("prompt64", 0, 64), ("prompt256", 0, 256),
+                                            ("decode8_prompt64", 8, 64)):
+            slots = [engine.acquire() for _ in range(n_decoding + 1)]
+            if n_decoding:
+                engine.step([StepEntry(s, p, []) for s, p in zip(slots, model.prompts(n_decoding, 300, 300))])
+            new = model.prompts(1, n_prompt, n_prompt)[0]
+
+            def step():
+                engine.step([StepEntry(s, [7], [0]) for s in slots[:-1]] + [StepEntry(slots[-1], new, [n_prompt - 1])])
+
+            def reset():
+                engine.truncate(slots[-1], 0)
+                for s in slots[:-1]:
+                    engine.truncate(s, 300)
+            rows_allowed = engine.graph_step_rows
+            graph_ms = timed(step, reset)
+            engine.graph_step_rows = 0
+            eager_ms = timed(step, reset)
+            engine.graph_step_rows = rows_allowed
+            short_steps[label] = {"graph_ms": graph_ms, "eager_ms": eager_ms}
+            for s in slots:
+                engine.release(s)
+
     # ---- decode at the headline batch
     progress(f"decode at batch {args.batch}")
     runs = model.decode_run(args.batch, PROMPT_LO, PROMPT_HI, args.steps, args.warmup, args.repeats,
@@ -363,6 +407,8 @@ def main() -> int:
     }
     if prefill_fp32:
         line["prefill_fp32"] = prefill_fp32
+    if short_steps:
+        line["short_steps"] = short_steps
     if continuation:
         line["continuation"] = continuation
     if packed:

@@ -8,10 +8,13 @@ runs one sequence with one position scalar (src/graph_builder.hpp:222-231,
 src/engine.cpp:138-145); packing, slots and per-row positions are this
 engine's own. One-token steps are captured once per batch-size bucket into a
 HIP graph and replayed (the reference's build-once, replay-many decode:
-src/engine.cpp:151-269).
+src/engine.cpp:151-269); so are short prompt steps and steps that mix prompts
+with one-token entries, per bucket of their sizes (rows, sequences, longest run
+of new tokens, keys, wanted places).
 """
 from __future__ import annotations
 
+import collections
 import dataclasses
 import warnings
 
@@ -33,6 +36,11 @@ _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.
            "fp32": torch.float32}
 
 GRAPH_MAX_BUCKET = 256
+# Steps other than all-one-token ones are captured too when they have at most so many rows: a
+# longer prompt keeps the GPU busy for longer than the host needs to issue it, and its sizes
+# rarely come again. So many such graphs are kept, the least recently used one goes first.
+GRAPH_MAX_STEP_ROWS = 512
+GRAPH_MAX_STEP_PLANS = 24
 
 
 class StepError(ValueError):
@@ -64,10 +72,14 @@ class _Meta:
         return {name: buf[o:o + n] for name, (o, n) in self.offsets.items()}
 
 
+def _pow2(n: int, least: int = 1) -> int:
+    return max(least, 1 << (max(n, 1) - 1).bit_length())
+
+
 class _GraphBucket:
-    def __init__(self, size: int, device):
+    def __init__(self, size: int, device, seqs: int | None = None, wants: int | None = None):
         self.size = size
-        self.meta = _Meta(size, size, size)
+        self.meta = _Meta(size, size if seqs is None else seqs, size if wants is None else wants)
         self.dev = torch.zeros(self.meta.total, dtype=torch.int32, device=device)
         self.views = self.meta.views(self.dev)
         self.pool = ScratchPool(device)
@@ -83,13 +95,15 @@ class Engine:
                  max_slots: int | None = None, max_seq_len: int | None = None,
                  device: str = "cuda:0", fast_kernels: bool = True, use_graphs: bool = True,
                  tune_library: bool = False, beyond_max_positions: bool = False, profile: bool = False,
-                 sync_each_launch: bool = False):
+                 sync_each_launch: bool = False, graph_step_rows: int = GRAPH_MAX_STEP_ROWS):
         """max_seq_len: the longest sequence (default: the positions the model's configuration
         allows; more than that is refused unless beyond_max_positions says it is meant).
         tune_library: let the library's autotuner choose the kernel of each tall bfloat16
         matrix product the first time its shape is seen (kernels/library_tuning.py).
         profile: time every kernel with a pair of events (kernels/profiler.py; steps then run
         without HIP graphs); profile_summary() gives the table.
+        graph_step_rows: prompt steps and mixed steps of up to so many rows are captured as HIP
+        graphs too, one per bucket of their sizes (0: only one-token steps are).
         sync_each_launch: a debugging mode (the reference's sync_after_each_op, src/engine.cpp:318-334):
         steps run without HIP graphs and the host waits for the GPU after every launch, so that
         a fault is reported with the name of the op that raised it."""
@@ -144,12 +158,14 @@ class Engine:
         self.use_graphs = use_graphs and self.model.graph_safe() and not profile and not sync_each_launch
         self._buckets: dict[tuple[int, bool], _GraphBucket] = {}
         self._uneven_sticky: dict[int, bool] = {}     # per bucket size: the flag of the step before
+        self.graph_step_rows = graph_step_rows
+        self._plans: collections.OrderedDict[tuple, _GraphBucket] = collections.OrderedDict()
         self._pinned = [torch.empty(1 << 16, dtype=torch.int32).pin_memory() for _ in range(4)]
         self._pinned_events: list[torch.cuda.Event | None] = [None] * 4
         self._pinned_next = 0
         self._iota_cache = np.arange(64, dtype=np.int32)
         self.stats = {"steps": 0, "graph_replays": 0, "graph_captures": 0, "eager_steps": 0,
-                      "graph_capture_failures": 0}
+                      "graph_capture_failures": 0, "step_graph_captures": 0, "step_graph_replays": 0}
         self.capture_failures: list[str] = []         # one line per bucket whose capture failed
 
     # -- slots ----------------------------------------------------------------
@@ -218,8 +234,11 @@ class Engine:
         every_wanted = all(list(e.want) == [0] for e in entries)
         self.stats["steps"] += 1
         with profiler.active(self.profiler), profiler.sync_each_launch(self.sync_each_launch):
+            plan = None
             if self.use_graphs and all_single and every_wanted and len(entries) <= GRAPH_MAX_BUCKET:
                 logits = self._graph_step(entries, device_tokens)
+            elif self.use_graphs and device_tokens is None and (plan := self._step_plan(entries, all_single)):
+                logits = self._planned_step(entries, plan)
             else:
                 logits = self._eager_step(entries, all_single, device_tokens)
         self.cache.commit(growth)
@@ -253,6 +272,7 @@ class Engine:
         v["positions"][:] = 0
         v["seq_slot"][:] = -1
         v["seq_start"][:] = 0
+        v["want_rows"][:] = 0               # places beyond the wanted ones name row 0: never an index out of range
         if all(len(e.tokens) == 1 for e in entries):
             # one token a sequence: whole columns at once
             k = len(entries)
@@ -334,6 +354,7 @@ class Engine:
         ctx.host = {"q_lens": [len(e.tokens) for e in entries],
                     "starts": [self.cache.length(e.slot) for e in entries],
                     "slots": [e.slot for e in entries]}
+        ctx.most_keys = max(s + n for s, n in zip(ctx.host["starts"], ctx.host["q_lens"]))
         want = meta.views(host.numpy())["want_rows"][:nw]
         ctx.want_all = nw == rows and bool((want == np.arange(rows, dtype=np.int32)).all())
         self.stats["eager_steps"] += 1
@@ -358,6 +379,7 @@ class Engine:
             ctx = self._context(bucket.views, size, size, 1, True, bucket.pool)
             ctx.want_all = True
             ctx.uneven_keys = uneven
+            ctx.padded = True
             if bucket.uses == 1:
                 # first use: run eagerly; it also sizes the bucket's scratch pool
                 return self._bucket_eager(bucket, ctx, n)
@@ -392,6 +414,79 @@ class Engine:
         bucket.graph.replay()
         self.stats["graph_replays"] += 1
         return bucket.logits[:n]
+
+    # -- prompt steps and mixed steps as graphs ------------------------------------
+    def _step_plan(self, entries, all_single: bool):
+        """The bucket of sizes a step that is not all one-token (or does not want every row)
+        runs in as a graph, or None when it runs eagerly: (rows, sequences, longest run of new
+        tokens, most keys of a sequence after the step, wanted places, every row wanted in
+        order, all one-token), each rounded up to a power of two. The sizes decide every
+        grid, so steps of one bucket replay one graph; rows and sequences beyond the step's
+        own are padding (row_seq -1, slot -1) that every kernel passes over."""
+        rows = sum(len(e.tokens) for e in entries)
+        if rows > self.graph_step_rows:
+            return None
+        wants = sum(len(e.want) for e in entries)
+        want_all = wants == rows and all(list(e.want) == list(range(len(e.tokens))) for e in entries)
+        R = _pow2(rows, 16)
+        most = max(self.cache.length(e.slot) + len(e.tokens) for e in entries)
+        keys = min(_pow2(most, 256), max(self.cache.max_seq_len, 256))
+        return (R, _pow2(len(entries)), min(_pow2(max(len(e.tokens) for e in entries)), R), keys,
+                R if want_all else (_pow2(wants) if wants else 0), want_all, all_single)
+
+    def _planned_step(self, entries, plan):
+        R, S, Q, keys, W, want_all, all_single = plan
+        bucket = self._plans.get(plan)
+        if bucket is None:
+            if len(self._plans) >= GRAPH_MAX_STEP_PLANS:
+                self._plans.popitem(last=False)          # the least recently used graph and its buffers
+            bucket = self._plans[plan] = _GraphBucket(R, self.device, S, max(W, 1))
+        self._plans.move_to_end(plan)
+        host, idx, nw = self._pack(entries, bucket.meta, R, S)
+        self._upload(host, idx, bucket.dev)
+        rows = sum(len(e.tokens) for e in entries)
+        bucket.uses += 1
+        n_out = rows if want_all else nw
+
+        def forward(ctx):
+            return self.model.forward(bucket.views["tokens"], ctx, self.caches, bucket.views["want_rows"], W)
+
+        if bucket.graph is None:
+            ctx = self._context(bucket.views, R, S, Q, all_single, bucket.pool)
+            ctx.want_all = want_all
+            ctx.most_keys = keys
+            ctx.padded = True
+            if bucket.uses == 1 or bucket.capture_failed is not None:
+                bucket.pool.reset()          # first use: eagerly; it also sizes the bucket's scratch pool
+                self.stats["eager_steps"] += 1
+                logits = forward(ctx)
+                return None if logits is None or n_out == 0 else logits[:n_out]
+            bucket.pool.reset()
+            bucket.pool.frozen = True
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            try:
+                with library_tuning.no_new_tuning(), torch.cuda.graph(graph):
+                    bucket.pool.reset()
+                    bucket.logits = forward(ctx)
+            except Exception as exc:
+                bucket.capture_failed = f"step of {plan}: {exc!r}"
+                self.capture_failures.append(bucket.capture_failed)
+                self.stats["graph_capture_failures"] += 1
+                bucket.pool.frozen = False
+                del graph
+                torch.cuda.synchronize()
+                bucket.pool.reset()
+                self.stats["eager_steps"] += 1
+                logits = forward(ctx)       # the step's own errors are raised again here
+                warnings.warn(f"capturing the {bucket.capture_failed} as a HIP graph failed; steps of these "
+                              "sizes run without a graph from here on", stacklevel=3)
+                return None if logits is None or n_out == 0 else logits[:n_out]
+            bucket.graph = graph
+            self.stats["step_graph_captures"] += 1
+        bucket.graph.replay()
+        self.stats["step_graph_replays"] += 1
+        return None if bucket.logits is None or n_out == 0 else bucket.logits[:n_out]
 
     def _bucket_eager(self, bucket, ctx, n: int):
         """The bucket's step without a graph, on its own buffers."""

@@ -138,12 +138,16 @@ class Attention(Mixer):
                                  self.scale, ctx.max_keys, ws)
         else:
             # few queries against many keys (a continuation of a long sequence): the keys in parts
-            most = max(s + n for s, n in zip(ctx.host["starts"], ctx.host["q_lens"])) if ctx.host else ctx.max_keys
+            most = ctx.most_keys
             if self.window > 0:
                 most = min(most, self.window + ctx.max_q_len)
             parts = ops.attention_prefill_parts(ctx.num_seqs, ctx.max_q_len, H, hd, most)
             ws = ctx.alloc((ops.attention_prefill_workspace_floats(rows, H, hd, parts),), torch.float32) \
                 if parts > 1 else None
+            if ctx.padded:
+                # the prompt kernels write the rows of sequences only: padding rows hold zeros (their
+                # parts too, whose join then gives zeros), never what the buffer held before
+                (ws if ws is not None else out).zero_()
             ops.attention_prefill(out, q, cache.kpool, cache.vpool, ctx.cu_seqlens, ctx.seq_slot,
                                   ctx.seq_start, cache.page_table, ctx.num_seqs, ctx.max_q_len,
                                   rows, H, KVH, hd, self.window, self.scale, parts=parts, workspace=ws)

@@ -140,13 +140,16 @@ class StepContext:
         self.cu_seqlens = cu_seqlens      # int32 [num_seqs + 1] first row of each sequence
         self.seq_start = seq_start        # int32 [num_seqs] cached length before this step
         self.max_q_len = max_q_len        # longest run of new tokens of one sequence
-        self.max_keys = max_keys          # upper bound of any sequence's length after the step
+        self.max_keys = max_keys          # upper bound of any sequence's length (the cache's)
+        self.most_keys = max_keys         # the most keys a sequence of this step has after it, or a bound on that
         self.all_single = all_single      # every sequence brings exactly one token
         self.env = env
         self.scratch = scratch            # ScratchPool: alloc(shape, dtype)
         self.host = host                  # {"q_lens", "starts", "slots"}: lists per sequence, eager steps only
         self.uneven_keys = False          # one sequence has several times the keys of the others (a hint for the grids)
         self.want_all = False             # the wanted rows are all rows, in order
+        self.padded = False               # the step may hold padding rows and sequences (row_seq -1, slot -1: a step that
+                                          # runs as a graph of its bucket of sizes); a part leaves such rows finite
         self.next_norm = None             # the norm that reads the stream after the running block (set by the model)
         self.sink = None                  # ResidualSink offered to the running mixer / feed-forward
 

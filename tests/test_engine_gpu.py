@@ -633,3 +633,100 @@ def test_sync_each_launch_mode_gives_the_same_logits(model_dirs, plain_models):
             assert eng.stats["graph_replays"] == 0
     assert torch.equal(outs[0], outs[1])
     close(outs[1], plain_logits(plain_models, "D", ids), "float32")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_short_prompt_and_mixed_steps_replay_a_graph(model_dirs, plain_models, name, dtype):
+    """Prompt steps and mixed steps of up to a few hundred rows run as HIP graphs, one per bucket of
+    their sizes: the first step of a bucket runs eagerly, the second is captured, later ones replay.
+    Steps of different lengths that share a bucket (prompts of 37, 41 and 60 tokens; three one-token
+    entries beside a prompt of 33 to 50) replay the same graph; every logit is the plain
+    implementation's, and in 32-bit bit for bit what an engine without such graphs gives."""
+    import hector_engine_amd as he
+    opts = dict(max_tokens=4096, max_slots=8, max_seq_len=1024, beyond_max_positions=True)
+    eng = he.Engine(model_dirs[name], dtype=dtype, **opts)
+    plain_eng = he.Engine(model_dirs[name], dtype=dtype, graph_step_rows=0, **opts)
+    vocab = plain_models[name][0]["vocab_size"]
+
+    def both(make_entries):
+        a = eng.step(make_entries(eng))
+        b = plain_eng.step(make_entries(plain_eng))
+        if dtype == "float32":
+            assert torch.equal(a, b)
+        return a.clone()
+
+    # whole prompts of lengths that share the bucket of 64 rows, all positions wanted
+    for i, n in enumerate((37, 41, 60, 33, 64)):
+        ids = rand_ids(vocab, n, 800 + i)
+        slots = {}
+
+        def prompt(e, ids=ids, n=n):
+            slots[e] = e.acquire()
+            return [entry(slots[e], ids, range(n))]
+        got = both(prompt)
+        close(got, plain_logits(plain_models, name, ids), dtype)
+        for e, s in slots.items():
+            e.release(s)
+    assert eng.stats["step_graph_captures"] == 1 and eng.stats["step_graph_replays"] == 4
+    assert plain_eng.stats["step_graph_captures"] == 0
+    # three sequences that decode, and a prompt that joins them: five mixed steps in a row, the
+    # joining prompt of another length each time, only some places wanted
+    requests = [rand_ids(vocab, n, 820 + i) for i, n in enumerate((30, 52, 75))]
+    held = {e: [e.acquire() for _ in requests] for e in (eng, plain_eng)}
+    fed = [20, 40, 60]
+    both(lambda e: [entry(s, r[:n], [n - 1]) for s, r, n in zip(held[e], requests, fed)])
+    rows = [[] for _ in requests]
+    for step, n in enumerate((33, 50, 41, 36, 48)):
+        joiner = rand_ids(vocab, n, 840 + step)
+        extra = {}
+
+        def mixed(e, joiner=joiner, n=n):
+            extra[e] = e.acquire()
+            return [entry(s, [r[k]], [0]) for s, r, k in zip(held[e], requests, fed)] \
+                + [entry(extra[e], joiner, [0, n // 2, n - 1])]
+        got = both(mixed)
+        for i in range(3):
+            rows[i].append(got[i:i + 1])
+            fed[i] += 1
+        close(got[3:], plain_logits(plain_models, name, joiner)[[0, n // 2, n - 1]], dtype)
+        for e, s in extra.items():
+            e.release(s)
+    for i, r in enumerate(requests):
+        close(torch.cat(rows[i]), plain_logits(plain_models, name, r[:fed[i]])[fed[i] - 5:], dtype)
+    assert eng.stats["step_graph_captures"] >= 2 and eng.stats["step_graph_replays"] >= 4 + 3
+    assert not eng.capture_failures
+    for e, ss in held.items():
+        for s in ss:
+            e.release(s)
+        assert e.cache.free_pages == e.cache.num_pages
+
+
+def test_step_graphs_are_kept_least_recently_used_first_out(model_dirs, plain_models):
+    """No more graphs of prompt steps are kept than GRAPH_MAX_STEP_PLANS: the one used longest ago
+    goes, and a bucket that comes again after that is captured anew, with the same logits."""
+    import hector_engine_amd as he
+    from hector_engine_amd.engine import engine as engine_module
+    eng = he.Engine(model_dirs["A"], dtype="float32", max_tokens=4096, max_slots=8, max_seq_len=512,
+                    beyond_max_positions=True)
+    ids = rand_ids(256, 300, 860)
+    want = plain_logits(plain_models, "A", ids[:20])
+
+    def run(n_seqs, n, places):
+        slots = [eng.acquire() for _ in range(n_seqs)]
+        out = eng.step([entry(s, ids[:n], places) for s in slots]).clone()
+        for s in slots:
+            eng.release(s)
+        return out
+    first = [run(1, 20, [19]) for _ in range(3)]
+    close(first[2], want[19:20], "float32")
+    assert len(eng._plans) == 1
+    # 24 other buckets: 1, 2, 4 or 8 sequences, runs of 2 to 64 new tokens, two places wanted of each
+    for s in (1, 2, 3, 5):
+        for n in (2, 3, 5, 9, 17, 33):
+            run(s, n, [0, n - 1])
+    assert len(eng._plans) == engine_module.GRAPH_MAX_STEP_PLANS == 24
+    captures = eng.stats["step_graph_captures"]
+    again = [run(1, 20, [19]) for _ in range(3)]
+    assert eng.stats["step_graph_captures"] == captures + 1
+    assert all(torch.equal(a, first[0]) for a in again + first)
