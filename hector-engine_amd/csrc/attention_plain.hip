@@ -1,21 +1,89 @@
-// Plain attention over the paged cache: one wavefront per (query row, head),
-// keys visited one by one in ascending position with an online softmax in
-// fp32. The result for a query depends only on its own position and the cache
-// rows [first, p], never on how the step was cut or batched, so prompt steps
-// and one-token steps give identical bits. It is the 32-bit path's attention
-// and the reference beside the MFMA kernels.
+// Plain attention over the paged cache in fp32, in one fixed order per (query, head): the keys
+// are taken page by page (64 positions, by absolute position), inside a page one by one in
+// ascending position with an online softmax begun afresh, and the pages' results (m, l, sums)
+// are joined one after the other in ascending position. The result for a query depends only on
+// its own position and the cache rows [first, p], never on how the step was cut or batched, so
+// prompt steps and one-token steps give identical bits. It is the 32-bit path's attention and
+// the reference beside the MFMA kernels.
 //
 // For the query at absolute position p: first = window > 0 ? max(0, p+1-window) : 0,
 // s_j = (q . k_j) * scale for j in [first, p], out = sum_j softmax(s)_j v_j,
 // kv head = h / (H / KVH)   (reference: kernels/attention.cu:155-316, :664-773, :60).
+//
+// Two launches keep that order and give the same bits: one wavefront per (query, head) that walks
+// the pages itself; or, for steps of few queries over many keys (one-token steps), a wavefront
+// per (query, head, page) that leaves its page's result in a workspace, and a second kernel that
+// joins them in order (one wavefront alone would walk thousands of keys while the chip idles:
+// a one-token step of 28 heads over 2,048 keys took 2.4 ms so).
+// No multiply and add of this file is fused unless it is written as an fma: the same lines are
+// compiled into several kernels that must give the same bits.
+#pragma clang fp contract(off)
 #include "cache_layout.h"
 #include "hector_kernels.h"
 
 #define AP_MAX_PER_LANE 8
 
+struct ApState {
+  float m, l;
+  float acc[AP_MAX_PER_LANE];
+};
+
+// The online softmax of the keys [j_lo, j_hi] of one page (they lie in the same page), begun afresh.
+// Every multiply-add is written out as an fma: these lines are compiled into several kernels,
+// and the compiler would otherwise be free to fuse each copy its own way.
+template <typename T>
+__device__ __forceinline__ void ap_page(ApState& st, const float (&qv)[AP_MAX_PER_LANE], const T* kpool,
+                                        const T* vpool, int page, int num_pages, int KVH, int kvh, int hd,
+                                        int j_lo, int j_hi, float scale, int lane, int npl) {
+  st.m = -INFINITY;
+  st.l = 0.f;
+#pragma unroll
+  for (int i = 0; i < AP_MAX_PER_LANE; ++i) st.acc[i] = 0.f;
+  if (page < 0 || page >= num_pages) return;  // never for an admitted batch
+  // the pages are stored in the MFMA kernels' operand order (cache_layout.h)
+  const int64_t base = ((int64_t)page * KVH + kvh) * he_k_page_elems(hd);
+  const int64_t vbase = ((int64_t)page * KVH + kvh) * he_v_page_elems(hd);
+  const int KS = he_k_steps(hd), NT = he_v_tiles(hd);
+  for (int j = j_lo; j <= j_hi; ++j) {
+    const int off = j & (HE_PAGE_TOKENS - 1);
+    float part = 0.f;
+#pragma unroll
+    for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
+      const int d = lane + i * HE_WAVE;
+      if (i < npl && d < hd) part = fmaf(qv[i], to_float(kpool[base + he_k_index(off, d, KS)]), part);
+    }
+    const float s = wave_sum(part) * scale;
+    const float m_new = fmaxf(st.m, s);
+    const float alpha = expf(st.m - m_new);
+    const float w = expf(s - m_new);
+    st.l = fmaf(st.l, alpha, w);
+#pragma unroll
+    for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
+      const int d = lane + i * HE_WAVE;
+      if (i < npl && d < hd) st.acc[i] = fmaf(st.acc[i], alpha, w * to_float(vpool[vbase + he_v_index(off, d, NT)]));
+    }
+    st.m = m_new;
+  }
+}
+
+// total <- total joined with the result of the next page (one that had keys).
+__device__ __forceinline__ void ap_join(ApState& total, const ApState& st) {
+  if (!(st.m > -INFINITY)) return;
+  const float m_new = fmaxf(total.m, st.m);
+  const float a = total.m > -INFINITY ? expf(total.m - m_new) : 0.f;
+  const float b = expf(st.m - m_new);
+  total.l = fmaf(total.l, a, st.l * b);
+#pragma unroll
+  for (int i = 0; i < AP_MAX_PER_LANE; ++i) total.acc[i] = fmaf(total.acc[i], a, st.acc[i] * b);
+  total.m = m_new;
+}
+
+// grid (rows, ceil(H / 4), pages): pages == 1: the wavefront walks all pages of its query and stores
+// the result; pages > 1: it takes the page (first >> 6) + blockIdx.z alone and stores (m, l, sums)
+// into ws [row][head][pages][hd + 2], if the query has such a page.
 template <typename T>
 __global__ __launch_bounds__(256) void attention_plain_kernel(
-    T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ kpool,
+    T* __restrict__ out, float* __restrict__ ws, const T* __restrict__ q, const T* __restrict__ kpool,
     const T* __restrict__ vpool, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ row_seq, const int32_t* __restrict__ seq_slot,
     const int32_t* __restrict__ page_table, int max_blocks, int num_pages, int H, int KVH, int hd,
@@ -24,14 +92,16 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(
   const int h = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int64_t row = blockIdx.x;
   if (h >= H) return;
+  const bool split = gridDim.z > 1;
   T* o = out + (row * H + h) * (int64_t)hd;
   const int seq = row_seq[row];
   const int npl = (hd + HE_WAVE - 1) / HE_WAVE;
   if (seq < 0) {
-    for (int i = 0; i < npl; ++i) {
-      const int d = lane + i * HE_WAVE;
-      if (d < hd) o[d] = from_float<T>(0.f);
-    }
+    if (!split)
+      for (int i = 0; i < npl; ++i) {
+        const int d = lane + i * HE_WAVE;
+        if (d < hd) o[d] = from_float<T>(0.f);
+      }
     return;
   }
   const int p = positions[row];
@@ -39,73 +109,154 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(
   const int kvh = h / (H / KVH);
   const int first = window > 0 ? max(0, p + 1 - window) : 0;
   const int32_t* pt = page_table + (int64_t)slot * max_blocks;
+  const int c_first = first >> HE_PAGE_SHIFT, c_last = p >> HE_PAGE_SHIFT;
+  if (split && c_first + (int)blockIdx.z > c_last) return;
 
-  float qv[AP_MAX_PER_LANE], acc[AP_MAX_PER_LANE];
+  float qv[AP_MAX_PER_LANE];
   const T* qrow = q + (row * H + h) * (int64_t)hd;
 #pragma unroll
   for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
     const int d = lane + i * HE_WAVE;
     qv[i] = (i < npl && d < hd) ? to_float(qrow[d]) : 0.f;
-    acc[i] = 0.f;
   }
-  float m = -INFINITY, l = 0.f;
-  for (int j = first; j <= p; ++j) {
-    const int page = pt[j >> HE_PAGE_SHIFT];
-    if (page < 0 || page >= num_pages) continue;  // never for an admitted batch
-    const int off = j & (HE_PAGE_TOKENS - 1);
-    // the pages are stored in the MFMA kernels' operand order (cache_layout.h)
-    const int64_t base = ((int64_t)page * KVH + kvh) * he_k_page_elems(hd);
-    const int64_t vbase = ((int64_t)page * KVH + kvh) * he_v_page_elems(hd);
-    const int KS = he_k_steps(hd), NT = he_v_tiles(hd);
-    float part = 0.f;
+  ApState st;
+  if (split) {
+    const int c = c_first + blockIdx.z;
+    ap_page<T>(st, qv, kpool, vpool, pt[c], num_pages, KVH, kvh, hd, max(first, c << HE_PAGE_SHIFT),
+               min(p, (c << HE_PAGE_SHIFT) + HE_PAGE_TOKENS - 1), scale, lane, npl);
+    float* w = ws + ((row * H + h) * (int64_t)gridDim.z + blockIdx.z) * (hd + 2);
 #pragma unroll
     for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
       const int d = lane + i * HE_WAVE;
-      if (i < npl && d < hd) part = fmaf(qv[i], to_float(kpool[base + he_k_index(off, d, KS)]), part);
+      if (i < npl && d < hd) w[d] = st.acc[i];
     }
-    const float s = wave_sum(part) * scale;
-    const float m_new = fmaxf(m, s);
-    const float alpha = expf(m - m_new);
-    const float w = expf(s - m_new);
-    l = l * alpha + w;
-#pragma unroll
-    for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
-      const int d = lane + i * HE_WAVE;
-      if (i < npl && d < hd) acc[i] = acc[i] * alpha + w * to_float(vpool[vbase + he_v_index(off, d, NT)]);
-    }
-    m = m_new;
+    if (lane == 0) w[hd] = st.m, w[hd + 1] = st.l;
+    return;
   }
-  const float inv = l > 0.f ? 1.f / l : 0.f;
+  ApState total;
+  total.m = -INFINITY;
+  total.l = 0.f;
+#pragma unroll
+  for (int i = 0; i < AP_MAX_PER_LANE; ++i) total.acc[i] = 0.f;
+  for (int c = c_first; c <= c_last; ++c) {
+    ap_page<T>(st, qv, kpool, vpool, pt[c], num_pages, KVH, kvh, hd, max(first, c << HE_PAGE_SHIFT),
+               min(p, (c << HE_PAGE_SHIFT) + HE_PAGE_TOKENS - 1), scale, lane, npl);
+    ap_join(total, st);
+  }
+  const float inv = total.l > 0.f ? 1.f / total.l : 0.f;
 #pragma unroll
   for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
     const int d = lane + i * HE_WAVE;
-    if (i < npl && d < hd) o[d] = from_float<T>(acc[i] * inv);
+    if (i < npl && d < hd) o[d] = from_float<T>(total.acc[i] * inv);
   }
+}
+
+// Joins the pages' results of a split launch in ascending position. grid (rows, ceil(H / 4)).
+template <typename T>
+__global__ __launch_bounds__(256) void attention_plain_join_kernel(
+    T* __restrict__ out, const float* __restrict__ ws, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ row_seq, int H, int hd, int window, int pages) {
+  const int lane = threadIdx.x & (HE_WAVE - 1);
+  const int h = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int64_t row = blockIdx.x;
+  if (h >= H) return;
+  T* o = out + (row * H + h) * (int64_t)hd;
+  const int npl = (hd + HE_WAVE - 1) / HE_WAVE;
+  ApState total, st;
+  total.m = -INFINITY;
+  total.l = 0.f;
+#pragma unroll
+  for (int i = 0; i < AP_MAX_PER_LANE; ++i) total.acc[i] = 0.f;
+  if (row_seq[row] >= 0) {
+    const int p = positions[row];
+    const int first = window > 0 ? max(0, p + 1 - window) : 0;
+    const int count = (p >> HE_PAGE_SHIFT) - (first >> HE_PAGE_SHIFT) + 1;
+    if (count > pages) {
+      // the caller's bound on the keys was too low: no part of the result may pass for one
+#pragma unroll
+      for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
+        const int d = lane + i * HE_WAVE;
+        if (i < npl && d < hd) o[d] = from_float<T>(NAN);
+      }
+      return;
+    }
+    for (int z = 0; z < count; ++z) {
+      const float* w = ws + ((row * H + h) * (int64_t)pages + z) * (hd + 2);
+#pragma unroll
+      for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
+        const int d = lane + i * HE_WAVE;
+        st.acc[i] = (i < npl && d < hd) ? w[d] : 0.f;
+      }
+      st.m = w[hd];
+      st.l = w[hd + 1];
+      ap_join(total, st);
+    }
+  }
+  const float inv = total.l > 0.f ? 1.f / total.l : 0.f;
+#pragma unroll
+  for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
+    const int d = lane + i * HE_WAVE;
+    if (i < npl && d < hd) o[d] = from_float<T>(total.acc[i] * inv);
+  }
+}
+
+// Pages a query of this step has at most (what a split launch needs room for), given the most keys
+// a sequence holds after the step.
+static int ap_pages(int most_keys, int window) {
+  int pages = (most_keys + HE_PAGE_TOKENS - 1) / HE_PAGE_TOKENS;
+  if (window > 0) pages = min(pages, (window + HE_PAGE_TOKENS - 2) / HE_PAGE_TOKENS + 1);
+  return max(pages, 1);
+}
+
+// Floats of workspace with which the step's attention runs page by page in parallel (0: one
+// wavefront per query and head walks the pages itself; that is the better launch for a step with
+// many queries).
+extern "C" int64_t he_attention_plain_workspace_floats(int rows, int H, int hd, int most_keys, int window) {
+  if (rows <= 0 || H <= 0 || hd <= 0 || most_keys <= 0) return 0;
+  const int pages = ap_pages(most_keys, window);
+  if (pages < 2 || (int64_t)rows * H > 8 * he_cus()) return 0;
+  return (int64_t)rows * H * pages * (hd + 2);
 }
 
 extern "C" int he_attention_plain(void* out, const void* q, const void* kpool, const void* vpool,
                                   const void* positions, const void* row_seq, const void* seq_slot,
                                   const void* page_table, int max_blocks, int num_pages, int rows,
                                   int H, int KVH, int hd, int window, float scale, int dtype,
+                                  int most_keys, void* workspace_f32, int64_t workspace_floats,
                                   void* stream) {
   HE_REQUIRE(rows >= 0 && H > 0 && KVH > 0 && hd > 0, "he_attention_plain: bad sizes");
   HE_REQUIRE(H % KVH == 0, "he_attention_plain: heads %d not a multiple of kv heads %d", H, KVH);
   HE_REQUIRE(hd <= AP_MAX_PER_LANE * HE_WAVE, "he_attention_plain: head_dim %d above %d", hd,
              AP_MAX_PER_LANE * HE_WAVE);
+  HE_REQUIRE(dtype == HE_BF16 || dtype == HE_F32, "he_attention_plain: unknown dtype %d", dtype);
   if (rows == 0) return 0;
-  dim3 grid(rows, (H + 3) / 4);
+  // page by page in parallel when the caller brought room for it (the same bits either way)
+  const int64_t need = he_attention_plain_workspace_floats(rows, H, hd, most_keys, window);
+  const bool split = need > 0 && workspace_f32 != nullptr && workspace_floats >= need;
+  const int pages = split ? ap_pages(most_keys, window) : 1;
+  HE_REQUIRE(pages <= 65535, "he_attention_plain: %d pages of keys are too many for one launch", pages);
+  dim3 grid(rows, (H + 3) / 4, pages);
+  float* ws = (float*)workspace_f32;
   hipStream_t s = (hipStream_t)stream;
-#define AP_LAUNCH(T)                                                                       \
-  attention_plain_kernel<T><<<grid, 256, 0, s>>>(                                          \
-      (T*)out, (const T*)q, (const T*)kpool, (const T*)vpool, (const int32_t*)positions,   \
-      (const int32_t*)row_seq, (const int32_t*)seq_slot, (const int32_t*)page_table,       \
+#define AP_LAUNCH(T)                                                                           \
+  attention_plain_kernel<T><<<grid, 256, 0, s>>>(                                              \
+      (T*)out, ws, (const T*)q, (const T*)kpool, (const T*)vpool, (const int32_t*)positions,   \
+      (const int32_t*)row_seq, (const int32_t*)seq_slot, (const int32_t*)page_table,           \
       max_blocks, num_pages, H, KVH, hd, window, scale)
+#define AP_JOIN(T)                                                                             \
+  attention_plain_join_kernel<T><<<dim3(rows, (H + 3) / 4), 256, 0, s>>>(                      \
+      (T*)out, ws, (const int32_t*)positions, (const int32_t*)row_seq, H, hd, window, pages)
   if (dtype == HE_BF16)
     AP_LAUNCH(bf16_t);
-  else if (dtype == HE_F32)
-    AP_LAUNCH(float);
   else
-    HE_REQUIRE(false, "he_attention_plain: unknown dtype %d", dtype);
+    AP_LAUNCH(float);
+  int rc = he_check_launch("he_attention_plain");
+  if (rc || !split) return rc;
+  if (dtype == HE_BF16)
+    AP_JOIN(bf16_t);
+  else
+    AP_JOIN(float);
 #undef AP_LAUNCH
+#undef AP_JOIN
   return he_check_launch("he_attention_plain");
 }

@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 18
+#define HE_ABI_VERSION 19
 
 #ifdef __cplusplus
 extern "C" {
@@ -44,9 +44,14 @@ int he_rmsnorm_rows(void* out, const void* x, const void* weight, int rows, int 
                     void* stream);
 
 // ---- matrix products: C[M,N] = A[M,K] * W[N,K]^T (+ bias) -------------------
+// he_gemm_plain: fp32 FMA sums in one fixed order per element (segments of 128 k, each a chain in
+// ascending k, added in segment order). With a workspace of he_gemm_plain_workspace_floats(M, N, K)
+// floats (0 for more than 8 rows) a product of few rows runs through kernels made for it; the
+// result is the same bit for bit.
+int64_t he_gemm_plain_workspace_floats(int M, int N, int K);
 int he_gemm_plain(void* C, const void* A, const void* W, const void* bias, int M, int N, int K,
                   int64_t lda, int64_t ldw, int64_t ldc, int in_dtype, int out_dtype,
-                  int bias_dtype, void* stream);
+                  int bias_dtype, void* workspace_f32, int64_t workspace_floats, void* stream);
 // bf16 MFMA product for M <= HE_BLOCKSPLIT_MAX_M with K cut inside the workgroup (NW
 // wavefronts, one slice each, added in LDS): complete in one launch.
 #define HE_BLOCKSPLIT_MAX_M 32
@@ -106,10 +111,17 @@ int he_qkv_rope_cache(void* q_out, void* kpool, void* vpool, const void* q_in, c
                       int H, int KVH, int hd, int dtype, void* stream);
 
 // ---- attention over the paged cache ----------------------------------------
+// he_attention_plain: fp32 sums in one fixed order per (query, head): page by page (64 positions),
+// inside a page key by key with an online softmax begun afresh, the pages joined in ascending
+// position. most_keys: no sequence holds more keys after the step. With a workspace of
+// he_attention_plain_workspace_floats floats (0 for a step of many queries) the pages of a query
+// run in parallel and a second kernel joins them; the result is the same bit for bit.
+int64_t he_attention_plain_workspace_floats(int rows, int H, int hd, int most_keys, int window);
 int he_attention_plain(void* out, const void* q, const void* kpool, const void* vpool,
                        const void* positions, const void* row_seq, const void* seq_slot,
                        const void* page_table, int max_blocks, int num_pages, int rows, int H,
-                       int KVH, int hd, int window, float scale, int dtype, void* stream);
+                       int KVH, int hd, int window, float scale, int dtype, int most_keys,
+                       void* workspace_f32, int64_t workspace_floats, void* stream);
 // bf16, one query row per sequence (decode): split over the keys, then merged.
 int he_attention_decode_bf16(void* out, const void* q, const void* kpool, const void* vpool,
                              const void* positions, const void* row_seq, const void* seq_slot,

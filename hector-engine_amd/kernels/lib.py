@@ -16,7 +16,7 @@ _lib = None
 
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 
-EXPECTED_ABI = 18
+EXPECTED_ABI = 19
 
 c_int, c_i64, c_f32, c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
@@ -32,8 +32,9 @@ _SIGNATURES = {
     "he_silu_mul": [c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_ptr],
     "he_add_rmsnorm": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_f32, c_int, c_int, c_ptr],
     "he_rmsnorm_rows": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_i64, c_i64, c_f32, c_int, c_int, c_ptr],
+    "he_gemm_plain_workspace_floats": [c_int, c_int, c_int],
     "he_gemm_plain": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_i64, c_i64, c_i64,
-                      c_int, c_int, c_int, c_ptr],
+                      c_int, c_int, c_int, c_ptr, c_i64, c_ptr],
     "he_gemm_blocksplit_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_int,
                                 c_int, c_int, c_int, c_ptr],
     "he_gemm_blocksplit_blocks": [c_int, c_int, c_int],
@@ -52,8 +53,9 @@ _SIGNATURES = {
     "he_qkv_rope_cache": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_ptr,
                           c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_ptr, c_int, c_int,
                           c_int, c_int, c_int, c_int, c_ptr],
+    "he_attention_plain_workspace_floats": [c_int, c_int, c_int, c_int, c_int],
     "he_attention_plain": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int,
-                           c_int, c_int, c_int, c_int, c_int, c_f32, c_int, c_ptr],
+                           c_int, c_int, c_int, c_int, c_int, c_f32, c_int, c_int, c_ptr, c_i64, c_ptr],
     "he_attention_decode_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_int, c_ptr,
                                  c_i64, c_ptr],
@@ -79,6 +81,8 @@ _SIGNATURES = {
     "he_sample_rows": [c_ptr, c_ptr, c_int, c_int, c_i64, c_ptr, c_f32, c_int, c_f32, c_ptr],
 }
 _RESTYPES = {
+    "he_attention_plain_workspace_floats": c_i64,
+    "he_gemm_plain_workspace_floats": c_i64,
     "he_attention_decode_workspace_floats": c_i64,
     "he_attention_decode_fused_workspace_floats": c_i64,
     "he_attention_prefill_workspace_floats": c_i64,

@@ -171,9 +171,17 @@ def rmsnorm_rows(out, x, weight, rows: int, D: int, x_stride: int, out_stride: i
                                  dtype_code(weight.dtype) if weight is not None else F32, _stream()))
 
 
+def gemm_plain_workspace_floats(M: int, N: int, K: int) -> int:
+    """Floats of workspace with which gemm_plain runs a product of few rows through the kernels made
+    for it (0: none needed)."""
+    return int(_lib.load().he_gemm_plain_workspace_floats(M, N, K))
+
+
 @_op("gemm_plain")
-def gemm_plain(out, a, w, bias, M: int) -> None:
-    """out[M,N] = a[M,K] . w[N,K]^T (+ bias), fixed summation order."""
+def gemm_plain(out, a, w, bias, M: int, workspace=None) -> None:
+    """out[M,N] = a[M,K] . w[N,K]^T (+ bias), fixed summation order. workspace: fp32, of
+    gemm_plain_workspace_floats(M, N, K) elements or more, for a product of few rows (the result
+    is the same bit for bit without it, and slower)."""
     N, K = w.shape
     _need(a, "a")
     _need(w, "w", a.dtype)
@@ -183,9 +191,12 @@ def gemm_plain(out, a, w, bias, M: int) -> None:
     if bias is not None:
         _need(bias, "bias", shape=(N,))
     L = _lib.load()
+    if workspace is not None:
+        _need(workspace, "workspace", torch.float32)
     _lib.check(L.he_gemm_plain(out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, K,
                                K, N, dtype_code(a.dtype), dtype_code(out.dtype),
-                               dtype_code(bias.dtype) if bias is not None else F32, _stream()))
+                               dtype_code(bias.dtype) if bias is not None else F32,
+                               _ptr(workspace), workspace.numel() if workspace is not None else 0, _stream()))
 
 
 BLOCKSPLIT_MAX_M = 32
@@ -486,8 +497,14 @@ def _check_attention(out, q, kpool, vpool, page_table, rows, H, KVH, hd):
 
 @_op("attention_plain")
 def attention_plain(out, q, kpool, vpool, positions, row_seq, seq_slot, page_table, rows: int,
-                    H: int, KVH: int, hd: int, window: int, scale: float) -> None:
+                    H: int, KVH: int, hd: int, window: int, scale: float, most_keys: int = 0,
+                    workspace=None) -> None:
+    """most_keys: a bound on the keys any sequence holds after the step, and workspace: fp32, of
+    attention_plain_workspace_floats elements or more: the pages of a query then run in parallel
+    (a step of few queries over many keys); the result is the same bit for bit without them."""
     _check_attention(out, q, kpool, vpool, page_table, rows, H, KVH, hd)
+    if workspace is not None:
+        _need(workspace, "workspace", torch.float32)
     for name, t in (("positions", positions), ("row_seq", row_seq), ("seq_slot", seq_slot)):
         _need(t, name, torch.int32)
     if positions.numel() < rows or row_seq.numel() < rows:
@@ -496,7 +513,12 @@ def attention_plain(out, q, kpool, vpool, positions, row_seq, seq_slot, page_tab
     _lib.check(L.he_attention_plain(
         out.data_ptr(), q.data_ptr(), kpool.data_ptr(), vpool.data_ptr(), positions.data_ptr(),
         row_seq.data_ptr(), seq_slot.data_ptr(), page_table.data_ptr(), page_table.shape[1],
-        kpool.shape[0], rows, H, KVH, hd, window, float(scale), dtype_code(q.dtype), _stream()))
+        kpool.shape[0], rows, H, KVH, hd, window, float(scale), dtype_code(q.dtype), int(most_keys),
+        _ptr(workspace), workspace.numel() if workspace is not None else 0, _stream()))
+
+
+def attention_plain_workspace_floats(rows: int, H: int, hd: int, most_keys: int, window: int) -> int:
+    return int(_lib.load().he_attention_plain_workspace_floats(rows, H, hd, most_keys, window))
 
 
 def attention_decode_workspace_floats(rows: int, H: int, KVH: int, hd: int, max_keys: int) -> int:

@@ -127,9 +127,11 @@ class Attention(Mixer):
                            ctx.seq_slot, cache.page_table, inv_freq, r, rows, H, KVH, hd, writes)
         out = ctx.alloc((rows, H * hd))
         if not self.fast:
+            floats = ops.attention_plain_workspace_floats(rows, H, hd, ctx.most_keys, self.window)
+            ws = ctx.alloc((floats,), torch.float32) if floats else None
             ops.attention_plain(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
                                 ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,
-                                self.scale)
+                                self.scale, ctx.most_keys, ws)
         elif ctx.all_single:
             floats = ops.attention_decode_workspace_floats(rows, H, KVH, hd, ctx.max_keys)
             ws = ctx.alloc((max(floats, 1),), torch.float32)

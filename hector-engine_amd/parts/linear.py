@@ -110,13 +110,13 @@ class Linear:
             if act == torch.float32:
                 if out_dtype != torch.float32:
                     raise TypeError("float32 activations give float32 outputs")
-                ops.gemm_plain(out, x, w, bias, rows)
+                self._plain(out, x, bias, rows, ctx)
                 return out
             # weight kept in 32-bit under bfloat16 activations
             x32 = ctx.alloc((rows, K), torch.float32)
             x32.copy_(x[:rows])
             y32 = out if out_dtype == torch.float32 else ctx.alloc((rows, N), torch.float32)
-            ops.gemm_plain(y32, x32, w, bias, rows)
+            self._plain(y32, x32, bias, rows, ctx)
             if y32 is not out:
                 out[:rows].copy_(y32)
             return out
@@ -124,12 +124,19 @@ class Linear:
             raise TypeError(f"Linear: weight {w.dtype} with activations {act} is not supported")
         if not ctx.env.fast_kernels or K % 8 != 0:
             # the plain kernel also under bfloat16; the MFMA kernels take K in steps of 8
-            ops.gemm_plain(out, x, w, bias, rows)
+            self._plain(out, x, bias, rows, ctx)
             return out
         if library_tuning.enabled() and not library_tuning.worth_tuning(rows):
             with library_tuning.no_new_tuning():
                 return self._library(x, bias, rows, out, out_dtype, ctx)
         return self._library(x, bias, rows, out, out_dtype, ctx)
+
+    def _plain(self, out, x, bias, rows: int, ctx: StepContext) -> None:
+        """The plain product (fixed summation order); with few rows through its kernels for them,
+        which want a workspace for their segment sums."""
+        floats = ops.gemm_plain_workspace_floats(rows, *self.weight.shape)
+        ws = ctx.alloc((floats,), torch.float32) if floats else None
+        ops.gemm_plain(out, x, self.weight, bias, rows, workspace=ws)
 
     def _library_slices(self, rows: int) -> int:
         """K slices for the library's product of a long-K weight with few output columns at up to

@@ -123,6 +123,40 @@ def test_gemm_plain_rows_do_not_depend_on_the_batch(ops):
         assert torch.equal(one.cpu()[0], full.cpu()[r])      # bit-equal
 
 
+@pytest.mark.parametrize("N,K", [(33, 100), (301, 136), (64, 256), (130, 257), (70, 1000), (5, 3), (200, 515)])
+def test_gemm_plain_for_few_rows_gives_the_bits_of_the_tile_kernel(ops, N, K):
+    """The plain product has one summation order (segments of 128 k, each a chain in ascending k, added
+    in segment order): its kernels for up to 8 rows, which take a workspace, and its tile kernel
+    give the same bits, with a bias or without, for widths that are no multiple of anything; a row of
+    a product of 70 rows equals the same row alone; and a workspace that is too small is not used."""
+    w, b = rnd(N, K, seed=13), rnd(N, seed=14)
+    a = rnd(70, K, seed=12)
+    full = torch.empty(70, N, device="cuda")
+    ops.gemm_plain(full, dev(a), dev(w), dev(b), 70)
+    ref = a.double() @ w.double().T + b.double()
+    assert torch.allclose(full.cpu().double(), ref, rtol=1e-5, atol=1e-6 * K)      # sums of K products of size one
+    for M in (1, 2, 3, 4, 5, 8):
+        floats = ops.gemm_plain_workspace_floats(M, N, K)
+        assert floats == -(-K // 128) * M * N
+        rows = dev(a[7:7 + M].contiguous())
+        tiled = torch.empty(M, N, device="cuda")
+        ops.gemm_plain(tiled, rows, dev(w), dev(b), M)
+        few = torch.full((M, N), 7.0, device="cuda")
+        ops.gemm_plain(few, rows, dev(w), dev(b), M, workspace=torch.empty(floats + 5, device="cuda"))
+        assert torch.equal(few, tiled) and torch.equal(few.cpu(), full.cpu()[7:7 + M])
+        ops.gemm_plain(few, rows, dev(w), None, M, workspace=torch.empty(floats, device="cuda"))
+        ops.gemm_plain(tiled, rows, dev(w), None, M, workspace=torch.empty(max(floats - 1, 1), device="cuda"))
+        assert torch.equal(few, tiled)
+    assert ops.gemm_plain_workspace_floats(9, N, K) == 0
+    # bfloat16 operands through the same kernels (the plain path of a bfloat16 model)
+    a16, w16 = a[:4].bfloat16().contiguous(), w.bfloat16()
+    tiled = torch.empty(4, N, dtype=torch.bfloat16, device="cuda")
+    few = torch.empty(4, N, dtype=torch.bfloat16, device="cuda")
+    ops.gemm_plain(tiled, dev(a16), dev(w16), None, 4)
+    ops.gemm_plain(few, dev(a16), dev(w16), None, 4, workspace=torch.empty(ops.gemm_plain_workspace_floats(4, N, K), device="cuda"))
+    assert torch.equal(few, tiled)
+
+
 def test_splitk_reduce_and_the_gated_activation_add_slices_in_order(ops):
     """K slices of a product are added in index order (+ bias) by splitk_reduce, and by the gated
     activation while it reads them."""
@@ -502,6 +536,14 @@ def attention_case(ops, kind, dtype, H, KVH, hd, window, lengths, q_lens, seed, 
     if kind == "plain":
         ops.attention_plain(out, dev(q), *args, dev(positions), dev(row_seq), dev(seq_slot),
                             dev(table), rows + pad, H, KVH, hd, window, scale)
+        # page by page in parallel (a bound on the keys and a workspace): the same bits
+        most = max(lengths) + 3
+        floats = ops.attention_plain_workspace_floats(rows + pad, H, hd, most, window)
+        if floats:
+            again = torch.full((rows + pad, H * hd), 7.0, dtype=dtype, device="cuda")
+            ops.attention_plain(again, dev(q), *args, dev(positions), dev(row_seq), dev(seq_slot), dev(table),
+                                rows + pad, H, KVH, hd, window, scale, most, torch.empty(floats, device="cuda"))
+            assert torch.equal(again, out)
     elif kind == "decode":
         max_keys = 4096
         ws = torch.empty(ops.attention_decode_workspace_floats(rows + pad, H, KVH, hd, max_keys), device="cuda")
@@ -534,6 +576,19 @@ def test_attention_plain(ops, dtype, H, KVH, hd, window):
     tol = 3e-6 if dtype == torch.float32 else 2 ** -6
     for g, w in zip(got, want):
         assert torch.allclose(g, w, rtol=tol, atol=tol)
+    assert ops.attention_plain_workspace_floats(11, H, hd, 203, window) == \
+        11 * H * (hd + 2) * (min(4, 3) if window else 4)       # 203 keys lie in 4 pages, a window of 70 in 3 at most
+    assert ops.attention_plain_workspace_floats(100000, H, hd, 203, window) == 0      # many queries: one wavefront each
+    # a bound on the keys that is too low must not pass for a result
+    if dtype == torch.float32 and not window:
+        slots, table, kpool, vpool = paged_setup([200], KVH, hd, dtype, 3)
+        q = rnd(1, H * hd, seed=5)
+        out = torch.zeros(1, H * hd, device="cuda")
+        ops.attention_plain(out, dev(q), dev(kpool), dev(vpool), dev(torch.tensor([199], dtype=torch.int32)),
+                            dev(torch.zeros(1, dtype=torch.int32)), dev(torch.tensor(slots, dtype=torch.int32)), dev(table),
+                            1, H, KVH, hd, 0, 0.1, 128, torch.empty(ops.attention_plain_workspace_floats(1, H, hd, 128, 0),
+                                                                   device="cuda"))
+        assert torch.isnan(out).all()
 
 
 @pytest.mark.parametrize("H,KVH,hd", ATT_SHAPES + [(40, 2, 32)])
