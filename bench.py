@@ -99,6 +99,8 @@ def main() -> int:
     ap.add_argument("--short-steps", action="store_true",
                     help="also time prompt steps of 16, 64 and 256 tokens and a step of 8 one-token entries plus a "
                          "64-token prompt, as replayed graphs and issued launch by launch; reported as \"short_steps\"")
+    ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16",
+                    help="float32: the whole measurement in true 32-bit (no library products, no extra points)")
     ap.add_argument("--no-tune", action="store_true",
                     help="leave the library's default kernels for the tall matrix products")
     args = ap.parse_args()
@@ -265,7 +267,10 @@ def main() -> int:
 
     progress(f"{MODEL}: random weights, {args.layers} layers")
     max_batch = 2 * args.batch if args.no_points else max(2 * args.batch, BIG_BATCH)
-    model = Model(SHAPE, args.layers, "bfloat16", max_batch, CONTEXT, not args.no_tune)
+    fp32 = args.dtype == "float32"
+    if fp32:
+        args.no_tune = True
+    model = Model(SHAPE, args.layers, args.dtype, max_batch, CONTEXT, not args.no_tune)
     engine, load_s = model.engine, model.load_s
 
     # ---- prefill of one 2,048-token prompt
@@ -299,16 +304,21 @@ def main() -> int:
         short_steps = {}
 
         def timed(step, reset):
-            times = []
+            """(wall ms, ms between two events around the step on the GPU's own clock), medians."""
+            times, spans = [], []
             for run in range(7):
                 reset()
+                before, after = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
+                before.record()
                 step()
+                after.record()
                 torch.cuda.synchronize()
                 if run > 2:               # the bucket's first step runs eagerly, its second is captured
                     times.append(time.perf_counter() - t0)
-            return round(sorted(times)[len(times) // 2] * 1e3, 3)
+                    spans.append(before.elapsed_time(after))
+            return round(sorted(times)[len(times) // 2] * 1e3, 3), round(sorted(spans)[len(spans) // 2], 3)
 
         for label, n_decoding, n_prompt in (("prompt16", 0, 16), ("prompt64", 0, 64), ("prompt256", 0, 256),
                                             ("decode8_prompt64", 8, 64)):
@@ -325,11 +335,11 @@ def main() -> int:
                 for s in slots[:-1]:
                     engine.truncate(s, 300)
             rows_allowed = engine.graph_step_rows
-            graph_ms = timed(step, reset)
+            graph_ms, graph_gpu_ms = timed(step, reset)
             engine.graph_step_rows = 0
-            eager_ms = timed(step, reset)
+            eager_ms, _ = timed(step, reset)
             engine.graph_step_rows = rows_allowed
-            short_steps[label] = {"graph_ms": graph_ms, "eager_ms": eager_ms}
+            short_steps[label] = {"graph_ms": graph_ms, "graph_gpu_ms": graph_gpu_ms, "eager_ms": eager_ms}
             for s in slots:
                 engine.release(s)
 
@@ -344,7 +354,7 @@ def main() -> int:
     if not args.no_points:
         for b in (1, BIG_BATCH):
             point(f"decode_b{b}", model, b, PROMPT_LO, PROMPT_HI, args.steps, max(3, args.warmup // 2), args.repeats)
-    extra = not args.no_extra and not args.no_points and args.shape == "7b" and args.layers == FULL_LAYERS
+    extra = not args.no_extra and not args.no_points and args.shape == "7b" and args.layers == FULL_LAYERS and not fp32
     prefill_fp32 = None
     if extra:
         # the large batch behind long prompts: 32 steps a run keep the sequences inside the context
@@ -367,7 +377,7 @@ def main() -> int:
 
     PROMPTS = PROMPT_LO if PROMPT_LO == PROMPT_HI else f"{PROMPT_LO}-{PROMPT_HI}"
     line = {
-        "metric": f"decode tok/s @ bs {args.batch}, {MODEL} bf16, context {CONTEXT}, prompts {PROMPTS}",
+        "metric": f"decode tok/s @ bs {args.batch}, {MODEL} {'fp32' if fp32 else 'bf16'}, context {CONTEXT}, prompts {PROMPTS}",
         "value": round(args.batch / step_s, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -377,7 +387,7 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": "fp32" if fp32 else "bf16",
         "data": "synthetic token ids (uniform), random N(0, 0.02) weights",
         "config": {
             "model": MODEL, "layers": args.layers, "layers_full": FULL_LAYERS,
@@ -393,7 +403,7 @@ def main() -> int:
         },
         "prefill": {"value": round(PROMPT / prefill_s, 1), "tokens": PROMPT,
                     "ms": round(prefill_s * 1e3, 3),
-                    "frac": round(flops / prefill_s / BF16_PEAK_FLOPS, 4)},
+                    "frac": round(flops / prefill_s / (FP32_PEAK_FLOPS if fp32 else BF16_PEAK_FLOPS), 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)},
         "points": points,
@@ -414,7 +424,8 @@ def main() -> int:
     if packed:
         line["prefill_packed"] = {"value": round(packed["tokens"] / packed["seconds"], 1), "tokens": packed["tokens"],
                                   "ms": round(packed["seconds"] * 1e3, 3),
-                                  "frac": round(packed["flops"] / packed["seconds"] / BF16_PEAK_FLOPS, 4)}
+                                  "frac": round(packed["flops"] / packed["seconds"]
+                                                / (FP32_PEAK_FLOPS if fp32 else BF16_PEAK_FLOPS), 4)}
     print(json.dumps(line))
     return 0
 
