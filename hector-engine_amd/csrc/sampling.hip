@@ -237,14 +237,18 @@ extern "C" int he_apply_penalties(void* logits_f32, int rows, int V, int64_t row
 // queued steps needs no token on the host in between: window [rows][W] is a ring (the token
 // appended as number n lies at n % W), appended[row] counts what was ever appended. One
 // workgroup a row first appends last_ids[row] (the token sampled by the step before; null:
-// nothing), then counts the distinct ids among the last min(appended, W) tokens and changes
-// each one's logit once, with the arithmetic of penalties_kernel.
+// nothing), then counts the distinct ids among the last min(appended, W) tokens in a hash table
+// in LDS (open addressing, twice as many places as the window has tokens: linear in the window)
+// and changes each one's logit once, with the arithmetic of penalties_kernel. The result
+// depends on the counts alone, not on the order in which the threads meet the ids.
 #define PEN_WINDOW_MAX 4096
+#define PEN_TABLE_MAX (2 * PEN_WINDOW_MAX)
 __global__ __launch_bounds__(256) void penalties_window_kernel(
     float* __restrict__ logits, int V, int64_t stride, int32_t* __restrict__ window,
     int32_t* __restrict__ appended, int W, const int32_t* __restrict__ last_ids, float rep,
     float freq, float pres) {
-  __shared__ int32_t ids[PEN_WINDOW_MAX];
+  __shared__ int32_t keys[PEN_TABLE_MAX];     // -1: free
+  __shared__ int32_t counts[PEN_TABLE_MAX];
   float* x = logits + blockIdx.x * stride;
   int32_t* ring = window + (int64_t)blockIdx.x * W;
   int total = appended[blockIdx.x];
@@ -252,26 +256,32 @@ __global__ __launch_bounds__(256) void penalties_window_kernel(
   const int at = total % W;
   if (last_ids != nullptr) ++total;
   const int n = total < W ? total : W;
-  for (int i = threadIdx.x; i < n; i += blockDim.x) ids[i] = last_ids != nullptr && i == at ? fresh : ring[i];
+  int places = 64;
+  while (places < 2 * n) places <<= 1;        // at most PEN_TABLE_MAX, as n <= W <= PEN_WINDOW_MAX
+  for (int i = threadIdx.x; i < places; i += blockDim.x) keys[i] = -1, counts[i] = 0;
   __syncthreads();          // every thread has read the count before it is written
-  if (threadIdx.x == 0 && last_ids != nullptr) {
-    ring[at] = fresh;
-    appended[blockIdx.x] = total;
-  }
+  if (threadIdx.x == 0 && last_ids != nullptr) appended[blockIdx.x] = total;
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
-    const int id = ids[i];
+    const int id = last_ids != nullptr && i == at ? fresh : ring[i];
+    if (last_ids != nullptr && i == at) ring[at] = fresh;
     if (id < 0 || id >= V) continue;
-    int count = 0;
-    bool first = true;
-    for (int j = 0; j < n; ++j) {
-      const bool same = ids[j] == id;
-      count += same;
-      first = first && !(same && j < i);
+    unsigned h = ((unsigned)id * 2654435761u) >> 7;
+    for (int probe = 0; probe < places; ++probe, ++h) {   // a free place exists: the table is at most half full
+      const int slot = h & (places - 1);
+      const int seen = atomicCAS(&keys[slot], -1, id);
+      if (seen == -1 || seen == id) {
+        atomicAdd(&counts[slot], 1);
+        break;
+      }
     }
-    if (!first) continue;
+  }
+  __syncthreads();
+  for (int slot = threadIdx.x; slot < places; slot += blockDim.x) {
+    const int id = keys[slot];
+    if (id < 0) continue;
     float v = x[id];
     if (rep != 1.0f) v = v > 0.f ? v / rep : v * rep;
-    if (freq != 0.0f) v -= freq * (float)count;
+    if (freq != 0.0f) v -= freq * (float)counts[slot];
     if (pres != 0.0f) v -= pres;
     x[id] = v;
   }

@@ -95,11 +95,10 @@ class PendingIds:
 
 
 READS_IN_FLIGHT = 64
-# The kernel that keeps the penalty window on the device counts the distinct ids of a window by
-# comparing its entries with one another in LDS: quadratic in the window. Up to this many
-# entries that costs less than the trip to the host it saves; longer windows (the kernel takes
-# up to ops.PENALTY_WINDOW_MAX) are counted on the host, step by step, which is linear.
-WINDOW_ON_DEVICE_MAX = 1024
+# The longest penalty window that is kept on the device for runs of queued steps (the kernel
+# counts its distinct ids in a hash table in LDS, linear in the window); longer windows are
+# counted on the host, step by step.
+WINDOW_ON_DEVICE_MAX = ops.PENALTY_WINDOW_MAX
 
 
 class Sampler:
