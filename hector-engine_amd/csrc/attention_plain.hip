@@ -23,65 +23,87 @@
 
 #define AP_MAX_PER_LANE 8
 
+// NPL: head elements a lane holds (head_dim / 64 rounded up to 1, 2, 4 or 8)
+template <int NPL>
 struct ApState {
   float m, l;
-  float acc[AP_MAX_PER_LANE];
+  float acc[NPL];
 };
 
 // The online softmax of the keys [j_lo, j_hi] of one page (they lie in the same page), begun afresh.
 // Every multiply-add is written out as an fma: these lines are compiled into several kernels,
 // and the compiler would otherwise be free to fuse each copy its own way.
-template <typename T>
-__device__ __forceinline__ void ap_page(ApState& st, const float (&qv)[AP_MAX_PER_LANE], const T* kpool,
+template <typename T, int NPL>
+__device__ __forceinline__ void ap_page(ApState<NPL>& st, const float (&qv)[NPL], const T* kpool,
                                         const T* vpool, int page, int num_pages, int KVH, int kvh, int hd,
                                         int j_lo, int j_hi, float scale, int lane, int npl) {
   st.m = -INFINITY;
   st.l = 0.f;
 #pragma unroll
-  for (int i = 0; i < AP_MAX_PER_LANE; ++i) st.acc[i] = 0.f;
+  for (int i = 0; i < NPL; ++i) st.acc[i] = 0.f;
   if (page < 0 || page >= num_pages) return;  // never for an admitted batch
   // the pages are stored in the MFMA kernels' operand order (cache_layout.h)
   const int64_t base = ((int64_t)page * KVH + kvh) * he_k_page_elems(hd);
   const int64_t vbase = ((int64_t)page * KVH + kvh) * he_v_page_elems(hd);
   const int KS = he_k_steps(hd), NT = he_v_tiles(hd);
-  for (int j = j_lo; j <= j_hi; ++j) {
-    const int off = j & (HE_PAGE_TOKENS - 1);
-    float part = 0.f;
+  // Four keys at a time: their key and value elements are asked for together, ahead of the chain of
+  // the softmax, which then takes the keys one by one in ascending position as before (a key at a
+  // time, each load was waited for before the next was asked for: 1 us a key).
+  constexpr int GROUP = 4;
+  for (int j0 = j_lo; j0 <= j_hi; j0 += GROUP) {
+    float kv[GROUP][NPL], vv[GROUP][NPL];
 #pragma unroll
-    for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
-      const int d = lane + i * HE_WAVE;
-      if (i < npl && d < hd) part = fmaf(qv[i], to_float(kpool[base + he_k_index(off, d, KS)]), part);
-    }
-    const float s = wave_sum(part) * scale;
-    const float m_new = fmaxf(st.m, s);
-    const float alpha = expf(st.m - m_new);
-    const float w = expf(s - m_new);
-    st.l = fmaf(st.l, alpha, w);
+    for (int g = 0; g < GROUP; ++g) {
+      const int off = min(j0 + g, j_hi) & (HE_PAGE_TOKENS - 1);
 #pragma unroll
-    for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
-      const int d = lane + i * HE_WAVE;
-      if (i < npl && d < hd) st.acc[i] = fmaf(st.acc[i], alpha, w * to_float(vpool[vbase + he_v_index(off, d, NT)]));
+      for (int i = 0; i < NPL; ++i) {
+        const int d = lane + i * HE_WAVE;
+        const bool has = i < npl && d < hd;
+        kv[g][i] = has ? to_float(kpool[base + he_k_index(off, d, KS)]) : 0.f;
+        vv[g][i] = has ? to_float(vpool[vbase + he_v_index(off, d, NT)]) : 0.f;
+      }
     }
-    st.m = m_new;
+#pragma unroll
+    for (int g = 0; g < GROUP; ++g) {
+      if (j0 + g > j_hi) break;
+      float part = 0.f;
+#pragma unroll
+      for (int i = 0; i < NPL; ++i) {
+        const int d = lane + i * HE_WAVE;
+        if (i < npl && d < hd) part = fmaf(qv[i], kv[g][i], part);
+      }
+      const float s = wave_sum(part) * scale;
+      const float m_new = fmaxf(st.m, s);
+      const float alpha = expf(st.m - m_new);
+      const float w = expf(s - m_new);
+      st.l = fmaf(st.l, alpha, w);
+#pragma unroll
+      for (int i = 0; i < NPL; ++i) {
+        const int d = lane + i * HE_WAVE;
+        if (i < npl && d < hd) st.acc[i] = fmaf(st.acc[i], alpha, w * vv[g][i]);
+      }
+      st.m = m_new;
+    }
   }
 }
 
 // total <- total joined with the result of the next page (one that had keys).
-__device__ __forceinline__ void ap_join(ApState& total, const ApState& st) {
+template <int NPL>
+__device__ __forceinline__ void ap_join(ApState<NPL>& total, const ApState<NPL>& st) {
   if (!(st.m > -INFINITY)) return;
   const float m_new = fmaxf(total.m, st.m);
   const float a = total.m > -INFINITY ? expf(total.m - m_new) : 0.f;
   const float b = expf(st.m - m_new);
   total.l = fmaf(total.l, a, st.l * b);
 #pragma unroll
-  for (int i = 0; i < AP_MAX_PER_LANE; ++i) total.acc[i] = fmaf(total.acc[i], a, st.acc[i] * b);
+  for (int i = 0; i < NPL; ++i) total.acc[i] = fmaf(total.acc[i], a, st.acc[i] * b);
   total.m = m_new;
 }
 
 // grid (rows, ceil(H / 4), pages): pages == 1: the wavefront walks all pages of its query and stores
 // the result; pages > 1: it takes the page (first >> 6) + blockIdx.z alone and stores (m, l, sums)
 // into ws [row][head][pages][hd + 2], if the query has such a page.
-template <typename T>
+template <typename T, int NPL>
 __global__ __launch_bounds__(256) void attention_plain_kernel(
     T* __restrict__ out, float* __restrict__ ws, const T* __restrict__ q, const T* __restrict__ kpool,
     const T* __restrict__ vpool, const int32_t* __restrict__ positions,
@@ -112,47 +134,47 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(
   const int c_first = first >> HE_PAGE_SHIFT, c_last = p >> HE_PAGE_SHIFT;
   if (split && c_first + (int)blockIdx.z > c_last) return;
 
-  float qv[AP_MAX_PER_LANE];
+  float qv[NPL];
   const T* qrow = q + (row * H + h) * (int64_t)hd;
 #pragma unroll
-  for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
+  for (int i = 0; i < NPL; ++i) {
     const int d = lane + i * HE_WAVE;
     qv[i] = (i < npl && d < hd) ? to_float(qrow[d]) : 0.f;
   }
-  ApState st;
+  ApState<NPL> st;
   if (split) {
     const int c = c_first + blockIdx.z;
-    ap_page<T>(st, qv, kpool, vpool, pt[c], num_pages, KVH, kvh, hd, max(first, c << HE_PAGE_SHIFT),
+    ap_page<T, NPL>(st, qv, kpool, vpool, pt[c], num_pages, KVH, kvh, hd, max(first, c << HE_PAGE_SHIFT),
                min(p, (c << HE_PAGE_SHIFT) + HE_PAGE_TOKENS - 1), scale, lane, npl);
     float* w = ws + ((row * H + h) * (int64_t)gridDim.z + blockIdx.z) * (hd + 2);
 #pragma unroll
-    for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
+    for (int i = 0; i < NPL; ++i) {
       const int d = lane + i * HE_WAVE;
       if (i < npl && d < hd) w[d] = st.acc[i];
     }
     if (lane == 0) w[hd] = st.m, w[hd + 1] = st.l;
     return;
   }
-  ApState total;
+  ApState<NPL> total;
   total.m = -INFINITY;
   total.l = 0.f;
 #pragma unroll
-  for (int i = 0; i < AP_MAX_PER_LANE; ++i) total.acc[i] = 0.f;
+  for (int i = 0; i < NPL; ++i) total.acc[i] = 0.f;
   for (int c = c_first; c <= c_last; ++c) {
-    ap_page<T>(st, qv, kpool, vpool, pt[c], num_pages, KVH, kvh, hd, max(first, c << HE_PAGE_SHIFT),
+    ap_page<T, NPL>(st, qv, kpool, vpool, pt[c], num_pages, KVH, kvh, hd, max(first, c << HE_PAGE_SHIFT),
                min(p, (c << HE_PAGE_SHIFT) + HE_PAGE_TOKENS - 1), scale, lane, npl);
     ap_join(total, st);
   }
   const float inv = total.l > 0.f ? 1.f / total.l : 0.f;
 #pragma unroll
-  for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
+  for (int i = 0; i < NPL; ++i) {
     const int d = lane + i * HE_WAVE;
     if (i < npl && d < hd) o[d] = from_float<T>(total.acc[i] * inv);
   }
 }
 
 // Joins the pages' results of a split launch in ascending position. grid (rows, ceil(H / 4)).
-template <typename T>
+template <typename T, int NPL>
 __global__ __launch_bounds__(256) void attention_plain_join_kernel(
     T* __restrict__ out, const float* __restrict__ ws, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ row_seq, int H, int hd, int window, int pages) {
@@ -162,11 +184,11 @@ __global__ __launch_bounds__(256) void attention_plain_join_kernel(
   if (h >= H) return;
   T* o = out + (row * H + h) * (int64_t)hd;
   const int npl = (hd + HE_WAVE - 1) / HE_WAVE;
-  ApState total, st;
+  ApState<NPL> total, st;
   total.m = -INFINITY;
   total.l = 0.f;
 #pragma unroll
-  for (int i = 0; i < AP_MAX_PER_LANE; ++i) total.acc[i] = 0.f;
+  for (int i = 0; i < NPL; ++i) total.acc[i] = 0.f;
   if (row_seq[row] >= 0) {
     const int p = positions[row];
     const int first = window > 0 ? max(0, p + 1 - window) : 0;
@@ -174,7 +196,7 @@ __global__ __launch_bounds__(256) void attention_plain_join_kernel(
     if (count > pages) {
       // the caller's bound on the keys was too low: no part of the result may pass for one
 #pragma unroll
-      for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
+      for (int i = 0; i < NPL; ++i) {
         const int d = lane + i * HE_WAVE;
         if (i < npl && d < hd) o[d] = from_float<T>(NAN);
       }
@@ -183,7 +205,7 @@ __global__ __launch_bounds__(256) void attention_plain_join_kernel(
     for (int z = 0; z < count; ++z) {
       const float* w = ws + ((row * H + h) * (int64_t)pages + z) * (hd + 2);
 #pragma unroll
-      for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
+      for (int i = 0; i < NPL; ++i) {
         const int d = lane + i * HE_WAVE;
         st.acc[i] = (i < npl && d < hd) ? w[d] : 0.f;
       }
@@ -194,7 +216,7 @@ __global__ __launch_bounds__(256) void attention_plain_join_kernel(
   }
   const float inv = total.l > 0.f ? 1.f / total.l : 0.f;
 #pragma unroll
-  for (int i = 0; i < AP_MAX_PER_LANE; ++i) {
+  for (int i = 0; i < NPL; ++i) {
     const int d = lane + i * HE_WAVE;
     if (i < npl && d < hd) o[d] = from_float<T>(total.acc[i] * inv);
   }
@@ -238,24 +260,32 @@ extern "C" int he_attention_plain(void* out, const void* q, const void* kpool, c
   dim3 grid(rows, (H + 3) / 4, pages);
   float* ws = (float*)workspace_f32;
   hipStream_t s = (hipStream_t)stream;
-#define AP_LAUNCH(T)                                                                           \
-  attention_plain_kernel<T><<<grid, 256, 0, s>>>(                                              \
+#define AP_LAUNCH(T, NPL)                                                                      \
+  attention_plain_kernel<T, NPL><<<grid, 256, 0, s>>>(                                         \
       (T*)out, ws, (const T*)q, (const T*)kpool, (const T*)vpool, (const int32_t*)positions,   \
       (const int32_t*)row_seq, (const int32_t*)seq_slot, (const int32_t*)page_table,           \
       max_blocks, num_pages, H, KVH, hd, window, scale)
-#define AP_JOIN(T)                                                                             \
-  attention_plain_join_kernel<T><<<dim3(rows, (H + 3) / 4), 256, 0, s>>>(                      \
+#define AP_JOIN(T, NPL)                                                                        \
+  attention_plain_join_kernel<T, NPL><<<dim3(rows, (H + 3) / 4), 256, 0, s>>>(                 \
       (T*)out, ws, (const int32_t*)positions, (const int32_t*)row_seq, H, hd, window, pages)
-  if (dtype == HE_BF16)
-    AP_LAUNCH(bf16_t);
-  else
-    AP_LAUNCH(float);
+  const int npl = (hd + HE_WAVE - 1) / HE_WAVE;   // elements a lane holds: 1, 2, up to 4, up to 8
+#define AP_BY_SIZE(WHAT)                                  \
+  if (dtype == HE_BF16) {                                 \
+    if (npl <= 1) WHAT(bf16_t, 1);                        \
+    else if (npl <= 2) WHAT(bf16_t, 2);                   \
+    else if (npl <= 4) WHAT(bf16_t, 4);                   \
+    else WHAT(bf16_t, 8);                                 \
+  } else {                                                \
+    if (npl <= 1) WHAT(float, 1);                         \
+    else if (npl <= 2) WHAT(float, 2);                    \
+    else if (npl <= 4) WHAT(float, 4);                    \
+    else WHAT(float, 8);                                  \
+  }
+  AP_BY_SIZE(AP_LAUNCH)
   int rc = he_check_launch("he_attention_plain");
   if (rc || !split) return rc;
-  if (dtype == HE_BF16)
-    AP_JOIN(bf16_t);
-  else
-    AP_JOIN(float);
+  AP_BY_SIZE(AP_JOIN)
+#undef AP_BY_SIZE
 #undef AP_LAUNCH
 #undef AP_JOIN
   return he_check_launch("he_attention_plain");

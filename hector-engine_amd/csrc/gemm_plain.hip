@@ -178,7 +178,15 @@ __global__ __launch_bounds__(256) void gemm_plain_rows_sum_kernel(
   const int n = blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
   if (n >= N) return;
   float total = 0.f;
-  for (int s = 0; s < segments; ++s) total += partial[((int64_t)s * M + m) * N + n];
+  int s = 0;
+  for (; s + 8 <= segments; s += 8) {   // eight sums on their way at a time; added in segment order
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = partial[((int64_t)(s + u) * M + m) * N + n];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) total += v[u];
+  }
+  for (; s < segments; ++s) total += partial[((int64_t)s * M + m) * N + n];
   if (bias != nullptr) total += load_param(bias, n, bias_dtype);
   C[(int64_t)m * ldc + n] = from_float<TC>(total);
 }
