@@ -156,8 +156,9 @@ class Engine:
         self.profiler = profiler.OpProfiler() if profile else None
         self.sync_each_launch = sync_each_launch
         self.use_graphs = use_graphs and self.model.graph_safe() and not profile and not sync_each_launch
-        self._buckets: dict[tuple[int, bool], _GraphBucket] = {}
-        self._uneven_sticky: dict[int, bool] = {}     # per bucket size: the flag of the step before
+        self._buckets: dict[tuple[int, tuple], _GraphBucket] = {}
+        self._hint_fns = self.model.step_hints()      # what parts want to know of a one-token step (parts/base.py)
+        self._hints_before: dict[int, tuple] = {}     # per bucket size: the hints of the step before
         self.graph_step_rows = graph_step_rows
         self._plans: collections.OrderedDict[tuple, _GraphBucket] = collections.OrderedDict()
         self._pinned = [torch.empty(1 << 16, dtype=torch.int32).pin_memory() for _ in range(4)]
@@ -326,16 +327,13 @@ class Engine:
                            max_q_len=max_q_len, max_keys=self.cache.max_seq_len,
                            all_single=all_single, env=self.env, scratch=pool)
 
-    def _uneven_keys(self, entries, was: bool = False) -> bool:
-        """Whether one sequence of a one-token step has several times the keys of the others (and
-        thousands of them): the attention kernels then cut every sequence's keys across more
-        workgroups, or the long sequence would be left to a few of them. A step with the flag has a
-        graph of its own. was: the flag of the step before; it then stays up until the longest
-        sequence has fewer than three times the mean (four to raise it), so that a batch at the
-        edge does not go back and forth between two graphs."""
-        lens = [self.cache.length(e.slot) for e in entries]
-        longest = max(lens)
-        return longest >= 4096 and longest * len(lens) >= (3 if was else 4) * sum(lens)
+    def _step_hints(self, entries, before: tuple | None = None) -> tuple:
+        """What the parts' step_hint functions say of a one-token step of these entries, one value
+        per function (before: the values of the bucket's step before)."""
+        if not self._hint_fns:
+            return ()
+        lengths = [self.cache.length(e.slot) for e in entries]
+        return tuple(fn(lengths, None if before is None else before[i]) for i, fn in enumerate(self._hint_fns))
 
     def _eager_step(self, entries, all_single: bool, device_tokens=None):
         rows = sum(len(e.tokens) for e in entries)
@@ -350,7 +348,8 @@ class Engine:
             views["tokens"][:len(entries)].copy_(device_tokens)
         ctx = self._context(views, rows, len(entries), max(len(e.tokens) for e in entries),
                             all_single, self.scratch)
-        ctx.uneven_keys = all_single and self._uneven_keys(entries)
+        if all_single:
+            ctx.hints = dict(zip(self._hint_fns, self._step_hints(entries)))
         ctx.host = {"q_lens": [len(e.tokens) for e in entries],
                     "starts": [self.cache.length(e.slot) for e in entries],
                     "slots": [e.slot for e in entries]}
@@ -363,10 +362,10 @@ class Engine:
     def _graph_step(self, entries, device_tokens=None):
         n = len(entries)
         size = 1 << (n - 1).bit_length()
-        uneven = self._uneven_sticky[size] = self._uneven_keys(entries, self._uneven_sticky.get(size, False))
-        bucket = self._buckets.get((size, uneven))
+        hints = self._hints_before[size] = self._step_hints(entries, self._hints_before.get(size))
+        bucket = self._buckets.get((size, hints))
         if bucket is None:
-            bucket = self._buckets[(size, uneven)] = _GraphBucket(size, self.device)
+            bucket = self._buckets[(size, hints)] = _GraphBucket(size, self.device)
         # every row of the bucket gets logits; padding rows are inert (row_seq -1)
         padded = [StepEntry(e.slot, e.tokens, [0]) for e in entries]
         host, idx, _ = self._pack(padded, bucket.meta, size, size)
@@ -378,7 +377,7 @@ class Engine:
         if bucket.graph is None:
             ctx = self._context(bucket.views, size, size, 1, True, bucket.pool)
             ctx.want_all = True
-            ctx.uneven_keys = uneven
+            ctx.hints = dict(zip(self._hint_fns, hints))
             ctx.padded = True
             if bucket.uses == 1:
                 # first use: run eagerly; it also sizes the bucket's scratch pool
@@ -399,7 +398,7 @@ class Engine:
                 # eagerly below: an error that is the step's own (a kernel's refusal, a part's
                 # bug) is raised again there and reaches the caller; only a failure of the
                 # capture itself ends in the fallback.
-                bucket.capture_failed = f"{size} rows{', uneven' if uneven else ''}: {exc!r}"
+                bucket.capture_failed = f"{size} rows{f', hints {hints}' if any(hints) else ''}: {exc!r}"
                 self.capture_failures.append(bucket.capture_failed)
                 self.stats["graph_capture_failures"] += 1
                 bucket.pool.frozen = False

@@ -48,6 +48,17 @@ class DecoderModel:
             todo += p.children()
         return True
 
+    def step_hints(self) -> list:
+        """The distinct step_hint functions of the model's parts, in a fixed order."""
+        found, todo = [], list(self.parts())
+        while todo:
+            p = todo.pop(0)
+            fn = getattr(p, "step_hint", None)
+            if fn is not None and fn not in found:
+                found.append(fn)
+            todo += p.children()
+        return found
+
     def tensor_specs(self):
         specs = {}
         for p in self.parts():

@@ -21,9 +21,20 @@ from .base import (BuildEnv, KVNeed, LayerCache, Mixer, PartSpec, PieceRows, Ste
 from .linear import Linear
 
 
+def keys_uneven(lengths: list[int], before=None) -> bool:
+    """Whether one sequence of a one-token step has several times the keys of the others (and
+    thousands of them): the one-token attention then cuts every sequence's keys across more
+    workgroups, or the long sequence would be left to a few of them. Once up (`before`), the flag
+    stays up until the longest sequence has fewer than three times the mean (four to raise it), so
+    that a batch at the edge does not go back and forth between two graphs."""
+    longest = max(lengths)
+    return longest >= 4096 and longest * len(lengths) >= (3 if before else 4) * sum(lengths)
+
+
 @register_part("mixer", "attention")
 class Attention(Mixer):
     accepts_normed_rows = True
+    step_hint = staticmethod(keys_uneven)
 
     def __init__(self, params: dict, prefix: str, env: BuildEnv):
         super().__init__(prefix, env)
@@ -105,12 +116,13 @@ class Attention(Mixer):
             qkv = proj(x, rows, ctx, use_bias=False)
             pieces = self.o_proj.reads_pieces(rows, ctx)       # the layout the output product reads best
             out = ctx.alloc(ops.pieces_shape(rows, H * hd) if pieces else (rows, H * hd))
-            floats = ops.attention_decode_fused_workspace_floats(rows, H, KVH, hd, ctx.max_keys, ctx.uneven_keys)
+            uneven = bool(ctx.hints.get(keys_uneven, False))
+            floats = ops.attention_decode_fused_workspace_floats(rows, H, KVH, hd, ctx.max_keys, uneven)
             ws = ctx.alloc((floats,), torch.float32) if floats else None
             ops.attention_decode_fused(out, qkv, proj.bias, cache.kpool, cache.vpool, ctx.positions,
                                        ctx.row_seq, ctx.seq_slot, cache.page_table, rot[0], rot[1],
                                        rows, H, KVH, hd, self.window, self.scale, ctx.max_keys,
-                                       writes, ws, out_pieces=pieces, spread=ctx.uneven_keys)
+                                       writes, ws, out_pieces=pieces, spread=uneven)
             return self.o_proj(PieceRows(out) if pieces else out, rows, ctx, sink=ctx.take_sink())
         # With a rotation (or no encoding) the bias is added inside the fused kernel;
         # any other encoding sees q and k with their bias already added.

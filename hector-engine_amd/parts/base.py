@@ -146,7 +146,7 @@ class StepContext:
         self.env = env
         self.scratch = scratch            # ScratchPool: alloc(shape, dtype)
         self.host = host                  # {"q_lens", "starts", "slots"}: lists per sequence, eager steps only
-        self.uneven_keys = False          # one sequence has several times the keys of the others (a hint for the grids)
+        self.hints: dict = {}             # what the parts' step_hint functions said of this step (function -> value)
         self.want_all = False             # the wanted rows are all rows, in order
         self.padded = False               # the step may hold padding rows and sequences (row_seq -1, slot -1: a step that
                                           # runs as a graph of its bucket of sizes); a part leaves such rows finite
@@ -184,6 +184,13 @@ class Part:
     # False for a part that plans on the host from ctx.host (sequence lengths as Python
     # lists); one-token steps of a model holding such a part are not captured into graphs.
     graph_safe = True
+    # A part whose launches for a one-token step should depend on what the host knows of the
+    # step names a function here: step_hint(lengths, before) -> a hashable value, where `lengths`
+    # are the cached lengths of the step's sequences and `before` is the value it gave for the
+    # bucket's step before (None at first). The engine calls each distinct function once a step
+    # (parts that name the same function share the call), runs steps with different values as
+    # different graphs, and hands the values over as ctx.hints[function]. None: no such wish.
+    step_hint = None
 
     def __init__(self, prefix: str, env: BuildEnv):
         self.prefix = prefix

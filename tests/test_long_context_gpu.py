@@ -379,7 +379,7 @@ def test_engine_one_long_sequence_among_short_ones(tmp_path):
         entries = lambda live: [StepEntry(slots[i], [reqs[i][fed[i]]], [0]) for i in live]   # noqa: E731
         for t in range(steps):
             live = list(range(len(reqs)))
-            assert eng._uneven_keys(entries(live))
+            assert eng._step_hints(entries(live)) == (True,)
             out = eng.step(entries(live))
             for j, i in enumerate(live):
                 close(out[j:j + 1], want[i][fed[i]:fed[i] + 1], dtype)
@@ -388,7 +388,7 @@ def test_engine_one_long_sequence_among_short_ones(tmp_path):
         eng.release(slots[0])
         for t in range(3):
             live = list(range(1, len(reqs)))
-            assert not eng._uneven_keys(entries(live))
+            assert eng._step_hints(entries(live)) == (False,)
             out = eng.step(entries(live))
             for j, i in enumerate(live):
                 close(out[j:j + 1], want[i][fed[i]:fed[i] + 1], dtype)

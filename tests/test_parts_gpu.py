@@ -316,7 +316,14 @@ def toys(fw):
     class RunningMeanOnDevice(parts.Mixer):
         """The same mixer, planned on the device: its state rows are found through ctx.seq_slot
         and updated by index there, so that one-token steps can be captured into HIP graphs.
-        Padding rows (row_seq -1) add zeros to a row of the state."""
+        Padding rows (row_seq -1) add zeros to a row of the state. It also names a step hint of
+        its own (whether a sequence of the step holds 30 tokens or more): the engine keys its
+        one-token graphs by it and hands the value over."""
+        seen_hints = set()
+
+        @staticmethod
+        def step_hint(lengths, before):
+            return max(lengths) >= 30
 
         def __init__(self, params, prefix, env):
             super().__init__(prefix, env)
@@ -333,6 +340,8 @@ def toys(fw):
 
         def forward(self, x, ctx, cache):
             D, rows = self.D, ctx.rows
+            if ctx.all_single:
+                type(self).seen_hints.add(ctx.hints[type(self).step_hint])
             st = cache.state.view(torch.float32)                       # [slots, D + 1]
             seq = ctx.row_seq[:rows].long()
             valid = seq >= 0
@@ -816,3 +825,7 @@ def test_state_of_fixed_size_under_graph_replay(fw, toys, tmp_path, dtype):
         for i in batch:
             close(torch.cat(got[i]), want[i], dtype)
     assert eng.stats["graph_replays"] > 40 and eng.stats["graph_captures"] >= 2
+    # the toy's own step hint reached it, with both of its values, and each value has graphs of its own
+    mixer = type(eng.model.blocks[1].mixer)
+    assert mixer.seen_hints == {False, True}
+    assert {hints[-1] for _, hints in eng._buckets} == {False, True}

@@ -21,14 +21,14 @@ def test_which_library_products_are_cut_along_k():
 
 
 def test_which_one_token_steps_count_as_uneven():
-    """The engine's flag for a step in which one sequence has several times the keys of the others: the longest
-    has 4096 or more and at least four times the mean; a single sequence, equal lengths or short ones do not count."""
-    import types
-    from hector_engine_amd.engine.engine import Engine, StepEntry
+    """The attention part's hint for a one-token step in which one sequence has several times the keys of the
+    others: the longest has 4096 or more and at least four times the mean; a single sequence, equal lengths or
+    short ones do not count."""
+    from hector_engine_amd.parts.attention import Attention, keys_uneven
+    assert Attention.step_hint is keys_uneven
 
     def uneven(lengths, was=False):
-        fake = types.SimpleNamespace(cache=types.SimpleNamespace(length=lambda slot: lengths[slot]))
-        return Engine._uneven_keys(fake, [StepEntry(i, [1], [0]) for i in range(len(lengths))], was)
+        return keys_uneven(lengths, was)
     assert uneven([30000] + [200] * 7) and uneven([30000, 30000] + [500] * 62) and uneven([4096, 10, 10, 10, 10])
     assert not uneven([30000]) and not uneven([8000] * 8) and not uneven([16000, 16000] + [1000] * 6)
     assert not uneven([4000, 10, 10, 10, 10]) and not uneven([5000, 4000, 3000])
