@@ -10,8 +10,9 @@
 // s_j = (q . k_j) * scale for j in [first, p], out = sum_j softmax(s)_j v_j,
 // kv head = h / (H / KVH)   (reference: kernels/attention.cu:155-316, :664-773, :60).
 //
-// Two launches keep that order and give the same bits: one wavefront per (query, head) that walks
-// the pages itself; or, for steps of few queries over many keys (one-token steps), a wavefront
+// Three launches keep that order and give the same bits: one wavefront per (query, head) that walks
+// the pages itself (or, in a step of many queries, per four neighbouring queries, which share what
+// they fetch); or, for steps of few queries over many keys (one-token steps), a wavefront
 // per (query, head, page) that leaves its page's result in a workspace, and a second kernel that
 // joins them in order (one wavefront alone would walk thousands of keys while the chip idles:
 // a one-token step of 28 heads over 2,048 keys took 2.4 ms so).
@@ -29,6 +30,29 @@ struct ApState {
   float m, l;
   float acc[NPL];
 };
+
+// One key joins the running softmax of a page: k, v are this lane's elements of the key and its value.
+template <int NPL>
+__device__ __forceinline__ void ap_key(ApState<NPL>& st, const float (&qv)[NPL], const float (&k)[NPL],
+                                       const float (&v)[NPL], float scale, int lane, int npl, int hd) {
+  float part = 0.f;
+#pragma unroll
+  for (int i = 0; i < NPL; ++i) {
+    const int d = lane + i * HE_WAVE;
+    if (i < npl && d < hd) part = fmaf(qv[i], k[i], part);
+  }
+  const float s = wave_sum(part) * scale;
+  const float m_new = fmaxf(st.m, s);
+  const float alpha = expf(st.m - m_new);
+  const float w = expf(s - m_new);
+  st.l = fmaf(st.l, alpha, w);
+#pragma unroll
+  for (int i = 0; i < NPL; ++i) {
+    const int d = lane + i * HE_WAVE;
+    if (i < npl && d < hd) st.acc[i] = fmaf(st.acc[i], alpha, w * v[i]);
+  }
+  st.m = m_new;
+}
 
 // The online softmax of the keys [j_lo, j_hi] of one page (they lie in the same page), begun afresh.
 // Every multiply-add is written out as an fma: these lines are compiled into several kernels,
@@ -66,23 +90,7 @@ __device__ __forceinline__ void ap_page(ApState<NPL>& st, const float (&qv)[NPL]
 #pragma unroll
     for (int g = 0; g < GROUP; ++g) {
       if (j0 + g > j_hi) break;
-      float part = 0.f;
-#pragma unroll
-      for (int i = 0; i < NPL; ++i) {
-        const int d = lane + i * HE_WAVE;
-        if (i < npl && d < hd) part = fmaf(qv[i], kv[g][i], part);
-      }
-      const float s = wave_sum(part) * scale;
-      const float m_new = fmaxf(st.m, s);
-      const float alpha = expf(st.m - m_new);
-      const float w = expf(s - m_new);
-      st.l = fmaf(st.l, alpha, w);
-#pragma unroll
-      for (int i = 0; i < NPL; ++i) {
-        const int d = lane + i * HE_WAVE;
-        if (i < npl && d < hd) st.acc[i] = fmaf(st.acc[i], alpha, w * vv[g][i]);
-      }
-      st.m = m_new;
+      ap_key<NPL>(st, qv, kv[g], vv[g], scale, lane, npl, hd);
     }
   }
 }
@@ -171,6 +179,129 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(
     const int d = lane + i * HE_WAVE;
     if (i < npl && d < hd) o[d] = from_float<T>(total.acc[i] * inv);
   }
+}
+
+// Four neighbouring queries of one sequence and head in one wavefront (whole prompts): every key
+// and value is fetched once for the four, and each query still takes its own keys [first, p] page by
+// page in the order above, so the bits are those of the kernel that takes a query at a time. A
+// group of four rows that is not four consecutive positions of one sequence (the end of a
+// sequence, padding) is taken query by query. grid (ceil(rows / 4), ceil(H / 4)).
+#define AP_ROWS 4
+template <typename T, int NPL>
+__global__ __launch_bounds__(256) void attention_plain_rows_kernel(
+    T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ kpool, const T* __restrict__ vpool,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
+    const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ page_table, int max_blocks,
+    int num_pages, int rows, int H, int KVH, int hd, int window, float scale) {
+  const int lane = threadIdx.x & (HE_WAVE - 1);
+  const int h = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (h >= H) return;
+  const int64_t row0 = (int64_t)blockIdx.x * AP_ROWS;
+  const int npl = (hd + HE_WAVE - 1) / HE_WAVE;
+  const int kvh = h / (H / KVH);
+  const int n_rows = (int)min((int64_t)AP_ROWS, rows - row0);
+  const int seq0 = row_seq[row0], p0 = positions[row0];
+  bool together = n_rows == AP_ROWS && seq0 >= 0;
+  for (int r = 1; r < n_rows; ++r) together = together && row_seq[row0 + r] == seq0 && positions[row0 + r] == p0 + r;
+  auto store = [&](int64_t row, const ApState<NPL>& total) {
+    T* o = out + (row * H + h) * (int64_t)hd;
+    const float inv = total.l > 0.f ? 1.f / total.l : 0.f;
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+      const int d = lane + i * HE_WAVE;
+      if (i < npl && d < hd) o[d] = from_float<T>(total.acc[i] * inv);
+    }
+  };
+  auto load_q = [&](float (&qv)[NPL], int64_t row) {
+    const T* qrow = q + (row * H + h) * (int64_t)hd;
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+      const int d = lane + i * HE_WAVE;
+      qv[i] = (i < npl && d < hd) ? to_float(qrow[d]) : 0.f;
+    }
+  };
+  if (!together) {
+    for (int r = 0; r < n_rows; ++r) {
+      const int64_t row = row0 + r;
+      ApState<NPL> total, st;
+      total.m = -INFINITY;
+      total.l = 0.f;
+#pragma unroll
+      for (int i = 0; i < NPL; ++i) total.acc[i] = 0.f;
+      const int seq = row_seq[row];
+      if (seq >= 0) {
+        const int p = positions[row];
+        const int first = window > 0 ? max(0, p + 1 - window) : 0;
+        const int32_t* pt = page_table + (int64_t)seq_slot[seq] * max_blocks;
+        float qv[NPL];
+        load_q(qv, row);
+        for (int c = first >> HE_PAGE_SHIFT; c <= (p >> HE_PAGE_SHIFT); ++c) {
+          ap_page<T, NPL>(st, qv, kpool, vpool, pt[c], num_pages, KVH, kvh, hd, max(first, c << HE_PAGE_SHIFT),
+                          min(p, (c << HE_PAGE_SHIFT) + HE_PAGE_TOKENS - 1), scale, lane, npl);
+          ap_join(total, st);
+        }
+      }
+      store(row, total);
+    }
+    return;
+  }
+  const int32_t* pt = page_table + (int64_t)seq_slot[seq0] * max_blocks;
+  float qv[AP_ROWS][NPL];
+  ApState<NPL> total[AP_ROWS], st[AP_ROWS];
+  int first[AP_ROWS];
+#pragma unroll
+  for (int r = 0; r < AP_ROWS; ++r) {
+    load_q(qv[r], row0 + r);
+    first[r] = window > 0 ? max(0, p0 + r + 1 - window) : 0;
+    total[r].m = -INFINITY;
+    total[r].l = 0.f;
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) total[r].acc[i] = 0.f;
+  }
+  const int KS = he_k_steps(hd), NT = he_v_tiles(hd);
+  const int p_last = p0 + AP_ROWS - 1;
+  for (int c = first[0] >> HE_PAGE_SHIFT; c <= (p_last >> HE_PAGE_SHIFT); ++c) {
+#pragma unroll
+    for (int r = 0; r < AP_ROWS; ++r) {
+      st[r].m = -INFINITY;
+      st[r].l = 0.f;
+#pragma unroll
+      for (int i = 0; i < NPL; ++i) st[r].acc[i] = 0.f;
+    }
+    const int page = pt[c];
+    if (page >= 0 && page < num_pages) {
+      const int64_t base = ((int64_t)page * KVH + kvh) * he_k_page_elems(hd);
+      const int64_t vbase = ((int64_t)page * KVH + kvh) * he_v_page_elems(hd);
+      const int j_lo = max(first[0], c << HE_PAGE_SHIFT), j_hi = min(p_last, (c << HE_PAGE_SHIFT) + HE_PAGE_TOKENS - 1);
+      constexpr int GROUP = 4;
+      for (int j0 = j_lo; j0 <= j_hi; j0 += GROUP) {
+        float kv[GROUP][NPL], vv[GROUP][NPL];
+#pragma unroll
+        for (int g = 0; g < GROUP; ++g) {
+          const int off = min(j0 + g, j_hi) & (HE_PAGE_TOKENS - 1);
+#pragma unroll
+          for (int i = 0; i < NPL; ++i) {
+            const int d = lane + i * HE_WAVE;
+            const bool has = i < npl && d < hd;
+            kv[g][i] = has ? to_float(kpool[base + he_k_index(off, d, KS)]) : 0.f;
+            vv[g][i] = has ? to_float(vpool[vbase + he_v_index(off, d, NT)]) : 0.f;
+          }
+        }
+#pragma unroll
+        for (int g = 0; g < GROUP; ++g) {
+          const int j = j0 + g;
+          if (j > j_hi) break;
+#pragma unroll
+          for (int r = 0; r < AP_ROWS; ++r)
+            if (j >= first[r] && j <= p0 + r) ap_key<NPL>(st[r], qv[r], kv[g], vv[g], scale, lane, npl, hd);
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < AP_ROWS; ++r) ap_join(total[r], st[r]);
+  }
+#pragma unroll
+  for (int r = 0; r < AP_ROWS; ++r) store(row0 + r, total[r]);
 }
 
 // Joins the pages' results of a split launch in ascending position. grid (rows, ceil(H / 4)).
@@ -281,11 +412,21 @@ extern "C" int he_attention_plain(void* out, const void* q, const void* kpool, c
     else if (npl <= 4) WHAT(float, 4);                    \
     else WHAT(float, 8);                                  \
   }
+#define AP_ROWS_LAUNCH(T, NPL)                                                                          \
+  attention_plain_rows_kernel<T, NPL><<<dim3((rows + AP_ROWS - 1) / AP_ROWS, (H + 3) / 4), 256, 0, s>>>(   \
+      (T*)out, (const T*)q, (const T*)kpool, (const T*)vpool, (const int32_t*)positions,               \
+      (const int32_t*)row_seq, (const int32_t*)seq_slot, (const int32_t*)page_table, max_blocks,       \
+      num_pages, rows, H, KVH, hd, window, scale)
+  if (!split && rows >= 64) {      // a step of many queries: four neighbours a wavefront share their keys
+    AP_BY_SIZE(AP_ROWS_LAUNCH)
+    return he_check_launch("he_attention_plain");
+  }
   AP_BY_SIZE(AP_LAUNCH)
   int rc = he_check_launch("he_attention_plain");
   if (rc || !split) return rc;
   AP_BY_SIZE(AP_JOIN)
 #undef AP_BY_SIZE
+#undef AP_ROWS_LAUNCH
 #undef AP_LAUNCH
 #undef AP_JOIN
   return he_check_launch("he_attention_plain");

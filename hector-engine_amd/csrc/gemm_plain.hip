@@ -7,8 +7,9 @@
 // The order: K is cut into segments of GP_SEG (128) consecutive k. The sum of a segment is one
 // chain of FMAs over its k in ascending order, begun at zero; the element is the segment
 // sums added one after the other in segment order, begun at zero; then the bias.
-// Two kernels keep this order and give the same bits:
-//   tiles   64 x 64 outputs a workgroup, staged through LDS, every thread 4 x 4 outputs;
+// Three kernels keep this order and give the same bits:
+//   tiles   64 x 64 outputs a workgroup, staged through LDS, every thread 4 x 4 outputs
+//           (128 x 128 and 8 x 8 for fp32 steps of 128 rows or more);
 //   rows    for up to GP_ROWS_MAX_M rows (the one-token steps): a thread owns one weight
 //           row and one segment and walks it with all M activation rows at once, so a product
 //           has N * ceil(K / GP_SEG) threads however few its rows are; the segment sums go
@@ -110,6 +111,101 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 8))) voi
       float v = total[i][j];
       if (bias != nullptr) v += load_param(bias, n, bias_dtype);
       C[m * ldc + n] = from_float<TC>(v);
+    }
+  }
+}
+
+// The same product and order in tiles of 128 x 128 outputs, every thread 8 x 8 of them (two
+// groups of four rows by two groups of four columns, 64 apart, so that the operand reads from LDS
+// are whole 16-byte reads of neighbouring lanes): four times the products per LDS read of the
+// 64 x 64 kernel. For fp32 operands and steps of 128 rows or more (whole prompts).
+#define GPW_BM 128
+#define GPW_BN 128
+__global__ __launch_bounds__(256) void gemm_plain_wide_kernel(
+    float* __restrict__ C, const float* __restrict__ A, const float* __restrict__ W,
+    const void* __restrict__ bias, int bias_dtype, int M, int N, int K, int64_t lda, int64_t ldw,
+    int64_t ldc) {
+  __shared__ __attribute__((aligned(16))) float As[GP_BK][GPW_BM + 4];
+  __shared__ __attribute__((aligned(16))) float Ws[GP_BK][GPW_BN + 4];
+  const int tid = threadIdx.x;
+  const int tx = tid & 15;  // along N
+  const int ty = tid >> 4;  // along M
+  const int m0 = blockIdx.y * GPW_BM;
+  const int n0 = blockIdx.x * GPW_BN;
+  const int lrow = tid >> 2;       // 0..63 (and + 64)
+  const int lk = (tid & 3) * 4;    // 0,4,8,12
+  float acc[8][8], total[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = 0.f, total[i][j] = 0.f;
+  const bool a_vec = m0 + GPW_BM <= M && (lda & 3) == 0 && (((uintptr_t)A) & 15) == 0;
+  const bool w_vec = n0 + GPW_BN <= N && (ldw & 3) == 0 && (((uintptr_t)W) & 15) == 0;
+  for (int k0 = 0; k0 < K; k0 += GP_BK) {
+    const bool whole = k0 + GP_BK <= K;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int r = lrow + 64 * half;
+      const int am = m0 + r, wn = n0 + r;
+      if (a_vec && whole) {
+        const float4 v = *reinterpret_cast<const float4*>(A + am * lda + k0 + lk);
+        As[lk][r] = v.x, As[lk + 1][r] = v.y, As[lk + 2][r] = v.z, As[lk + 3][r] = v.w;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int k = k0 + lk + j;
+          As[lk + j][r] = (am < M && k < K) ? A[am * lda + k] : 0.f;
+        }
+      }
+      if (w_vec && whole) {
+        const float4 v = *reinterpret_cast<const float4*>(W + wn * ldw + k0 + lk);
+        Ws[lk][r] = v.x, Ws[lk + 1][r] = v.y, Ws[lk + 2][r] = v.z, Ws[lk + 3][r] = v.w;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int k = k0 + lk + j;
+          Ws[lk + j][r] = (wn < N && k < K) ? W[wn * ldw + k] : 0.f;
+        }
+      }
+    }
+    __syncthreads();
+#define GPW_STEP(kk)                                                                               \
+  {                                                                                                \
+    const float4 a0 = *reinterpret_cast<const float4*>(&As[kk][ty * 4]);                           \
+    const float4 a1 = *reinterpret_cast<const float4*>(&As[kk][64 + ty * 4]);                      \
+    const float4 b0 = *reinterpret_cast<const float4*>(&Ws[kk][tx * 4]);                           \
+    const float4 b1 = *reinterpret_cast<const float4*>(&Ws[kk][64 + tx * 4]);                      \
+    const float a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};                           \
+    const float b[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};                           \
+    _Pragma("unroll") for (int i = 0; i < 8; ++i)                                                  \
+        _Pragma("unroll") for (int j = 0; j < 8; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);     \
+  }
+    if (whole) {
+#pragma unroll
+      for (int kk = 0; kk < GP_BK; ++kk) GPW_STEP(kk)
+    } else {
+      for (int kk = 0; kk < K - k0; ++kk) GPW_STEP(kk)
+    }
+#undef GPW_STEP
+    __syncthreads();
+    if ((k0 + GP_BK) % GP_SEG == 0 || k0 + GP_BK >= K) {   // the segment ends here
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) total[i][j] += acc[i][j], acc[i][j] = 0.f;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int m = m0 + (i >> 2) * 64 + ty * 4 + (i & 3);
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int n = n0 + (j >> 2) * 64 + tx * 4 + (j & 3);
+      if (n >= N) continue;
+      float v = total[i][j];
+      if (bias != nullptr) v += load_param(bias, n, bias_dtype);
+      C[m * ldc + n] = v;
     }
   }
 }
@@ -243,7 +339,11 @@ extern "C" int he_gemm_plain(void* C, const void* A, const void* W, const void* 
   }
   dim3 grid((N + GP_BN - 1) / GP_BN, (M + GP_BM - 1) / GP_BM);
   HE_REQUIRE(grid.y <= 65535, "he_gemm_plain: M=%d too large for one launch", M);
-  if (in_dtype == HE_F32 && out_dtype == HE_F32)
+  if (in_dtype == HE_F32 && out_dtype == HE_F32 && M >= GPW_BM) {
+    dim3 wide((N + GPW_BN - 1) / GPW_BN, (M + GPW_BM - 1) / GPW_BM);
+    gemm_plain_wide_kernel<<<wide, 256, 0, s>>>((float*)C, (const float*)A, (const float*)W, bias, bias_dtype, M, N,
+                                                K, lda, ldw, ldc);
+  } else if (in_dtype == HE_F32 && out_dtype == HE_F32)
     gemm_plain_kernel<float, float, float><<<grid, 256, 0, s>>>(
         (float*)C, (const float*)A, (const float*)W, bias, bias_dtype, M, N, K, lda, ldw, ldc);
   else if (in_dtype == HE_BF16 && out_dtype == HE_BF16)

@@ -135,6 +135,12 @@ def test_gemm_plain_for_few_rows_gives_the_bits_of_the_tile_kernel(ops, N, K):
     ops.gemm_plain(full, dev(a), dev(w), dev(b), 70)
     ref = a.double() @ w.double().T + b.double()
     assert torch.allclose(full.cpu().double(), ref, rtol=1e-5, atol=1e-6 * K)      # sums of K products of size one
+    # a step of 128 rows or more runs in tiles of 128 x 128: the same bits for the rows both hold
+    more = torch.cat([a, rnd(133, K, seed=15)])
+    wide = torch.empty(203, N, device="cuda")
+    ops.gemm_plain(wide, dev(more), dev(w), dev(b), 203)
+    assert torch.equal(wide[:70], full)
+    assert torch.allclose(wide.cpu().double(), more.double() @ w.double().T + b.double(), rtol=1e-5, atol=1e-6 * K)
     for M in (1, 2, 3, 4, 5, 8):
         floats = ops.gemm_plain_workspace_floats(M, N, K)
         assert floats == -(-K // 128) * M * N
@@ -589,6 +595,43 @@ def test_attention_plain(ops, dtype, H, KVH, hd, window):
                             1, H, KVH, hd, 0, 0.1, 128, torch.empty(ops.attention_plain_workspace_floats(1, H, hd, 128, 0),
                                                                    device="cuda"))
         assert torch.isnan(out).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,KVH,hd", [(6, 3, 48), (28, 4, 128), (2, 1, 256), (3, 1, 320)])
+@pytest.mark.parametrize("window", [0, 70])
+def test_attention_plain_of_many_queries_gives_the_bits_of_one_at_a_time(ops, dtype, H, KVH, hd, window):
+    """A step of 64 rows or more takes four neighbouring queries of a sequence in one wavefront (they
+    share the keys they fetch); a step of fewer rows takes them one by one: the same rows, cut into
+    steps of at most 40, give the same bits. Sequences that end inside a group of four, a
+    continuation (70 new tokens behind 130) and a single token are among them."""
+    lengths, q_lens = [150, 200, 67, 1, 90], [150, 70, 67, 1, 3]
+    slots, table, kpool, vpool = paged_setup(lengths, KVH, hd, dtype, 50)
+    ks = [rnd(n, KVH, hd, seed=60 + i).to(dtype) for i, n in enumerate(lengths)]
+    vs = [rnd(n, KVH, hd, seed=70 + i).to(dtype) for i, n in enumerate(lengths)]
+    fill_cache(table, slots, kpool, vpool, ks, vs)
+    qs = [rnd(m, H, hd, seed=80 + i, scale=2.0).to(dtype) for i, m in enumerate(q_lens)]
+    rows = sum(q_lens)
+    q = torch.cat(qs).reshape(rows, H * hd)
+    positions = torch.cat([torch.arange(n - m, n) for n, m in zip(lengths, q_lens)]).int()
+    row_seq = torch.cat([torch.full((m,), i) for i, m in enumerate(q_lens)]).int()
+    seq_slot = torch.tensor(slots, dtype=torch.int32)
+    scale = 1.0 / math.sqrt(hd)
+    whole = torch.full((rows, H * hd), 7.0, dtype=dtype, device="cuda")
+    ops.attention_plain(whole, dev(q), dev(kpool), dev(vpool), dev(positions), dev(row_seq), dev(seq_slot),
+                        dev(table), rows, H, KVH, hd, window, scale)
+    r = 0
+    for i, (n, m) in enumerate(zip(lengths, q_lens)):
+        want = P.attention(qs[i].double(), ks[i].double(), vs[i].double(), torch.arange(n - m, n), torch.arange(n), window)
+        tol = 3e-6 if dtype == torch.float32 else 2 ** -6
+        assert torch.allclose(whole.cpu()[r:r + m].double().reshape(want.shape), want, rtol=tol, atol=tol)
+        r += m
+    for lo in range(0, rows, 37):
+        hi = min(rows, lo + 37)
+        part = torch.full((hi - lo, H * hd), 7.0, dtype=dtype, device="cuda")
+        ops.attention_plain(part, dev(q[lo:hi].contiguous()), dev(kpool), dev(vpool), dev(positions[lo:hi].contiguous()),
+                            dev(row_seq[lo:hi].contiguous()), dev(seq_slot), dev(table), hi - lo, H, KVH, hd, window, scale)
+        assert torch.equal(part, whole[lo:hi])
 
 
 @pytest.mark.parametrize("H,KVH,hd", ATT_SHAPES + [(40, 2, 32)])
