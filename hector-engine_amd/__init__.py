@@ -13,8 +13,8 @@ bookkeeping import without a GPU.
 from __future__ import annotations
 
 __all__ = ["Engine", "StepEntry", "generate", "GenerationResult", "SamplingConfig", "Sampler",
-           "load_config", "register_architecture", "register_part", "register_init", "write_random_model",
-           "build_kernels"]
+           "load_config", "register_architecture", "register_part", "register_init", "register_route",
+           "write_random_model", "build_kernels"]
 
 _LAZY = {
     "Engine": ("engine.engine", "Engine"),
@@ -27,6 +27,7 @@ _LAZY = {
     "register_architecture": ("registry", "register_architecture"),
     "register_part": ("parts.base", "register_part"),
     "register_init": ("weights.random_init", "register_init"),
+    "register_route": ("kernels.routes", "register_route"),
     "write_random_model": ("weights.random_init", "write_random_model"),
 }
 

@@ -12,13 +12,22 @@ scale 1/sqrt(head_dim) (src/graph_builder.cpp:1328); then o = a Wo^T.
 from __future__ import annotations
 
 import math
+from dataclasses import dataclass
 
 import torch
 
-from ..kernels import kv_layout, ops
+from ..kernels import kv_layout, ops, routes
 from .base import (BuildEnv, KVNeed, LayerCache, Mixer, PartSpec, PieceRows, StepContext, TensorSpec,
                    build_part, param, register_part)
 from .linear import Linear
+
+
+@dataclass(frozen=True)
+class AttentionCase:
+    """What a route of "attention" decides by."""
+    all_single: bool    # every sequence of the step brings one token
+    fast: bool          # sizes and environment allow the MFMA kernels
+    fusable: bool       # head size and position encoding are ones the fused one-token kernel takes
 
 
 def keys_uneven(lengths: list[int], before=None) -> bool:
@@ -103,29 +112,43 @@ class Attention(Mixer):
         self.position.bind(tensors)
 
     def forward(self, x, ctx: StepContext, cache: LayerCache):
+        if cache.writes and not self.kv_projection:
+            raise RuntimeError(f"{self.prefix}: a mixer without k/v projections must read another run's cache")
+        rot = self.position.rotary()
+        case = AttentionCase(
+            all_single=ctx.all_single, fast=self.fast,
+            fusable=not self.position.custom and rot is not None
+            and ops.attention_decode_fused_ok(self.H, self.KVH, self.hd, rot[1]))
+        return routes.choose("attention", (ctx.env.dtype,), case).run(self, x, ctx, cache)
+
+    # ---- the routes' bodies ----
+
+    def _run_fused_one_token(self, x, ctx: StepContext, cache: LayerCache):
+        """One-token steps: bias, rotation, cache write and attention in one launch."""
+        rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.hd
+        proj = self.qkv if cache.writes else self.q_only
+        rot = self.position.rotary()
+        qkv = proj(x, rows, ctx, use_bias=False)
+        pieces = self.o_proj.reads_pieces(rows, ctx)       # the layout the output product reads best
+        out = ctx.alloc(ops.pieces_shape(rows, H * hd) if pieces else (rows, H * hd))
+        uneven = bool(ctx.hints.get(keys_uneven, False))
+        floats = ops.attention_decode_fused_workspace_floats(rows, H, KVH, hd, ctx.max_keys, uneven)
+        ws = ctx.alloc((floats,), torch.float32) if floats else None
+        ops.attention_decode_fused(out, qkv, proj.bias, cache.kpool, cache.vpool, ctx.positions,
+                                   ctx.row_seq, ctx.seq_slot, cache.page_table, rot[0], rot[1],
+                                   rows, H, KVH, hd, self.window, self.scale, ctx.max_keys,
+                                   cache.writes, ws, out_pieces=pieces, spread=uneven)
+        return self.o_proj(PieceRows(out) if pieces else out, rows, ctx, sink=ctx.take_sink())
+
+    def _encoded_q(self, x, ctx: StepContext, cache: LayerCache):
+        """q with bias and position encoding, after the new keys and values went into the cache."""
         rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.hd
         writes = cache.writes
-        if writes and not self.kv_projection:
-            raise RuntimeError(f"{self.prefix}: a mixer without k/v projections must read another run's cache")
         proj = self.qkv if writes else self.q_only
         rot = self.position.rotary()
-        fused_bias = not self.position.custom
-        if self.fast and ctx.all_single and fused_bias and rot is not None \
-                and ops.attention_decode_fused_ok(H, KVH, hd, rot[1]):
-            # one-token steps: bias, rotation, cache write and attention in one launch
-            qkv = proj(x, rows, ctx, use_bias=False)
-            pieces = self.o_proj.reads_pieces(rows, ctx)       # the layout the output product reads best
-            out = ctx.alloc(ops.pieces_shape(rows, H * hd) if pieces else (rows, H * hd))
-            uneven = bool(ctx.hints.get(keys_uneven, False))
-            floats = ops.attention_decode_fused_workspace_floats(rows, H, KVH, hd, ctx.max_keys, uneven)
-            ws = ctx.alloc((floats,), torch.float32) if floats else None
-            ops.attention_decode_fused(out, qkv, proj.bias, cache.kpool, cache.vpool, ctx.positions,
-                                       ctx.row_seq, ctx.seq_slot, cache.page_table, rot[0], rot[1],
-                                       rows, H, KVH, hd, self.window, self.scale, ctx.max_keys,
-                                       writes, ws, out_pieces=pieces, spread=uneven)
-            return self.o_proj(PieceRows(out) if pieces else out, rows, ctx, sink=ctx.take_sink())
         # With a rotation (or no encoding) the bias is added inside the fused kernel;
         # any other encoding sees q and k with their bias already added.
+        fused_bias = not self.position.custom
         qkv = proj(x, rows, ctx, use_bias=not fused_bias)
         if not fused_bias:
             q_cols, kv_cols = H * hd, KVH * hd
@@ -137,32 +160,58 @@ class Attention(Mixer):
         ops.qkv_rope_cache(q, cache.kpool, cache.vpool, qkv, H * hd, KVH * hd,
                            proj.bias if fused_bias else None, ctx.positions, ctx.row_seq,
                            ctx.seq_slot, cache.page_table, inv_freq, r, rows, H, KVH, hd, writes)
+        return q
+
+    def _run_plain(self, x, ctx: StepContext, cache: LayerCache):
+        """The plain kernel: one fixed order per (query, head), in the precision of the cache."""
+        rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.hd
+        q = self._encoded_q(x, ctx, cache)
         out = ctx.alloc((rows, H * hd))
-        if not self.fast:
-            floats = ops.attention_plain_workspace_floats(rows, H, hd, ctx.most_keys, self.window)
-            ws = ctx.alloc((floats,), torch.float32) if floats else None
-            ops.attention_plain(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
-                                ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,
-                                self.scale, ctx.most_keys, ws)
-        elif ctx.all_single:
-            floats = ops.attention_decode_workspace_floats(rows, H, KVH, hd, ctx.max_keys)
-            ws = ctx.alloc((max(floats, 1),), torch.float32)
-            ops.attention_decode(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
-                                 ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,
-                                 self.scale, ctx.max_keys, ws)
-        else:
-            # few queries against many keys (a continuation of a long sequence): the keys in parts
-            most = ctx.most_keys
-            if self.window > 0:
-                most = min(most, self.window + ctx.max_q_len)
-            parts = ops.attention_prefill_parts(ctx.num_seqs, ctx.max_q_len, H, hd, most)
-            ws = ctx.alloc((ops.attention_prefill_workspace_floats(rows, H, hd, parts),), torch.float32) \
-                if parts > 1 else None
-            if ctx.padded:
-                # the prompt kernels write the rows of sequences only: padding rows hold zeros (their
-                # parts too, whose join then gives zeros), never what the buffer held before
-                (ws if ws is not None else out).zero_()
-            ops.attention_prefill(out, q, cache.kpool, cache.vpool, ctx.cu_seqlens, ctx.seq_slot,
-                                  ctx.seq_start, cache.page_table, ctx.num_seqs, ctx.max_q_len,
-                                  rows, H, KVH, hd, self.window, self.scale, parts=parts, workspace=ws)
+        floats = ops.attention_plain_workspace_floats(rows, H, hd, ctx.most_keys, self.window)
+        ws = ctx.alloc((floats,), torch.float32) if floats else None
+        ops.attention_plain(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
+                            ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,
+                            self.scale, ctx.most_keys, ws)
         return self.o_proj(out, rows, ctx, sink=ctx.take_sink())
+
+    def _run_mfma_one_token(self, x, ctx: StepContext, cache: LayerCache):
+        """One-token steps of the head sizes and encodings the fused kernel does not take."""
+        rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.hd
+        q = self._encoded_q(x, ctx, cache)
+        out = ctx.alloc((rows, H * hd))
+        floats = ops.attention_decode_workspace_floats(rows, H, KVH, hd, ctx.max_keys)
+        ws = ctx.alloc((max(floats, 1),), torch.float32)
+        ops.attention_decode(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
+                             ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,
+                             self.scale, ctx.max_keys, ws)
+        return self.o_proj(out, rows, ctx, sink=ctx.take_sink())
+
+    def _run_mfma_prompt(self, x, ctx: StepContext, cache: LayerCache):
+        """Prompt steps and mixed steps."""
+        rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.hd
+        q = self._encoded_q(x, ctx, cache)
+        out = ctx.alloc((rows, H * hd))
+        # few queries against many keys (a continuation of a long sequence): the keys in parts
+        most = ctx.most_keys
+        if self.window > 0:
+            most = min(most, self.window + ctx.max_q_len)
+        parts = ops.attention_prefill_parts(ctx.num_seqs, ctx.max_q_len, H, hd, most)
+        ws = ctx.alloc((ops.attention_prefill_workspace_floats(rows, H, hd, parts),), torch.float32) \
+            if parts > 1 else None
+        if ctx.padded:
+            # the prompt kernels write the rows of sequences only: padding rows hold zeros (their
+            # parts too, whose join then gives zeros), never what the buffer held before
+            (ws if ws is not None else out).zero_()
+        ops.attention_prefill(out, q, cache.kpool, cache.vpool, ctx.cu_seqlens, ctx.seq_slot,
+                              ctx.seq_start, cache.page_table, ctx.num_seqs, ctx.max_q_len,
+                              rows, H, KVH, hd, self.window, self.scale, parts=parts, workspace=ws)
+        return self.o_proj(out, rows, ctx, sink=ctx.take_sink())
+
+
+_BF16 = (torch.bfloat16,)
+routes.register_route("attention", _BF16, "fused_one_token",
+                      lambda c: c.fast and c.all_single and c.fusable, Attention._run_fused_one_token)
+routes.register_route("attention", _BF16, "plain", lambda c: not c.fast, Attention._run_plain)
+routes.register_route("attention", _BF16, "mfma_one_token", lambda c: c.all_single, Attention._run_mfma_one_token)
+routes.register_route("attention", _BF16, "mfma_prompt", lambda c: True, Attention._run_mfma_prompt)
+routes.register_route("attention", (torch.float32,), "plain", lambda c: True, Attention._run_plain)

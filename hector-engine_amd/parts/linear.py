@@ -1,6 +1,8 @@
 """The linear layer all parts share: y[M,N] = x[M,K] . W[N,K]^T (+ bias).
 
-Which kernel runs is decided by precision and row count:
+Which kernel runs is looked up in the table of kernel routes (kernels.routes) under
+("linear", (weight dtype, activation dtype)) with the step's row count; the routes this file
+registers:
   float32 weights          -> the plain FMA kernel (fixed summation order per element);
                               a weight that was stored in 32-bit stays 32-bit and runs
                               through it also under bfloat16 activations
@@ -29,10 +31,23 @@ the gated product) writes so after asking reads_pieces().
 """
 from __future__ import annotations
 
+from dataclasses import dataclass
+
 import torch
 
-from ..kernels import library_tuning, ops, profiler
+from ..kernels import library_tuning, ops, profiler, routes
 from .base import NormedRows, PieceRows, ResidualSink, StepContext
+
+BF16, F32 = torch.bfloat16, torch.float32
+
+
+@dataclass(frozen=True)
+class ProductCase:
+    """What a route of "linear" decides by."""
+    rows: int
+    N: int
+    K: int
+    fast: bool          # the environment allows the MFMA kernels and the library
 
 
 def _operand(x):
@@ -54,15 +69,19 @@ class Linear:
         self.out_features, self.in_features = weight.shape
         self._plans: dict[bool, tuple[int, int]] = {}
 
-    def _mfma_rows(self, rows: int, ctx: StepContext, act: torch.dtype) -> bool:
-        """Whether one of the MFMA kernels of this library runs this product."""
-        K = self.weight.shape[1]
-        return (self.weight.dtype == torch.bfloat16 and act == torch.bfloat16
-                and ctx.env.fast_kernels and K % 8 == 0 and 0 < rows <= ops.ROWS_MAX_M)
+    def route(self, rows: int, ctx: StepContext, act: torch.dtype) -> routes.Route:
+        """The kernel route of this product at this many rows of this activation dtype."""
+        N, K = self.weight.shape
+        return routes.choose("linear", (self.weight.dtype, act), ProductCase(rows, N, K, ctx.env.fast_kernels))
+
+    def _has(self, trait: str, rows: int, ctx: StepContext, act: torch.dtype) -> bool:
+        if not routes.routes_of("linear", (self.weight.dtype, act)):
+            return False
+        return trait in self.route(rows, ctx, act).traits
 
     def reads_pieces(self, rows: int, ctx: StepContext) -> bool:
         """Whether bf16 input rows may come piece-major (PieceRows)."""
-        return self._mfma_rows(rows, ctx, torch.bfloat16)
+        return self._has("pieces", rows, ctx, BF16)
 
     def _plan(self, rows: int) -> tuple[int, int]:
         """(workgroups along N, K slices) of the 17-to-64-row kernel for this weight."""
@@ -76,55 +95,71 @@ class Linear:
                  sink: ResidualSink | None = None):
         """x: a tensor, NormedRows or PieceRows. With a sink the result may go into the
         residual stream directly; the call then returns None."""
-        w = self.weight
-        N, K = w.shape
         bias = self.bias if use_bias else None
+        act = _operand(x)[0]
+        return self.route(rows, ctx, act).run(self, x, rows, ctx, bias, out_dtype or act, out, sink)
+
+    # ---- the routes' bodies ----
+
+    def _run_mfma(self, x, rows, ctx, bias, out_dtype, out, sink):
+        """Up to 64 rows of bf16: the block-split kernel (up to 16 rows) or the rows kernel."""
+        w = self.weight
+        N = w.shape[0]
         act, a, scale, pieces = _operand(x)
-        out_dtype = out_dtype or act
-        if self._mfma_rows(rows, ctx, act):
-            if sink is not None and out is None and out_dtype == act \
-                    and sink.stream.rows == rows and sink.stream.resid.shape[-1] == N:
-                return self._into_residual(x, bias, rows, ctx, sink)
-            if out is None:
-                out = ctx.alloc((rows, N), out_dtype)
-            if rows <= ops.BLOCKSPLIT_PIECES_MAX_M:
-                ops.gemm_blocksplit(out, a, w, bias, rows, row_scale=scale, x_pieces=pieces)
-                return out
-            splits = self._plan(rows)[1]
-            if splits == 1:
-                ops.gemm_rows(out, None, a, w, bias, rows, row_scale=scale, x_pieces=pieces)
-                return out
-            partial = ctx.alloc((splits, rows, N), torch.float32)
-            ops.gemm_rows(None, partial, a, w, None, rows, row_scale=scale, x_pieces=pieces)
-            ops.splitk_reduce(out, partial, bias, rows, splits)
+        if sink is not None and out is None and out_dtype == act \
+                and sink.stream.rows == rows and sink.stream.resid.shape[-1] == N:
+            return self._into_residual(x, bias, rows, ctx, sink)
+        if out is None:
+            out = ctx.alloc((rows, N), out_dtype)
+        if rows <= ops.BLOCKSPLIT_PIECES_MAX_M:
+            ops.gemm_blocksplit(out, a, w, bias, rows, row_scale=scale, x_pieces=pieces)
             return out
+        splits = self._plan(rows)[1]
+        if splits == 1:
+            ops.gemm_rows(out, None, a, w, bias, rows, row_scale=scale, x_pieces=pieces)
+            return out
+        partial = ctx.alloc((splits, rows, N), torch.float32)
+        ops.gemm_rows(None, partial, a, w, None, rows, row_scale=scale, x_pieces=pieces)
+        ops.splitk_reduce(out, partial, bias, rows, splits)
+        return out
+
+    def _dense(self, x, rows, ctx, out_dtype, out):
+        """(x as a plain tensor, the result buffer) for the routes that read row-major rows."""
         if isinstance(x, PieceRows):
             raise TypeError("Linear: piece-major rows for a product that does not read them (ask reads_pieces)")
         if isinstance(x, NormedRows):
             x = x.tensor(ctx)
-        if rows == 0:
-            return out if out is not None else ctx.alloc((0, N), out_dtype)
         if out is None:
-            out = ctx.alloc((rows, N), out_dtype)
-        if w.dtype == torch.float32:
-            if act == torch.float32:
-                if out_dtype != torch.float32:
-                    raise TypeError("float32 activations give float32 outputs")
-                self._plain(out, x, bias, rows, ctx)
-                return out
-            # weight kept in 32-bit under bfloat16 activations
-            x32 = ctx.alloc((rows, K), torch.float32)
-            x32.copy_(x[:rows])
-            y32 = out if out_dtype == torch.float32 else ctx.alloc((rows, N), torch.float32)
-            self._plain(y32, x32, bias, rows, ctx)
-            if y32 is not out:
-                out[:rows].copy_(y32)
+            out = ctx.alloc((rows, self.weight.shape[0]), out_dtype)
+        return x, out
+
+    def _run_plain(self, x, rows, ctx, bias, out_dtype, out, sink):
+        """The plain kernel (fixed summation order) in the precision of its operands."""
+        x, out = self._dense(x, rows, ctx, out_dtype, out)
+        if rows == 0:
             return out
-        if w.dtype != torch.bfloat16 or act != torch.bfloat16:
-            raise TypeError(f"Linear: weight {w.dtype} with activations {act} is not supported")
-        if not ctx.env.fast_kernels or K % 8 != 0:
-            # the plain kernel also under bfloat16; the MFMA kernels take K in steps of 8
-            self._plain(out, x, bias, rows, ctx)
+        if x.dtype == torch.float32 and out_dtype != torch.float32:
+            raise TypeError("float32 activations give float32 outputs")
+        self._plain(out, x, bias, rows, ctx)
+        return out
+
+    def _run_plain_widened(self, x, rows, ctx, bias, out_dtype, out, sink):
+        """A weight kept in 32-bit under bfloat16 activations: the rows widened, the plain kernel."""
+        x, out = self._dense(x, rows, ctx, out_dtype, out)
+        if rows == 0:
+            return out
+        N, K = self.weight.shape
+        x32 = ctx.alloc((rows, K), torch.float32)
+        x32.copy_(x[:rows])
+        y32 = out if out_dtype == torch.float32 else ctx.alloc((rows, N), torch.float32)
+        self._plain(y32, x32, bias, rows, ctx)
+        if y32 is not out:
+            out[:rows].copy_(y32)
+        return out
+
+    def _run_library(self, x, rows, ctx, bias, out_dtype, out, sink):
+        x, out = self._dense(x, rows, ctx, out_dtype, out)
+        if rows == 0:
             return out
         if library_tuning.enabled() and not library_tuning.worth_tuning(rows):
             with library_tuning.no_new_tuning():
@@ -213,7 +248,7 @@ class Linear:
 
     def gated_silu_rows(self, rows: int, ctx: StepContext, act: torch.dtype) -> bool:
         """Whether gated_silu applies to this many rows of this dtype."""
-        return self._mfma_rows(rows, ctx, act) and self.weight.shape[0] % 2 == 0
+        return self._has("gated", rows, ctx, act) and self.weight.shape[0] % 2 == 0
 
     def gated_silu(self, x, rows: int, ctx: StepContext, out: torch.Tensor,
                    out_pieces: bool = False) -> None:
@@ -242,3 +277,15 @@ class Linear:
     def gated_pieces(self, rows: int) -> bool:
         """Whether gated_silu can write its result piece-major at this many rows."""
         return rows <= ops.BLOCKSPLIT_PIECES_MAX_M or self._plan(rows)[1] == 1
+
+
+def _mfma_takes(case: ProductCase) -> bool:
+    # the MFMA kernels take K in steps of 8
+    return case.fast and case.K % 8 == 0 and 0 < case.rows <= ops.ROWS_MAX_M
+
+
+routes.register_route("linear", (BF16, BF16), "mfma", _mfma_takes, Linear._run_mfma, traits=("pieces", "gated"))
+routes.register_route("linear", (BF16, BF16), "plain", lambda c: not c.fast or c.K % 8 != 0, Linear._run_plain)
+routes.register_route("linear", (BF16, BF16), "library", lambda c: True, Linear._run_library)
+routes.register_route("linear", (F32, F32), "plain", lambda c: True, Linear._run_plain)
+routes.register_route("linear", (F32, BF16), "plain_widened", lambda c: True, Linear._run_plain_widened)

@@ -241,6 +241,37 @@ def test_a_weight_stored_in_32_bit_stays_so_under_bfloat16(fw):
     assert torch.allclose(out.cpu().double(), want, rtol=2 ** -7, atol=2 ** -7)
 
 
+def test_a_kernel_route_registered_from_outside_is_the_one_that_runs(fw):
+    """Another kernel for a product is added by registering a route: here one in front of the
+    others that takes three rows of a 40-wide weight, counts its calls and runs the plain kernel.
+    The Linear part is not edited for it; other sizes keep their routes."""
+    from hector_engine_amd.kernels import routes
+    from hector_engine_amd.parts.linear import Linear
+    env = env_for(fw, torch.bfloat16)
+    calls = []
+
+    def run(lin, x, rows, ctx, bias, out_dtype, out, sink):
+        calls.append(rows)
+        return Linear._run_plain(lin, x, rows, ctx, bias, out_dtype, out, sink)
+    key = (torch.bfloat16, torch.bfloat16)
+    routes.register_route("linear", key, "toy_three_rows", lambda c: c.rows == 3 and c.N == 40, run, before="mfma")
+    try:
+        w, b = rnd(40, 48, seed=1, scale=0.1).to(torch.bfloat16), rnd(40, seed=2).to(torch.bfloat16)
+        lin = Linear(w.cuda(), b.cuda())
+        for rows in (3, 5):
+            ctx = make_ctx(fw, env, [rows], [0], [0])
+            assert lin.route(rows, ctx, torch.bfloat16).name == ("toy_three_rows" if rows == 3 else "mfma")
+            assert not lin.reads_pieces(3, ctx) and lin.reads_pieces(5, ctx)
+            x = rnd(rows, 48, seed=3).to(torch.bfloat16)
+            out = lin(x.cuda(), rows, ctx)
+            want = x.double() @ w.double().T + b.double()
+            assert torch.allclose(out.cpu().double(), want, rtol=2 ** -7, atol=2 ** -7)
+        assert calls == [3]
+    finally:
+        routes.unregister_route("linear", key, "toy_three_rows")
+    assert [r.name for r in routes.routes_of("linear", key)] == ["mfma", "plain", "library"]
+
+
 @pytest.mark.parametrize("rows", [65, 200, 512, 513])
 @pytest.mark.parametrize("N,K,bias", [(72, 8192, True), (300, 9024, False), (40, 8200, True)])
 def test_a_long_k_product_in_slices_through_the_library(fw, rows, N, K, bias):

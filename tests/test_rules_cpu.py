@@ -1,8 +1,70 @@
-"""Host-side rules that choose how a step runs: which library products are cut along K, which
-one-token steps count as uneven."""
+"""Host-side rules that choose how a step runs: the table of kernel routes, which library products
+are cut along K, which one-token steps count as uneven."""
 import torch
 
 import hector_engine_amd  # noqa: F401
+
+
+def test_kernel_routes_are_tried_in_order_and_say_what_is_registered():
+    """The table keyed by (operation, dtypes): the first route that takes the case wins, `before`
+    puts a narrower route in front, a name is registered once per key, unknown dtypes and a case
+    nobody takes are errors that list what there is."""
+    import pytest
+    from hector_engine_amd.kernels import routes
+    f16 = (torch.float16,)
+    routes.register_route("toy_op", f16, "general", lambda c: c < 100, lambda: "general")
+    try:
+        routes.register_route("toy_op", f16, "small", lambda c: c < 10, lambda: "small", traits=("tiny",),
+                              before="general")
+        assert [r.name for r in routes.routes_of("toy_op", f16)] == ["small", "general"]
+        assert routes.choose("toy_op", f16, 3).run() == "small" and "tiny" in routes.choose("toy_op", f16, 3).traits
+        assert routes.choose("toy_op", f16, 30).run() == "general"
+        assert routes.table()["toy_op (float16)"] == ["small", "general"]
+        with pytest.raises(ValueError, match="registered already"):
+            routes.register_route("toy_op", f16, "small", lambda c: True, lambda: None)
+        with pytest.raises(ValueError, match="'nowhere'.*not registered"):
+            routes.register_route("toy_op", f16, "other", lambda c: True, lambda: None, before="nowhere")
+        with pytest.raises(ValueError, match="none of the routes .*small.*general.*takes 1000"):
+            routes.choose("toy_op", f16, 1000)
+        with pytest.raises(TypeError, match=r"toy_op: no kernel for \(float64\); registered: \(float16\)"):
+            routes.choose("toy_op", (torch.float64,), 1)
+    finally:
+        for name in [r.name for r in routes.routes_of("toy_op", f16)]:
+            routes.unregister_route("toy_op", f16, name)
+    assert routes.routes_of("toy_op", f16) == []
+    with pytest.raises(ValueError, match="not registered"):
+        routes.unregister_route("toy_op", f16, "small")
+
+
+def test_which_route_a_product_and_an_attention_step_take():
+    """The routes the parts register: products by dtypes, row count, K and the environment;
+    attention by the cache's dtype, the step's kind and what the fused kernel takes."""
+    import pytest
+    from hector_engine_amd.kernels import routes
+    from hector_engine_amd.parts.attention import AttentionCase
+    from hector_engine_amd.parts.linear import ProductCase
+    bf, f32 = torch.bfloat16, torch.float32
+    table = routes.table()
+    assert table["linear (bfloat16, bfloat16)"] == ["mfma", "plain", "library"]
+    assert table["linear (float32, float32)"] == ["plain"] and table["linear (float32, bfloat16)"] == ["plain_widened"]
+    assert table["attention (bfloat16)"] == ["fused_one_token", "plain", "mfma_one_token", "mfma_prompt"]
+    assert table["attention (float32)"] == ["plain"]
+
+    def product(rows, K=3584, fast=True, dtypes=(bf, bf)):
+        return routes.choose("linear", dtypes, ProductCase(rows, 512, K, fast)).name
+    assert [product(r) for r in (0, 1, 16, 17, 64, 65, 2048)] == ["library"] + ["mfma"] * 4 + ["library"] * 2
+    assert product(8, K=3580) == "plain" and product(300, K=3580) == "plain"     # K not in steps of 8
+    assert product(8, fast=False) == "plain" and product(300, fast=False) == "plain"
+    assert product(8, dtypes=(f32, f32)) == "plain" and product(8, dtypes=(f32, bf)) == "plain_widened"
+    with pytest.raises(TypeError, match=r"linear: no kernel for \(float16, bfloat16\); registered: .*\(bfloat16, bfloat16\)"):
+        product(8, dtypes=(torch.float16, bf))
+
+    def attention(all_single, fast=True, fusable=True, dtype=bf):
+        return routes.choose("attention", (dtype,), AttentionCase(all_single, fast, fusable)).name
+    assert attention(True) == "fused_one_token" and attention(True, fusable=False) == "mfma_one_token"
+    assert attention(False) == "mfma_prompt" and attention(False, fusable=False) == "mfma_prompt"
+    assert attention(True, fast=False) == "plain" and attention(False, fast=False) == "plain"
+    assert attention(True, fast=False, dtype=f32) == "plain"
 
 
 def test_which_library_products_are_cut_along_k():
