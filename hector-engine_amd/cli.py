@@ -13,7 +13,8 @@ HELIOS_TOPK, HELIOS_TOPP, HELIOS_SEED, and HELIOS_CTX (helios_chat.cpp:549); a
 flag wins over its variable. Options of this library's own: --random CONFIG.json
 --seed N (random weights instead of a folder), --tokens / --tokens-file,
 --max-new-tokens, --temperature, --top-k, --top-p, --sampler-seed, --max-seq,
---slots, --dtype, --stop-ids, --no-graph, --tune-gemm, --profile, --sync-each-launch.
+--slots, --dtype, --stop-ids, --no-graph, --tune-gemm, --profile, --sync-each-launch,
+--stream (print each sequence's ids as they come).
 Without --stop-ids a sequence ends at the model's own end-of-sequence ids: `eos_token_id` of
 the folder's generation_config.json, else of its config.json.
 It prints the generated ids and the reference's closing report
@@ -84,6 +85,8 @@ def parse_args(argv: list[str]):
                     help="time every kernel with a pair of events (no HIP graphs) and print the table")
     ap.add_argument("--sync-each-launch", action="store_true",
                     help="debugging: wait for the GPU after every launch and name the op in an error")
+    ap.add_argument("--stream", action="store_true",
+                    help="print every token id as it comes ([sequence] + id), before the closing report")
     ap.add_argument("rest", nargs="*")
     ns = ap.parse_args(argv)
     rest = list(ns.rest)
@@ -177,8 +180,12 @@ def main(argv: list[str] | None = None) -> int:
     print(f"Model: {what}  ({config.architecture}, {ns.dtype})  loaded in "
           f"{(time.perf_counter() - start) * 1e3:.0f} ms")
     t0 = time.perf_counter()
+    on_token = None
+    if ns.stream:
+        def on_token(i, tok):
+            print(f"[{i}] + {tok}", flush=True)
     results = he.generate(engine, prompts, max_new_tokens=max_tokens, sampling=sampling,
-                          stop_ids=stop_ids, batch_size=slots)
+                          stop_ids=stop_ids, batch_size=slots, on_token=on_token)
     total_ms = (time.perf_counter() - t0) * 1e3
     for i, r in enumerate(results):
         print(f"[{i}] prompt {r.prompt_tokens} tokens -> {len(r.tokens)} tokens ({r.finish_reason}): "

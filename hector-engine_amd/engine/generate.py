@@ -74,7 +74,8 @@ RUN_OF_STEPS = 8
 def generate(engine, prompts: list[list[int]], *, max_new_tokens: int = 100, sampling=None,
              stop_ids=None, include_stop: bool = False, batch_size: int | None = None,
              cancel: Callable[[], bool] | None = None, sample_fn=None, sampler=None,
-             run_of_steps: int = RUN_OF_STEPS) -> list[GenerationResult]:
+             run_of_steps: int = RUN_OF_STEPS, on_token: Callable[[int, int], None] | None = None,
+             on_prefill: Callable[[list[int], float], None] | None = None) -> list[GenerationResult]:
     """Generates for every prompt; returns results in the order of `prompts`.
 
     stop_ids: the token ids that end a sequence; None: the model's own (engine.stop_ids: the
@@ -83,6 +84,12 @@ def generate(engine, prompts: list[list[int]], *, max_new_tokens: int = 100, sam
     sampler: an object with the library Sampler's interface (config, sample, sample_device,
     uniforms_device, read_later) in place of one made from `sampling`; sample_fn: a plain
     function (logits, requests, steps, contexts) -> ids, which runs step by step.
+
+    on_token(request index, token) is called for every token that becomes part of a result, in
+    the order of each sequence (the reference hands text out as it comes through its on_text
+    callback: src/inference_session.cpp:636-645; here the ids); with queued steps the tokens of a
+    run arrive together when the run has been read. on_prefill(request indices, ms) is called
+    once per batch after its prompt step (:603).
 
     run_of_steps: with a sampler, up to so many one-token steps are queued at a time, each
     step's ids going into the next on the device (and into the penalty windows, which then live
@@ -125,7 +132,7 @@ def generate(engine, prompts: list[list[int]], *, max_new_tokens: int = 100, sam
                 raise RuntimeError("the cache holds other sequences and no request fits beside them")
             continue
         _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, include_stop,
-                   cancel, sample_fn, sampler, run_of_steps)
+                   cancel, sample_fn, sampler, run_of_steps, on_token, on_prefill)
     return results
 
 
@@ -167,7 +174,7 @@ def _run_of_steps(engine, sampler, slots: list[int], tokens: list[int], seqs: li
 
 
 def _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, include_stop, cancel,
-               sample_fn, sampler=None, run_of_steps: int = 1) -> None:
+               sample_fn, sampler=None, run_of_steps: int = 1, on_token=None, on_prefill=None) -> None:
     slots = {i: engine.acquire() for i in admitted}
     out: dict[int, list[int]] = {i: [] for i in admitted}
     t0 = time.perf_counter()
@@ -176,6 +183,8 @@ def _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, inc
         active = list(admitted)
         tokens = sample_fn(logits, active, [0] * len(active), [out[i] for i in active])
         prefill_ms = (time.perf_counter() - t0) * 1e3
+        if on_prefill is not None:
+            on_prefill(list(admitted), prefill_ms)
         t1 = time.perf_counter()
 
         def finish(i, reason):
@@ -189,6 +198,8 @@ def _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, inc
             keep, reason = after_token(tok, len(out[i]), max_new_tokens, length, engine.max_seq_len, stop_ids)
             if keep or include_stop:
                 out[i].append(tok)
+                if on_token is not None:
+                    on_token(i, tok)
             if reason is not None:
                 finish(i, reason)
             return reason is None

@@ -229,9 +229,12 @@ def test_command_line_flags(model_dirs, plain_models, tmp_path):
     out = subprocess.run([sys.executable, exe, folder, "5,17,3", "2", "--max-seq", "1000"], capture_output=True,
                          text=True, timeout=120)
     assert out.returncode != 0 and "256 positions" in out.stderr
-    out = subprocess.run([sys.executable, exe, folder, "5,17,3", "40", "--max-seq", "16", "--dtype", "float32"],
-                         capture_output=True, text=True, timeout=120)
+    out = subprocess.run([sys.executable, exe, folder, "5,17,3", "40", "--max-seq", "16", "--dtype", "float32",
+                          "--stream"], capture_output=True, text=True, timeout=120)
     assert out.returncode == 0 and "-> 14 tokens (stop)" in out.stdout, out.stdout + out.stderr
+    # --stream: every id on a line of its own as it comes, the same ids as the closing report's
+    streamed = [line.split("+ ")[1] for line in out.stdout.splitlines() if line.startswith("[0] + ")]
+    assert len(streamed) == 14 and "(stop): " + ",".join(streamed) in out.stdout
 
 
 def test_command_line_with_the_library_tuner(model_dirs, tmp_path):

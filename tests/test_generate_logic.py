@@ -247,3 +247,21 @@ def test_cancel_is_seen_inside_a_run():
     assert r.finish_reason == "cancelled" and 1 <= len(r.tokens) <= 5
     assert r.tokens == expected([1, 2], len(r.tokens))[0]
     assert eng.cache.book.slots.available == 3 and eng.cache.free_pages == 16
+
+
+def test_tokens_are_handed_out_as_they_come():
+    """on_token sees every token of every result, per sequence in order and nothing else (a stop
+    token only with include_stop); on_prefill once per batch with its requests. Step by step and
+    with queued runs alike."""
+    prompts = [[1, 2, 3], [4] * 9, [7, 7, 7, 7, 7]]
+    stop = {expected(prompts[1], 3)[0][2]}
+    for include_stop in (False, True):
+        for kwargs in (dict(sample_fn=pick), dict(sampler=FakeSampler(), run_of_steps=8)):
+            seen = {i: [] for i in range(3)}
+            batches = []
+            res = generate(FakeEngine(slots=2), prompts, max_new_tokens=6, stop_ids=stop,
+                           include_stop=include_stop, on_token=lambda i, t: seen[i].append(t),
+                           on_prefill=lambda ids, ms: batches.append(ids), **kwargs)
+            assert [seen[i] for i in range(3)] == [r.tokens for r in res]
+            assert (res[1].tokens[-1] in stop) == include_stop
+            assert batches == [[0, 1], [2]]
