@@ -16,7 +16,6 @@ import dataclasses
 import time
 from typing import Callable
 
-import torch
 
 from ..cache.pages import blocks_for
 from .engine import StepEntry

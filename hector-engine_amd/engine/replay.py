@@ -15,8 +15,6 @@ from __future__ import annotations
 import json
 import os
 
-import numpy as np
-
 from .engine import Engine, StepEntry
 
 

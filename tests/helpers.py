@@ -1,5 +1,4 @@
 """Helpers shared by the GPU tests."""
-import numpy as np
 import torch
 
 

@@ -10,7 +10,6 @@ head, at a place chosen for what is special about it: the first key, a page's ed
 of a slice of the keys, the oldest key of a window and the one before it."""
 import math
 
-import numpy as np
 import pytest
 import torch
 

@@ -4,7 +4,6 @@ encoding and toy schedules (a layer named twice, a layer that reads another
 layer's cache) are registered here, built and stepped without a change to the
 framework's files. The toys are test fixtures, not models."""
 import dataclasses
-import math
 import os
 
 import pytest

@@ -6,7 +6,6 @@ window) fails it."""
 import math
 
 import numpy as np
-import pytest
 import torch
 
 from tests.plain import qwen2_plain as P
