@@ -39,26 +39,29 @@
 
 // Tilings measured on MI355X (graph-timed sweeps over R, U and NW at the Qwen2.5-7B, Qwen2.5-32B
 // and Qwen2-72B shapes). The rule depends on the sizes only, so a product always runs the same way.
+// What counts is how many weight rows fall to a compute unit, so the bounds on N are written in
+// rows a unit (on the MI355X's 256 units: 256 a unit = 65536 rows, the output head; 64 a unit =
+// 16384, gate||up; 16 a unit = 4096); the bounds on K are lengths of a weight row.
 static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int U, int NW) {
   BlockSplitPlan p;
   const int cus = he_cus();
   p.MT = (M + 15) / 16;
   int r, u, nw;
-  if (N >= 65536) {                 // output head
+  if (N >= 256 * cus) {             // 256 rows or more a unit: the output head
     if (M <= 8) r = 2, u = 1, nw = 8;
     else if (p.MT == 1) r = 4, u = 2, nw = 4;
     else r = 2, u = 2, nw = 4;
   } else if (K >= 8192) {           // long K
     const int groups = (N + 31) / 32, last_round = groups % cus;   // with two tiles a workgroup
-    if (N < 4096) {                 // few weight rows: one tile a workgroup, or the chip is not filled
+    if (N < 16 * cus) {             // few weight rows: one tile a workgroup, or the chip is not filled
       r = 1, u = 1, nw = p.MT == 1 ? 8 : 4;
     } else if (p.MT == 2) {
       r = 2, u = 2, nw = 4;
-    } else if (M > 8 && N >= 10240) {
+    } else if (M > 8 && N >= 40 * cus) {
       r = 4, u = 2, nw = 4;         // the activation rows are read half as often
     } else if (groups < cus) {
       r = 2, u = 1, nw = 8;         // under one workgroup a compute unit: more wavefronts each
-    } else if (groups < 1024 && last_round > 0 && last_round <= 128) {
+    } else if (groups < 4 * cus && last_round > 0 && last_round <= cus / 2) {
       r = 1, u = 1, nw = 8;         // the last round of whole tiles would fill under half of the chip:
                                     // the rows are dealt out below, 20 a workgroup for 10240
     } else if (K >= 16384) {
@@ -66,12 +69,12 @@ static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int
     } else {
       r = 2, u = 4, nw = 4;
     }
-  } else if (N >= 16384) {          // wide N (gate||up)
+  } else if (N >= 64 * cus) {       // wide N (gate||up)
     r = 2, u = 1, nw = 8;
     if (p.MT == 2 || K < 5120) u = 2, nw = 4;   // 37888 x 3584 at 8 rows: 47.7 us against 48.5 us
     else if (M > 8) r = 4;
   } else {                          // small products (q||k||v, o)
-    r = N >= 4096 ? 2 : 1;
+    r = N >= 16 * cus ? 2 : 1;
     u = p.MT == 1 && K < 5120 ? 4 : 1;   // 5120 x 5120 at 8 rows: 12.8 us unrolled once, 13.5 us four times
     nw = 8;
   }
@@ -82,7 +85,7 @@ static BlockSplitPlan blocksplit_plan(int M, int N, int K, int gated, int R, int
   // empty. A workgroup's rows are an even number: a gate stays with its up, and outputs can be
   // stored in pairs.
   int rows = 0;
-  if (R <= 0 && r <= 2 && N >= 2048 && N < 65536) {
+  if (R <= 0 && r <= 2 && N >= 8 * cus && N < 256 * cus) {
     const int rounds = (N + cus * 32 - 1) / (cus * 32);
     rows = ((N + cus * rounds - 1) / (cus * rounds) + 1) & ~1;
     r = rows > 16 ? 2 : 1;

@@ -33,23 +33,24 @@
 // others; above 32 rows one workgroup of sixteen wavefronts a compute unit); narrow ones are cut along K until the grid holds about a workgroup a compute unit.
 static RowsPlan rows_plan(int M, int N, int K, int R, int NWV, int splits) {
   RowsPlan p;
+  const int cus = he_cus();   // the bounds on N are weight rows a compute unit (256 units: 65536, 16384, 4096 rows)
   p.MT = M <= 32 ? 2 : 4;
   if (R <= 0 || NWV <= 0) {
-    if (N >= 65536) R = p.MT == 4 ? 1 : 2, NWV = p.MT == 4 ? 16 : 8;   // the output head (at 64 rows 223.6 -> 216.2 us)
-    else if (N >= 16384) R = 1, NWV = p.MT == 4 ? 16 : 8;  // gate||up: at 33 to 64 rows one workgroup a compute
+    if (N >= 256 * cus) R = p.MT == 4 ? 1 : 2, NWV = p.MT == 4 ? 16 : 8;   // the output head (at 64 rows 223.6 -> 216.2 us)
+    else if (N >= 64 * cus) R = 1, NWV = p.MT == 4 ? 16 : 8;  // gate||up: at 33 to 64 rows one workgroup a compute
                                                            // unit, so that the unit fetches the activation rows
                                                            // once, not twice (gate||up at 64 rows 61.1 -> 57.2 us;
                                                            // without that copying it takes 53.6)
-    else R = 1, NWV = (K >= 8192 || N >= 4096) ? 8 : 4;
+    else R = 1, NWV = (K >= 8192 || N >= 16 * cus) ? 8 : 4;
   }
   p.R = R;
   p.NWV = NWV;
   const int cap = 16 * R * NWV;
   int rows = cap;
-  if (N >= 16384 && splits <= 1) {
+  if (N >= 64 * cus && splits <= 1) {
     // dealt out evenly over the workgroups the chip holds at once: one a compute unit where a workgroup
     // has 256 rows (the head; sixteen wavefronts), two otherwise
-    const int slots = he_cus() * ((R == 2 && NWV == 8) || NWV == 16 ? 1 : 2);
+    const int slots = cus * ((R == 2 && NWV == 8) || NWV == 16 ? 1 : 2);
     const int rounds = (N + slots * cap - 1) / (slots * cap);
     rows = ((N + slots * rounds - 1) / (slots * rounds) + 3) & ~3;
     if (rows > cap) rows = cap;
@@ -59,7 +60,7 @@ static RowsPlan rows_plan(int M, int N, int K, int R, int NWV, int splits) {
   int s = splits;
   if (s <= 0) {
     s = 1;
-    while (p.groups * s < he_cus() * 3 / 4 && K / (2 * s) >= 512 && s < 32) s *= 2;   // 192 workgroups on 256 units
+    while (p.groups * s < cus * 3 / 4 && K / (2 * s) >= 512 && s < 32) s *= 2;   // 192 workgroups on 256 units
   }
   int ks = (K + s - 1) / s;
   ks = (ks + ROWS_KC - 1) / ROWS_KC * ROWS_KC;
