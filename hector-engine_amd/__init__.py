@@ -12,7 +12,7 @@ bookkeeping import without a GPU.
 """
 from __future__ import annotations
 
-__all__ = ["Engine", "StepEntry", "generate", "GenerationResult", "SamplingConfig", "Sampler",
+__all__ = ["Engine", "StepEntry", "generate", "GenerationResult", "Session", "SamplingConfig", "Sampler",
            "load_config", "register_architecture", "register_part", "register_init", "register_route",
            "write_random_model", "build_kernels"]
 
@@ -21,6 +21,7 @@ _LAZY = {
     "StepEntry": ("engine.engine", "StepEntry"),
     "generate": ("engine.generate", "generate"),
     "GenerationResult": ("engine.generate", "GenerationResult"),
+    "Session": ("engine.session", "Session"),
     "SamplingConfig": ("sampling.sampler", "SamplingConfig"),
     "Sampler": ("sampling.sampler", "Sampler"),
     "load_config": ("registry", "load_config"),

@@ -173,8 +173,12 @@ def _run_of_steps(engine, sampler, slots: list[int], tokens: list[int], seqs: li
 
 
 def _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, include_stop, cancel,
-               sample_fn, sampler=None, run_of_steps: int = 1, on_token=None, on_prefill=None) -> None:
-    slots = {i: engine.acquire() for i in admitted}
+               sample_fn, sampler=None, run_of_steps: int = 1, on_token=None, on_prefill=None,
+               held: dict[int, int] | None = None) -> None:
+    """One batch from its prompt step to its last sequence's end. held: request -> a slot the
+    caller holds and keeps (a session's turn: `prompts` then continue what the slots hold);
+    without it the batch takes slots of its own and gives each back as its sequence ends."""
+    slots = dict(held) if held is not None else {i: engine.acquire() for i in admitted}
     out: dict[int, list[int]] = {i: [] for i in admitted}
     t0 = time.perf_counter()
     try:
@@ -189,7 +193,9 @@ def _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, inc
         def finish(i, reason):
             results[i] = GenerationResult(out[i], reason, len(prompts[i]), prefill_ms,
                                           (time.perf_counter() - t1) * 1e3)
-            engine.release(slots.pop(i))     # the slot goes back at once
+            slot = slots.pop(i)
+            if held is None:
+                engine.release(slot)         # the slot goes back at once
 
         def decide(i, tok, length) -> bool:
             """Records a sampled token of request i whose cache held `length` tokens when it was
@@ -234,4 +240,6 @@ def _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, inc
             active = [i for i in active if going[i]]
     finally:
         for i in list(slots):
-            engine.release(slots.pop(i))
+            slot = slots.pop(i)
+            if held is None:
+                engine.release(slot)

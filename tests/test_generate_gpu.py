@@ -305,3 +305,49 @@ def test_default_stop_ids_are_the_model_folders_own(he, model_dirs, plain_models
     eng = he.Engine(folder, dtype="float32", max_tokens=1024, max_seq_len=128)
     assert eng.stop_ids == [stop[0]]
     assert he.generate(eng, prompts[:1], max_new_tokens=10)[0].tokens == want[0]
+
+
+@pytest.mark.parametrize("name", ["A", "B", "D"])
+def test_a_session_of_turns_equals_plain_on_the_whole_context(he, model_dirs, plain_models, name):
+    """A session keeps its slot: the second turn's tokens continue the first turn's context, the
+    token that ended the first turn under its budget goes in front of them, every turn samples
+    with numbers of its own (seed + turn), a stop token is neither given out nor left in the
+    cache, and a rewind to the first turn's end followed by the same turn gives the same tokens.
+    Configuration B keeps a window in some layers (a session then steps one token at a time where
+    a stop token could come)."""
+    cfg, w = plain_models[name]
+    V = cfg["vocab_size"]
+    p1, p2, p3 = rand_ids(V, 11, 1), rand_ids(V, 4, 2), rand_ids(V, 70, 3)
+    eng = he.Engine(model_dirs[name], dtype="float32", max_tokens=1024, max_slots=2, max_seq_len=512,
+                    beyond_max_positions=True)
+    with he.Session(eng, stop_ids=()) as ses:
+        r1 = ses.turn(p1, 9)
+        assert r1.tokens == P.generate(cfg, w, p1, 9) and r1.finish_reason == "max_tokens"
+        ctx = p1 + r1.tokens
+        assert ses.position == len(ctx) - 1
+        sampling = he.SamplingConfig(temperature=0.8, seed=7)
+        r2 = ses.turn(p2, 10, sampling=sampling)
+        assert r2.tokens == P.generate(cfg, w, ctx + p2, 10, temperature=0.8, seed=7 + 1)
+        at = ses.position
+        ctx2 = ctx + p2 + r2.tokens
+        # a long third turn (a prompt step of 70 tokens behind a context), then taken back and run again
+        want3 = P.generate(cfg, w, ctx2 + p3, 6)
+        assert ses.turn(p3, 6).tokens == want3
+        if any(g.window for g in eng.cache.book.groups):
+            # layers that keep a window have given pages back that the shorter sequence would read
+            from hector_engine_amd.cache import CacheError
+            with pytest.raises(CacheError, match="keeps a window"):
+                ses.rewind(at)
+        else:
+            ses.rewind(at)
+            ses.turns -= 1
+            assert ses.turn([r2.tokens[-1]] + p3, 6).tokens == want3
+    assert eng.cache.free_pages == eng.cache.num_pages
+    # a stop token: the turn ends before it, the next turn continues behind the tokens given out
+    stop = {P.generate(cfg, w, p1, 9)[4]}
+    with he.Session(eng, stop_ids=stop) as ses:
+        r = ses.turn(p1, 9)
+        want = P.generate(cfg, w, p1, 9, stop_ids=stop)
+        assert r.tokens == want and r.finish_reason == "eos" and ses.position == len(p1) + len(want)
+        assert ses.turn(p2, 5).tokens == P.generate(cfg, w, p1 + want + p2, 5, stop_ids=stop)
+    assert eng.cache.free_pages == eng.cache.num_pages

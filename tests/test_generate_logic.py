@@ -44,6 +44,10 @@ class FakeEngine:
     def length(self, s):
         return self.cache.book.length[s]
 
+    def truncate(self, s, length):
+        self.cache.book.truncate(s, length)
+        del self.history[s][length:]
+
     def step(self, entries, device_tokens=None):
         """device_tokens: as the engine takes them, the tokens of a one-token step in place of
         the entries' own (here a plain list: the fake has no device)."""
@@ -265,3 +269,84 @@ def test_tokens_are_handed_out_as_they_come():
             assert [seen[i] for i in range(3)] == [r.tokens for r in res]
             assert (res[1].tokens[-1] in stop) == include_stop
             assert batches == [[0, 1], [2]]
+
+
+def test_a_session_continues_its_slot_turn_after_turn():
+    """Turns of a session against one long run: the second turn sees the first turn's tokens, the
+    generated ones and the token that ended the first turn under its budget (sampled, not yet
+    fed: it goes in front of the second turn's tokens). Step by step and with queued runs."""
+    from hector_engine_amd.engine.session import Session
+    p1, p2 = [1, 2, 3], [9, 8]
+    for run_of_steps in (1, 8):
+        eng = FakeEngine()
+        with Session(eng, stop_ids=(), make_sampler=lambda config: FakeSampler()) as ses:
+            r1 = ses.turn(p1, 5, run_of_steps=run_of_steps)
+            assert (r1.tokens, r1.finish_reason) == expected(p1, 5) and r1.prompt_tokens == 3
+            assert ses.position == 3 + 4 and ses.unfed == [r1.tokens[-1]]
+            r2 = ses.turn(p2, 6, run_of_steps=run_of_steps)
+            assert (r2.tokens, r2.finish_reason) == expected(p1 + r1.tokens + p2, 6) and r2.prompt_tokens == 3
+            assert eng.history[ses.slot] == p1 + r1.tokens + p2 + r2.tokens[:-1]
+            seen = []
+            r3 = ses.turn([4], 3, on_token=seen.append, run_of_steps=run_of_steps)
+            assert seen == r3.tokens == expected(p1 + r1.tokens + p2 + r2.tokens + [4], 3)[0]
+            assert ses.turns == 3 and eng.cache.book.slots.available == 2
+        assert eng.cache.book.slots.available == 3 and eng.cache.free_pages == 16 and not eng.history
+
+
+def test_a_session_takes_back_what_a_late_read_stop_token_fed():
+    """With queued steps the stop token is read while the next step, which feeds it, is already
+    queued. A session keeps its slot, so that step is taken back: the slot holds the turn's tokens
+    and the generated ones before the stop token, and the next turn continues from there."""
+    from hector_engine_amd.engine.session import Session
+    p1 = [1, 2, 3]
+    stop = {expected(p1, 3)[0][2]}                     # the third token of the first turn
+    eng = FakeEngine()
+    ses = Session(eng, stop_ids=stop, make_sampler=lambda config: FakeSampler())
+    r1 = ses.turn(p1, 12, run_of_steps=8)
+    assert (r1.tokens, r1.finish_reason) == expected(p1, 12, stop) and len(r1.tokens) == 2
+    assert eng.history[ses.slot] == p1 + r1.tokens and ses.position == 5 and ses.unfed == []
+    assert max(len(step) for step in eng.log) == 1 and len(eng.log) == 1 + 3      # the prompt, two tokens, the surplus step
+    r2 = ses.turn([7], 4, run_of_steps=8)
+    assert r2.tokens == expected(p1 + r1.tokens + [7], 4, stop)[0]
+    # include_stop: the stop token is part of the result and still not fed
+    ses.reset()
+    r = ses.turn(p1, 12, include_stop=True, run_of_steps=8)
+    assert r.tokens[:-1] == r1.tokens and r.tokens[-1] in stop and eng.history[ses.slot] == p1 + r1.tokens
+    ses.close()
+    assert eng.cache.book.slots.available == 3 and eng.cache.free_pages == 16
+    with pytest.raises(RuntimeError, match="closed"):
+        ses.turn([1])
+
+
+def test_a_session_refuses_a_turn_without_room_and_takes_a_failed_turn_back():
+    from hector_engine_amd.engine.session import Session
+    eng = FakeEngine(max_blocks=1)                      # 64 positions
+    ses = Session(eng, stop_ids=(), make_sampler=lambda config: FakeSampler())
+    ses.turn([1] * 40, 4, run_of_steps=1)
+    at = ses.position
+    held = list(eng.history[ses.slot])
+    r = ses.turn([2] * 30, 4)
+    assert r.finish_reason == "context_full" and r.tokens == [] and ses.position == at and eng.history[ses.slot] == held
+    with pytest.raises(ValueError, match="empty turn"):
+        Session(eng, stop_ids=(), make_sampler=lambda config: FakeSampler()).turn([])
+    # the step after the turn's third fails: the slot holds again what it held before the turn
+    calls = {"n": 0}
+    step = eng.step
+
+    def failing(entries, device_tokens=None):
+        calls["n"] += 1
+        if calls["n"] == 3:
+            raise RuntimeError("boom")
+        return step(entries, device_tokens)
+    eng.step = failing
+    unfed = list(ses.unfed)
+    with pytest.raises(RuntimeError, match="boom"):
+        ses.turn([3, 4], 6, run_of_steps=1)
+    assert ses.position == at and eng.history[ses.slot] == held and ses.unfed == unfed
+    eng.step = step
+    r = ses.turn([3, 4], 2, run_of_steps=1)
+    assert r.tokens == expected(held + unfed + [3, 4], 2)[0]
+    # the room ends inside a turn: "stop", and the next turn is refused
+    r = ses.turn([5] * 8, 40, run_of_steps=1)
+    assert r.finish_reason == "stop" and ses.position == 64 and len(ses.unfed) == 1
+    assert ses.turn([1], 2).finish_reason == "context_full"
