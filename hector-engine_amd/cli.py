@@ -14,7 +14,9 @@ flag wins over its variable. Options of this library's own: --random CONFIG.json
 --seed N (random weights instead of a folder), --tokens / --tokens-file,
 --max-new-tokens, --temperature, --top-k, --top-p, --sampler-seed, --max-seq,
 --slots, --dtype, --stop-ids, --no-graph, --tune-gemm, --profile, --sync-each-launch,
---stream (print each sequence's ids as they come).
+--stream (print each sequence's ids as they come), --chat (one conversation: every line of
+standard input is a turn of token ids, answered with the generated ids, the context staying in
+the cache as in the reference's helios_chat; prompts given on the command line are the first turns).
 Without --stop-ids a sequence ends at the model's own end-of-sequence ids: `eos_token_id` of
 the folder's generation_config.json, else of its config.json.
 It prints the generated ids and the reference's closing report
@@ -87,6 +89,8 @@ def parse_args(argv: list[str]):
                     help="debugging: wait for the GPU after every launch and name the op in an error")
     ap.add_argument("--stream", action="store_true",
                     help="print every token id as it comes ([sequence] + id), before the closing report")
+    ap.add_argument("--chat", action="store_true",
+                    help="one conversation in one slot: each prompt, then each line of standard input, is a turn")
     ap.add_argument("rest", nargs="*")
     ns = ap.parse_args(argv)
     rest = list(ns.rest)
@@ -162,14 +166,14 @@ def main(argv: list[str] | None = None) -> int:
     else:
         config = he.load_config(model)
     prompts = gather_prompts(ns, prompt)
-    if not prompts:
+    if not prompts and not ns.chat:
         first = config.bos_token_id if getattr(config, "bos_token_id", None) is not None else 0
         prompts = [[first]]
     ctx = context_length(ns, model_spec(config).max_positions)
     sampling = he.SamplingConfig(**sampling_options(ns, temperature))
     # None: the model's own end-of-sequence ids (generation_config.json, else config.json)
     stop_ids = [int(t) for t in ns.stop_ids.split(",") if t] if ns.stop_ids is not None else None
-    slots = max(1, min(len(prompts), ns.slots or len(prompts)))
+    slots = 1 if ns.chat else max(1, min(len(prompts), ns.slots or len(prompts)))
     pages = slots * ((ctx + 63) // 64)
     start = time.perf_counter()
     source = dict(config=config, seed=ns.seed) if ns.random is not None else dict(model_dir=model)
@@ -179,6 +183,8 @@ def main(argv: list[str] | None = None) -> int:
     what = f"random weights for {ns.random}, seed {ns.seed}" if ns.random is not None else model
     print(f"Model: {what}  ({config.architecture}, {ns.dtype})  loaded in "
           f"{(time.perf_counter() - start) * 1e3:.0f} ms")
+    if ns.chat:
+        return chat(he, engine, ns, prompts, sampling, stop_ids, max_tokens)
     t0 = time.perf_counter()
     on_token = None
     if ns.stream:
@@ -199,6 +205,29 @@ def main(argv: list[str] | None = None) -> int:
     print(f"Time: {total_ms:.0f} ms")
     print(f"Speed: {gen * 1000.0 / decode_ms if decode_ms > 0 else 0.0:.1f} tok/s")
     print("============================================")
+    if ns.profile:
+        print(engine.profile_summary())
+    return 0
+
+
+def chat(he, engine, ns, first_turns, sampling, stop_ids, max_tokens) -> int:
+    """Turn after turn in one session: the prompts of the command line, then every line of standard
+    input (token ids; an empty line or the end of the input ends the conversation)."""
+    def turns():
+        yield from first_turns
+        for line in sys.stdin:
+            ids = parse_prompts(line.split("#", 1)[0])
+            if not ids:
+                return
+            yield ids[0]
+    with he.Session(engine, sampling, stop_ids) as session:
+        for n, ids in enumerate(turns()):
+            on_token = (lambda tok: print(f"[turn {n}] + {tok}", flush=True)) if ns.stream else None
+            r = session.turn(ids, max_tokens, on_token=on_token)
+            speed = len(r.tokens) * 1000.0 / r.decode_ms if r.decode_ms > 0 else 0.0
+            print(f"[turn {n}] {r.prompt_tokens} tokens in ({r.prefill_ms:.0f} ms) -> {len(r.tokens)} tokens "
+                  f"({r.finish_reason}, {speed:.1f} tok/s, context {session.position}): "
+                  + ",".join(str(t) for t in r.tokens), flush=True)
     if ns.profile:
         print(engine.profile_summary())
     return 0

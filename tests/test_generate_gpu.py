@@ -237,6 +237,23 @@ def test_command_line_flags(model_dirs, plain_models, tmp_path):
     assert len(streamed) == 14 and "(stop): " + ",".join(streamed) in out.stdout
 
 
+def test_command_line_chat(model_dirs, plain_models):
+    """--chat: the prompt of the command line is the first turn, every line of standard input a
+    further one; each answer continues the whole context."""
+    cfg, w = plain_models["A"]
+    exe = os.path.join(ROOT, "bin", "hector_generate")
+    out = subprocess.run([sys.executable, exe, model_dirs["A"], "5,17,3", "6", "--dtype", "float32", "--chat",
+                          "--stop-ids", ""], input="9,2,77\n4 4\n\n8,8\n", capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    t0 = P.generate(cfg, w, [5, 17, 3], 6)
+    t1 = P.generate(cfg, w, [5, 17, 3] + t0 + [9, 2, 77], 6)
+    t2 = P.generate(cfg, w, [5, 17, 3] + t0 + [9, 2, 77] + t1 + [4, 4], 6)
+    for n, (fed, t) in enumerate([(3, t0), (4, t1), (3, t2)]):
+        assert f"[turn {n}] {fed} tokens in" in out.stdout and "(max_tokens, " in out.stdout
+        assert "): " + ",".join(map(str, t)) in out.stdout
+    assert "[turn 3]" not in out.stdout           # the empty line ended the conversation
+
+
 def test_command_line_with_the_library_tuner(model_dirs, tmp_path):
     """--tune-gemm: tall bfloat16 products go through the library's tuner (its own process, since the
     tuner is process-wide); the same tokens as without it where the decision is clear."""
