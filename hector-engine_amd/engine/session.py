@@ -95,6 +95,25 @@ class Session:
         self.turns += 1
         return result
 
+    def feed(self, tokens: list[int]) -> bool:
+        """Puts tokens behind what the slot holds without generating (a system prompt, a turn of the
+        other side). False, with nothing touched, if they do not fit."""
+        from .engine import StepEntry
+        engine, slot = self.engine, self._slot()
+        feed = self.unfed + [int(t) for t in tokens]
+        if not feed:
+            return True
+        before = engine.length(slot)
+        if before + len(feed) > engine.max_seq_len:
+            return False
+        try:
+            engine.step([StepEntry(slot, feed, [])])
+        except BaseException:
+            self._take_back(before)
+            raise
+        self.unfed = []
+        return True
+
     def _take_back(self, length: int) -> None:
         try:
             self.engine.truncate(self.slot, length)

@@ -338,7 +338,8 @@ def test_a_session_of_turns_equals_plain_on_the_whole_context(he, model_dirs, pl
     eng = he.Engine(model_dirs[name], dtype="float32", max_tokens=1024, max_slots=2, max_seq_len=512,
                     beyond_max_positions=True)
     with he.Session(eng, stop_ids=()) as ses:
-        r1 = ses.turn(p1, 9)
+        assert ses.feed(p1[:4]) and ses.position == 4        # context without an answer, then the turn's rest
+        r1 = ses.turn(p1[4:], 9)
         assert r1.tokens == P.generate(cfg, w, p1, 9) and r1.finish_reason == "max_tokens"
         ctx = p1 + r1.tokens
         assert ses.position == len(ctx) - 1

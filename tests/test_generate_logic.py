@@ -58,6 +58,8 @@ class FakeEngine:
             self.cache.book.reserve(e.slot, new)
             self.cache.book.commit(e.slot, new)
             self.history[e.slot] += list(e.tokens) if device_tokens is None else [device_tokens[k]]
+            if not e.want:
+                continue
             assert list(e.want) == [len(e.tokens) - 1]
             h = self.history[e.slot]
             rows.append((sum(h) + len(h)) % V)
@@ -280,8 +282,9 @@ def test_a_session_continues_its_slot_turn_after_turn():
     for run_of_steps in (1, 8):
         eng = FakeEngine()
         with Session(eng, stop_ids=(), make_sampler=lambda config: FakeSampler()) as ses:
-            r1 = ses.turn(p1, 5, run_of_steps=run_of_steps)
-            assert (r1.tokens, r1.finish_reason) == expected(p1, 5) and r1.prompt_tokens == 3
+            assert ses.feed(p1[:2]) and ses.position == 2 and not ses.feed([1] * 300) and ses.position == 2
+            r1 = ses.turn(p1[2:], 5, run_of_steps=run_of_steps)
+            assert (r1.tokens, r1.finish_reason) == expected(p1, 5) and r1.prompt_tokens == 1
             assert ses.position == 3 + 4 and ses.unfed == [r1.tokens[-1]]
             r2 = ses.turn(p2, 6, run_of_steps=run_of_steps)
             assert (r2.tokens, r2.finish_reason) == expected(p1 + r1.tokens + p2, 6) and r2.prompt_tokens == 3
