@@ -31,20 +31,30 @@ struct ApState {
   float acc[NPL];
 };
 
-// One key joins the running softmax of a page: k, v are this lane's elements of the key and its value.
+// The score of one key: k holds this lane's elements of the key. It does not depend on the keys
+// before it, so the scores of a group of keys are computed side by side ahead of the chain below.
 template <int NPL>
-__device__ __forceinline__ void ap_key(ApState<NPL>& st, const float (&qv)[NPL], const float (&k)[NPL],
-                                       const float (&v)[NPL], float scale, int lane, int npl, int hd) {
+__device__ __forceinline__ float ap_score(const float (&qv)[NPL], const float (&k)[NPL], float scale, int lane,
+                                          int npl, int hd) {
   float part = 0.f;
 #pragma unroll
   for (int i = 0; i < NPL; ++i) {
     const int d = lane + i * HE_WAVE;
     if (i < npl && d < hd) part = fmaf(qv[i], k[i], part);
   }
-  const float s = wave_sum(part) * scale;
-  const float m_new = fmaxf(st.m, s);
-  const float alpha = expf(st.m - m_new);
-  const float w = expf(s - m_new);
+  return wave_sum(part) * scale;
+}
+
+// One key joins the running softmax of a page: s is its score, v this lane's elements of its value.
+// Of the two weights exp(m - m_new) and exp(s - m_new) one is exp(0) = 1: one exponential a key.
+template <int NPL>
+__device__ __forceinline__ void ap_update(ApState<NPL>& st, float s, const float (&v)[NPL], int lane, int npl,
+                                          int hd) {
+  const bool up = s > st.m;                 // the reference point moves to s
+  const float m_new = up ? s : st.m;
+  const float e = expf(up ? st.m - s : s - st.m);
+  const float alpha = up ? e : 1.f;
+  const float w = up ? 1.f : e;
   st.l = fmaf(st.l, alpha, w);
 #pragma unroll
   for (int i = 0; i < NPL; ++i) {
@@ -52,6 +62,26 @@ __device__ __forceinline__ void ap_key(ApState<NPL>& st, const float (&qv)[NPL],
     if (i < npl && d < hd) st.acc[i] = fmaf(st.acc[i], alpha, w * v[i]);
   }
   st.m = m_new;
+}
+
+#define AP_GROUP 4
+// The key and value elements of this lane for the AP_GROUP keys from j0 on (positions beyond j_hi
+// read key j_hi again: no load stands behind a condition, so the compiler counts what is in flight).
+template <typename T, int NPL>
+__device__ __forceinline__ void ap_fetch(float (&kv)[AP_GROUP][NPL], float (&vv)[AP_GROUP][NPL], const T* kpage,
+                                         const T* vpage, int j0, int j_hi, int KS, int NT, int lane, int npl,
+                                         int hd) {
+#pragma unroll
+  for (int g = 0; g < AP_GROUP; ++g) {
+    const int off = min(j0 + g, j_hi) & (HE_PAGE_TOKENS - 1);
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+      const int d = lane + i * HE_WAVE;
+      const bool has = i < npl && d < hd;
+      kv[g][i] = has ? to_float(kpage[he_k_index(off, d, KS)]) : 0.f;
+      vv[g][i] = has ? to_float(vpage[he_v_index(off, d, NT)]) : 0.f;
+    }
+  }
 }
 
 // The online softmax of the keys [j_lo, j_hi] of one page (they lie in the same page), begun afresh.
@@ -67,31 +97,29 @@ __device__ __forceinline__ void ap_page(ApState<NPL>& st, const float (&qv)[NPL]
   for (int i = 0; i < NPL; ++i) st.acc[i] = 0.f;
   if (page < 0 || page >= num_pages) return;  // never for an admitted batch
   // the pages are stored in the MFMA kernels' operand order (cache_layout.h)
-  const int64_t base = ((int64_t)page * KVH + kvh) * he_k_page_elems(hd);
-  const int64_t vbase = ((int64_t)page * KVH + kvh) * he_v_page_elems(hd);
+  const T* kpage = kpool + ((int64_t)page * KVH + kvh) * he_k_page_elems(hd);
+  const T* vpage = vpool + ((int64_t)page * KVH + kvh) * he_v_page_elems(hd);
   const int KS = he_k_steps(hd), NT = he_v_tiles(hd);
-  // Four keys at a time: their key and value elements are asked for together, ahead of the chain of
-  // the softmax, which then takes the keys one by one in ascending position as before (a key at a
-  // time, each load was waited for before the next was asked for: 1 us a key).
-  constexpr int GROUP = 4;
-  for (int j0 = j_lo; j0 <= j_hi; j0 += GROUP) {
-    float kv[GROUP][NPL], vv[GROUP][NPL];
+  // Four keys at a time, in two sets of registers: while the chain of the softmax takes the keys of
+  // one set one by one in ascending position, the elements of the next four are on their way (a key
+  // at a time, each load was waited for before the next was asked for: 1 us a key; four at a time
+  // without the second set, a wait of its own for every four: a page of 64 keys 39 us).
+  float ka[AP_GROUP][NPL], va[AP_GROUP][NPL], kb[AP_GROUP][NPL], vb[AP_GROUP][NPL];
+  ap_fetch<T, NPL>(ka, va, kpage, vpage, j_lo, j_hi, KS, NT, lane, npl, hd);
+  for (int j0 = j_lo; j0 <= j_hi; j0 += 2 * AP_GROUP) {
+    ap_fetch<T, NPL>(kb, vb, kpage, vpage, j0 + AP_GROUP, j_hi, KS, NT, lane, npl, hd);
+    float sc[AP_GROUP];
 #pragma unroll
-    for (int g = 0; g < GROUP; ++g) {
-      const int off = min(j0 + g, j_hi) & (HE_PAGE_TOKENS - 1);
+    for (int g = 0; g < AP_GROUP; ++g) sc[g] = ap_score<NPL>(qv, ka[g], scale, lane, npl, hd);
 #pragma unroll
-      for (int i = 0; i < NPL; ++i) {
-        const int d = lane + i * HE_WAVE;
-        const bool has = i < npl && d < hd;
-        kv[g][i] = has ? to_float(kpool[base + he_k_index(off, d, KS)]) : 0.f;
-        vv[g][i] = has ? to_float(vpool[vbase + he_v_index(off, d, NT)]) : 0.f;
-      }
-    }
+    for (int g = 0; g < AP_GROUP; ++g)
+      if (j0 + g <= j_hi) ap_update<NPL>(st, sc[g], va[g], lane, npl, hd);
+    ap_fetch<T, NPL>(ka, va, kpage, vpage, j0 + 2 * AP_GROUP, j_hi, KS, NT, lane, npl, hd);
 #pragma unroll
-    for (int g = 0; g < GROUP; ++g) {
-      if (j0 + g > j_hi) break;
-      ap_key<NPL>(st, qv, kv[g], vv[g], scale, lane, npl, hd);
-    }
+    for (int g = 0; g < AP_GROUP; ++g) sc[g] = ap_score<NPL>(qv, kb[g], scale, lane, npl, hd);
+#pragma unroll
+    for (int g = 0; g < AP_GROUP; ++g)
+      if (j0 + AP_GROUP + g <= j_hi) ap_update<NPL>(st, sc[g], vb[g], lane, npl, hd);
   }
 }
 
@@ -273,27 +301,36 @@ __global__ __launch_bounds__(256) void attention_plain_rows_kernel(
       const int64_t base = ((int64_t)page * KVH + kvh) * he_k_page_elems(hd);
       const int64_t vbase = ((int64_t)page * KVH + kvh) * he_v_page_elems(hd);
       const int j_lo = max(first[0], c << HE_PAGE_SHIFT), j_hi = min(p_last, (c << HE_PAGE_SHIFT) + HE_PAGE_TOKENS - 1);
-      constexpr int GROUP = 4;
-      for (int j0 = j_lo; j0 <= j_hi; j0 += GROUP) {
-        float kv[GROUP][NPL], vv[GROUP][NPL];
+      const T* kpage = kpool + base;
+      const T* vpage = vpool + vbase;
+      // two sets of registers, as in ap_page: the next four keys are on their way while these are taken
+      float ka[AP_GROUP][NPL], va[AP_GROUP][NPL], kb[AP_GROUP][NPL], vb[AP_GROUP][NPL];
+      ap_fetch<T, NPL>(ka, va, kpage, vpage, j_lo, j_hi, KS, NT, lane, npl, hd);
+      for (int j0 = j_lo; j0 <= j_hi; j0 += 2 * AP_GROUP) {
+        ap_fetch<T, NPL>(kb, vb, kpage, vpage, j0 + AP_GROUP, j_hi, KS, NT, lane, npl, hd);
+        float sc[AP_GROUP][AP_ROWS];
 #pragma unroll
-        for (int g = 0; g < GROUP; ++g) {
-          const int off = min(j0 + g, j_hi) & (HE_PAGE_TOKENS - 1);
+        for (int g = 0; g < AP_GROUP; ++g)
 #pragma unroll
-          for (int i = 0; i < NPL; ++i) {
-            const int d = lane + i * HE_WAVE;
-            const bool has = i < npl && d < hd;
-            kv[g][i] = has ? to_float(kpool[base + he_k_index(off, d, KS)]) : 0.f;
-            vv[g][i] = has ? to_float(vpool[vbase + he_v_index(off, d, NT)]) : 0.f;
-          }
-        }
+          for (int r = 0; r < AP_ROWS; ++r) sc[g][r] = ap_score<NPL>(qv[r], ka[g], scale, lane, npl, hd);
 #pragma unroll
-        for (int g = 0; g < GROUP; ++g) {
+        for (int g = 0; g < AP_GROUP; ++g) {
           const int j = j0 + g;
-          if (j > j_hi) break;
 #pragma unroll
           for (int r = 0; r < AP_ROWS; ++r)
-            if (j >= first[r] && j <= p0 + r) ap_key<NPL>(st[r], qv[r], kv[g], vv[g], scale, lane, npl, hd);
+            if (j <= j_hi && j >= first[r] && j <= p0 + r) ap_update<NPL>(st[r], sc[g][r], va[g], lane, npl, hd);
+        }
+        ap_fetch<T, NPL>(ka, va, kpage, vpage, j0 + 2 * AP_GROUP, j_hi, KS, NT, lane, npl, hd);
+#pragma unroll
+        for (int g = 0; g < AP_GROUP; ++g)
+#pragma unroll
+          for (int r = 0; r < AP_ROWS; ++r) sc[g][r] = ap_score<NPL>(qv[r], kb[g], scale, lane, npl, hd);
+#pragma unroll
+        for (int g = 0; g < AP_GROUP; ++g) {
+          const int j = j0 + AP_GROUP + g;
+#pragma unroll
+          for (int r = 0; r < AP_ROWS; ++r)
+            if (j <= j_hi && j >= first[r] && j <= p0 + r) ap_update<NPL>(st[r], sc[g][r], vb[g], lane, npl, hd);
         }
       }
     }
@@ -315,7 +352,7 @@ __global__ __launch_bounds__(256) void attention_plain_join_kernel(
   if (h >= H) return;
   T* o = out + (row * H + h) * (int64_t)hd;
   const int npl = (hd + HE_WAVE - 1) / HE_WAVE;
-  ApState<NPL> total, st;
+  ApState<NPL> total;
   total.m = -INFINITY;
   total.l = 0.f;
 #pragma unroll
@@ -333,16 +370,25 @@ __global__ __launch_bounds__(256) void attention_plain_join_kernel(
       }
       return;
     }
-    for (int z = 0; z < count; ++z) {
-      const float* w = ws + ((row * H + h) * (int64_t)pages + z) * (hd + 2);
+    // eight pages' results are asked for together and then joined one after the other in order
+    // (one at a time, every page waited for its own loads: 17 us for 33 pages)
+    constexpr int AHEAD = 8;
+    for (int z0 = 0; z0 < count; z0 += AHEAD) {
+      ApState<NPL> part[AHEAD];
 #pragma unroll
-      for (int i = 0; i < NPL; ++i) {
-        const int d = lane + i * HE_WAVE;
-        st.acc[i] = (i < npl && d < hd) ? w[d] : 0.f;
+      for (int u = 0; u < AHEAD; ++u) {
+        const float* w = ws + ((row * H + h) * (int64_t)pages + min(z0 + u, count - 1)) * (hd + 2);
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) {
+          const int d = lane + i * HE_WAVE;
+          part[u].acc[i] = (i < npl && d < hd) ? w[d] : 0.f;
+        }
+        part[u].m = w[hd];
+        part[u].l = w[hd + 1];
       }
-      st.m = w[hd];
-      st.l = w[hd + 1];
-      ap_join(total, st);
+#pragma unroll
+      for (int u = 0; u < AHEAD; ++u)
+        if (z0 + u < count) ap_join(total, part[u]);
     }
   }
   const float inv = total.l > 0.f ? 1.f / total.l : 0.f;

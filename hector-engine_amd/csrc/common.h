@@ -116,15 +116,39 @@ __device__ __forceinline__ float xor16_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// The value of lane i ^ 8, 4, 2, 1 through the data-parallel path of the vector ALU (DPP): a
+// rotation by 8 inside a row of 16 lanes; the mirror image of a half row, then of its quads;
+// permutations inside a quad. All 64 lanes must be active.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x) {
+  return __uint_as_float((unsigned)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(x), CTRL, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float lane_xor8(float x) { return dpp_move<0x128>(x); }                  // row_ror:8
+__device__ __forceinline__ float lane_xor4(float x) { return dpp_move<0x1B>(dpp_move<0x141>(x)); }  // row_half_mirror, quad_perm:[3,2,1,0]
+__device__ __forceinline__ float lane_xor2(float x) { return dpp_move<0x4E>(x); }                   // quad_perm:[2,3,0,1]
+__device__ __forceinline__ float lane_xor1(float x) { return dpp_move<0xB1>(x); }                   // quad_perm:[1,0,3,2]
+
+// Sum and maximum over the wavefront, every lane gets the result: the butterfly lane i with lane
+// i ^ 32, 16, 8, 4, 2, 1 in that order (an addition gives both lanes of a pair the same bits). Through
+// the lane swaps and DPP it is a dozen vector-ALU instructions; six __shfl_xor go through the LDS
+// crossbar one after the other (a key of the plain attention 0.6 us, most of it this sum).
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = HE_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, HE_WAVE);
+  v = xor32_sum(v);
+  v = xor16_sum(v);
+  v += lane_xor8(v);
+  v += lane_xor4(v);
+  v += lane_xor2(v);
+  v += lane_xor1(v);
   return v;
 }
 
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = HE_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, HE_WAVE));
+  v = xor32_max(v);
+  v = xor16_max(v);
+  v = fmaxf(v, lane_xor8(v));
+  v = fmaxf(v, lane_xor4(v));
+  v = fmaxf(v, lane_xor2(v));
+  v = fmaxf(v, lane_xor1(v));
   return v;
 }
 

@@ -267,6 +267,83 @@ __global__ __launch_bounds__(256) void gemm_plain_rows_kernel(
   }
 }
 
+// The same sums for 32-bit weights whose K is whole segments, with the weights fetched line by
+// line: in the kernel above the 64 lanes of a load touch 64 cache lines (each lane its own row), and
+// the rate at which a compute unit looks lines up bounds it (3.6 TB/s at the Qwen2.5-7B shape). Here
+// eight neighbouring lanes fetch the 128 bytes of one row, a load touches eight lines, and the
+// wavefront turns the tile round in LDS: 32 k of its 64 rows at a time (two such chunks on their
+// way while one is multiplied), the values go into the wavefront's own LDS region as
+// [16-byte piece][row, 65 to a piece][4], from which lane n reads the pieces of row n one after the
+// other (a read of 64 lanes is one KiB on end) and extends its chain of FMAs in ascending k. The
+// region is the wavefront's own: LDS runs a wavefront's writes and reads in program order, so no
+// barrier is needed, and the compiler keeps stores and loads that may name the same address in
+// order. (A wavefront-scope fence here kept the staging registers in scratch memory.) grid and
+// block as above.
+#define GP_TURN_ROWS 65
+template <int MT>
+__global__ __launch_bounds__(256) void gemm_plain_rows_turned_kernel(
+    float* __restrict__ partial, const float* __restrict__ A, const float* __restrict__ W, int M, int N, int K,
+    int64_t lda, int64_t ldw, int segments) {
+  __shared__ float4 turned[4][8 * GP_TURN_ROWS];
+  const int lane = threadIdx.x;
+  const int n0 = blockIdx.x * 64;
+  const int seg = __builtin_amdgcn_readfirstlane(blockIdx.y * 4 + threadIdx.y);
+  if (seg >= segments) return;
+  const int k_begin = seg * GP_SEG;
+  // load i of a chunk of 32 k: row 8 i + lane / 8 of the tile, piece lane % 8 of its 128 bytes
+  const int lrow = lane >> 3, piece = lane & 7;
+  const float* src[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) src[i] = W + (int64_t)min(n0 + 8 * i + lrow, N - 1) * ldw + k_begin + 4 * piece;
+  float4 w0[8], w1[8];   // two chunks of 32 k on their way while a third is multiplied
+#pragma unroll
+  for (int i = 0; i < 8; ++i) w0[i] = *reinterpret_cast<const float4*>(src[i]);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) w1[i] = *reinterpret_cast<const float4*>(src[i] + 32);
+  float acc[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) acc[m] = 0.f;
+  const float* arow[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) arow[m] = A + (int64_t)min(m, M - 1) * lda + k_begin;
+  float4* mine = turned[threadIdx.y];
+#define GP_TURN(WV_, C_)                                                                          \
+  {                                                                                               \
+    _Pragma("unroll") for (int i = 0; i < 8; ++i) mine[piece * GP_TURN_ROWS + 8 * i + lrow] = WV_[i]; \
+    __builtin_amdgcn_wave_barrier();                                                              \
+    _Pragma("unroll") for (int p = 0; p < 8; ++p) {                                               \
+      const float4 w4 = mine[p * GP_TURN_ROWS + lane];                                            \
+      const float w[4] = {w4.x, w4.y, w4.z, w4.w};                                                \
+      _Pragma("unroll") for (int e = 0; e < 4; ++e)                                               \
+        _Pragma("unroll") for (int m = 0; m < MT; ++m)                                            \
+          acc[m] = fmaf(arow[m][32 * (C_) + 4 * p + e], w[e], acc[m]);                            \
+    }                                                                                             \
+    __builtin_amdgcn_wave_barrier();                                                              \
+  }
+  // (the scheduler would ask for all four chunks at once and then spill two of them: each
+  // sched_barrier keeps a group of loads where it is written)
+  __builtin_amdgcn_sched_barrier(0);
+  GP_TURN(w0, 0)
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) w0[i] = *reinterpret_cast<const float4*>(src[i] + 64);
+  __builtin_amdgcn_sched_barrier(0);
+  GP_TURN(w1, 1)
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) w1[i] = *reinterpret_cast<const float4*>(src[i] + 96);
+  __builtin_amdgcn_sched_barrier(0);
+  GP_TURN(w0, 2)
+  GP_TURN(w1, 3)
+#undef GP_TURN
+  const int n = n0 + lane;
+  if (n < N) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+      if (m < M) partial[((int64_t)seg * M + m) * N + n] = acc[m];
+  }
+}
+
 template <typename TC>
 __global__ __launch_bounds__(256) void gemm_plain_rows_sum_kernel(
     TC* __restrict__ C, const float* __restrict__ partial, const void* __restrict__ bias, int bias_dtype,
@@ -300,9 +377,16 @@ static int launch_rows(void* C, const void* A, const void* W, const void* bias, 
   const int segments = (K + GP_SEG - 1) / GP_SEG;
   dim3 grid((N + 63) / 64, (segments + 3) / 4), block(64, 4);
   HE_REQUIRE(grid.y <= 65535, "he_gemm_plain: K=%d too long for one launch", K);
+  // 32-bit weights in whole segments, rows 16-byte aligned: fetched line by line and turned round in LDS
+  constexpr bool f32 = sizeof(TA) == 4 && sizeof(TW) == 4;
+  const bool turned = f32 && K % GP_SEG == 0 && (ldw & 3) == 0 && (((uintptr_t)W) & 15) == 0;
 #define GP_ROWS(MT_)                                                                                  \
-  gemm_plain_rows_kernel<MT_, TA, TW><<<grid, block, 0, s>>>(ws, (const TA*)A, (const TW*)W, M, N, K, \
-                                                             lda, ldw, segments)
+  if (turned)                                                                                         \
+    gemm_plain_rows_turned_kernel<MT_><<<grid, block, 0, s>>>(ws, (const float*)A, (const float*)W, M, N, K, \
+                                                              lda, ldw, segments);                    \
+  else                                                                                                \
+    gemm_plain_rows_kernel<MT_, TA, TW><<<grid, block, 0, s>>>(ws, (const TA*)A, (const TW*)W, M, N, K, \
+                                                               lda, ldw, segments)
   if (M == 1) GP_ROWS(1);
   else if (M == 2) GP_ROWS(2);
   else if (M <= 4) GP_ROWS(4);

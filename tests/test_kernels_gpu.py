@@ -123,7 +123,8 @@ def test_gemm_plain_rows_do_not_depend_on_the_batch(ops):
         assert torch.equal(one.cpu()[0], full.cpu()[r])      # bit-equal
 
 
-@pytest.mark.parametrize("N,K", [(33, 100), (301, 136), (64, 256), (130, 257), (70, 1000), (5, 3), (200, 515)])
+@pytest.mark.parametrize("N,K", [(33, 100), (301, 136), (64, 256), (130, 257), (70, 1000), (5, 3), (200, 515),
+                                 (301, 384), (130, 128), (70, 1024), (7, 640)])   # K in whole segments: the kernel that turns the tile round
 def test_gemm_plain_for_few_rows_gives_the_bits_of_the_tile_kernel(ops, N, K):
     """The plain product has one summation order (segments of 128 k, each a chain in ascending k, added
     in segment order): its kernels for up to 8 rows, which take a workspace, and its tile kernel
