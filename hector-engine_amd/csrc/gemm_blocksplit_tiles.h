@@ -395,8 +395,8 @@ __global__ __launch_bounds__(64 * bs_max_waves(MT, R, U)) void gemm_blocksplit_k
           bs_store4<bf16_t>(reinterpret_cast<bf16_t*>(fu.xg) + at, xgv, out_align, valid);
       }
       // the four lane groups hold the row's other columns of this tile
-      sq += __shfl_xor(sq, 16, HE_WAVE);
-      sq += __shfl_xor(sq, 32, HE_WAVE);
+      sq = xor16_sum(sq);     // lane swaps, not the LDS crossbar: the same sums
+      sq = xor32_sum(sq);
       if (olg == 0) row_sq[ot][olr] = sq;
     }
   }

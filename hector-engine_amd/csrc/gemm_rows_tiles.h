@@ -367,8 +367,8 @@ __global__ __launch_bounds__(64 * NWV) void gemm_rows_kernel(
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
       float s = sq[t];
-      s += __shfl_xor(s, 16, HE_WAVE);
-      s += __shfl_xor(s, 32, HE_WAVE);
+      s = xor16_sum(s);     // lane swaps, not the LDS crossbar: the same sums
+      s = xor32_sum(s);
       if (lg == 0) row_sq[wave][16 * t + lr] = s;
     }
     __syncthreads();
