@@ -120,13 +120,22 @@ __device__ __forceinline__ float xor16_sum(float x) {
 // rotation by 8 inside a row of 16 lanes; the mirror image of a half row, then of its quads;
 // permutations inside a quad. All 64 lanes must be active.
 template <int CTRL>
-__device__ __forceinline__ float dpp_move(float x) {
-  return __uint_as_float((unsigned)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(x), CTRL, 0xF, 0xF, false));
+__device__ __forceinline__ unsigned dpp_bits(unsigned x) {
+  return (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, 0xF, 0xF, false);
 }
-__device__ __forceinline__ float lane_xor8(float x) { return dpp_move<0x128>(x); }                  // row_ror:8
-__device__ __forceinline__ float lane_xor4(float x) { return dpp_move<0x1B>(dpp_move<0x141>(x)); }  // row_half_mirror, quad_perm:[3,2,1,0]
-__device__ __forceinline__ float lane_xor2(float x) { return dpp_move<0x4E>(x); }                   // quad_perm:[2,3,0,1]
-__device__ __forceinline__ float lane_xor1(float x) { return dpp_move<0xB1>(x); }                   // quad_perm:[1,0,3,2]
+// OFF: 8, 4, 2 or 1
+template <int OFF>
+__device__ __forceinline__ unsigned lane_xor_bits(unsigned x) {
+  static_assert(OFF == 8 || OFF == 4 || OFF == 2 || OFF == 1, "lane_xor_bits: 8, 4, 2 or 1");
+  if (OFF == 8) return dpp_bits<0x128>(x);                    // row_ror:8
+  if (OFF == 4) return dpp_bits<0x1B>(dpp_bits<0x141>(x));    // row_half_mirror, quad_perm:[3,2,1,0]
+  if (OFF == 2) return dpp_bits<0x4E>(x);                     // quad_perm:[2,3,0,1]
+  return dpp_bits<0xB1>(x);                                   // quad_perm:[1,0,3,2]
+}
+__device__ __forceinline__ float lane_xor8(float x) { return __uint_as_float(lane_xor_bits<8>(__float_as_uint(x))); }
+__device__ __forceinline__ float lane_xor4(float x) { return __uint_as_float(lane_xor_bits<4>(__float_as_uint(x))); }
+__device__ __forceinline__ float lane_xor2(float x) { return __uint_as_float(lane_xor_bits<2>(__float_as_uint(x))); }
+__device__ __forceinline__ float lane_xor1(float x) { return __uint_as_float(lane_xor_bits<1>(__float_as_uint(x))); }
 
 // Sum and maximum over the wavefront, every lane gets the result: the butterfly lane i with lane
 // i ^ 32, 16, 8, 4, 2, 1 in that order (an addition gives both lanes of a pair the same bits). Through

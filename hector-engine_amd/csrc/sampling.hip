@@ -35,16 +35,33 @@ __device__ __forceinline__ void argmax_take(float& best, int& bi, float v, int i
   }
 }
 
+// Reduces (best, bi) over the wavefront, every lane gets the result: the butterfly lane i with lane
+// i ^ 32, 16, 8, 4, 2, 1 through lane swaps and DPP (which of two candidates wins does not depend
+// on the order they are compared in). All 64 lanes must be active.
+__device__ __forceinline__ void argmax_wave(float& best, int& bi) {
+  {
+    const auto v = __builtin_amdgcn_permlane32_swap(__float_as_uint(best), __float_as_uint(best), false, false);
+    const auto i = __builtin_amdgcn_permlane32_swap((unsigned)bi, (unsigned)bi, false, false);
+    best = __uint_as_float(v[0]), bi = (int)i[0];
+    argmax_take(best, bi, __uint_as_float(v[1]), (int)i[1]);
+  }
+  {
+    const auto v = __builtin_amdgcn_permlane16_swap(__float_as_uint(best), __float_as_uint(best), false, false);
+    const auto i = __builtin_amdgcn_permlane16_swap((unsigned)bi, (unsigned)bi, false, false);
+    best = __uint_as_float(v[0]), bi = (int)i[0];
+    argmax_take(best, bi, __uint_as_float(v[1]), (int)i[1]);
+  }
+  argmax_take(best, bi, __uint_as_float(lane_xor_bits<8>(__float_as_uint(best))), (int)lane_xor_bits<8>((unsigned)bi));
+  argmax_take(best, bi, __uint_as_float(lane_xor_bits<4>(__float_as_uint(best))), (int)lane_xor_bits<4>((unsigned)bi));
+  argmax_take(best, bi, __uint_as_float(lane_xor_bits<2>(__float_as_uint(best))), (int)lane_xor_bits<2>((unsigned)bi));
+  argmax_take(best, bi, __uint_as_float(lane_xor_bits<1>(__float_as_uint(best))), (int)lane_xor_bits<1>((unsigned)bi));
+}
+
 // Reduces (best, bi) over the workgroup; valid in thread 0.
 __device__ __forceinline__ void argmax_block(float& best, int& bi) {
   __shared__ float sval[ARGMAX_THREADS / HE_WAVE];
   __shared__ int sidx[ARGMAX_THREADS / HE_WAVE];
-#pragma unroll
-  for (int off = HE_WAVE / 2; off > 0; off >>= 1) {
-    const float ov = __shfl_xor(best, off, HE_WAVE);
-    const int oi = __shfl_xor(bi, off, HE_WAVE);
-    argmax_take(best, bi, ov, oi);
-  }
+  argmax_wave(best, bi);
   const int lane = threadIdx.x & (HE_WAVE - 1), wave = threadIdx.x >> 6;
   if (lane == 0) {
     sval[wave] = best;
@@ -63,16 +80,27 @@ __global__ __launch_bounds__(ARGMAX_THREADS) void argmax_parts_kernel(
   const int lo = blockIdx.x * ARGMAX_PART, hi = min(V, lo + ARGMAX_PART);
   float best = -INFINITY;
   int bi = 0x7fffffff;
-  const bool vec = ((stride & 3) == 0) && ((((uintptr_t)logits) & 15) == 0);
+  const bool vec = V >= 4 && ((stride & 3) == 0) && ((((uintptr_t)logits) & 15) == 0);
   if (vec) {
-    for (int i = lo + 4 * threadIdx.x; i < hi; i += 4 * ARGMAX_THREADS) {
+    // a thread's eight loads of four values go out together (one after the other, each waited for
+    // the one before: 8 us a part); a load that would pass the part's end reads the row's start
+    // and is not used, the few elements behind the last whole four are taken one by one
+    constexpr int LOADS = ARGMAX_PART / (4 * ARGMAX_THREADS);
+    float4 v[LOADS];
+#pragma unroll
+    for (int u = 0; u < LOADS; ++u) {
+      const int i = lo + 4 * (int)threadIdx.x + 4 * ARGMAX_THREADS * u;
+      v[u] = *reinterpret_cast<const float4*>(x + (i + 4 <= hi ? i : 0));
+    }
+#pragma unroll
+    for (int u = 0; u < LOADS; ++u) {
+      const int i = lo + 4 * (int)threadIdx.x + 4 * ARGMAX_THREADS * u;
       if (i + 4 <= hi) {
-        const float4 v = *reinterpret_cast<const float4*>(x + i);
-        argmax_take(best, bi, v.x, i);
-        argmax_take(best, bi, v.y, i + 1);
-        argmax_take(best, bi, v.z, i + 2);
-        argmax_take(best, bi, v.w, i + 3);
-      } else {
+        argmax_take(best, bi, v[u].x, i);
+        argmax_take(best, bi, v[u].y, i + 1);
+        argmax_take(best, bi, v[u].z, i + 2);
+        argmax_take(best, bi, v[u].w, i + 3);
+      } else if (i < hi) {
         for (int j = i; j < hi; ++j) argmax_take(best, bi, x[j], j);
       }
     }
@@ -99,12 +127,7 @@ __global__ __launch_bounds__(HE_WAVE) void argmax_join_kernel(int32_t* __restric
   int bi = 0x7fffffff;
   for (int p = threadIdx.x; p < parts; p += HE_WAVE)
     argmax_take(best, bi, part_val[blockIdx.x * parts + p], part_idx[blockIdx.x * parts + p]);
-#pragma unroll
-  for (int off = HE_WAVE / 2; off > 0; off >>= 1) {
-    const float ov = __shfl_xor(best, off, HE_WAVE);
-    const int oi = __shfl_xor(bi, off, HE_WAVE);
-    argmax_take(best, bi, ov, oi);
-  }
+  argmax_wave(best, bi);
   if (threadIdx.x == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
 }
 
