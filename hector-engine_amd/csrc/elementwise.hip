@@ -17,6 +17,22 @@ __global__ void embedding_kernel(float* __restrict__ out, const T* __restrict__ 
     return;
   }
   const T* row = table + (int64_t)id * D;
+  if (sizeof(T) == 2 && (D & 7) == 0 && (((uintptr_t)table | (uintptr_t)out) & 15) == 0) {
+    // eight elements a thread and turn: one 16-byte load, two 16-byte stores
+    for (int i = 8 * threadIdx.x; i < D; i += 8 * blockDim.x) {
+      const uint4 v = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(row) + i);
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      float f[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        f[2 * j] = __uint_as_float(w[j] << 16);
+        f[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+      }
+      *reinterpret_cast<float4*>(o + i) = make_float4(f[0], f[1], f[2], f[3]);
+      *reinterpret_cast<float4*>(o + i + 4) = make_float4(f[4], f[5], f[6], f[7]);
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = to_float(row[i]);
 }
 
@@ -48,6 +64,11 @@ __global__ void gather_rows_f32_kernel(float* __restrict__ out, const float* __r
     return;
   }
   const float* in = src + (int64_t)idx * D;
+  if ((D & 3) == 0 && (((uintptr_t)src | (uintptr_t)out) & 15) == 0) {
+    for (int i = 4 * threadIdx.x; i < D; i += 4 * blockDim.x)
+      *reinterpret_cast<float4*>(o + i) = *reinterpret_cast<const float4*>(in + i);
+    return;
+  }
   for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = in[i];
 }
 
