@@ -29,6 +29,11 @@ class Route:
 
 
 _table: dict[tuple[str, tuple], list[Route]] = {}
+_version = 0      # counts the changes of the table: what a part remembers of a choice holds for one version
+
+
+def version() -> int:
+    return _version
 
 
 def register_route(op: str, dtypes: tuple, name: str, takes: Callable[[Any], bool],
@@ -38,6 +43,8 @@ def register_route(op: str, dtypes: tuple, name: str, takes: Callable[[Any], boo
     routes = _table.setdefault((op, tuple(dtypes)), [])
     if any(r.name == name for r in routes):
         raise ValueError(f"route {name!r} of {op!r} {_names(dtypes)} is registered already")
+    global _version
+    _version += 1
     route = Route(name, takes, run, frozenset(traits))
     if before is None:
         routes.append(route)
@@ -54,6 +61,8 @@ def unregister_route(op: str, dtypes: tuple, name: str) -> None:
     left = [r for r in routes if r.name != name]
     if len(left) == len(routes):
         raise ValueError(f"route {name!r} of {op!r} {_names(dtypes)} is not registered")
+    global _version
+    _version += 1
     _table[(op, tuple(dtypes))] = left
 
 

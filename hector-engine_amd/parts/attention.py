@@ -63,6 +63,8 @@ class Attention(Mixer):
         self.qkv: Linear | None = None
         self.q_only: Linear | None = None
         self.o_proj: Linear | None = None
+        self._chosen: dict[tuple, routes.Route] = {}      # (all one-token, dtype) -> route, for one version of the table
+        self._chosen_version = -1
         self.fast = env.dtype == torch.bfloat16 and getattr(env, "fast_kernels", True) \
             and self.hd % 16 == 0 and self.hd <= 256 and self.scale > 0   # else the plain kernel
 
@@ -114,12 +116,19 @@ class Attention(Mixer):
     def forward(self, x, ctx: StepContext, cache: LayerCache):
         if cache.writes and not self.kv_projection:
             raise RuntimeError(f"{self.prefix}: a mixer without k/v projections must read another run's cache")
-        rot = self.position.rotary()
-        case = AttentionCase(
-            all_single=ctx.all_single, fast=self.fast,
-            fusable=not self.position.custom and rot is not None
-            and ops.attention_decode_fused_ok(self.H, self.KVH, self.hd, rot[1]))
-        return routes.choose("attention", (ctx.env.dtype,), case).run(self, x, ctx, cache)
+        if self._chosen_version != routes.version():
+            self._chosen.clear()
+            self._chosen_version = routes.version()
+        key = (ctx.all_single, ctx.env.dtype)
+        route = self._chosen.get(key)
+        if route is None:
+            rot = self.position.rotary()
+            case = AttentionCase(
+                all_single=ctx.all_single, fast=self.fast,
+                fusable=not self.position.custom and rot is not None
+                and ops.attention_decode_fused_ok(self.H, self.KVH, self.hd, rot[1]))
+            route = self._chosen[key] = routes.choose("attention", (ctx.env.dtype,), case)
+        return route.run(self, x, ctx, cache)
 
     # ---- the routes' bodies ----
 

@@ -68,11 +68,22 @@ class Linear:
         self.bias = bias
         self.out_features, self.in_features = weight.shape
         self._plans: dict[bool, tuple[int, int]] = {}
+        self._chosen: dict[tuple, routes.Route] = {}     # (rows, activations, fast) -> route, for one version of the table
+        self._chosen_version = -1
 
     def route(self, rows: int, ctx: StepContext, act: torch.dtype) -> routes.Route:
-        """The kernel route of this product at this many rows of this activation dtype."""
-        N, K = self.weight.shape
-        return routes.choose("linear", (self.weight.dtype, act), ProductCase(rows, N, K, ctx.env.fast_kernels))
+        """The kernel route of this product at this many rows of this activation dtype (remembered
+        per row count while the table of routes does not change: a step asks a hundred times)."""
+        if self._chosen_version != routes.version() or len(self._chosen) > 256:
+            self._chosen.clear()
+            self._chosen_version = routes.version()
+        key = (rows, act, ctx.env.fast_kernels)
+        route = self._chosen.get(key)
+        if route is None:
+            N, K = self.weight.shape
+            route = routes.choose("linear", (self.weight.dtype, act), ProductCase(rows, N, K, ctx.env.fast_kernels))
+            self._chosen[key] = route
+        return route
 
     def _has(self, trait: str, rows: int, ctx: StepContext, act: torch.dtype) -> bool:
         if not routes.routes_of("linear", (self.weight.dtype, act)):
