@@ -18,6 +18,7 @@ from __future__ import annotations
 
 import dataclasses
 
+import numpy as np
 import torch
 
 from ..parts.base import KVNeed, LayerCache
@@ -44,6 +45,8 @@ class _Group:
         self.kpool = torch.zeros((len(runs), num_pages, need.kv_heads, need.k_elems), dtype=dtype, device=device)
         self.vpool = torch.zeros((len(runs), num_pages, need.kv_heads, need.v_elems), dtype=dtype, device=device)
         self.page_table = torch.full((max_slots, max_blocks), -1, dtype=torch.int32, device=device)
+        # the same table on the host: a step can take its sequences' rows along with its metadata
+        self.host_table = np.full((max_slots, max_blocks), -1, dtype=np.int32)
 
 
 class PagedCache:
@@ -155,11 +158,18 @@ class PagedCache:
             idx.append(slot * self.max_blocks + block)
             val.append(page)
         for gi, (idx, val) in by_group.items():
+            self.groups[gi].host_table.reshape(-1)[idx] = val
             packed = torch.tensor([idx, val], dtype=torch.int64).to(self.device)
             self.groups[gi].page_table.view(-1).index_copy_(0, packed[0], packed[1].to(torch.int32))
 
     def _clear(self, entries) -> None:
         self._write([(gi, slot, block, -1) for gi, slot, block in entries])
+
+    def rows_of_tables(self, slots: list[int], out: np.ndarray) -> None:
+        """out[g, r, :] = the page table row of slots[r] in group g (int32 [groups, rows or more,
+        max_blocks]; rows beyond the slots keep what they hold)."""
+        for gi, g in enumerate(self.groups):
+            out[gi, :len(slots)] = g.host_table[slots]
 
     # -- views for the layers -----------------------------------------------
     def layer_cache(self, run: int) -> LayerCache:

@@ -122,10 +122,23 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
   const bool h_ok = lr < GT;
   const int h = kvh * G + 16 * ht + min(lr, GT - 1);
   // loads that need nothing but the row: issued first, used last
+  // seq_slot null: the page table has a row per row of the step (the host has gathered the
+  // sequences' page numbers into the step's metadata), so its address needs nothing but the row and
+  // its lines are asked for at once: with the table of the cache the numbers come at the end of a
+  // chain row -> sequence -> slot -> table (3.0 us after the kernel's start, measured with time
+  // stamps inside it, the table's line from memory every time: the weights of a layer have passed
+  // through the caches since the layer before read it).
+  const bool by_row = seq_slot == nullptr;
+  // (an ordinary load whose value is "used" by an empty statement at the kernel's end: the compiler
+  // keeps the load, counts it, and holds its register until then. Written as inline assembly the
+  // load's register counted as free at once, and what arrived later overwrote whatever lived there
+  // by then; a volatile load bypasses the caches and is waited for where it stands.)
+  int touched = 0;
+  if (by_row && lane < ((max_blocks * 4 + 127) >> 7)) touched = page_table[(int64_t)row * max_blocks + 32 * lane];
   const uint16_t* qkv_row = qkv + (int64_t)row * qkv_stride;
   QLoads<NT> ql;
   q_issue<NT>(ql, qkv_row + (int64_t)h * HD, bias, bias_dtype, h * HD, lg);
-  const float freq = lane < HD / 2 ? inv_freq[lane] : 0.f;
+  const float freq = inv_freq[min(lane, HD / 2 - 1)];   // no condition in front of the load (the lanes beyond take no angle)
   const int seq = row_seq[row];
   const int Z = gridDim.z, z = blockIdx.z;
   // where dims d.. of head (column) hg of this tile go: row-major [rows, H HD], or piece-major
@@ -139,7 +152,7 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
       for (int i = threadIdx.x; i < GT * HD; i += blockDim.x) *out_at(i / HD, i % HD) = 0;
     return;
   }
-  const int slot = seq_slot[seq];
+  const int slot = by_row ? row : seq_slot[seq];
   const int p = positions[row];
   const int n_keys = p + 1;
   const int first = window > 0 ? max(0, n_keys - window) : 0;
@@ -162,7 +175,12 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
   if (early) attend_pages<NT>(cursor, pt, max_blocks, kb_begin);
   float qx[NT / 2][8];
   q_biased<NT>(qx, ql, bias, bias_dtype, h * HD, h_ok, lg);
-  const float angle = (float)p * freq;
+  // The angle is formed here, ahead of the loads of the first keys: its frequency was asked for at
+  // the top, and a wait for it behind those loads would be a wait for them too (loads complete in
+  // order): the sines and the rotation of q, which are meant to run while the keys are on their way,
+  // ran after them (2.4 us of the kernel's 11).
+  float angle = (float)p * freq;
+  asm volatile("" : "+v"(angle));
   __builtin_amdgcn_sched_barrier(0);
   if (early) attend_first<NT>(cursor, kpool, vpool, num_pages, KVH, kvh, kb_begin, lr, lg);
   float sn = 0.f, c = 1.f;                   // lane j < HD / 2: angle j of position p
@@ -260,6 +278,7 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
       }
     }
   }
+  asm volatile("" :: "v"(touched));
 }
 
 // Wavefronts per workgroup and workgroups per (sequence, kv head, head tile), measured on

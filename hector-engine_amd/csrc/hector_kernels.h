@@ -135,6 +135,8 @@ int64_t he_attention_decode_workspace_floats(int rows, int H, int KVH, int hd, i
 // when the sizes are taken (head_dim 64 or 128, rotated whole). out_pieces: out lies piece-major
 // (as he_gemm_blocksplit_fused_bf16 reads it with x_pieces). spread: one sequence of the step has
 // several times the keys of the others; every sequence's keys are then cut across more workgroups.
+// seq_slot null: page_table has a row per row of the step ([rows, max_blocks], the page numbers of
+// the row's sequence) instead of a row per slot.
 int he_attention_decode_fused_ok(int H, int KVH, int hd, int rotary_dim);
 int64_t he_attention_decode_fused_workspace_floats(int rows, int H, int KVH, int hd, int max_keys,
                                                    int spread);

@@ -41,6 +41,7 @@ GRAPH_MAX_BUCKET = 256
 # rarely come again. So many such graphs are kept, the least recently used one goes first.
 GRAPH_MAX_STEP_ROWS = 512
 GRAPH_MAX_STEP_PLANS = 24
+ROW_TABLES_MAX_BYTES = 256 * 1024     # page table rows that a one-token step takes along with its metadata
 
 
 class StepError(ValueError):
@@ -59,13 +60,18 @@ class _Meta:
 
     FIELDS = ("tokens", "positions", "row_seq", "seq_slot", "cu_seqlens", "seq_start", "want_rows")
 
-    def __init__(self, rows: int, seqs: int, wants: int):
+    def __init__(self, rows: int, seqs: int, wants: int, row_tables: int = 0):
+        """row_tables: ints of room behind the fields for the page table rows of the step's rows."""
         sizes = (rows, rows, rows, seqs, seqs + 1, seqs, max(wants, 1))
         self.offsets = {}
         off = 0
         for name, n in zip(self.FIELDS, sizes):
             self.offsets[name] = (off, n)
             off += n
+        if row_tables:
+            off = (off + 31) // 32 * 32          # from a cache line's start
+            self.offsets["row_tables"] = (off, row_tables)
+            off += row_tables
         self.total = off
 
     def views(self, buf):
@@ -77,9 +83,10 @@ def _pow2(n: int, least: int = 1) -> int:
 
 
 class _GraphBucket:
-    def __init__(self, size: int, device, seqs: int | None = None, wants: int | None = None):
+    def __init__(self, size: int, device, seqs: int | None = None, wants: int | None = None,
+                 row_tables: int = 0):
         self.size = size
-        self.meta = _Meta(size, size if seqs is None else seqs, size if wants is None else wants)
+        self.meta = _Meta(size, size if seqs is None else seqs, size if wants is None else wants, row_tables)
         self.dev = torch.zeros(self.meta.total, dtype=torch.int32, device=device)
         self.views = self.meta.views(self.dev)
         self.pool = ScratchPool(device)
@@ -364,12 +371,23 @@ class Engine:
         size = 1 << (n - 1).bit_length()
         hints = self._hints_before[size] = self._step_hints(entries, self._hints_before.get(size))
         bucket = self._buckets.get((size, hints))
+        groups, blocks = len(self.cache.groups), self.cache.max_blocks
+        # The page table rows of the step's rows travel with its metadata (where they are few KiB):
+        # a mixer then has its pages' numbers without the chain row -> sequence -> slot -> table,
+        # each link of which is a trip to memory in every layer (7B shape, batch 8: 3.0 us of the
+        # one-token attention's 12.8; with the rows beside the metadata the step takes 2 % less).
+        by_row = groups * size * blocks if groups * size * blocks * 4 <= ROW_TABLES_MAX_BYTES else 0
         if bucket is None:
-            bucket = self._buckets[(size, hints)] = _GraphBucket(size, self.device)
+            bucket = self._buckets[(size, hints)] = _GraphBucket(size, self.device, row_tables=by_row)
         # every row of the bucket gets logits; padding rows are inert (row_seq -1)
         padded = [StepEntry(e.slot, e.tokens, [0]) for e in entries]
         host, idx, _ = self._pack(padded, bucket.meta, size, size)
         host.numpy()[bucket.meta.offsets["want_rows"][0]:][:size] = np.arange(size, dtype=np.int32)
+        if by_row:
+            o, count = bucket.meta.offsets["row_tables"]
+            tables = host.numpy()[o:o + count].reshape(groups, size, blocks)
+            tables[:, n:] = -1
+            self.cache.rows_of_tables([e.slot for e in entries], tables)
         self._upload(host, idx, bucket.dev)
         if device_tokens is not None:
             bucket.views["tokens"][:n].copy_(device_tokens)
@@ -379,6 +397,9 @@ class Engine:
             ctx.want_all = True
             ctx.hints = dict(zip(self._hint_fns, hints))
             ctx.padded = True
+            if by_row:
+                dev_tables = bucket.views["row_tables"].view(groups, size, blocks)
+                ctx.row_tables = {g.page_table.data_ptr(): dev_tables[gi] for gi, g in enumerate(self.cache.groups)}
             if bucket.uses == 1:
                 # first use: run eagerly; it also sizes the bucket's scratch pool
                 return self._bucket_eager(bucket, ctx, n)

@@ -563,7 +563,9 @@ def attention_decode_fused(out, qkv, bias, kpool, vpool, positions, row_seq, seq
     others (every sequence's keys are then cut across more workgroups; the workspace is asked for
     with the same flag). qkv: bf16 [rows, (H + 2 KVH) hd] without bias; q columns
     alone where the run reads another run's cache (write_kv False). out_pieces: out is written
-    piece-major for exactly `rows` rows (see :func:`to_pieces`)."""
+    piece-major for exactly `rows` rows (see :func:`to_pieces`). seq_slot None: page_table has a row
+    per row of the step ([rows or more, blocks]: the page numbers of the row's sequence), not a
+    row per slot; the kernel then asks for them at its start, without the chain through the slot."""
     width = (H + 2 * KVH) * hd if write_kv else H * hd
     _need(qkv, "qkv", torch.bfloat16)
     _need(out, "out", torch.bfloat16)
@@ -574,10 +576,12 @@ def attention_decode_fused(out, qkv, bias, kpool, vpool, positions, row_seq, seq
     _need(kpool, "kpool", torch.bfloat16, (None, KVH, layout.k_page_elems(hd)))
     _need(vpool, "vpool", torch.bfloat16, (None, KVH, layout.v_page_elems(hd)))
     _need(page_table, "page_table", torch.int32)
-    for name, t in (("positions", positions), ("row_seq", row_seq), ("seq_slot", seq_slot)):
+    for name, t in (("positions", positions), ("row_seq", row_seq)) + ((("seq_slot", seq_slot),) if seq_slot is not None else ()):
         _need(t, name, torch.int32)
     if positions.numel() < rows or row_seq.numel() < rows or page_table.dim() != 2:
         raise ValueError("attention_decode_fused: metadata shorter than the row count")
+    if seq_slot is None and page_table.shape[0] < rows:
+        raise ValueError("attention_decode_fused: a page table by rows needs a row per row of the step")
     if bias is not None:
         _need(bias, "bias", shape=(width,))
     _need(inv_freq, "inv_freq", torch.float32, (rotary_dim // 2,))
@@ -587,7 +591,7 @@ def attention_decode_fused(out, qkv, bias, kpool, vpool, positions, row_seq, seq
     _lib.check(L.he_attention_decode_fused_bf16(
         out.data_ptr(), qkv.data_ptr(), width, _ptr(bias),
         dtype_code(bias.dtype) if bias is not None else F32, kpool.data_ptr(), vpool.data_ptr(),
-        positions.data_ptr(), row_seq.data_ptr(), seq_slot.data_ptr(), page_table.data_ptr(),
+        positions.data_ptr(), row_seq.data_ptr(), _ptr(seq_slot), page_table.data_ptr(),
         page_table.shape[1], kpool.shape[0], inv_freq.data_ptr(), rotary_dim, rows, H, KVH, hd,
         window, float(scale), max_keys, int(spread), int(write_kv), int(out_pieces), _ptr(workspace),
         workspace.numel() if workspace is not None else 0, _stream()))

@@ -143,8 +143,11 @@ class Attention(Mixer):
         uneven = bool(ctx.hints.get(keys_uneven, False))
         floats = ops.attention_decode_fused_workspace_floats(rows, H, KVH, hd, ctx.max_keys, uneven)
         ws = ctx.alloc((floats,), torch.float32) if floats else None
+        # the page numbers of the step's rows, where the host has put them beside the step's metadata
+        by_row = ctx.row_tables.get(cache.page_table.data_ptr())
         ops.attention_decode_fused(out, qkv, proj.bias, cache.kpool, cache.vpool, ctx.positions,
-                                   ctx.row_seq, ctx.seq_slot, cache.page_table, rot[0], rot[1],
+                                   ctx.row_seq, None if by_row is not None else ctx.seq_slot,
+                                   by_row if by_row is not None else cache.page_table, rot[0], rot[1],
                                    rows, H, KVH, hd, self.window, self.scale, ctx.max_keys,
                                    cache.writes, ws, out_pieces=pieces, spread=uneven)
         return self.o_proj(PieceRows(out) if pieces else out, rows, ctx, sink=ctx.take_sink())

@@ -150,6 +150,10 @@ class StepContext:
         self.want_all = False             # the wanted rows are all rows, in order
         self.padded = False               # the step may hold padding rows and sequences (row_seq -1, slot -1: a step that
                                           # runs as a graph of its bucket of sizes); a part leaves such rows finite
+        self.row_tables: dict = {}        # a cache group's page table (its data_ptr) -> int32 [rows, blocks]: the table
+                                          # rows of the step's rows, gathered by the host into the step's metadata
+                                          # (one-token steps that replay a graph; a mixer may read it in place of
+                                          # LayerCache.page_table[seq_slot[row_seq[row]]] and skip that chain)
         self.next_norm = None             # the norm that reads the stream after the running block (set by the model)
         self.sink = None                  # ResidualSink offered to the running mixer / feed-forward
 

@@ -199,3 +199,53 @@ def test_random_traffic_with_truncation_keeps_every_invariant():
     for s in list(live):
         b.release(s)
     assert all(g.pool.available == 40 for g in b.groups)
+
+
+def test_the_host_copy_of_the_page_tables_follows_the_device_tables():
+    """The cache keeps its page tables twice, for the kernels and for the step's metadata: after
+    every kind of traffic (growth, a window that moves on, truncation, release, a slot used again)
+    both say the same, in a group that keeps all keys and in one that keeps a window."""
+    import numpy as np
+    import torch
+    from hector_engine_amd.cache.paged import PagedCache, RunPlan
+    from hector_engine_amd.parts.base import KVNeed
+    plans = [RunPlan(KVNeed(2, 16), None), RunPlan(KVNeed(2, 16, window=100), None), RunPlan(None, 0)]
+    cache = PagedCache(plans, max_tokens=64 * 24, max_slots=4, max_seq_len=64 * 8, dtype=torch.float32,
+                       device="cpu")
+    rng = random.Random(5)
+    held: dict[int, int] = {}
+
+    def check():
+        for g in cache.groups:
+            assert np.array_equal(g.host_table, g.page_table.numpy())
+        slots = sorted(held)
+        out = np.full((len(cache.groups), len(slots) + 2, cache.max_blocks), 7, dtype=np.int32)
+        cache.rows_of_tables(slots, out)
+        for gi, g in enumerate(cache.groups):
+            assert np.array_equal(out[gi, :len(slots)], g.page_table.numpy()[slots])
+            assert (out[gi, len(slots):] == 7).all()
+
+    for _ in range(300):
+        move = rng.random()
+        try:
+            if move < 0.2 and len(held) < cache.max_slots:
+                held[cache.acquire()] = 0
+            elif move < 0.75 and held:
+                s = rng.choice(sorted(held))
+                n = held[s] + rng.choice([1, 1, 1, 63, 64, 130])
+                cache.reserve([(s, n)])
+                cache.commit([(s, n)])
+                held[s] = n
+            elif move < 0.85 and held:
+                s = rng.choice(sorted(held))
+                n = rng.randrange(held[s] + 1)
+                cache.truncate(s, n)
+                held[s] = n
+            elif held:
+                s = rng.choice(sorted(held))
+                cache.release(s)
+                del held[s]
+        except (CacheFull, CacheError):
+            pass
+        check()
+    assert any((g.host_table >= 0).any() for g in cache.groups)

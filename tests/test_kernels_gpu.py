@@ -825,6 +825,13 @@ def test_attention_decode_fused(ops, H, KVH, hd, window, write_kv, copies):
                                    dev(row_seq), dev(seq_slot), dev(table), dev(inv), hd, rows, H, KVH,
                                    hd, window, 1.0 / math.sqrt(hd), 4096, write_kv, ws, out_pieces=True)
         assert torch.equal(from_pieces(out2).cpu(), out.cpu())
+    # the page numbers handed over row by row (a padding row's are -1) instead of through the slots
+    by_row = torch.stack([table[slots[s]] if s >= 0 else torch.full_like(table[0], -1) for s in order])
+    out3 = torch.full((rows, H * hd), 7.0, dtype=torch.bfloat16, device="cuda")
+    ops.attention_decode_fused(out3, dev(qkv_rows), dev(bias), dev(kp), dev(vp), dev(positions), dev(row_seq),
+                               None, dev(by_row), dev(inv), hd, rows, H, KVH, hd, window,
+                               1.0 / math.sqrt(hd), 4096, write_kv, ws)
+    assert torch.equal(out3.cpu(), out.cpu())
 
 
 def test_attention_decode_fused_refuses_other_sizes(ops):
