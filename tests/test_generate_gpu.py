@@ -324,6 +324,53 @@ def test_default_stop_ids_are_the_model_folders_own(he, model_dirs, plain_models
     assert he.generate(eng, prompts[:1], max_new_tokens=10)[0].tokens == want[0]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_two_sessions_on_one_engine_share_the_weights_and_nothing_else(he, model_dirs, plain_models, name, dtype):
+    """Several sessions over one loaded model, as the reference attaches sessions to one Model
+    (src/inference_session.hpp:126-144): each has its slot, its sampler and its turn count, and
+    turns that alternate between them give what each conversation gives alone. The second
+    session samples, the first is greedy; a closed session's slot is taken by a third."""
+    cfg, w = plain_models[name]
+    V = cfg["vocab_size"]
+    a1, a2, b1, b2, c1 = (rand_ids(V, n, 40 + i) for i, n in enumerate((9, 5, 66, 3, 12)))
+    eng = he.Engine(model_dirs[name], dtype=dtype, max_tokens=1024, max_slots=2, max_seq_len=512,
+                    beyond_max_positions=True)
+    exact = dtype == "float32"
+    hot = he.SamplingConfig(temperature=0.8, seed=3)
+    sa, sb = he.Session(eng, stop_ids=()), he.Session(eng, hot, stop_ids=())
+    assert sa.slot != sb.slot
+    ra1 = sa.turn(a1, 7)
+    rb1 = sb.turn(b1, 6)
+    ra2 = sa.turn(a2, 8)
+    rb2 = sb.turn(b2, 5)
+    if exact:
+        assert ra1.tokens == P.generate(cfg, w, a1, 7)
+        assert rb1.tokens == P.generate(cfg, w, b1, 6, temperature=0.8, seed=3)
+        assert ra2.tokens == P.generate(cfg, w, a1 + ra1.tokens + a2, 8)
+        assert rb2.tokens == P.generate(cfg, w, b1 + rb1.tokens + b2, 5, temperature=0.8, seed=4)
+    else:   # bfloat16: each conversation alone in a fresh engine gives the same tokens
+        alone = he.Engine(model_dirs[name], dtype=dtype, max_tokens=1024, max_slots=1, max_seq_len=512,
+                          beyond_max_positions=True)
+        with he.Session(alone, stop_ids=()) as s:
+            assert [s.turn(a1, 7).tokens, s.turn(a2, 8).tokens] == [ra1.tokens, ra2.tokens]
+        with he.Session(alone, hot, stop_ids=()) as s:
+            assert [s.turn(b1, 6).tokens, s.turn(b2, 5).tokens] == [rb1.tokens, rb2.tokens]
+    assert sa.position == len(a1) + 7 + len(a2) + 8 - 1 and sb.position == len(b1) + 6 + len(b2) + 5 - 1
+    freed = sa.slot
+    sa.close()
+    with he.Session(eng, stop_ids=()) as sc:      # the freed slot, used again beside the running one
+        assert sc.slot == freed
+        rc = sc.turn(c1, 6)
+        if exact:
+            assert rc.tokens == P.generate(cfg, w, c1, 6)
+        rb3 = sb.turn(a2, 4)
+        if exact:
+            assert rb3.tokens == P.generate(cfg, w, b1 + rb1.tokens + b2 + rb2.tokens + a2, 4, temperature=0.8, seed=5)
+    sb.close()
+    assert eng.cache.free_pages == eng.cache.num_pages
+
+
 @pytest.mark.parametrize("name", ["A", "B", "D"])
 def test_a_session_of_turns_equals_plain_on_the_whole_context(he, model_dirs, plain_models, name):
     """A session keeps its slot: the second turn's tokens continue the first turn's context, the
