@@ -67,7 +67,8 @@ def after_token(token: int, generated: int, max_new_tokens: int, length: int, ma
     return True, None
 
 
-RUN_OF_STEPS = 8
+RUN_OF_STEPS = 8        # one-token steps queued ahead of the host's reading of their ids
+LONGEST_RUN = 256       # steps after which a run of queued steps ends in any case
 
 
 def generate(engine, prompts: list[list[int]], *, max_new_tokens: int = 100, sampling=None,
@@ -86,19 +87,20 @@ def generate(engine, prompts: list[list[int]], *, max_new_tokens: int = 100, sam
 
     on_token(request index, token) is called for every token that becomes part of a result, in
     the order of each sequence (the reference hands text out as it comes through its on_text
-    callback: src/inference_session.cpp:636-645; here the ids); with queued steps the tokens of a
-    run arrive together when the run has been read. on_prefill(request indices, ms) is called
+    callback: src/inference_session.cpp:636-645; here the ids); with queued steps a token arrives
+    when the host reads its step's ids, run_of_steps steps behind the queue. on_prefill(request indices, ms) is called
     once per batch after its prompt step (:603).
 
-    run_of_steps: with a sampler, up to so many one-token steps are queued at a time, each
-    step's ids going into the next on the device (and into the penalty windows, which then live
-    there for the run). The tokens are the same as step
-    by step. When nothing can end a sequence inside a run but its token budget or its cache
-    room (no stop ids, no `cancel`), the run never reaches past those and the host reads all
-    its ids at the end. Otherwise the host reads the ids of a step while the next one runs,
-    and queues nothing more once it has seen a stop token or `cancel` says so: a sequence that
-    has sampled its stop token is stepped once more at most (the step that was already
-    queued), then gives its slot back and leaves the batch."""
+    run_of_steps: with a sampler, one-token steps are queued ahead of the host, each step's ids
+    going into the next on the device (and into the penalty windows, which then live there for
+    the run). The tokens are the same as step by step. When nothing can end a sequence inside a
+    run but its token budget or its cache room (no stop ids, no `cancel`), the run never reaches
+    past those, and the host reads a step's ids (and hands them to on_token) when
+    run_of_steps - 1 further steps are queued behind it: the device does not wait for the host
+    between steps. Otherwise the host reads the ids of a step while the next one runs, and
+    queues nothing more once it has seen a stop token or `cancel` says so: a sequence that has
+    sampled its stop token is stepped once more at most (the step that was already queued), then
+    gives its slot back and leaves the batch. 1 or less: step by step."""
     from ..sampling import Sampler, SamplingConfig
     from ..sampling.sampler import READS_IN_FLIGHT
     if sample_fn is None:
@@ -147,28 +149,44 @@ def steps_in_run(generated: list[int], lengths: list[int], max_new_tokens: int, 
 
 def _run_of_steps(engine, sampler, slots: list[int], tokens: list[int], seqs: list[int],
                   steps: list[int], count: int, stop_ids=frozenset(), cancel=None,
-                  contexts: list[list[int]] | None = None) -> list[list[int]]:
-    """Feeds `tokens` and queues up to `count` one-token steps; returns the sampled ids of the
-    steps that ran, [steps][rows]. With stop ids or `cancel`, the ids of step j are read while
-    step j + 1 runs, and the run ends with the step that was queued when a stop token (or the
-    cancellation) was seen."""
-    uniforms = None if sampler.config.is_greedy else sampler.uniforms_device(seqs, steps, count)
+                  contexts: list[list[int]] | None = None, ahead: int = RUN_OF_STEPS,
+                  on_ids=None) -> list[list[int]]:
+    """Feeds `tokens` and queues up to `count` one-token steps, each step's ids going into the
+    next on the device; returns the sampled ids of the steps that ran, [steps][rows]. The host
+    reads the ids of a step when `ahead` - 1 further steps have been queued behind it, so inside
+    a run the device never waits for the host. With stop ids or `cancel`, the ids of step j are
+    read while step j + 1 runs, and the run ends with the step that was queued when a stop token
+    (or the cancellation) was seen. on_ids(j, ids) hands over the ids of step j once a later
+    step's have been read: every step of the run but its last, whose ids the caller feeds next."""
+    from ..sampling.sampler import READS_IN_FLIGHT
     # the penalty windows (the generated tokens, the ones fed now included) go to the device once
     window = sampler.window_device(contexts) if sampler.config.has_penalties and contexts is not None else None
     watch = bool(stop_ids) or cancel is not None
-    reads, ids, device_ids = [], [], None
+    depth = 1 if watch else max(1, min(ahead, READS_IN_FLIGHT) - 1)
+    draws = max(1, ahead)          # random draws go up for so many steps at a time, while earlier steps run
+    reads, ids, device_ids, uniforms = [], [], None, None
+
+    def take() -> None:
+        """Reads the oldest step not yet read."""
+        ids.append(reads[len(ids)].wait())
+        if on_ids is not None and len(ids) >= 2:
+            on_ids(len(ids) - 2, ids[-2])
+
     for j in range(count):
+        if not sampler.config.is_greedy and j % draws == 0:
+            uniforms = sampler.uniforms_device(seqs, [t + j for t in steps], min(draws, count - j))
         entries = [StepEntry(s, [t], [0]) for s, t in zip(slots, tokens)]
         logits = engine.step(entries, device_tokens=device_ids)
         more = {} if window is None else {"window": window, "last_ids": device_ids}
         device_ids = sampler.sample_device(logits, seqs, [t + j for t in steps],
-                                           uniforms=None if uniforms is None else uniforms[j], **more)
+                                           uniforms=None if uniforms is None else uniforms[j % draws], **more)
         reads.append(sampler.read_later(device_ids))
-        if watch and j >= 1:
-            ids.append(reads[j - 1].wait())
-            if not stop_ids.isdisjoint(ids[-1]) or (cancel is not None and cancel()):
+        if j >= depth:
+            take()
+            if watch and (not stop_ids.isdisjoint(ids[-1]) or (cancel is not None and cancel())):
                 break
-    ids += [r.wait() for r in reads[len(ids):]]
+    while len(ids) < len(reads):
+        take()
     return ids
 
 
@@ -220,23 +238,26 @@ def _run_batch(engine, prompts, admitted, results, max_new_tokens, stop_ids, inc
                 break
             count = 1 if sampler is None else steps_in_run(
                 [len(out[i]) for i in active], [engine.length(slots[i]) for i in active],
-                max_new_tokens, engine.max_seq_len, run_of_steps)
+                max_new_tokens, engine.max_seq_len, LONGEST_RUN)
             if count == 1:
                 logits = engine.step([StepEntry(slots[i], [tok], [0]) for i, tok in feed])
                 tokens = sample_fn(logits, active, [len(out[i]) for i in active], [out[i] for i in active])
                 continue
+            # all but the last step of the run are decided as their ids are read, each with the cache
+            # length of its moment; a sequence that ends inside the run drops the rest of its ids
+            before = {i: engine.length(slots[i]) for i in active}
+            going = dict.fromkeys(active, True)
+            row_of = list(active)
+
+            def decide_step(j, row):
+                for col, i in enumerate(row_of):
+                    if going[i]:
+                        going[i] = decide(i, row[col], before[i] + j + 1)
+
             run = _run_of_steps(engine, sampler, [slots[i] for i in active], [tok for _, tok in feed],
                                 active, [len(out[i]) for i in active], count, stop_ids, cancel,
-                                [out[i] for i in active])
-            count = len(run)            # fewer when a stop token was seen on the way
-            # all but the last step of the run are decided here, each with the cache length of its
-            # moment; a sequence that ends inside the run drops the rest of its ids
-            going = dict.fromkeys(active, True)
-            for j in range(count - 1):
-                for col, i in enumerate(active):
-                    if going[i]:
-                        going[i] = decide(i, run[j][col], engine.length(slots[i]) - (count - 1 - j))
-            tokens = [run[count - 1][col] for col, i in enumerate(active) if going[i]]
+                                [out[i] for i in active], run_of_steps, decide_step)
+            tokens = [run[-1][col] for col, i in enumerate(active) if going[i]]
             active = [i for i in active if going[i]]
     finally:
         for i in list(slots):

@@ -241,6 +241,36 @@ def test_runs_without_stop_ids_read_their_ids_once():
     assert eng.cache.book.slots.available == 3
 
 
+def test_the_host_reads_ids_a_fixed_number_of_steps_behind_the_queue():
+    """Without stop ids one run reaches to the budget, far beyond run_of_steps; the host has read
+    (and handed out) the ids of step j by the time step j + run_of_steps is queued, and never
+    looks at a step's ids before run_of_steps - 1 further steps are queued behind it: the device
+    has work queued while the host waits. With stop ids the host is one step behind."""
+    for ahead, stop in ((8, ()), (3, ()), (8, {(1 + 2 + 2) % V + 99})):       # the last: a stop id that never comes
+        eng, sampler = FakeEngine(), FakeSampler()
+        seen_at_step = []                 # tokens handed out when one-token step k was queued
+        handed = []
+        step = eng.step
+
+        def logged_step(entries, device_tokens=None):
+            if all(len(e.tokens) == 1 for e in entries):
+                seen_at_step.append(len(handed))
+            return step(entries, device_tokens)
+
+        eng.step = logged_step
+        r = generate(eng, [[1, 2]], max_new_tokens=40, sampler=sampler, run_of_steps=ahead,
+                     stop_ids=stop, on_token=lambda i, tok: handed.append(tok))[0]
+        assert (r.tokens, r.finish_reason) == expected([1, 2], 40) and handed == r.tokens
+        assert len(seen_at_step) == 39     # one run: the prompt step gave the first token, none wasted
+        lag = 2 if stop else ahead
+        for k, n in enumerate(seen_at_step):
+            # token 0 came from the prompt step; step k samples token k + 1. The loop hands a step's ids
+            # out once the next step's ids are read, hence one step more than the reading itself.
+            assert n >= min(1, k + 1) + max(0, k - lag), (k, n)
+            assert n <= 1 + max(0, k - (1 if stop else ahead - 1)), (k, n)
+        assert sampler.waits == 39
+
+
 def test_cancel_is_seen_inside_a_run():
     eng = FakeEngine()
     calls = {"n": 0}
