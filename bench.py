@@ -18,9 +18,9 @@ leaves them out), each with its share of the HBM peak in `points_roofline_frac`:
                      `prefill_fp32`, the 2,048-token prompt in 32-bit against the fp32 peak
 
 A step is one decode step of the whole batch: the engine's step function (HIP
-graph replay) plus greedy sampling. As in the library's generation loop, 8 steps are
-queued at a time: the chosen ids go into the next step on the device, and the host
-reads them once per run of 8.
+graph replay) plus greedy sampling. As in the library's generation loop, steps are
+queued ahead of the host: the chosen ids go into the next step on the device, and the host
+reads a step's ids when 7 further steps are queued behind it.
 
 Procedure (the reference quotes medians with their range over repeated runs:
 tools/HQS_DECODE_OPTIMIZATION_PLAN.md:54-65): after the warm-up steps, `--repeats` (5) runs of
