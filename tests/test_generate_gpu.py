@@ -173,6 +173,26 @@ def test_penalties(he, model_dirs, plain_models):
     assert got == want and got != plainly
 
 
+def test_one_long_run_of_queued_steps_with_draws_and_penalties(he, model_dirs, plain_models):
+    """Without stop ids the whole generation is one run of queued steps: 150 of them here, far
+    more than the host keeps reads in flight, with random draws that go up eight steps at a time,
+    a penalty window on the device that wraps round many times. Token for token what the plain loop
+    gives, handed out in order."""
+    cfg, w = plain_models["A"]
+    prompts = prompts_for(cfg, [5, 21], 500)
+    eng = he.Engine(model_dirs["A"], dtype="float32", max_tokens=1024, max_seq_len=512, beyond_max_positions=True)
+    sampling = he.SamplingConfig(temperature=0.9, top_k=12, top_p=0.95, seed=11, repetition_penalty=1.2,
+                                 frequency_penalty=0.1, presence_penalty=0.1, penalty_window=7)
+    seen = {0: [], 1: []}
+    got = he.generate(eng, prompts, max_new_tokens=150, sampling=sampling, stop_ids=(),
+                      on_token=lambda i, tok: seen[i].append(tok))
+    for i, (p, r) in enumerate(zip(prompts, got)):
+        want = P.generate(cfg, w, p, 150, 0.9, 12, 0.95, 11, i, (), 1.2, 0.1, 0.1, 7)
+        assert r.tokens == want and r.finish_reason == "max_tokens" and seen[i] == want
+    assert eng.stats["graph_replays"] >= 140
+    assert eng.cache.free_pages == eng.cache.num_pages
+
+
 def test_cache_room_ends_a_sequence(he, model_dirs):
     eng = he.Engine(model_dirs["A"], dtype="bfloat16", max_tokens=128, max_slots=2, max_seq_len=64)
     r = he.generate(eng, [[1] * 60, [2] * 64], max_new_tokens=20)
