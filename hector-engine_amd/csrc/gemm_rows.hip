@@ -60,7 +60,9 @@ static RowsPlan rows_plan(int M, int N, int K, int R, int NWV, int splits) {
   int s = splits;
   if (s <= 0) {
     s = 1;
-    while (p.groups * s < cus * 3 / 4 && K / (2 * s) >= 512 && s < 32) s *= 2;   // 192 workgroups on 256 units
+    // 192 workgroups on 256 units, slices of four chunks or more (q||k||v of 4608 x 3584 at 64 rows: 36 groups
+    // in 7 slices of 512 take 15.9 us with their sum, in 4 slices of 896 17.8 us)
+    while (p.groups * s < cus * 3 / 4 && K / (2 * s) >= 256 && s < 32) s *= 2;
   }
   int ks = (K + s - 1) / s;
   ks = (ks + ROWS_KC - 1) / ROWS_KC * ROWS_KC;
