@@ -80,6 +80,40 @@ __device__ __forceinline__ void q_biased(float (&x)[NT / 2][8], const QLoads<NT>
   }
 }
 
+// The projection row from the K slices of its product: the product of 17 to 64 rows is cut along K
+// across workgroups and leaves fp32 sums [slices][rows][width] (gemm_rows.hip). Added in slice
+// order and rounded to bfloat16, the values are the bits he_splitk_reduce would have written, and
+// its launch is not needed. The loads of up to eight slices go out together.
+template <typename V>
+__device__ __forceinline__ V slices_sum(const float* part, int slices, int64_t slice_stride);
+template <>
+__device__ __forceinline__ float4 slices_sum<float4>(const float* part, int slices, int64_t slice_stride) {
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int s0 = 0; s0 < slices; s0 += 8) {
+    float4 v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const float4*>(part + (int64_t)min(s0 + j, slices - 1) * slice_stride);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (s0 + j < slices) acc.x += v[j].x, acc.y += v[j].y, acc.z += v[j].z, acc.w += v[j].w;
+  }
+  return acc;
+}
+template <>
+__device__ __forceinline__ float slices_sum<float>(const float* part, int slices, int64_t slice_stride) {
+  float acc = 0.f;
+  for (int s0 = 0; s0 < slices; s0 += 8) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = part[(int64_t)min(s0 + j, slices - 1) * slice_stride];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (s0 + j < slices) acc += v[j];
+  }
+  return acc;
+}
+__device__ __forceinline__ float as_bf16(float v) { return bf16_bits_to_float(float_to_bf16_bits(v)); }
+
 template <int NT>
 __device__ __forceinline__ void rotate_q(bf16x8* qf, float (&x)[NT / 2][8], int lg, float sn, float c) {
   constexpr int KS = NT / 2;
@@ -101,10 +135,13 @@ __device__ __forceinline__ void rotate_q(bf16x8* qf, float (&x)[NT / 2][8], int 
                            pack2_bf16(x[ks][4], x[ks][5]), pack2_bf16(x[ks][6], x[ks][7])));
 }
 
-template <int NT>
+// SLICED: qkv is null and the projection row comes as the fp32 sums of its K slices,
+// qkv_part [qkv_slices][.][qkv_stride], slice_stride elements from slice to slice.
+template <int NT, bool SLICED>
 __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
     uint16_t* __restrict__ out, float* __restrict__ ws_o, float* __restrict__ ws_ml,
-    const uint16_t* __restrict__ qkv, int64_t qkv_stride,
+    const uint16_t* __restrict__ qkv, const float* __restrict__ qkv_part, int qkv_slices,
+    int64_t slice_stride, int64_t qkv_stride,
     const void* __restrict__ bias, int bias_dtype, uint16_t* kpool, uint16_t* vpool,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
     const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ page_table, int max_blocks,
@@ -136,9 +173,10 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
   // by then; a volatile load bypasses the caches and is waited for where it stands.)
   int touched = 0;
   if (by_row && lane < ((max_blocks * 4 + 127) >> 7)) touched = page_table[(int64_t)row * max_blocks + 32 * lane];
-  const uint16_t* qkv_row = qkv + (int64_t)row * qkv_stride;
+  const uint16_t* qkv_row = SLICED ? nullptr : qkv + (int64_t)row * qkv_stride;
+  const float* part_row = SLICED ? qkv_part + (int64_t)row * qkv_stride : nullptr;
   QLoads<NT> ql;
-  q_issue<NT>(ql, qkv_row + (int64_t)h * HD, bias, bias_dtype, h * HD, lg);
+  if (!SLICED) q_issue<NT>(ql, qkv_row + (int64_t)h * HD, bias, bias_dtype, h * HD, lg);
   const float freq = inv_freq[min(lane, HD / 2 - 1)];   // no condition in front of the load (the lanes beyond take no angle)
   const int seq = row_seq[row];
   const int Z = gridDim.z, z = blockIdx.z;
@@ -185,7 +223,7 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
   AttendCursor<NT> cursor;
   if (early) attend_pages<NT>(cursor, pt, max_blocks, kb_begin);
   float qx[NT / 2][8];
-  q_biased<NT>(qx, ql, bias, bias_dtype, h * HD, h_ok, lg);
+  if (!SLICED) q_biased<NT>(qx, ql, bias, bias_dtype, h * HD, h_ok, lg);
   // The angle is formed here, ahead of the loads of the first keys: its frequency was asked for at
   // the top, and a wait for it behind those loads would be a wait for them too (loads complete in
   // order): the sines and the rotation of q, which are meant to run while the keys are on their way,
@@ -194,6 +232,31 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
   asm volatile("" : "+v"(angle));
   __builtin_amdgcn_sched_barrier(0);
   if (early) attend_first<NT>(cursor, kpool, vpool, num_pages, KVH, kvh, kb_begin, lr, lg);
+  if (SLICED) {
+    // The workgroup adds the slices of its heads' q once, four neighbouring values a thread, and hands
+    // the sums round through LDS (the buffer the join uses at the end); every wavefront then takes its
+    // operand's values from there. Summed wavefront by wavefront the same values would be fetched
+    // as many times as the workgroup has wavefronts, a round trip a slice.
+    const int h0 = kvh * G + 16 * ht;
+    for (int v4 = threadIdx.x; v4 < GT * (HD / 4); v4 += blockDim.x) {
+      const int col = h0 * HD + 4 * v4;
+      const float4 sum = slices_sum<float4>(part_row + col, qkv_slices, slice_stride);
+      float q4[4] = {as_bf16(sum.x), as_bf16(sum.y), as_bf16(sum.z), as_bf16(sum.w)};
+      if (bias != nullptr)
+        for (int i = 0; i < 4; ++i) q4[i] += load_param(bias, col + i, bias_dtype);
+      *reinterpret_cast<float4*>(lds + 4 * v4) = make_float4(q4[0], q4[1], q4[2], q4[3]);
+    }
+    __syncthreads();
+    const float* ql_row = lds + min(lr, GT - 1) * HD + 8 * lg;
+#pragma unroll
+    for (int ks = 0; ks < NT / 2; ++ks) {
+      const float4 a = *reinterpret_cast<const float4*>(ql_row + 32 * ks);
+      const float4 b = *reinterpret_cast<const float4*>(ql_row + 32 * ks + 4);
+      qx[ks][0] = h_ok ? a.x : 0.f, qx[ks][1] = h_ok ? a.y : 0.f, qx[ks][2] = h_ok ? a.z : 0.f, qx[ks][3] = h_ok ? a.w : 0.f;
+      qx[ks][4] = h_ok ? b.x : 0.f, qx[ks][5] = h_ok ? b.y : 0.f, qx[ks][6] = h_ok ? b.z : 0.f, qx[ks][7] = h_ok ? b.w : 0.f;
+    }
+    __syncthreads();     // the buffer is written again when the wavefronts' slices are joined
+  }
   float sn = 0.f, c = 1.f;                   // lane j < HD / 2: angle j of position p
   if (has_keys && lane < HD / 2) sincos_angle(angle, &sn, &c);
 
@@ -209,8 +272,10 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
       uint16_t* vpage = vpool + ((int64_t)page * KVH + kvh) * he_v_page_elems(HD);
       if (lane < half) {                     // half <= 64: one pair per lane
         const int j = lane;
-        float x0 = bf16_bits_to_float(qkv_row[k_col + j]);
-        float x1 = bf16_bits_to_float(qkv_row[k_col + j + half]);
+        float x0 = SLICED ? as_bf16(slices_sum<float>(part_row + k_col + j, qkv_slices, slice_stride))
+                          : bf16_bits_to_float(qkv_row[k_col + j]);
+        float x1 = SLICED ? as_bf16(slices_sum<float>(part_row + k_col + j + half, qkv_slices, slice_stride))
+                          : bf16_bits_to_float(qkv_row[k_col + j + half]);
         if (bias) {
           x0 += load_param(bias, k_col + j, bias_dtype);
           x1 += load_param(bias, k_col + j + half, bias_dtype);
@@ -219,7 +284,8 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
         kpage[he_k_index(off, j + half, KS)] = float_to_bf16_bits(x0 * sn + x1 * c);
       }
       for (int d = lane; d < HD; d += 64) {
-        float x = bf16_bits_to_float(qkv_row[v_col + d]);
+        float x = SLICED ? as_bf16(slices_sum<float>(part_row + v_col + d, qkv_slices, slice_stride))
+                         : bf16_bits_to_float(qkv_row[v_col + d]);
         if (bias) x += load_param(bias, v_col + d, bias_dtype);
         vpage[he_v_index(off, d, NT)] = float_to_bf16_bits(x);
       }
@@ -344,7 +410,9 @@ extern "C" int64_t he_attention_decode_fused_workspace_floats(int rows, int H, i
   return Z == 1 ? 0 : (int64_t)rows * H * Z * (hd + 2);
 }
 
-extern "C" int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_t qkv_stride,
+extern "C" int he_attention_decode_fused_bf16(void* out, const void* qkv, const void* qkv_part,
+                                              int qkv_slices, int64_t qkv_slice_stride,
+                                              int64_t qkv_stride,
                                               const void* bias, int bias_dtype, void* kpool,
                                               void* vpool, const void* positions,
                                               const void* row_seq, const void* seq_slot,
@@ -361,6 +429,12 @@ extern "C" int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_
              "he_attention_decode_fused_bf16: sizes H=%d KVH=%d head_dim=%d rotary_dim=%d are not "
              "taken (head_dim 64 or 128, rotated whole)", H, KVH, hd, rotary_dim);
   HE_REQUIRE(rows <= 65535, "he_attention_decode_fused_bf16: %d rows above 65535", rows);
+  HE_REQUIRE((qkv != nullptr) != (qkv_part != nullptr),
+             "he_attention_decode_fused_bf16: the projection rows come as bfloat16 rows or as K slices, one of the two");
+  HE_REQUIRE(qkv_part == nullptr || (qkv_slices >= 1 && qkv_slices <= 64 && (((uintptr_t)qkv_part) & 15) == 0 &&
+                                     qkv_slice_stride >= (int64_t)rows * qkv_stride && (qkv_slice_stride & 3) == 0),
+             "he_attention_decode_fused_bf16: %d K slices (1 to 64) of %lld elements each, 16-byte aligned, for %d rows of %lld",
+             qkv_slices, (long long)qkv_slice_stride, rows, (long long)qkv_stride);
   HE_REQUIRE((qkv_stride & 7) == 0 && (((uintptr_t)qkv) & 15) == 0 &&
                  (((uintptr_t)kpool) & 15) == 0 && (((uintptr_t)vpool) & 15) == 0 &&
                  (((uintptr_t)out) & 7) == 0,
@@ -382,15 +456,18 @@ extern "C" int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_
   const size_t lds = (size_t)nw * gt * (hd + 2) * sizeof(float);
   hipStream_t s = (hipStream_t)stream;
   dim3 grid(KVH * head_tiles, rows, Z);
-#define FUSED(NTV)                                                                              \
-  case NTV:                                                                                     \
-    attention_decode_fused_kernel<NTV><<<grid, 64 * nw, lds, s>>>(                              \
-        (uint16_t*)out, ws_o, ws_ml, (const uint16_t*)qkv, qkv_stride, bias, bias_dtype,        \
+#define FUSED_LAUNCH(NTV, SL)                                                                   \
+    attention_decode_fused_kernel<NTV, SL><<<grid, 64 * nw, lds, s>>>(                          \
+        (uint16_t*)out, ws_o, ws_ml, (const uint16_t*)qkv, (const float*)qkv_part, qkv_slices,  \
+        qkv_slice_stride, qkv_stride, bias, bias_dtype,                                         \
         (uint16_t*)kpool,                                                                       \
         (uint16_t*)vpool, (const int32_t*)positions, (const int32_t*)row_seq,                   \
         (const int32_t*)seq_slot, (const int32_t*)page_table, max_blocks, num_pages,            \
         (const float*)inv_freq, rotary_dim, H, KVH, head_tiles, window, scale, write_kv,        \
-        out_pieces);                                                                            \
+        out_pieces)
+#define FUSED(NTV)                                                                              \
+  case NTV:                                                                                     \
+    if (qkv_part != nullptr) FUSED_LAUNCH(NTV, true); else FUSED_LAUNCH(NTV, false);            \
     break;
   switch (hd / 16) {
     FUSED(4) FUSED(8)
@@ -398,6 +475,7 @@ extern "C" int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_
       HE_REQUIRE(false, "he_attention_decode_fused_bf16: head_dim %d", hd);
   }
 #undef FUSED
+#undef FUSED_LAUNCH
   const int rc = he_check_launch("he_attention_decode_fused_bf16");
   if (rc || Z == 1) return rc;
   return he_attention_merge_parts(out, ws_o, ws_ml, row_seq, rows, H, hd, Z, out_pieces, stream);

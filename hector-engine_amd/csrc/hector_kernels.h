@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 19
+#define HE_ABI_VERSION 20
 
 #ifdef __cplusplus
 extern "C" {
@@ -136,11 +136,15 @@ int64_t he_attention_decode_workspace_floats(int rows, int H, int KVH, int hd, i
 // (as he_gemm_blocksplit_fused_bf16 reads it with x_pieces). spread: one sequence of the step has
 // several times the keys of the others; every sequence's keys are then cut across more workgroups.
 // seq_slot null: page_table has a row per row of the step ([rows, max_blocks], the page numbers of
-// the row's sequence) instead of a row per slot.
+// the row's sequence) instead of a row per slot. qkv null: the projection rows come as the fp32
+// sums of their K slices, qkv_part [qkv_slices][.][qkv_stride] with qkv_slice_stride elements from
+// slice to slice (what he_gemm_rows_bf16 leaves when it cuts a product along K); the kernel adds
+// them in slice order and rounds to bfloat16, the bits he_splitk_reduce would have written.
 int he_attention_decode_fused_ok(int H, int KVH, int hd, int rotary_dim);
 int64_t he_attention_decode_fused_workspace_floats(int rows, int H, int KVH, int hd, int max_keys,
                                                    int spread);
-int he_attention_decode_fused_bf16(void* out, const void* qkv, int64_t qkv_stride, const void* bias,
+int he_attention_decode_fused_bf16(void* out, const void* qkv, const void* qkv_part, int qkv_slices,
+                                   int64_t qkv_slice_stride, int64_t qkv_stride, const void* bias,
                                    int bias_dtype, void* kpool, void* vpool, const void* positions,
                                    const void* row_seq, const void* seq_slot,
                                    const void* page_table, int max_blocks, int num_pages,

@@ -16,7 +16,7 @@ _lib = None
 
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 
-EXPECTED_ABI = 19
+EXPECTED_ABI = 20
 
 c_int, c_i64, c_f32, c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
@@ -62,7 +62,7 @@ _SIGNATURES = {
     "he_attention_decode_workspace_floats": [c_int, c_int, c_int, c_int, c_int],
     "he_attention_decode_fused_ok": [c_int, c_int, c_int, c_int],
     "he_attention_decode_fused_workspace_floats": [c_int, c_int, c_int, c_int, c_int, c_int],
-    "he_attention_decode_fused_bf16": [c_ptr, c_ptr, c_i64, c_ptr, c_int, c_ptr, c_ptr, c_ptr, c_ptr,
+    "he_attention_decode_fused_bf16": [c_ptr, c_ptr, c_ptr, c_int, c_i64, c_i64, c_ptr, c_int, c_ptr, c_ptr, c_ptr, c_ptr,
                                        c_ptr, c_ptr, c_int, c_int, c_ptr, c_int, c_int, c_int, c_int,
                                        c_int, c_int, c_f32, c_int, c_int, c_int, c_int, c_ptr, c_i64, c_ptr],
     "he_attention_prefill_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int,

@@ -561,16 +561,28 @@ def attention_decode_fused(out, qkv, bias, kpool, vpool, positions, row_seq, seq
     """One-token steps in one launch: bias, rotation of q and of the new key, cache write,
     attention over the cache, merge. spread: one sequence has several times the keys of the
     others (every sequence's keys are then cut across more workgroups; the workspace is asked for
-    with the same flag). qkv: bf16 [rows, (H + 2 KVH) hd] without bias; q columns
+    with the same flag). qkv: bf16 [rows, (H + 2 KVH) hd] without bias, or fp32 [slices, rows, width]:
+    the sums of the projection's K slices as gemm_rows leaves them; q columns
     alone where the run reads another run's cache (write_kv False). out_pieces: out is written
     piece-major for exactly `rows` rows (see :func:`to_pieces`). seq_slot None: page_table has a row
     per row of the step ([rows or more, blocks]: the page numbers of the row's sequence), not a
     row per slot; the kernel then asks for them at its start, without the chain through the slot."""
     width = (H + 2 * KVH) * hd if write_kv else H * hd
-    _need(qkv, "qkv", torch.bfloat16)
     _need(out, "out", torch.bfloat16)
-    if qkv.dim() != 2 or qkv.shape[1] != width or qkv.shape[0] < rows or out.numel() < rows * H * hd:
-        raise ValueError("attention_decode_fused: qkv/out do not match the head sizes and row count")
+    slices, slice_stride = 0, 0
+    if qkv.dtype == torch.float32:
+        # the fp32 sums of the projection's K slices, [slices, rows of the product, width] (gemm_rows):
+        # the kernel adds them itself, in slice order, and rounds as splitk_reduce would have
+        _need(qkv, "qkv (K slices)", torch.float32)
+        if qkv.dim() != 3 or qkv.shape[2] != width or qkv.shape[1] < rows:
+            raise ValueError("attention_decode_fused: K slices [slices, rows, width] do not match the head sizes and row count")
+        slices, slice_stride = qkv.shape[0], qkv.shape[1] * width
+    else:
+        _need(qkv, "qkv", torch.bfloat16)
+        if qkv.dim() != 2 or qkv.shape[1] != width or qkv.shape[0] < rows:
+            raise ValueError("attention_decode_fused: qkv does not match the head sizes and row count")
+    if out.numel() < rows * H * hd:
+        raise ValueError("attention_decode_fused: out does not match the head sizes and row count")
     if out_pieces:
         _need(out, "out", shape=pieces_shape(rows, H * hd))
     _need(kpool, "kpool", torch.bfloat16, (None, KVH, layout.k_page_elems(hd)))
@@ -589,7 +601,8 @@ def attention_decode_fused(out, qkv, bias, kpool, vpool, positions, row_seq, seq
         _need(workspace, "workspace", torch.float32)
     L = _lib.load()
     _lib.check(L.he_attention_decode_fused_bf16(
-        out.data_ptr(), qkv.data_ptr(), width, _ptr(bias),
+        out.data_ptr(), qkv.data_ptr() if not slices else None, qkv.data_ptr() if slices else None, slices,
+        slice_stride, width, _ptr(bias),
         dtype_code(bias.dtype) if bias is not None else F32, kpool.data_ptr(), vpool.data_ptr(),
         positions.data_ptr(), row_seq.data_ptr(), _ptr(seq_slot), page_table.data_ptr(),
         page_table.shape[1], kpool.shape[0], inv_freq.data_ptr(), rotary_dim, rows, H, KVH, hd,

@@ -137,7 +137,11 @@ class Attention(Mixer):
         rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.hd
         proj = self.qkv if cache.writes else self.q_only
         rot = self.position.rotary()
-        qkv = proj(x, rows, ctx, use_bias=False)
+        # where the projection is cut along K (17 to 64 rows), the kernel below adds the slices
+        # itself: the same bits, and the launch that would add them is not needed
+        qkv = proj.k_slices(x, rows, ctx)
+        if qkv is None:
+            qkv = proj(x, rows, ctx, use_bias=False)
         pieces = self.o_proj.reads_pieces(rows, ctx)       # the layout the output product reads best
         out = ctx.alloc(ops.pieces_shape(rows, H * hd) if pieces else (rows, H * hd))
         uneven = bool(ctx.hints.get(keys_uneven, False))

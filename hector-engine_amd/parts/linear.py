@@ -94,6 +94,22 @@ class Linear:
         """Whether bf16 input rows may come piece-major (PieceRows)."""
         return self._has("pieces", rows, ctx, BF16)
 
+    def k_slices(self, x, rows: int, ctx: StepContext):
+        """The product without bias as the fp32 sums of its K slices, [slices, rows, N], where the
+        kernel of this step cuts it along K across workgroups (17 to 64 rows of a weight with few
+        rows); None where it does not, and the caller calls the layer as usual. A reader that adds
+        the slices itself, in their order, and rounds to the activation dtype has the bits the
+        layer's own sum would have written, and saves that launch."""
+        act, a, scale, pieces = _operand(x)
+        if rows <= ops.BLOCKSPLIT_PIECES_MAX_M or not self._has("k_slices", rows, ctx, act):
+            return None
+        splits = self._plan(rows)[1]
+        if splits == 1:
+            return None
+        partial = ctx.alloc((splits, rows, self.weight.shape[0]), torch.float32)
+        ops.gemm_rows(None, partial, a, self.weight, None, rows, row_scale=scale, x_pieces=pieces)
+        return partial
+
     def _plan(self, rows: int) -> tuple[int, int]:
         """(workgroups along N, K slices) of the 17-to-64-row kernel for this weight."""
         key = rows <= 32
@@ -295,7 +311,8 @@ def _mfma_takes(case: ProductCase) -> bool:
     return case.fast and case.K % 8 == 0 and 0 < case.rows <= ops.ROWS_MAX_M
 
 
-routes.register_route("linear", (BF16, BF16), "mfma", _mfma_takes, Linear._run_mfma, traits=("pieces", "gated"))
+routes.register_route("linear", (BF16, BF16), "mfma", _mfma_takes, Linear._run_mfma,
+                      traits=("pieces", "gated", "k_slices"))
 routes.register_route("linear", (BF16, BF16), "plain", lambda c: not c.fast or c.K % 8 != 0, Linear._run_plain)
 routes.register_route("linear", (BF16, BF16), "library", lambda c: True, Linear._run_library)
 routes.register_route("linear", (F32, F32), "plain", lambda c: True, Linear._run_plain)

@@ -832,6 +832,25 @@ def test_attention_decode_fused(ops, H, KVH, hd, window, write_kv, copies):
                                None, dev(by_row), dev(inv), hd, rows, H, KVH, hd, window,
                                1.0 / math.sqrt(hd), 4096, write_kv, ws)
     assert torch.equal(out3.cpu(), out.cpu())
+    # the projection rows as the fp32 sums of K slices (what the rows kernel leaves at 17 to 64 rows):
+    # the kernel adds them in slice order and rounds as the kernel that sums them would have
+    S = 7 if copies == 1 else 3
+    parts = rnd(S, rows, width, seed=83, scale=0.6).cuda()
+    summed = torch.empty(rows, width, dtype=torch.bfloat16, device="cuda")
+    ops.splitk_reduce(summed, parts, None, rows, S)
+    outs, pools = [], []
+    for given in (summed, parts):
+        o = torch.full((rows, H * hd), 7.0, dtype=torch.bfloat16, device="cuda")
+        kq, vq = dev(kpool), dev(vpool)
+        ops.attention_decode_fused(o, given, dev(bias), kq, vq, dev(positions), dev(row_seq), dev(seq_slot),
+                                   dev(table), dev(inv), hd, rows, H, KVH, hd, window, 1.0 / math.sqrt(hd), 4096,
+                                   write_kv, ws)
+        outs.append(o.cpu())
+        pools.append((kq.cpu(), vq.cpu()))
+    assert torch.equal(outs[0], outs[1])
+    assert torch.equal(pools[0][0], pools[1][0]) and torch.equal(pools[0][1], pools[1][1])
+    if write_kv:
+        assert not torch.equal(pools[0][0], dev(kpool).cpu())      # the new rows did go in
 
 
 def test_attention_decode_fused_refuses_other_sizes(ops):
