@@ -58,6 +58,9 @@ def test_which_route_a_product_and_an_attention_step_take():
     assert product(8, dtypes=(f32, f32)) == "plain" and product(8, dtypes=(f32, bf)) == "plain_widened"
     with pytest.raises(TypeError, match=r"linear: no kernel for \(float16, bfloat16\); registered: .*\(bfloat16, bfloat16\)"):
         product(8, dtypes=(torch.float16, bf))
+    # what a part may ask a route for: piece-major rows, the gated epilogue, the K slices of a product
+    traits = {r.name: set(r.traits) for r in routes.routes_of("linear", (bf, bf))}
+    assert traits == {"mfma": {"pieces", "gated", "k_slices"}, "plain": set(), "library": set()}
 
     def attention(all_single, fast=True, fusable=True, dtype=bf):
         return routes.choose("attention", (dtype,), AttentionCase(all_single, fast, fusable)).name
