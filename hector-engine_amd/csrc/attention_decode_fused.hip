@@ -125,8 +125,10 @@ __device__ __forceinline__ void rotate_q(bf16x8* qf, float (&x)[NT / 2][8], int 
       const int i = 32 * ks + 8 * lg + j;
       const float si = __shfl(sn, i, HE_WAVE), ci = __shfl(c, i, HE_WAVE);
       const float a0 = x[ks][j], a1 = x[ks + HS][j];
-      x[ks][j] = a0 * ci - a1 * si;
-      x[ks + HS][j] = a0 * si + a1 * ci;
+      // one multiply-add each, written out: left to the compiler, the two instantiations of the
+      // kernel may fuse the two products differently and differ in a last bit
+      x[ks][j] = fmaf(a0, ci, -(a1 * si));
+      x[ks + HS][j] = fmaf(a0, si, a1 * ci);
     }
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks)
@@ -177,6 +179,15 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
   const float* part_row = SLICED ? qkv_part + (int64_t)row * qkv_stride : nullptr;
   QLoads<NT> ql;
   if (!SLICED) q_issue<NT>(ql, qkv_row + (int64_t)h * HD, bias, bias_dtype, h * HD, lg);
+  // SLICED: the first eight slices of the four q values this thread adds (see below) are asked for
+  // here, with everything else that needs nothing but the row
+  float4 q_early[8];
+  const int q_col = (kvh * G + 16 * ht) * HD + 4 * min((int)threadIdx.x, GT * (HD / 4) - 1);
+  if (SLICED) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      q_early[j] = *reinterpret_cast<const float4*>(part_row + q_col + (int64_t)min(j, qkv_slices - 1) * slice_stride);
+  }
   const float freq = inv_freq[min(lane, HD / 2 - 1)];   // no condition in front of the load (the lanes beyond take no angle)
   const int seq = row_seq[row];
   const int Z = gridDim.z, z = blockIdx.z;
@@ -240,7 +251,15 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
     const int h0 = kvh * G + 16 * ht;
     for (int v4 = threadIdx.x; v4 < GT * (HD / 4); v4 += blockDim.x) {
       const int col = h0 * HD + 4 * v4;
-      const float4 sum = slices_sum<float4>(part_row + col, qkv_slices, slice_stride);
+      float4 sum;
+      if (v4 == (int)threadIdx.x && qkv_slices <= 8) {      // the loads issued at the top
+        sum = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (j < qkv_slices) sum.x += q_early[j].x, sum.y += q_early[j].y, sum.z += q_early[j].z, sum.w += q_early[j].w;
+      } else {
+        sum = slices_sum<float4>(part_row + col, qkv_slices, slice_stride);
+      }
       float q4[4] = {as_bf16(sum.x), as_bf16(sum.y), as_bf16(sum.z), as_bf16(sum.w)};
       if (bias != nullptr)
         for (int i = 0; i < 4; ++i) q4[i] += load_param(bias, col + i, bias_dtype);
@@ -270,22 +289,46 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
       // the page in operand order (cache_layout.h)
       uint16_t* kpage = kpool + ((int64_t)page * KVH + kvh) * he_k_page_elems(HD);
       uint16_t* vpage = vpool + ((int64_t)page * KVH + kvh) * he_v_page_elems(HD);
+      // SLICED: the slices of this lane's two key values and (up to) two value values, all loads
+      // issued before the first sum (one after the other they were four round trips on the path the
+      // launch waits for)
+      float k_sl[2] = {0.f, 0.f}, v_sl[2] = {0.f, 0.f};
+      if (SLICED) {
+        const float* at[4] = {part_row + k_col + min(lane, half - 1), part_row + k_col + min(lane, half - 1) + half,
+                              part_row + v_col + min(lane, HD - 1), part_row + v_col + min(lane + 64, HD - 1)};
+        if (qkv_slices <= 8) {
+          float got[4][8];
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) got[q][j] = at[q][(int64_t)min(j, qkv_slices - 1) * slice_stride];
+          float sum[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (j < qkv_slices)
+#pragma unroll
+              for (int q = 0; q < 4; ++q) sum[q] += got[q][j];
+          k_sl[0] = as_bf16(sum[0]), k_sl[1] = as_bf16(sum[1]), v_sl[0] = as_bf16(sum[2]), v_sl[1] = as_bf16(sum[3]);
+        } else {
+          k_sl[0] = as_bf16(slices_sum<float>(at[0], qkv_slices, slice_stride));
+          k_sl[1] = as_bf16(slices_sum<float>(at[1], qkv_slices, slice_stride));
+          v_sl[0] = as_bf16(slices_sum<float>(at[2], qkv_slices, slice_stride));
+          v_sl[1] = as_bf16(slices_sum<float>(at[3], qkv_slices, slice_stride));
+        }
+      }
       if (lane < half) {                     // half <= 64: one pair per lane
         const int j = lane;
-        float x0 = SLICED ? as_bf16(slices_sum<float>(part_row + k_col + j, qkv_slices, slice_stride))
-                          : bf16_bits_to_float(qkv_row[k_col + j]);
-        float x1 = SLICED ? as_bf16(slices_sum<float>(part_row + k_col + j + half, qkv_slices, slice_stride))
-                          : bf16_bits_to_float(qkv_row[k_col + j + half]);
+        float x0 = SLICED ? k_sl[0] : bf16_bits_to_float(qkv_row[k_col + j]);
+        float x1 = SLICED ? k_sl[1] : bf16_bits_to_float(qkv_row[k_col + j + half]);
         if (bias) {
           x0 += load_param(bias, k_col + j, bias_dtype);
           x1 += load_param(bias, k_col + j + half, bias_dtype);
         }
-        kpage[he_k_index(off, j, KS)] = float_to_bf16_bits(x0 * c - x1 * sn);
-        kpage[he_k_index(off, j + half, KS)] = float_to_bf16_bits(x0 * sn + x1 * c);
+        kpage[he_k_index(off, j, KS)] = float_to_bf16_bits(fmaf(x0, c, -(x1 * sn)));
+        kpage[he_k_index(off, j + half, KS)] = float_to_bf16_bits(fmaf(x0, sn, x1 * c));
       }
       for (int d = lane; d < HD; d += 64) {
-        float x = SLICED ? as_bf16(slices_sum<float>(part_row + v_col + d, qkv_slices, slice_stride))
-                         : bf16_bits_to_float(qkv_row[v_col + d]);
+        float x = SLICED ? (d >= 64 ? v_sl[1] : v_sl[0]) : bf16_bits_to_float(qkv_row[v_col + d]);
         if (bias) x += load_param(bias, v_col + d, bias_dtype);
         vpage[he_v_index(off, d, NT)] = float_to_bf16_bits(x);
       }
