@@ -22,6 +22,11 @@ graph replay) plus greedy sampling. As in the library's generation loop, steps a
 queued ahead of the host: the chosen ids go into the next step on the device, and the host
 reads a step's ids when 7 further steps are queued behind it.
 
+The default warm-up of 64 steps is most of the first half second after the prompt step, during which
+the machine runs every kernel of the one-token step 4 to 6 % slower than afterwards (the reference
+leaves its first run and its thermal-low samples out: OPTIMIZATION_NOTES.md:114-117); `repeats` holds
+every timed run, the earlier ones still show it.
+
 Procedure (the reference quotes medians with their range over repeated runs:
 tools/HQS_DECODE_OPTIMIZATION_PLAN.md:54-65): after the warm-up steps, `--repeats` (5) runs of
 exactly `--steps` steps each are timed, each bracketed by a device synchronisation; `value` and
@@ -82,7 +87,7 @@ def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
-    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--warmup", type=int, default=64)
     ap.add_argument("--repeats", type=int, default=5, help="timed runs of --steps steps each; the median counts")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0 = all)")
