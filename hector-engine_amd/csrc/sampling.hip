@@ -331,7 +331,7 @@ typedef unsigned long long u64;
 // order-preserving map float -> uint32 (ascending)
 __device__ __forceinline__ uint32_t ordered_key(float x) {
   const uint32_t b = __float_as_uint(x);
-  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+  return b ^ ((uint32_t)((int32_t)b >> 31) | 0x80000000u);   // negative: all bits turned; else the sign bit set
 }
 __device__ __forceinline__ float key_to_float(uint32_t k) {
   const uint32_t b = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
@@ -339,7 +339,8 @@ __device__ __forceinline__ float key_to_float(uint32_t k) {
 }
 // NaN counts as -inf; -0.0 becomes +0.0, which it equals: as keys the two would differ, and equal
 // values are ordered by index alone.
-__device__ __forceinline__ float clean(float x) { return x != x ? -INFINITY : (x == 0.f ? 0.f : x); }
+// (x + 0 turns -0.0 into +0.0 and leaves everything else; the maximum with -inf is -inf for a NaN)
+__device__ __forceinline__ float clean(float x) { return fmaxf(x + 0.f, -INFINITY); }
 __device__ __forceinline__ u64 fixed_mass(float x, float m, float inv_temp) {
   const float w = expf((x - m) * inv_temp);
   return (u64)(w * SAMP_FIXED_ONE);
@@ -446,11 +447,13 @@ __device__ __forceinline__ void flush_runs(u64* hist, int bin, u64 run) {
 // Finds, in descending order inside `cut`, the element at which the cumulative
 // count (MASS = false) or mass (MASS = true) first reaches t (t >= 1), and
 // returns the set of everything up to and including it.
+// passes < 4: the descent stops with the upper 8 * passes bits of the key (the lower ones zero): the
+// key of the bin the element lies in, for a caller that wants a bound and not the element.
 template <bool MASS, typename Source>
 __device__ Cut descend(const Source& src, float m, float inv_temp, Cut cut, u64 t,
-                       SampShared& sh) {
+                       SampShared& sh, int passes = 4) {
   uint32_t prefix = 0;
-  for (int pass = 0; pass < 4; ++pass) {
+  for (int pass = 0; pass < passes; ++pass) {
     const int shift = 24 - 8 * pass;
     __syncthreads();
     if (threadIdx.x < 256) sh.hist[threadIdx.x] = 0;
@@ -649,43 +652,58 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_rows_kernel(
   __shared__ int list_n;
   const float* x = logits + blockIdx.x * stride;
 
-  // pass 1: row maximum
-  float best = -INFINITY;
-  if (((stride & 3) == 0) && ((((uintptr_t)logits) & 15) == 0)) {
-    // four loads on their way at a time: one workgroup reads the whole row, and a load takes
-    // about a microsecond
-    const int V4 = V & ~3;
-    for (int i0 = 4 * threadIdx.x; i0 < V4; i0 += 16 * SAMP_THREADS) {
-      float4 v[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int i = i0 + u * 4 * SAMP_THREADS;
-        v[u] = i < V4 ? *reinterpret_cast<const float4*>(x + i) : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-        best = fmaxf(fmaxf(best, clean(v[u].x)), fmaxf(clean(v[u].y), fmaxf(clean(v[u].z), clean(v[u].w))));
+  const bool aligned = ((stride & 3) == 0) && ((((uintptr_t)logits) & 15) == 0);
+  // With a top-k the kept set lies inside the list (or the whole row is walked instead) and the
+  // mass of the rest is never asked for: its 150,000 exponentials, most of the list pass, are left
+  // out, and the row's maximum, which nothing before the list needs then, is taken in that pass.
+  const bool need_rest = !(top_k > 0 && top_k < V);
+  const bool max_with_list = !need_rest && V > SAMP_LIST && aligned;
+
+  // the workgroup's maximum of `best`; false (index 0 stored) when the row has nothing finite
+  auto row_max = [&](float best, float* m_out) -> bool {
+    best = wave_max(best);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) sh.red[threadIdx.x >> 6] = (u64)__float_as_uint(best);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      float mm = -INFINITY;
+      for (int w = 0; w < SAMP_THREADS / HE_WAVE; ++w)
+        mm = fmaxf(mm, __uint_as_float((uint32_t)sh.red[w]));
+      sh.m = mm;
     }
-    for (int i = V4 + threadIdx.x; i < V; i += SAMP_THREADS) best = fmaxf(best, clean(x[i]));
-  } else {
-    for (int i = threadIdx.x; i < V; i += SAMP_THREADS) best = fmaxf(best, clean(x[i]));
-  }
-  best = wave_max(best);
-  if (threadIdx.x == 0) list_n = 0;
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) sh.red[threadIdx.x >> 6] = (u64)__float_as_uint(best);
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    float mm = -INFINITY;
-    for (int w = 0; w < SAMP_THREADS / HE_WAVE; ++w)
-      mm = fmaxf(mm, __uint_as_float((uint32_t)sh.red[w]));
-    sh.m = mm;
-  }
-  __syncthreads();
-  const float m = sh.m;
-  if (!(m > -INFINITY)) {  // nothing finite: fall back to index 0
-    if (threadIdx.x == 0) out[blockIdx.x] = 0;
-    return;
+    __syncthreads();
+    *m_out = sh.m;
+    if (!(sh.m > -INFINITY)) {
+      if (threadIdx.x == 0) out[blockIdx.x] = 0;
+      return false;
+    }
+    return true;
+  };
+
+  // pass 1: row maximum
+  float best = -INFINITY, m = -INFINITY;
+  if (!max_with_list) {
+    if (aligned) {
+      // four loads on their way at a time: one workgroup reads the whole row, and a load takes
+      // about a microsecond (more in flight gain nothing: a compute unit alone takes in about 64
+      // bytes a cycle, 4.5 us for a row of 152,064)
+      const int V4 = V & ~3;
+      for (int i0 = 4 * threadIdx.x; i0 < V4; i0 += 16 * SAMP_THREADS) {
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int i = i0 + u * 4 * SAMP_THREADS;
+          v[u] = i < V4 ? *reinterpret_cast<const float4*>(x + i) : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          best = fmaxf(fmaxf(best, clean(v[u].x)), fmaxf(clean(v[u].y), fmaxf(clean(v[u].z), clean(v[u].w))));
+      }
+      for (int i = V4 + threadIdx.x; i < V; i += SAMP_THREADS) best = fmaxf(best, clean(x[i]));
+    } else {
+      for (int i = threadIdx.x; i < V; i += SAMP_THREADS) best = fmaxf(best, clean(x[i]));
+    }
+    if (!row_max(best, &m)) return;   // nothing finite: index 0
   }
   const u64 u = (u64)uniforms[blockIdx.x];
   Cut pick;
@@ -707,8 +725,10 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_rows_kernel(
     none.any = 0;
     none.key = 0;
     none.ties = 0;
+    // the upper 24 bits of the key at that rank are bound enough: the list then takes the whole bin,
+    // 2^-15 of the value wide, a handful of elements more
     const u64 rank = ((u64)n * SAMP_AIM + V - 1) / V + 1;
-    threshold = descend<false>(sample, m, inv_temp, none, rank, sh).key;
+    threshold = descend<false>(sample, 0.f, inv_temp, none, rank, sh, 3).key;
     __syncthreads();
   }
 
@@ -732,12 +752,12 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_rows_kernel(
         list_v[wave * SEGMENT + at] = v;
         list_i[wave * SEGMENT + at] = i;
       }
-    } else if (in_range) {
+    } else if (in_range && need_rest) {
       rest_local += fixed_mass(v, m, inv_temp);
     }
     filled += __builtin_popcountll(appenders);
   };
-  if (V > SAMP_LIST && ((stride & 3) == 0) && ((((uintptr_t)logits) & 15) == 0)) {
+  if (V > SAMP_LIST && aligned) {
     // 16 bytes a load, four loads a group, the next group on its way while this one is looked
     // at; all lanes of a wavefront make the same number of turns
     const int V4 = V & ~3;
@@ -751,22 +771,52 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_rows_kernel(
         g[u] = at + u * STEP < V4 ? *reinterpret_cast<const float4*>(x + at + u * STEP) : make_float4(0.f, 0.f, 0.f, 0.f);
     };
     load_group(cur, i);
+    const unsigned long long below = (1ull << lane) - 1ull;     // the lanes in front of this one
     for (int gi = 0; gi < groups; ++gi) {
       load_group(nxt, i + 4 * STEP);
+      // A lane's sixteen elements of the group as a bit mask of those that go into the list (two in
+      // a hundred do); where the lane's first one goes follows from the counts of the lanes in front
+      // of it, taken bit by bit of the count through ballots: one such sum a group, not one ballot an
+      // element. The few elements that go are then fetched again by their index.
+      uint32_t mask = 0;
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int at = i + u * STEP;
-        const bool in = at < V4;
-        take(cur[u].x, at, in);
-        take(cur[u].y, at + 1, in);
-        take(cur[u].z, at + 2, in);
-        take(cur[u].w, at + 3, in);
+        const bool in = i + u * STEP < V4;
+        const float c4[4] = {cur[u].x, cur[u].y, cur[u].z, cur[u].w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const float v = clean(c4[c]);
+          if (in) best = fmaxf(best, v);      // (the row's maximum, where no pass before this one took it)
+          const bool mine = in && ordered_key(v) >= threshold;
+          mask |= (uint32_t)mine << (4 * u + c);
+          if (need_rest && in && !mine) rest_local += fixed_mass(v, m, inv_temp);
+        }
       }
+      const int count = __builtin_popcount(mask);
+      int before = 0, total = 0;
+#pragma unroll
+      for (int bit = 0; bit < 5; ++bit) {       // a lane has at most 16
+        const unsigned long long with = __builtin_amdgcn_ballot_w64((count >> bit) & 1);
+        before += __builtin_popcountll(with & below) << bit;
+        total += __builtin_popcountll(with) << bit;
+      }
+      int at = filled + before;
+      for (uint32_t left = mask; left != 0; left &= left - 1) {
+        const int e = __builtin_ctz(left);
+        const int idx = i + (e >> 2) * STEP + (e & 3);
+        if (at < SEGMENT) {
+          list_v[wave * SEGMENT + at] = clean(x[idx]);
+          list_i[wave * SEGMENT + at] = idx;
+        }
+        ++at;
+      }
+      filled += total;
 #pragma unroll
       for (int u = 0; u < 4; ++u) cur[u] = nxt[u];
       i += 4 * STEP;
     }
     const int j = V4 + threadIdx.x;
+    if (j < V) best = fmaxf(best, clean(x[j]));
     take(j < V ? x[j] : 0.f, j, j < V);   // at most three elements are left
   } else {
     const int turns = (V + SAMP_THREADS - 1) / SAMP_THREADS;
@@ -776,6 +826,7 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_rows_kernel(
     }
   }
   if (lane == 0 && filled > SEGMENT) list_n = 1;
+  if (max_with_list && !row_max(best, &m)) return;
   const u64 rest = block_sum_u64(rest_local, sh);   // its barriers also publish list_n
   ListSource list;
   list.v = list_v;
