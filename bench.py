@@ -32,7 +32,8 @@ tools/HQS_DECODE_OPTIMIZATION_PLAN.md:54-65): after the warm-up steps, `--repeat
 exactly `--steps` steps each are timed, each bracketed by a device synchronisation; `value` and
 `ms_per_step` are the median run's, `repeats` holds all of them. The same holds for the points at
 batch 1 and at the large batch. The prefill figure is the median of three whole-prompt steps of
-one 2,048-token prompt; `prefill_packed` is one step of `--batch` such prompts packed together.
+one 2,048-token prompt (a step of that size replays a HIP graph from its third use on, as in the engine's
+default configuration); `prefill_packed` is one step of `--batch` such prompts packed together.
 """
 from __future__ import annotations
 
@@ -183,16 +184,17 @@ def main() -> int:
 
         def prompt_step(self, tokens):
             """Seconds of one whole-prompt step of `tokens` tokens: a first run warms the library's
-            products, then the median of three."""
+            products, a second one is captured as a HIP graph where the engine keeps one for such a
+            step, then the median of three."""
             p = self.prompts(1, tokens, tokens)[0]
             times = []
-            for run in range(4):
+            for run in range(5):
                 slot = self.engine.acquire()
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
                 self.engine.step([StepEntry(slot, p, [tokens - 1])])
                 torch.cuda.synchronize()
-                if run > 0:
+                if run > 1:
                     times.append(time.perf_counter() - t0)
                 self.engine.release(slot)
             return sorted(times)[1]

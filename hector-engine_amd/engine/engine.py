@@ -41,6 +41,12 @@ GRAPH_MAX_BUCKET = 256
 # rarely come again. So many such graphs are kept, the least recently used one goes first.
 GRAPH_MAX_STEP_ROWS = 512
 GRAPH_MAX_STEP_PLANS = 24
+# A longer step is captured as it is, without padding rows (which the library's products would
+# compute), when its row count is a multiple of GRAPH_CHUNK_MULTIPLE up to GRAPH_MAX_CHUNK_ROWS: the
+# fixed chunks a long prompt is fed in come again and again (2,048 tokens at the Qwen2.5-7B shape:
+# 24.7 ms of kernels, 25.2 ms issued launch by launch).
+GRAPH_CHUNK_MULTIPLE = 256
+GRAPH_MAX_CHUNK_ROWS = 4096
 ROW_TABLES_MAX_BYTES = 256 * 1024     # page table rows that a one-token step takes along with its metadata
 
 
@@ -102,7 +108,8 @@ class Engine:
                  max_slots: int | None = None, max_seq_len: int | None = None,
                  device: str = "cuda:0", fast_kernels: bool = True, use_graphs: bool = True,
                  tune_library: bool = False, beyond_max_positions: bool = False, profile: bool = False,
-                 sync_each_launch: bool = False, graph_step_rows: int = GRAPH_MAX_STEP_ROWS):
+                 sync_each_launch: bool = False, graph_step_rows: int = GRAPH_MAX_STEP_ROWS,
+                 graph_chunk_rows: int = GRAPH_MAX_CHUNK_ROWS):
         """max_seq_len: the longest sequence (default: the positions the model's configuration
         allows; more than that is refused unless beyond_max_positions says it is meant).
         tune_library: let the library's autotuner choose the kernel of each tall bfloat16
@@ -111,6 +118,8 @@ class Engine:
         without HIP graphs); profile_summary() gives the table.
         graph_step_rows: prompt steps and mixed steps of up to so many rows are captured as HIP
         graphs too, one per bucket of their sizes (0: only one-token steps are).
+        graph_chunk_rows: longer steps are captured as well, unpadded, when their row count is a
+        multiple of 256 and at most this (fixed prompt chunks; 0, or graph_step_rows 0: none).
         sync_each_launch: a debugging mode (the reference's sync_after_each_op, src/engine.cpp:318-334):
         steps run without HIP graphs and the host waits for the GPU after every launch, so that
         a fault is reported with the name of the op that raised it."""
@@ -167,6 +176,7 @@ class Engine:
         self._hint_fns = self.model.step_hints()      # what parts want to know of a one-token step (parts/base.py)
         self._hints_before: dict[int, tuple] = {}     # per bucket size: the hints of the step before
         self.graph_step_rows = graph_step_rows
+        self.graph_chunk_rows = graph_chunk_rows
         self._plans: collections.OrderedDict[tuple, _GraphBucket] = collections.OrderedDict()
         self._pinned = [torch.empty(1 << 16, dtype=torch.int32).pin_memory() for _ in range(4)]
         self._pinned_events: list[torch.cuda.Event | None] = [None] * 4
@@ -440,15 +450,19 @@ class Engine:
         """The bucket of sizes a step that is not all one-token (or does not want every row)
         runs in as a graph, or None when it runs eagerly: (rows, sequences, longest run of new
         tokens, most keys of a sequence after the step, wanted places, every row wanted in
-        order, all one-token), each rounded up to a power of two. The sizes decide every
+        order, all one-token), each rounded up to a power of two (the rows of a longer step that
+        is a whole chunk stay as they are). The sizes decide every
         grid, so steps of one bucket replay one graph; rows and sequences beyond the step's
         own are padding (row_seq -1, slot -1) that every kernel passes over."""
         rows = sum(len(e.tokens) for e in entries)
-        if rows > self.graph_step_rows:
+        if rows <= self.graph_step_rows:
+            R = _pow2(rows, 16)
+        elif self.graph_step_rows and rows <= self.graph_chunk_rows and rows % GRAPH_CHUNK_MULTIPLE == 0:
+            R = rows                 # a whole chunk: its own bucket, no padding rows
+        else:
             return None
         wants = sum(len(e.want) for e in entries)
         want_all = wants == rows and all(list(e.want) == list(range(len(e.tokens))) for e in entries)
-        R = _pow2(rows, 16)
         most = max(self.cache.length(e.slot) + len(e.tokens) for e in entries)
         keys = min(_pow2(most, 256), max(self.cache.max_seq_len, 256))
         return (R, _pow2(len(entries)), min(_pow2(max(len(e.tokens) for e in entries)), R), keys,

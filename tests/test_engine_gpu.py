@@ -702,6 +702,53 @@ def test_short_prompt_and_mixed_steps_replay_a_graph(model_dirs, plain_models, n
         assert e.cache.free_pages == e.cache.num_pages
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_whole_chunks_of_a_long_prompt_replay_a_graph(model_dirs, plain_models, name, dtype):
+    """A step of more rows than the padded buckets take is captured as it is when its row count is a
+    multiple of 256: a prompt of 768 tokens fed in three chunks of 256 (each chunk a bucket of its
+    own, by the keys behind it), three requests in a row, so that every bucket runs eagerly, is
+    captured and is replayed; two prompts of 128 tokens packed into one such step; a step of 300 rows
+    runs eagerly. Every logit is the plain implementation's, and in 32-bit bit for bit what an engine
+    without such graphs gives."""
+    import hector_engine_amd as he
+    opts = dict(max_tokens=4096, max_slots=4, max_seq_len=1024, beyond_max_positions=True)
+    eng = he.Engine(model_dirs[name], dtype=dtype, graph_step_rows=64, **opts)
+    plain_eng = he.Engine(model_dirs[name], dtype=dtype, graph_step_rows=0, **opts)
+    vocab = plain_models[name][0]["vocab_size"]
+    for r in range(3):
+        ids = rand_ids(vocab, 768, 870 + r)
+        want = plain_logits(plain_models, name, ids)
+        slots = {e: e.acquire() for e in (eng, plain_eng)}
+        for c in range(3):
+            piece = ids[256 * c:256 * (c + 1)]
+            a, b = (e.step([entry(slots[e], piece, [0, 100, 255])]).clone() for e in (eng, plain_eng))
+            if dtype == "float32":
+                assert torch.equal(a, b)
+            close(a, want[[256 * c, 256 * c + 100, 256 * c + 255]], dtype)
+        for e, s in slots.items():
+            e.release(s)
+    assert eng.stats["step_graph_captures"] == 3 and eng.stats["step_graph_replays"] == 6
+    for r in range(3):
+        pair = [rand_ids(vocab, 128, 880 + 2 * r), rand_ids(vocab, 128, 881 + 2 * r)]
+        slots = {e: [e.acquire(), e.acquire()] for e in (eng, plain_eng)}
+        a, b = (e.step([entry(s, p, [127]) for s, p in zip(slots[e], pair)]).clone() for e in (eng, plain_eng))
+        if dtype == "float32":
+            assert torch.equal(a, b)
+        close(a, torch.cat([plain_logits(plain_models, name, p)[127:128] for p in pair]), dtype)
+        for e, ss in slots.items():
+            for s in ss:
+                e.release(s)
+    assert eng.stats["step_graph_captures"] == 4 and eng.stats["step_graph_replays"] == 8
+    ids = rand_ids(vocab, 300, 890)
+    slot = eng.acquire()
+    assert eng._step_plan([entry(slot, ids, [299])], False) is None
+    close(eng.step([entry(slot, ids, [299])]), plain_logits(plain_models, name, ids)[299:300], dtype)
+    eng.release(slot)
+    assert eng.stats["step_graph_captures"] == 4 and not eng.capture_failures
+    assert eng.cache.free_pages == eng.cache.num_pages
+
+
 def test_step_graphs_are_kept_least_recently_used_first_out(model_dirs, plain_models):
     """No more graphs of prompt steps are kept than GRAPH_MAX_STEP_PLANS: the one used longest ago
     goes, and a bucket that comes again after that is captured anew, with the same logits."""
