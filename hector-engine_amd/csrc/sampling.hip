@@ -360,6 +360,7 @@ struct SampShared {
   u64 t;
   uint32_t prefix;
   float m;
+  int few;      // elements gathered by choose_few
 };
 
 // Exact (integer) sum over the workgroup: wavefronts first, then their 16 sums in order.
@@ -597,20 +598,101 @@ __device__ int pick_index_list(const ListSource& src, Cut pick, SampShared& sh) 
   return after;
 }
 
+__device__ __forceinline__ u64 shfl_xor_u64(u64 v, int mask) {
+  const uint32_t lo = __shfl_xor((uint32_t)v, mask, HE_WAVE);
+  const uint32_t hi = __shfl_xor((uint32_t)(v >> 32), mask, HE_WAVE);
+  return ((u64)hi << 32) | lo;
+}
+__device__ __forceinline__ u64 shfl_u64(u64 v, int lane) {
+  const uint32_t lo = __shfl((uint32_t)v, lane, HE_WAVE);
+  const uint32_t hi = __shfl((uint32_t)(v >> 32), lane, HE_WAVE);
+  return ((u64)hi << 32) | lo;
+}
+
+// top-p and the draw after a top-k of at most a wavefront's width, in one wavefront: the
+// elements at or above the top-k's last key (`cut.key`) go one to a lane, are sorted by
+// descending value and ascending index, the first top_k of them keep their mass, and a
+// running sum over the lanes stands for the descents (12 passes over the list otherwise:
+// 20 us of a sampled step). The order and the masses are those of the descents, so the token
+// is the same. Returns false, with nothing decided, when more than a wavefront's width of
+// elements lie at or above that key (many ties at it).
+template <typename Source>
+__device__ bool choose_few(const Source& src, float m, float inv_temp, int top_k, float top_p,
+                           u64 u, Cut cut, SampShared& sh, int* index_out) {
+  __syncthreads();
+  if (threadIdx.x == 0) sh.few = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < src.n; i += SAMP_THREADS) {
+    if (!src.valid(i)) continue;
+    const uint32_t k = ordered_key(src.value(i));
+    if (k < cut.key) continue;
+    const int at = atomicAdd(&sh.few, 1);
+    if (at < HE_WAVE) sh.hist[at] = ((u64)k << 32) | (u64)(0xffffffffu - (uint32_t)src.index(i));
+  }
+  __syncthreads();
+  const int n = sh.few;
+  if (n > HE_WAVE) return false;
+  if (threadIdx.x < HE_WAVE) {
+    const int lane = threadIdx.x;
+    u64 e = lane < n ? sh.hist[lane] : 0ull;     // (an empty lane sorts behind every element)
+    // bitonic sort, descending over the lanes
+#pragma unroll
+    for (int size = 2; size <= HE_WAVE; size <<= 1) {
+#pragma unroll
+      for (int stride = size >> 1; stride > 0; stride >>= 1) {
+        const u64 other = shfl_xor_u64(e, stride);
+        const bool descending = (lane & size) == 0;
+        const bool first = (lane & stride) == 0;
+        const u64 hi = e > other ? e : other, lo = e > other ? other : e;
+        e = (first == descending) ? hi : lo;
+      }
+    }
+    const float v = key_to_float((uint32_t)(e >> 32));
+    const u64 mass = lane < top_k && lane < n ? fixed_mass(v, m, inv_temp) : 0ull;
+    u64 upto = mass;                             // inclusive running sum
+#pragma unroll
+    for (int off = 1; off < HE_WAVE; off <<= 1) {
+      const uint32_t lo = __shfl_up((uint32_t)upto, off, HE_WAVE);
+      const uint32_t hi = __shfl_up((uint32_t)(upto >> 32), off, HE_WAVE);
+      if (lane >= off) upto += ((u64)hi << 32) | lo;
+    }
+    u64 Z = shfl_u64(upto, HE_WAVE - 1);
+    int last = HE_WAVE - 1;                      // the last lane of the kept set
+    if (top_p > 0.f && top_p < 1.f) {
+      u64 target = (u64)ceil((double)top_p * (double)Z);
+      if (target < 1) target = 1;
+      if (target > Z) target = Z;
+      const unsigned long long reached = __builtin_amdgcn_ballot_w64(upto >= target);
+      last = __builtin_ctzll(reached);           // (Z > 0: the row's maximum is among the elements)
+      Z = shfl_u64(upto, last);
+    }
+    const u64 r = u * (Z >> 32) + ((u * (Z & 0xffffffffull)) >> 32);
+    const unsigned long long reached = __builtin_amdgcn_ballot_w64(lane <= last && upto >= r + 1);
+    const int pick = reached ? __builtin_ctzll(reached) : 0;
+    const u64 chosen = shfl_u64(e, pick);
+    if (lane == 0) sh.prefix = 0xffffffffu - (uint32_t)chosen;
+  }
+  __syncthreads();
+  *index_out = (int)sh.prefix;
+  return true;
+}
+
 // top-k, top-p and the draw on one source. rest: mass of the row's elements that are not
 // in the source (they all come after every element of the source in descending order).
 // Returns false when the answer needs elements outside the source (rest > 0 only).
 template <typename Source>
 __device__ bool choose(const Source& src, float m, float inv_temp, int top_k, float top_p, int V,
-                       u64 u, u64 rest, SampShared& sh, Cut* pick_out) {
+                       u64 u, u64 rest, SampShared& sh, Cut* pick_out, int* index_out) {
   Cut cut;
   cut.any = 0;
   cut.key = 0;
   cut.ties = 0;
+  *index_out = -1;
   if (top_k > 0 && top_k < V) {
     if ((u64)top_k > set_total<false>(src, m, inv_temp, cut, sh)) return false;
     cut = descend<false>(src, m, inv_temp, cut, (u64)top_k, sh);
     rest = 0;   // the set is inside the source
+    if (top_k <= HE_WAVE && choose_few(src, m, inv_temp, top_k, top_p, u, cut, sh, index_out)) return true;
   }
   u64 inside = set_total<true>(src, m, inv_temp, cut, sh);
   u64 Z = inside + rest;
@@ -832,8 +914,9 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_rows_kernel(
   list.v = list_v;
   list.idx = list_i;
   list.n = SAMP_LIST;
-  if (list_n == 0 && choose(list, m, inv_temp, top_k, top_p, V, u, rest, sh, &pick)) {
-    int res = pick_index_list(list, pick, sh);
+  int res;                             // the token, where choose() found it itself; else -1
+  if (list_n == 0 && choose(list, m, inv_temp, top_k, top_p, V, u, rest, sh, &pick, &res)) {
+    if (res < 0) res = pick_index_list(list, pick, sh);
     if (res < 0) res = pick_index_row(x, V, pick, s_counts);
     if (threadIdx.x == 0) out[blockIdx.x] = res;
     return;
@@ -841,8 +924,8 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_rows_kernel(
   RowSource row;
   row.x = x;
   row.n = V;
-  choose(row, m, inv_temp, top_k, top_p, V, u, 0, sh, &pick);
-  const int res = pick_index_row(x, V, pick, s_counts);
+  choose(row, m, inv_temp, top_k, top_p, V, u, 0, sh, &pick, &res);
+  if (res < 0) res = pick_index_row(x, V, pick, s_counts);
   if (threadIdx.x == 0) out[blockIdx.x] = res;
 }
 

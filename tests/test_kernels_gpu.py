@@ -1165,7 +1165,8 @@ def test_sample_rows_takes_both_zeros_as_equal(ops):
 
 
 @pytest.mark.parametrize("case", ["top_k beyond the list", "all equal", "ties at the threshold", "two values",
-                                  "deep nucleus"])
+                                  "deep nucleus", "a small top_k among thousands of ties",
+                                  "a small top_k that cuts through a few ties"])
 def test_sample_rows_list_and_whole_row_agree(ops, case):
     """The kernel works on a list of the row's largest elements and falls back to the whole row
     when that is not enough; both must give the plain implementation's token."""
@@ -1183,6 +1184,14 @@ def test_sample_rows_list_and_whole_row_agree(ops, case):
         x[:] = -4.0
         x[:, ::7] = 3.0
         top_p = 0.5
+    elif case == "a small top_k among thousands of ties":
+        x = torch.round(x * 2) / 2                 # more equal values at the top-k's edge than a wavefront has lanes
+        top_k, top_p = 40, 0.95
+    elif case == "a small top_k that cuts through a few ties":
+        for r in range(4):                         # ranks 37 to 43 hold one value: the top-k of 40 keeps the three
+            order = torch.argsort(-x[r], stable=True)   # of them with the lowest indices
+            x[r, order[37:44]] = x[r, order[37]]
+        top_k, top_p, temperature = 40, 0.999, 5.0   # flat, so that draws reach the edge
     elif case == "deep nucleus":
         top_p = 0.9999
         temperature = 3.0                          # flat: the nucleus reaches far beyond the list
