@@ -1190,7 +1190,7 @@ def test_sample_rows_list_and_whole_row_agree(ops, case):
     elif case == "a small top_k that cuts through a few ties":
         for r in range(4):                         # ranks 37 to 43 hold one value: the top-k of 40 keeps the three
             order = torch.argsort(-x[r], stable=True)   # of them with the lowest indices
-            x[r, order[37:44]] = x[r, order[37]]
+            x[r, order[37:44]] = x[r, order[37]].item()
         top_k, top_p, temperature = 40, 0.999, 5.0   # flat, so that draws reach the edge
     elif case == "deep nucleus":
         top_p = 0.9999
