@@ -105,6 +105,10 @@ def main() -> int:
     ap.add_argument("--short-steps", action="store_true",
                     help="also time prompt steps of 16, 64 and 256 tokens and a step of 8 one-token entries plus a "
                          "64-token prompt, as replayed graphs and issued launch by launch; reported as \"short_steps\"")
+    ap.add_argument("--generation", action="store_true",
+                    help="also time the generation loop (generate(): 72 new tokens after the decode batches' prompts, "
+                         "steps queued ahead of the host) at batch 1, --batch and the large batch, greedy and with "
+                         "the sampling presets; reported as \"generation\", decoded tokens a second")
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16",
                     help="float32: the whole measurement in true 32-bit (no library products, no extra points)")
     ap.add_argument("--no-tune", action="store_true",
@@ -270,7 +274,7 @@ def main() -> int:
         points_frac[name] = round(nbytes / s / 1e9 / HBM_PEAK_GBS, 4)
 
     progress(f"{MODEL}: random weights, {args.layers} layers")
-    max_batch = 2 * args.batch if args.no_points else max(2 * args.batch, BIG_BATCH)
+    max_batch = 2 * args.batch if args.no_points and not args.generation else max(2 * args.batch, BIG_BATCH)
     fp32 = args.dtype == "float32"
     if fp32:
         args.no_tune = True
@@ -358,6 +362,25 @@ def main() -> int:
     if not args.no_points:
         for b in (1, BIG_BATCH):
             point(f"decode_b{b}", model, b, PROMPT_LO, PROMPT_HI, args.steps, max(3, args.warmup // 2), args.repeats)
+
+    # ---- the generation loop: what a caller of generate() gets, sampling included
+    generation = None
+    if args.generation:
+        generation = {}
+        settings = {"greedy": he.SamplingConfig.deterministic(),
+                    "t0.8_k40_p0.9": he.SamplingConfig(temperature=0.8, top_k=40, top_p=0.9, seed=3),
+                    "t0.8": he.SamplingConfig(temperature=0.8, seed=3),
+                    "balanced": he.SamplingConfig.balanced(), "creative": he.SamplingConfig.creative()}
+        for b in sorted({1, args.batch, BIG_BATCH}):
+            progress(f"generation at batch {b}")
+            ps = model.prompts(b, PROMPT_LO, PROMPT_HI)
+            for name, sampling in settings.items():
+                he.generate(engine, ps, max_new_tokens=8, sampling=sampling)           # warm: graphs, buffers
+                results = he.generate(engine, ps, max_new_tokens=72, sampling=sampling)
+                torch.cuda.synchronize()
+                decode_ms = max(r.decode_ms for r in results)
+                tokens = sum(len(r.tokens) for r in results)
+                generation[f"b{b}_{name}"] = round((tokens - b) * 1e3 / decode_ms, 1)
     extra = not args.no_extra and not args.no_points and args.shape == "7b" and args.layers == FULL_LAYERS and not fp32
     prefill_fp32 = None
     if extra:
@@ -425,6 +448,8 @@ def main() -> int:
         line["short_steps"] = short_steps
     if continuation:
         line["continuation"] = continuation
+    if generation:
+        line["generation"] = generation
     if packed:
         line["prefill_packed"] = {"value": round(packed["tokens"] / packed["seconds"], 1), "tokens": packed["tokens"],
                                   "ms": round(packed["seconds"] * 1e3, 3),
