@@ -716,10 +716,14 @@ __device__ bool choose(const Source& src, float m, float inv_temp, int top_k, fl
 // elements - all whose key is at least a threshold - go into a list in LDS, and the mass
 // of all others is summed. The threshold is the value that a strided sample of the row
 // puts at the rank which aims at SAMP_AIM list elements (the list holds twice that; a row
-// no longer than the list goes in whole). top-k, top-p and the draw then run on the list.
-// When they need more than the list holds (a top-k beyond it, a nucleus or a draw that
-// reaches into the rest, a list that overflowed) the same steps run on the whole row
-// instead, many passes over it: rare, and the result is the same either way.
+// no longer than the list goes in whole). With a top-k nobody asks for the mass of the
+// others, and the maximum is taken in the list pass: one pass over the row. top-k, top-p
+// and the draw then run on the list (behind a top-k of at most 64 in one wavefront:
+// choose_few). When they need more than the list holds (a top-k beyond it, a nucleus or a
+// draw that reaches into the rest, a list that overflowed) the same steps run on the whole
+// row instead, many passes over it: rare for the peaked rows of a trained model (the rule
+// for nearly flat rows without a top-k, as random weights give them), and the result is
+// the same either way.
 #define SAMP_LIST 6144
 #define SAMP_AIM 3072
 #define SAMP_SAMPLE 4096
