@@ -47,6 +47,7 @@ GRAPH_MAX_STEP_PLANS = 24
 # 24.7 ms of kernels, 25.2 ms issued launch by launch).
 GRAPH_CHUNK_MULTIPLE = 256
 GRAPH_MAX_CHUNK_ROWS = 4096
+GRAPH_CHUNK_MAX_WANTS = 64      # (a bucket keeps its logits: thousands of wanted rows of a long vocabulary are gigabytes)
 ROW_TABLES_MAX_BYTES = 256 * 1024     # page table rows that a one-token step takes along with its metadata
 
 
@@ -119,7 +120,8 @@ class Engine:
         graph_step_rows: prompt steps and mixed steps of up to so many rows are captured as HIP
         graphs too, one per bucket of their sizes (0: only one-token steps are).
         graph_chunk_rows: longer steps are captured as well, unpadded, when their row count is a
-        multiple of 256 and at most this (fixed prompt chunks; 0, or graph_step_rows 0: none).
+        multiple of 256 and at most this and they want at most 64 places (fixed prompt chunks; 0,
+        or graph_step_rows 0: none).
         sync_each_launch: a debugging mode (the reference's sync_after_each_op, src/engine.cpp:318-334):
         steps run without HIP graphs and the host waits for the GPU after every launch, so that
         a fault is reported with the name of the op that raised it."""
@@ -455,13 +457,14 @@ class Engine:
         grid, so steps of one bucket replay one graph; rows and sequences beyond the step's
         own are padding (row_seq -1, slot -1) that every kernel passes over."""
         rows = sum(len(e.tokens) for e in entries)
+        wants = sum(len(e.want) for e in entries)
         if rows <= self.graph_step_rows:
             R = _pow2(rows, 16)
-        elif self.graph_step_rows and rows <= self.graph_chunk_rows and rows % GRAPH_CHUNK_MULTIPLE == 0:
+        elif self.graph_step_rows and rows <= self.graph_chunk_rows and rows % GRAPH_CHUNK_MULTIPLE == 0 \
+                and wants <= GRAPH_CHUNK_MAX_WANTS:
             R = rows                 # a whole chunk: its own bucket, no padding rows
         else:
             return None
-        wants = sum(len(e.want) for e in entries)
         want_all = wants == rows and all(list(e.want) == list(range(len(e.tokens))) for e in entries)
         most = max(self.cache.length(e.slot) + len(e.tokens) for e in entries)
         keys = min(_pow2(most, 256), max(self.cache.max_seq_len, 256))

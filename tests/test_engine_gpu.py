@@ -709,7 +709,7 @@ def test_whole_chunks_of_a_long_prompt_replay_a_graph(model_dirs, plain_models, 
     multiple of 256: a prompt of 768 tokens fed in three chunks of 256 (each chunk a bucket of its
     own, by the keys behind it), three requests in a row, so that every bucket runs eagerly, is
     captured and is replayed; two prompts of 128 tokens packed into one such step; a step of 300 rows
-    runs eagerly. Every logit is the plain implementation's, and in 32-bit bit for bit what an engine
+    runs eagerly, and so does a chunk of which every place is wanted. Every logit is the plain implementation's, and in 32-bit bit for bit what an engine
     without such graphs gives."""
     import hector_engine_amd as he
     opts = dict(max_tokens=4096, max_slots=4, max_seq_len=1024, beyond_max_positions=True)
@@ -743,6 +743,8 @@ def test_whole_chunks_of_a_long_prompt_replay_a_graph(model_dirs, plain_models, 
     ids = rand_ids(vocab, 300, 890)
     slot = eng.acquire()
     assert eng._step_plan([entry(slot, ids, [299])], False) is None
+    assert eng._step_plan([entry(slot, ids[:256], range(256))], False) is None     # a bucket would keep 256 rows of logits
+    assert eng._step_plan([entry(slot, ids[:256], [255])], False) is not None
     close(eng.step([entry(slot, ids, [299])]), plain_logits(plain_models, name, ids)[299:300], dtype)
     eng.release(slot)
     assert eng.stats["step_graph_captures"] == 4 and not eng.capture_failures
