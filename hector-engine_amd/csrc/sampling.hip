@@ -382,32 +382,58 @@ __device__ u64 block_sum_u64(u64 v, SampShared& sh) {
 
 // Where the elements come from: the whole row in global memory, or a list in LDS of the
 // row's largest elements (value and index), in no particular order.
+// for_each(f): f(value, index) for every element, the workgroup's threads sharing them out.
 struct RowSource {
   const float* x;
   int n;
-  __device__ __forceinline__ bool valid(int) const { return true; }
-  __device__ __forceinline__ float value(int i) const { return clean(x[i]); }
-  __device__ __forceinline__ int index(int i) const { return i; }
+  // Four 16-byte loads of a thread are on their way at a time where the row allows them: with
+  // one 4-byte load a turn a pass over a row of 152,064 waits 148 times for memory (50 us; the
+  // passes of a nearly flat row, whose draw lies beyond the list, took 340 us together).
+  template <typename F>
+  __device__ __forceinline__ void for_each(F&& f) const {
+    int done = 0;
+    if ((((uintptr_t)x) & 15) == 0) {
+      done = n & ~3;
+      for (int i0 = 4 * threadIdx.x; i0 < done; i0 += 16 * SAMP_THREADS) {
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int i = i0 + u * 4 * SAMP_THREADS;
+          v[u] = *reinterpret_cast<const float4*>(x + (i < done ? i : i0));
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int i = i0 + u * 4 * SAMP_THREADS;
+          if (i < done) {
+            f(clean(v[u].x), i);
+            f(clean(v[u].y), i + 1);
+            f(clean(v[u].z), i + 2);
+            f(clean(v[u].w), i + 3);
+          }
+        }
+      }
+    }
+    for (int i = done + threadIdx.x; i < n; i += SAMP_THREADS) f(clean(x[i]), i);
+  }
 };
 struct ListSource {   // n slots; a slot with index -1 is empty
   const float* v;
   const int* idx;
   int n;
-  __device__ __forceinline__ bool valid(int i) const { return idx[i] >= 0; }
-  __device__ __forceinline__ float value(int i) const { return v[i]; }
-  __device__ __forceinline__ int index(int i) const { return idx[i]; }
+  template <typename F>
+  __device__ __forceinline__ void for_each(F&& f) const {
+    for (int i = threadIdx.x; i < n; i += SAMP_THREADS)
+      if (idx[i] >= 0) f(v[i], idx[i]);
+  }
 };
 
 template <bool MASS, typename Source>
 __device__ u64 set_total(const Source& src, float m, float inv_temp, Cut cut, SampShared& sh) {
   u64 local = 0;
-  for (int i = threadIdx.x; i < src.n; i += SAMP_THREADS) {
-    if (!src.valid(i)) continue;
-    const float v = src.value(i);
-    const uint32_t k = ordered_key(v);
-    if (cut.any && k <= cut.key) continue;
+  src.for_each([&](float v, int) {
+    if (cut.any && ordered_key(v) <= cut.key) return;
     local += MASS ? fixed_mass(v, m, inv_temp) : 1ull;
-  }
+  });
   if (threadIdx.x == 0 && cut.any)
     local += (MASS ? fixed_mass(key_to_float(cut.key), m, inv_temp) : 1ull) * (u64)cut.ties;
   return block_sum_u64(local, sh);
@@ -461,12 +487,10 @@ __device__ Cut descend(const Source& src, float m, float inv_temp, Cut cut, u64 
     __syncthreads();
     int cur = -1;
     u64 run = 0;
-    for (int i = threadIdx.x; i < src.n; i += SAMP_THREADS) {
-      if (!src.valid(i)) continue;
-      const float v = src.value(i);
+    src.for_each([&](float v, int) {
       const uint32_t k = ordered_key(v);
-      if (pass > 0 && (k >> (shift + 8)) != (prefix >> (shift + 8))) continue;
-      if (cut.any && k <= cut.key) continue;
+      if (pass > 0 && (k >> (shift + 8)) != (prefix >> (shift + 8))) return;
+      if (cut.any && k <= cut.key) return;
       const int b = (k >> shift) & 255;
       if (b != cur) {
         if (cur >= 0) atomicAdd(&sh.hist[cur], run);
@@ -474,7 +498,7 @@ __device__ Cut descend(const Source& src, float m, float inv_temp, Cut cut, u64 
         run = 0;
       }
       run += MASS ? fixed_mass(v, m, inv_temp) : 1ull;
-    }
+    });
     flush_runs(sh.hist, cur, run);
     if (threadIdx.x == 0 && cut.any && cut.ties > 0 &&
         (pass == 0 || (cut.key >> (shift + 8)) == (prefix >> (shift + 8)))) {
@@ -541,32 +565,96 @@ __device__ Cut descend(const Source& src, float m, float inv_temp, Cut cut, u64 
   return r;
 }
 
-// The index of the pick.ties-th element, by ascending index, whose key equals pick.key.
-__device__ int pick_index_row(const float* x, int V, Cut pick, int* s_counts) {
-  __shared__ int s_res;
-  const int chunk = (V + SAMP_THREADS - 1) / SAMP_THREADS;
-  const int b = threadIdx.x * chunk;
-  const int e = min(V, b + chunk);
-  int cnt = 0;
-  for (int i = b; i < e; ++i) cnt += ordered_key(clean(x[i])) == pick.key;
-  s_counts[threadIdx.x] = cnt;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int want = (int)pick.ties, acc = 0, res = -1;
-    for (int th = 0; th < SAMP_THREADS && res < 0; ++th) {
-      if (acc + s_counts[th] >= want) {
-        const int bb = th * chunk, ee = min(V, bb + chunk);
-        for (int i = bb; i < ee; ++i) {
-          if (ordered_key(clean(x[i])) == pick.key && ++acc == want) {
-            res = i;
-            break;
-          }
-        }
+// For a lane's four elements from i on (i a multiple of 4), four such groups 256 elements apart:
+// bit c of mk[u] says that element i + 256 u + c lies before `e` and has the key. The loads of
+// the four groups go out together.
+__device__ __forceinline__ void row_masks(const float* x, int V, bool vec, int e, int i0,
+                                          uint32_t key, int mk[4]) {
+  const int full = vec ? (V & ~3) : 0;      // 16-byte loads stay before this index
+  float4 q[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int i = i0 + 256 * u;
+    q[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (full > 0) q[u] = *reinterpret_cast<const float4*>(x + (i < full && i < e ? i : 0));
+  }
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int i = i0 + 256 * u;
+    int m = 0;
+    if (i < e) {
+      if (i < full) {      // (e is a multiple of 256 or V itself: the four lie before it)
+        m = (int)(ordered_key(clean(q[u].x)) == key) | (int)(ordered_key(clean(q[u].y)) == key) << 1 |
+            (int)(ordered_key(clean(q[u].z)) == key) << 2 | (int)(ordered_key(clean(q[u].w)) == key) << 3;
       } else {
-        acc += s_counts[th];
+        for (int c = 0; c < 4; ++c)
+          if (i + c < e) m |= (int)(ordered_key(clean(x[i + c])) == key) << c;
       }
     }
-    s_res = res < 0 ? 0 : res;
+    mk[u] = m;
+  }
+}
+
+// The index of the pick.ties-th element, by ascending index, whose key equals pick.key. Every
+// wavefront counts the equal keys of a stretch of the row (256 elements a load, so that the
+// lanes read neighbouring addresses; a thread walking a stretch of its own read 64 cache lines
+// an instruction: 140 us for a row of 152,064); the wavefront in whose stretch the wanted one
+// lies walks it again and finds it through the lanes' counts.
+__device__ int pick_index_row(const float* x, int V, Cut pick, int* s_counts) {
+  __shared__ int s_res;
+  constexpr int WAVES = SAMP_THREADS / HE_WAVE;
+  const int lane = threadIdx.x & (HE_WAVE - 1), wave = threadIdx.x >> 6;
+  const bool vec = (((uintptr_t)x) & 15) == 0;
+  const int stretch = ((V + WAVES - 1) / WAVES + 255) & ~255;
+  const int b = min(V, wave * stretch), e = min(V, b + stretch);
+  int cnt = 0;
+  for (int i0 = b + 4 * lane; i0 < e; i0 += 1024) {
+    int mk[4];
+    row_masks(x, V, vec, e, i0, pick.key, mk);
+    cnt += __builtin_popcount(mk[0]) + __builtin_popcount(mk[1]) + __builtin_popcount(mk[2]) +
+           __builtin_popcount(mk[3]);
+  }
+#pragma unroll
+  for (int off = HE_WAVE / 2; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off, HE_WAVE);
+  __syncthreads();
+  if (lane == 0) s_counts[wave] = cnt;
+  if (threadIdx.x == 0) s_res = 0;              // fewer equal keys than the rank: index 0
+  __syncthreads();
+  int want = (int)pick.ties, holder = -1;
+  for (int w = 0; w < WAVES && holder < 0; ++w) {
+    if (want <= s_counts[w]) holder = w;
+    else want -= s_counts[w];
+  }
+  if (wave == holder) {
+    const unsigned long long below = (1ull << lane) - 1ull;
+    int passed = 0;
+    bool found = false;
+    for (int i0 = b + 4 * lane; i0 - 4 * lane < e && !found; i0 += 1024) {   // (the same turns in every lane)
+      int mk[4];
+      row_masks(x, V, vec, e, i0, pick.key, mk);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (found) continue;
+        const int c = __builtin_popcount(mk[u]);
+        int before = 0, total = 0;
+#pragma unroll
+        for (int bit = 0; bit < 3; ++bit) {       // a lane has at most 4
+          const unsigned long long with = __builtin_amdgcn_ballot_w64((c >> bit) & 1);
+          before += __builtin_popcountll(with & below) << bit;
+          total += __builtin_popcountll(with) << bit;
+        }
+        if (passed + total >= want) {
+          const int rank = want - passed - before;      // among this lane's: 1 .. c if it is here
+          if (rank >= 1 && rank <= c) {
+            int m = mk[u];
+            for (int k = 1; k < rank; ++k) m &= m - 1;
+            s_res = i0 + 256 * u + __builtin_ctz(m);
+          }
+          found = true;
+        }
+        passed += total;
+      }
+    }
   }
   __syncthreads();
   return s_res;
@@ -622,13 +710,12 @@ __device__ bool choose_few(const Source& src, float m, float inv_temp, int top_k
   __syncthreads();
   if (threadIdx.x == 0) sh.few = 0;
   __syncthreads();
-  for (int i = threadIdx.x; i < src.n; i += SAMP_THREADS) {
-    if (!src.valid(i)) continue;
-    const uint32_t k = ordered_key(src.value(i));
-    if (k < cut.key) continue;
+  src.for_each([&](float v, int index) {
+    const uint32_t k = ordered_key(v);
+    if (k < cut.key) return;
     const int at = atomicAdd(&sh.few, 1);
-    if (at < HE_WAVE) sh.hist[at] = ((u64)k << 32) | (u64)(0xffffffffu - (uint32_t)src.index(i));
-  }
+    if (at < HE_WAVE) sh.hist[at] = ((u64)k << 32) | (u64)(0xffffffffu - (uint32_t)index);
+  });
   __syncthreads();
   const int n = sh.few;
   if (n > HE_WAVE) return false;
